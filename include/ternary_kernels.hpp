@@ -1,0 +1,75 @@
+// Drop-in C++ operator interface over the C ABI (include/tllm_ternary.h).
+//
+// Re-declares the four ternary operators of the reference's `namespace ternary`
+// (include/kernels.cuh:11-40) with the same names, argument order and default stream,
+// so the call expressions in src/transformer.cpp:107-116, 132-142, 201-217, 266-278
+// compile unchanged against this header. `half` is HIP's __half (hip/hip_fp16.h) and the
+// stream is a hipStream_t. Like the reference these return void; a rejected call is
+// reported through the optional handler below instead of being silently dropped.
+#pragma once
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime_api.h>
+
+#include <cstdint>
+#include <cstdio>
+
+#include "tllm_ternary.h"
+
+namespace ternary {
+
+using error_handler_t = void (*)(const char *op, int code);
+
+inline void default_error_handler(const char *op, int code) {
+    std::fprintf(stderr, "[ternary] %s rejected: %s (%d)\n", op, tllm_error_string(code), code);
+}
+
+inline error_handler_t &error_handler() {
+    static error_handler_t h = default_error_handler;
+    return h;
+}
+
+inline void report(const char *op, int code) {
+    if (code != 0 && error_handler()) error_handler()(op, code);
+}
+
+// Reference include/kernels.cuh:11-14.
+inline void ternary_gemv(const uint32_t *nonzero_masks, const uint32_t *sign_masks,
+                         const half *scales, const half *input, half *output, int rows, int cols,
+                         int group_size, hipStream_t stream = 0) {
+    report("ternary_gemv",
+           tllm_ternary_gemv_f16(nonzero_masks, sign_masks,
+                                 reinterpret_cast<const uint16_t *>(scales),
+                                 reinterpret_cast<const uint16_t *>(input),
+                                 reinterpret_cast<uint16_t *>(output), rows, cols, group_size, stream));
+}
+
+// Reference include/kernels.cuh:19-24.
+inline void ternary_gemv_int8(const uint32_t *nonzero_masks, const uint32_t *sign_masks,
+                              const half *weight_scales, const int8_t *input_int8,
+                              float input_scale, half *output, int rows, int cols, int group_size,
+                              hipStream_t stream = 0) {
+    report("ternary_gemv_int8",
+           tllm_ternary_gemv_i8(nonzero_masks, sign_masks,
+                                reinterpret_cast<const uint16_t *>(weight_scales), input_int8,
+                                input_scale, reinterpret_cast<uint16_t *>(output), rows, cols,
+                                group_size, stream));
+}
+
+// Reference include/kernels.cuh:30-32.
+inline void quantize_absmax_int8(const half *input, int8_t *output, float *scale, int n,
+                                 hipStream_t stream = 0) {
+    report("quantize_absmax_int8",
+           tllm_quantize_absmax_i8(reinterpret_cast<const uint16_t *>(input), output, scale, n, stream));
+}
+
+// Reference include/kernels.cuh:37-40.
+inline void ternary_gemm(const half *A, const uint32_t *nz_B, const uint32_t *sign_B,
+                         const half *scales_B, half *C, int M, int N, int K, int group_size,
+                         hipStream_t stream = 0) {
+    report("ternary_gemm",
+           tllm_ternary_gemm_f16(reinterpret_cast<const uint16_t *>(A), nz_B, sign_B,
+                                 reinterpret_cast<const uint16_t *>(scales_B),
+                                 reinterpret_cast<uint16_t *>(C), M, N, K, group_size, stream));
+}
+
+}  // namespace ternary

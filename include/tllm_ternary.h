@@ -1,0 +1,132 @@
+/*
+ * C ABI of the MI355X ternary linear-layer operators.
+ *
+ * Weight layout (the .tllm dual-bitmask layout, reference include/model.h:17-36):
+ *   nonzero_masks  uint32 [rows, cols/32]   bit b of word j of row r <-> w[r, 32*j+b] != 0
+ *   sign_masks     uint32 [rows, cols/32]   same position, 1 <-> w > 0; ignored where nz bit is 0
+ *   scales         fp16   [rows, cols/group_size], one per `group_size` consecutive columns
+ * fp16 values cross this boundary as IEEE binary16 bit patterns (uint16_t).
+ * Every pointer is a borrowed DEVICE pointer unless said otherwise; the three weight
+ * arrays may live in separate allocations. Calls are asynchronous on `stream`.
+ *
+ * Return value: 0 on success; a negative TLLM_ERR_* code when the arguments are
+ * rejected before anything is launched; a positive value is a hipError_t from the
+ * launch. (The reference operators return void and check nothing; this is a strict
+ * superset. Unlike the reference, cols % group_size != 0 is rejected, not truncated.)
+ */
+#ifndef TLLM_TERNARY_H
+#define TLLM_TERNARY_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *tllm_stream_t; /* a hipStream_t; NULL is the default stream */
+
+enum {
+    TLLM_OK = 0,
+    TLLM_ERR_NULL_POINTER = -1, /* a required pointer is NULL */
+    TLLM_ERR_BAD_SHAPE = -2,    /* rows/cols/M/N/K/n < 1, or cols % 32 != 0 */
+    TLLM_ERR_BAD_GROUP = -3,    /* group_size < 32, group_size % 32 != 0 or cols % group_size != 0 */
+    TLLM_ERR_TOO_LARGE = -4,    /* an element count does not fit the index type, or exceeds a stated limit */
+    TLLM_ERR_ALIAS = -5,        /* output overlaps the activation input */
+    TLLM_ERR_BAD_PLAN = -6,     /* plan handle is NULL, or count < 1, or batch out of range */
+    TLLM_ERR_MISALIGNED = -7    /* masks/activations not 16-byte aligned, scales/outputs not 2-byte aligned */
+};
+
+/* Human-readable text for a negative TLLM_ERR_* code (host pointer, static storage). */
+const char *tllm_error_string(int code);
+
+/* ABI revision of this header. */
+int tllm_abi_version(void);
+
+/*
+ * y[r] = fp16( sum_g float(scales[r,g]) * sum_{k in g} w[r,k] * float(input[k]) ),  fp32 accumulation.
+ * Replaces ternary::ternary_gemv, reference include/kernels.cuh:11-14
+ * (kernels/ternary_gemv.cu:27-100). input fp16 [cols], output fp16 [rows].
+ */
+int tllm_ternary_gemv_f16(const uint32_t *nonzero_masks, const uint32_t *sign_masks,
+                          const uint16_t *scales, const uint16_t *input, uint16_t *output,
+                          int rows, int cols, int group_size, tllm_stream_t stream);
+
+/*
+ * y[r] = fp16( input_scale * sum_g float(weight_scales[r,g]) * float(sum_{k in g} w[r,k] * input_int8[k]) ).
+ * Replaces ternary::ternary_gemv_int8, reference include/kernels.cuh:19-24
+ * (kernels/ternary_gemv.cu:116-216). `input_scale` is passed by value from the host,
+ * as the reference does.
+ */
+int tllm_ternary_gemv_i8(const uint32_t *nonzero_masks, const uint32_t *sign_masks,
+                         const uint16_t *weight_scales, const int8_t *input_int8,
+                         float input_scale, uint16_t *output, int rows, int cols, int group_size,
+                         tllm_stream_t stream);
+
+/*
+ * Same as tllm_ternary_gemv_i8 but reads the activation scale from DEVICE memory
+ * (the float written by tllm_quantize_absmax_i8), so a decode step needs no
+ * device-to-host copy between the two calls. No counterpart in the reference, which
+ * copies the scale to the host first (src/transformer.cpp:134-142).
+ */
+int tllm_ternary_gemv_i8_dscale(const uint32_t *nonzero_masks, const uint32_t *sign_masks,
+                                const uint16_t *weight_scales, const int8_t *input_int8,
+                                const float *input_scale_device, uint16_t *output, int rows,
+                                int cols, int group_size, tllm_stream_t stream);
+
+/*
+ * absmax = max|input|; *scale = absmax > 0 ? absmax/127 : 1;
+ * output[i] = clamp(rint(input[i] * (127/absmax)), -127, 127)  (0 when absmax is 0).
+ * Replaces ternary::quantize_absmax_int8, reference include/kernels.cuh:30-32
+ * (kernels/activations.cu:88-151). `scale` is a device pointer to one float.
+ */
+int tllm_quantize_absmax_i8(const uint16_t *input, int8_t *output, float *scale, int n,
+                            tllm_stream_t stream);
+
+/*
+ * C[m,n] = fp16( sum_k float(scales_B[n, k/group]) * w[n,k] * float(A[m,k]) ),  fp32 accumulation.
+ * A fp16 [M,K] row-major, packed weight [N,K], C fp16 [M,N] row-major.
+ * Replaces ternary::ternary_gemm, reference include/kernels.cuh:37-40
+ * (kernels/ternary_gemm.cu:33-195). Any M >= 1 is accepted.
+ */
+int tllm_ternary_gemm_f16(const uint16_t *A, const uint32_t *nz_B, const uint32_t *sign_B,
+                          const uint16_t *scales_B, uint16_t *C, int M, int N, int K,
+                          int group_size, tllm_stream_t stream);
+
+/*
+ * Several independent ternary linears in ONE launch (e.g. q/k/v, gate/up, or a whole
+ * back-to-back projection sweep). Each problem is what one tllm_ternary_gemv_f16 /
+ * small-M tllm_ternary_gemm_f16 call would take: input fp16 [batch, cols],
+ * output fp16 [batch, rows]. The reference issues these as separate launches
+ * (src/transformer.cpp:206-217, 266-278).
+ */
+typedef struct tllm_linear_problem {
+    const uint32_t *nonzero_masks;
+    const uint32_t *sign_masks;
+    const uint16_t *scales;
+    const uint16_t *input;
+    uint16_t *output;
+    int32_t rows;
+    int32_t cols;
+    int32_t batch; /* 1..TLLM_MAX_PLAN_BATCH */
+    int32_t reserved;
+} tllm_linear_problem;
+
+enum { TLLM_MAX_PLAN_BATCH = 4 };
+
+typedef struct tllm_linear_plan tllm_linear_plan;
+
+/* Validates and copies `problems` (HOST array) into a device-resident schedule.
+ * Allocates device memory; not for the per-token path. group_size must be 128. */
+int tllm_linear_plan_create(tllm_linear_plan **plan, const tllm_linear_problem *problems,
+                            int count, int group_size);
+/* One launch over every problem of the plan. Allocation-free. */
+int tllm_linear_plan_launch(const tllm_linear_plan *plan, tllm_stream_t stream);
+/* Algorithmic weight-stream bytes (masks + scales) one launch reads. */
+int64_t tllm_linear_plan_weight_bytes(const tllm_linear_plan *plan);
+void tllm_linear_plan_destroy(tllm_linear_plan *plan);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TLLM_TERNARY_H */

@@ -1,0 +1,13 @@
+"""MI355X ternary linear-layer operators: a thin Python binding over the C-ABI library
+`lib/libtllm_ternary.so` (hand-written HIP, gfx950). There is no CPU or PyTorch fallback:
+every operator raises if the library is missing or a call is rejected."""
+from .ops import (  # noqa: F401
+    LinearPlan,
+    TllmError,
+    lib,
+    lib_path,
+    quantize_absmax_int8,
+    ternary_gemm,
+    ternary_gemv,
+    ternary_gemv_int8,
+)

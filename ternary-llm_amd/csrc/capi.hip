@@ -1,0 +1,165 @@
+// The C ABI: argument validation and dispatch. No kernel code lives here.
+#include <new>
+#include <vector>
+
+#include "common.h"
+
+namespace tllm {
+namespace {
+
+inline bool misaligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }
+
+inline bool overlaps(const void *a, size_t na, const void *b, size_t nb) {
+    const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), b0 = reinterpret_cast<uintptr_t>(b);
+    return a0 < b0 + nb && b0 < a0 + na;
+}
+
+// Checks shared by every operator over a packed rows x cols weight.
+int check_weight(const void *nz, const void *sg, const void *scales, int rows, int cols, int group) {
+    if (!nz || !sg || !scales) return TLLM_ERR_NULL_POINTER;
+    if (rows < 1 || cols < 1 || cols % 32 != 0) return TLLM_ERR_BAD_SHAPE;
+    if (group < 32 || group % 32 != 0 || cols % group != 0) return TLLM_ERR_BAD_GROUP;
+    if (misaligned(nz, 16) || misaligned(sg, 16) || misaligned(scales, 2)) return TLLM_ERR_MISALIGNED;
+    return TLLM_OK;
+}
+
+int check_linear(const Problem &p, int group) {
+    if (int e = check_weight(p.nz, p.sg, p.scales, p.rows, p.cols, group)) return e;
+    if (!p.x || !p.y) return TLLM_ERR_NULL_POINTER;
+    if (p.batch < 1) return TLLM_ERR_BAD_SHAPE;
+    if (misaligned(p.x, 16) || misaligned(p.y, 2)) return TLLM_ERR_MISALIGNED;
+    if ((int64_t)p.batch * p.cols > INT32_MAX || (int64_t)p.batch * p.rows > INT32_MAX)
+        return TLLM_ERR_TOO_LARGE;
+    if (overlaps(p.x, (size_t)p.batch * p.cols * 2, p.y, (size_t)p.batch * p.rows * 2))
+        return TLLM_ERR_ALIAS;
+    return TLLM_OK;
+}
+
+int run_linear(const Problem &p, int group, hipStream_t s) {
+    if (int e = check_linear(p, group)) return e;
+    return (int)dispatch_linear(p, group, s);
+}
+
+}  // namespace
+}  // namespace tllm
+
+using tllm::Problem;
+
+struct tllm_linear_plan {
+    std::vector<Problem> host;
+    tllm::PlanDevice dev;
+    int group;
+    int64_t weight_bytes;
+};
+
+extern "C" {
+
+const char *tllm_error_string(int code) {
+    switch (code) {
+        case TLLM_OK: return "ok";
+        case TLLM_ERR_NULL_POINTER: return "a required pointer is NULL";
+        case TLLM_ERR_BAD_SHAPE: return "bad shape: sizes must be >= 1 and cols a multiple of 32";
+        case TLLM_ERR_BAD_GROUP: return "bad group_size: must be a multiple of 32 that divides cols";
+        case TLLM_ERR_TOO_LARGE: return "size exceeds the supported maximum";
+        case TLLM_ERR_ALIAS: return "output overlaps the activation input";
+        case TLLM_ERR_BAD_PLAN: return "invalid plan, problem count or batch";
+        case TLLM_ERR_MISALIGNED: return "pointer alignment: masks/activations need 16 bytes, fp16 arrays 2";
+        default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error code";
+    }
+}
+
+int tllm_abi_version(void) { return 1; }
+
+int tllm_ternary_gemv_f16(const uint32_t *nonzero_masks, const uint32_t *sign_masks,
+                          const uint16_t *scales, const uint16_t *input, uint16_t *output,
+                          int rows, int cols, int group_size, tllm_stream_t stream) {
+    Problem p{nonzero_masks, sign_masks, scales, input, output, rows, cols, 1, 0};
+    return tllm::run_linear(p, group_size, (hipStream_t)stream);
+}
+
+int tllm_ternary_gemm_f16(const uint16_t *A, const uint32_t *nz_B, const uint32_t *sign_B,
+                          const uint16_t *scales_B, uint16_t *C, int M, int N, int K,
+                          int group_size, tllm_stream_t stream) {
+    if (M < 1) return TLLM_ERR_BAD_SHAPE;
+    Problem p{nz_B, sign_B, scales_B, A, C, N, K, M, 0};
+    return tllm::run_linear(p, group_size, (hipStream_t)stream);
+}
+
+static int gemv_i8_common(const uint32_t *nz, const uint32_t *sg, const uint16_t *scales,
+                          const int8_t *xq, float scale_value, const float *scale_dev,
+                          uint16_t *y, int rows, int cols, int group, tllm_stream_t stream) {
+    if (int e = tllm::check_weight(nz, sg, scales, rows, cols, group)) return e;
+    if (!xq || !y) return TLLM_ERR_NULL_POINTER;
+    if (tllm::misaligned(xq, 16) || tllm::misaligned(y, 2)) return TLLM_ERR_MISALIGNED;
+    if (tllm::overlaps(xq, (size_t)cols, y, (size_t)rows * 2)) return TLLM_ERR_ALIAS;
+    return (int)tllm::launch_gemv_rowwave_i8(nz, sg, scales, xq, scale_value, scale_dev, y, rows,
+                                             cols, group, (hipStream_t)stream);
+}
+
+int tllm_ternary_gemv_i8(const uint32_t *nonzero_masks, const uint32_t *sign_masks,
+                         const uint16_t *weight_scales, const int8_t *input_int8,
+                         float input_scale, uint16_t *output, int rows, int cols, int group_size,
+                         tllm_stream_t stream) {
+    return gemv_i8_common(nonzero_masks, sign_masks, weight_scales, input_int8, input_scale,
+                          nullptr, output, rows, cols, group_size, stream);
+}
+
+int tllm_ternary_gemv_i8_dscale(const uint32_t *nonzero_masks, const uint32_t *sign_masks,
+                                const uint16_t *weight_scales, const int8_t *input_int8,
+                                const float *input_scale_device, uint16_t *output, int rows,
+                                int cols, int group_size, tllm_stream_t stream) {
+    if (!input_scale_device) return TLLM_ERR_NULL_POINTER;
+    return gemv_i8_common(nonzero_masks, sign_masks, weight_scales, input_int8, 0.0f,
+                          input_scale_device, output, rows, cols, group_size, stream);
+}
+
+int tllm_quantize_absmax_i8(const uint16_t *input, int8_t *output, float *scale, int n,
+                            tllm_stream_t stream) {
+    if (!input || !output || !scale) return TLLM_ERR_NULL_POINTER;
+    if (n < 1) return TLLM_ERR_BAD_SHAPE;
+    if (tllm::misaligned(input, 2) || tllm::misaligned(scale, 4)) return TLLM_ERR_MISALIGNED;
+    return (int)tllm::launch_quantize_absmax_i8(input, output, scale, n, (hipStream_t)stream);
+}
+
+int tllm_linear_plan_create(tllm_linear_plan **plan, const tllm_linear_problem *problems,
+                            int count, int group_size) {
+    if (!plan || !problems) return TLLM_ERR_NULL_POINTER;
+    *plan = nullptr;
+    if (count < 1) return TLLM_ERR_BAD_PLAN;
+    if (group_size != 128) return TLLM_ERR_BAD_GROUP;
+    std::vector<Problem> host(count);
+    int64_t bytes = 0;
+    for (int i = 0; i < count; i++) {
+        const tllm_linear_problem &q = problems[i];
+        host[i] = Problem{q.nonzero_masks, q.sign_masks, q.scales, q.input, q.output,
+                          q.rows, q.cols, q.batch, 0};
+        if (q.batch < 1 || q.batch > TLLM_MAX_PLAN_BATCH) return TLLM_ERR_BAD_PLAN;
+        if (int e = tllm::check_linear(host[i], group_size)) return e;
+        bytes += (int64_t)q.rows * (q.cols / 32) * 8 + (int64_t)q.rows * (q.cols / group_size) * 2;
+    }
+    tllm_linear_plan *pl = new (std::nothrow) tllm_linear_plan{std::move(host), {}, group_size, bytes};
+    if (!pl) return TLLM_ERR_TOO_LARGE;
+    if (hipError_t e = tllm::plan_device_create(pl->host, &pl->dev)) {
+        delete pl;
+        return (int)e;
+    }
+    *plan = pl;
+    return TLLM_OK;
+}
+
+int tllm_linear_plan_launch(const tllm_linear_plan *plan, tllm_stream_t stream) {
+    if (!plan || plan->host.empty()) return TLLM_ERR_BAD_PLAN;
+    return (int)tllm::plan_device_launch(plan->dev, (hipStream_t)stream);
+}
+
+int64_t tllm_linear_plan_weight_bytes(const tllm_linear_plan *plan) {
+    return plan ? plan->weight_bytes : 0;
+}
+
+void tllm_linear_plan_destroy(tllm_linear_plan *plan) {
+    if (!plan) return;
+    tllm::plan_device_destroy(&plan->dev);
+    delete plan;
+}
+
+}  // extern "C"

@@ -1,0 +1,67 @@
+// Shared declarations of the ternary linear-layer library (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <vector>
+
+#include "../../include/tllm_ternary.h"
+
+namespace tllm {
+
+constexpr int kWave = 64;
+
+// One ternary linear: y[batch, rows] = x[batch, cols] * W^T with W packed as two bit planes.
+struct Problem {
+    const uint32_t *nz;
+    const uint32_t *sg;
+    const uint16_t *scales;
+    const uint16_t *x;
+    uint16_t *y;
+    int32_t rows;
+    int32_t cols;
+    int32_t batch;
+    int32_t reserved;
+};
+static_assert(sizeof(Problem) == sizeof(tllm_linear_problem), "ABI struct mirrors Problem");
+
+__device__ __forceinline__ float h2f(uint16_t bits) {
+    return (float)__builtin_bit_cast(_Float16, bits);
+}
+__device__ __forceinline__ uint16_t f2h(float v) {  // round to nearest even
+    return __builtin_bit_cast(uint16_t, (_Float16)v);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+// ---- launchers implemented in the kernel files; all return a hipError_t ----
+// General fallback (any group size that is a multiple of 32): one wave per output row.
+hipError_t launch_gemv_rowwave_f16(const Problem &p, int group, hipStream_t s);
+hipError_t launch_gemv_rowwave_f16_table(const Problem *table, int count, int max_rows,
+                                         int max_batch, int group, hipStream_t s);
+hipError_t launch_gemv_rowwave_i8(const uint32_t *nz, const uint32_t *sg, const uint16_t *scales,
+                                  const int8_t *xq, float scale_value, const float *scale_dev,
+                                  uint16_t *y, int rows, int cols, int group, hipStream_t s);
+hipError_t launch_quantize_absmax_i8(const uint16_t *x, int8_t *q, float *scale, int n,
+                                     hipStream_t s);
+
+// Picks the kernel for one linear (fast 128-group paths when they apply, else the row-wave kernel).
+hipError_t dispatch_linear(const Problem &p, int group, hipStream_t s);
+
+// Device-resident schedule of a multi-problem launch.
+struct PlanDevice {
+    Problem *problems = nullptr;  // device copy of the table
+    int count = 0;
+    int device = -1;
+    int max_rows = 0;
+    int max_batch = 0;
+};
+hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out);
+hipError_t plan_device_launch(const PlanDevice &plan, hipStream_t s);
+void plan_device_destroy(PlanDevice *plan);
+
+}  // namespace tllm

@@ -1,0 +1,42 @@
+// Compile-and-run check of the C++ drop-in interface: the call expressions below have
+// the shapes of the reference's callers (src/transformer.cpp:107-116 ternary_linear,
+// :132-142 ternary_linear_int8). With null pointers every call must be rejected by the
+// argument validation before any GPU work, so this runs on a host without a GPU.
+#include <cstdio>
+#include <cstdlib>
+
+#include "ternary_kernels.hpp"
+
+struct TernaryWeight {  // same fields as the reference's include/model.h:17-23
+    uint32_t *nonzero_masks = nullptr;
+    uint32_t *sign_masks = nullptr;
+    half *scales = nullptr;
+    int out_features = 0;
+    int in_features = 0;
+};
+
+static int rejected = 0;
+static void count_handler(const char *, int code) { rejected += code < 0; }
+
+int main() {
+    ternary::error_handler() = count_handler;
+    TernaryWeight w;
+    w.out_features = 2048;
+    w.in_features = 2048;
+    const half *input = nullptr;
+    half *output = nullptr;
+    int8_t *int8_buf_ = nullptr;
+    float *int8_scale_ = nullptr;
+    int gs = 128, n_tokens = 7, dim = 2048;
+    float h_scale = 0.5f;
+
+    ternary::ternary_gemv(w.nonzero_masks, w.sign_masks, w.scales, input, output, w.out_features,
+                          w.in_features, gs);
+    ternary::ternary_gemm(input, w.nonzero_masks, w.sign_masks, w.scales, output, n_tokens,
+                          w.out_features, w.in_features, gs);
+    ternary::quantize_absmax_int8(input, int8_buf_, int8_scale_, dim);
+    ternary::ternary_gemv_int8(w.nonzero_masks, w.sign_masks, w.scales, int8_buf_, h_scale, output,
+                               w.out_features, w.in_features, gs);
+    std::printf("rejected=%d\n", rejected);
+    return rejected == 4 ? 0 : 1;
+}

@@ -1,0 +1,74 @@
+"""Host-only checks of the drop-in boundary: every symbol include/tllm_ternary.h declares
+is exported, the argument validation rejects bad calls without touching a GPU, and the
+C++ interface compiles for the reference's call shapes."""
+import ctypes as C
+import os
+import re
+import subprocess
+
+import pytest
+
+import ternary_llm_amd as tl
+from ternary_llm_amd import ops
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_header_symbols_exported():
+    text = open(os.path.join(ROOT, "include", "tllm_ternary.h")).read()
+    declared = set(re.findall(r"\b(tllm_[a-z0-9_]+)\s*\(", text))
+    assert declared == set(ops.ABI_SYMBOLS)
+    L = tl.lib()
+    for name in declared:
+        assert hasattr(L, name), name
+    assert L.tllm_abi_version() == 1
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(ops, "_lib", None)
+    monkeypatch.setattr(ops, "_LIB_PATH", "/nonexistent/libtllm_ternary.so")
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops.lib()
+
+
+def _gemv(L, nz=0x1000, sg=0x2000, sc=0x3000, x=0x4000, y=0x5000, rows=4, cols=256, g=128):
+    return L.tllm_ternary_gemv_f16(nz, sg, sc, x, y, rows, cols, g, None)
+
+
+def test_validation_codes():
+    L = tl.lib()
+    assert _gemv(L, nz=None) == -1 and _gemv(L, y=None) == -1
+    assert _gemv(L, rows=0) == -2 and _gemv(L, cols=0) == -2 and _gemv(L, cols=250) == -2
+    assert _gemv(L, g=0) == -3 and _gemv(L, g=48) == -3
+    assert _gemv(L, cols=160, g=128) == -3          # cols % group != 0: rejected, not truncated
+    assert _gemv(L, x=0x4000, y=0x4010) == -5       # output inside the input
+    assert _gemv(L, nz=0x1004) == -7 and _gemv(L, x=0x4002) == -7 and _gemv(L, y=0x5001) == -7
+    assert L.tllm_ternary_gemm_f16(0x4000, 0x1000, 0x2000, 0x3000, 0x9000, 0, 4, 256, 128, None) == -2
+    assert L.tllm_quantize_absmax_i8(None, 0x10, 0x20, 4, None) == -1
+    assert L.tllm_quantize_absmax_i8(0x10, 0x20, 0x40, 0, None) == -2
+    assert L.tllm_ternary_gemv_i8(0x1000, 0x2000, 0x3000, None, 1.0, 0x5000, 4, 256, 128, None) == -1
+    assert L.tllm_ternary_gemv_i8_dscale(0x1000, 0x2000, 0x3000, 0x4000, None, 0x5000, 4, 256, 128, None) == -1
+    h = C.c_void_p(0)
+    assert L.tllm_linear_plan_create(C.byref(h), None, 1, 128) == -1
+    arr = (ops._Problem * 1)(ops._Problem(0x1000, 0x2000, 0x3000, 0x4000, 0x9000, 4, 256, 9, 0))
+    assert L.tllm_linear_plan_create(C.byref(h), arr, 1, 128) == -6   # batch > TLLM_MAX_PLAN_BATCH
+    assert L.tllm_linear_plan_create(C.byref(h), arr, 0, 128) == -6
+    assert L.tllm_linear_plan_create(C.byref(h), arr, 1, 64) == -3
+    assert L.tllm_linear_plan_launch(None, None) == -6
+    for code in range(-7, 1):
+        assert L.tllm_error_string(code)
+    with pytest.raises(tl.TllmError):
+        ops.check(-2)
+
+
+def test_cpp_dropin_call_shapes(tmp_path):
+    exe = tmp_path / "dropin_calls"
+    libdir = os.path.dirname(tl.lib_path())
+    # a plain host C++ translation unit, as the reference's src/transformer.cpp is
+    cmd = ["g++", "-std=c++17", "-D__HIP_PLATFORM_AMD__", "-I", "/opt/rocm/include",
+           "-I", os.path.join(ROOT, "include"), os.path.join(ROOT, "tests", "dropin_calls.cpp"),
+           "-L", libdir, "-ltllm_ternary", f"-Wl,-rpath,{libdir}", "-o", str(exe)]
+    subprocess.run(cmd, check=True, capture_output=True, text=True)
+    out = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert "rejected=4" in out.stdout

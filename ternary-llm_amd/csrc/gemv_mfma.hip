@@ -40,6 +40,16 @@ struct Tile {
     uint16_t sc[4];
 };
 
+// Weight streams are read through global-address-space pointers (pointers fetched from the
+// problem table would otherwise be treated as generic and use slower flat loads).
+typedef __attribute__((address_space(1))) const uint32_t GU32;
+typedef __attribute__((address_space(1))) const uint16_t GU16;
+typedef __attribute__((address_space(1))) const u4 GU4;
+template <class T>
+__device__ __forceinline__ __attribute__((address_space(1))) const T *as_global(const T *p) {
+    return (__attribute__((address_space(1))) const T *)p;
+}
+
 __device__ __forceinline__ float dpp_quad(float v, int ctrl_b1_or_4e) {
     // quad_perm swaps inside groups of 4 lanes; 0xB1 = [1,0,3,2], 0x4E = [2,3,0,1]
     int r = ctrl_b1_or_4e == 0xB1
@@ -165,85 +175,100 @@ __global__ __launch_bounds__(kThreads, 2) void gemv_mfma_kernel(Problem single, 
         const int bcol = li >> 2;               // batch column of this lane's D column
         const bool b_active = (li & 3) == lq && bcol < p.batch;
         float *my_part = partial + (size_t)wave * sc.range_rows * p.batch;
+        const bool part_lane = (li & 3) == 0 && bcol < p.batch;
 
-        bool first_slice = true;
-        for (int slice = wave; slice < slices; slice += kNW) {
-            // B operands of this slice (zero outside the lane's own group / batch column)
-            u4 B[kMfmaPerSlice];
-            {
+        // This wave's tiles: its slices (wave, wave + kNW, ...) times the 16-row blocks of the range,
+        // slice-major. Tile loads are issued three tiles ahead and never branch, so the hardware
+        // counters let two tiles stay in flight while one is being consumed.
+        const int n_rb = (nrows + kIterRows - 1) / kIterRows;
+        const int n_sl = slices > wave ? (slices - wave + kNW - 1) / kNW : 0;
+        const int n_tiles = n_sl * n_rb;
+        const GU32 *nz_g = as_global(p.nz);
+        const GU32 *sg_g = as_global(p.sg);
+        const GU16 *sc_g = as_global(p.scales);
+
+        // Groups past the end of a row (last slice when cols % 512 != 0) are read from the row's last
+        // group instead: their activations in the image are zero, so they add nothing.
+        auto load_tile = [&](int slice, int rb) -> Tile {
+            Tile t;
+            const int ga = min(4 * slice + lq, groups - 1);
+            const int gs = min(4 * slice + (li & 3), groups - 1);
+            const int ra = min(rb + li, p.rows - 1);
+            const size_t off = (size_t)ra * words + 4 * ga;
+            t.nz = *reinterpret_cast<const GU4 *>(nz_g + off);
+            t.sg = *reinterpret_cast<const GU4 *>(sg_g + off);
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int rs = min(rb + 4 * lq + v, p.rows - 1);
+                t.sc[v] = sc_g[(size_t)rs * groups + gs];
+            }
+            return t;
+        };
+
+        u4 B[kMfmaPerSlice];
+        f4 bias = {0.f, 0.f, 0.f, 0.f};
+        const u4 zero4 = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int t = 0; t < kMfmaPerSlice; t++) B[t] = zero4;
+
+        auto process = [&](const Tile &t, int slice, int rb) {
+            if (rb == r_begin) {
+                // new slice: its activations become the B operands (zero outside the lane's own
+                // group / batch column), and an all-zero weight row gives the "+1" term of the code
                 const u4 *src = reinterpret_cast<const u4 *>(image + (size_t)bcol * img_stride +
                                                              slice * kSliceCols) + lq;
+                if (b_active) {
 #pragma unroll
-                for (int t = 0; t < kMfmaPerSlice; t++) {
-                    u4 v = {0u, 0u, 0u, 0u};
-                    if (b_active) v = src[t * 4];
-                    B[t] = v;
+                    for (int k = 0; k < kMfmaPerSlice; k++) B[k] = src[k * 4];
                 }
+                bias = slice_product(zero4, zero4, B);
             }
-            // what an all-zero weight row yields; subtracting it removes the "+1" of the code
-            const u4 zero4 = {0u, 0u, 0u, 0u};
-            const f4 bias = slice_product(zero4, zero4, B);
-
-            // per-lane addressing
-            const int ga = 4 * slice + lq;        // group whose 128 weights this lane loads
-            const bool a_valid = ga < groups;
-            const int gs = 4 * slice + (li & 3);  // group whose scale this lane applies
-            const bool s_valid = gs < groups;
-            const size_t a_off = (size_t)slice * kSliceWords + 4 * lq;
-
-            auto load_tile = [&](int rb) -> Tile {
-                Tile t;
-                const int ra = min(rb + li, p.rows - 1);
-                t.nz = zero4;
-                t.sg = zero4;
-                if (a_valid) {
-                    t.nz = *reinterpret_cast<const u4 *>(p.nz + (size_t)ra * words + a_off);
-                    t.sg = *reinterpret_cast<const u4 *>(p.sg + (size_t)ra * words + a_off);
-                }
+            const f4 d = slice_product(t.nz, t.sg, B);
+            float r[4];
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                float x = h2f(t.sc[v]) * (d[v] - bias[v]);
+                x += dpp_quad(x, 0xB1);
+                x += dpp_quad(x, 0x4E);
+                r[v] = x;
+            }
+            if (part_lane) {
+                const bool first_slice = slice == wave;
 #pragma unroll
                 for (int v = 0; v < 4; v++) {
-                    const int rs = min(rb + 4 * lq + v, p.rows - 1);
-                    t.sc[v] = s_valid ? p.scales[(size_t)rs * groups + gs] : (uint16_t)0;
+                    float *dst = my_part + (size_t)(rb - r_begin + 4 * lq + v) * p.batch + bcol;
+                    *dst = first_slice ? r[v] : *dst + r[v];
                 }
+            }
+        };
+
+        if (n_tiles > 0) {
+            // load cursor (ls, lrb) runs three tiles ahead of the compute cursor (cs, crb)
+            int ls = wave, lrb = r_begin, cs = wave, crb = r_begin;
+            auto advance = [&](int &s_, int &rb_) {
+                rb_ += kIterRows;
+                if (rb_ >= r_end) { rb_ = r_begin; s_ += kNW; }
+            };
+            auto next_load = [&]() -> Tile {
+                // past the last tile the cursor is parked on it (a cached re-read, never out of range)
+                const Tile t = load_tile(ls < slices ? ls : cs, ls < slices ? lrb : crb);
+                if (ls < slices) advance(ls, lrb);
                 return t;
             };
-
-            auto process = [&](const Tile &t, int rb) {
-                const f4 d = slice_product(t.nz, t.sg, B);
-                float r[4];
-#pragma unroll
-                for (int v = 0; v < 4; v++) {
-                    float x = h2f(t.sc[v]) * (d[v] - bias[v]);
-                    x += dpp_quad(x, 0xB1);
-                    x += dpp_quad(x, 0x4E);
-                    r[v] = x;
-                }
-                if ((li & 3) == 0 && bcol < p.batch) {
-#pragma unroll
-                    for (int v = 0; v < 4; v++) {
-                        float *dst = my_part + (size_t)(rb - r_begin + 4 * lq + v) * p.batch + bcol;
-                        *dst = first_slice ? r[v] : *dst + r[v];
-                    }
-                }
-            };
-
-            // three tiles in flight, rotated by hand so no register copies are needed
-            Tile t0 = load_tile(r_begin), t1 = t0, t2 = t0;
-            if (r_begin + 16 < r_end) t1 = load_tile(r_begin + 16);
-            if (r_begin + 32 < r_end) t2 = load_tile(r_begin + 32);
-            for (int rb = r_begin; rb < r_end; rb += 48) {
-                process(t0, rb);
-                if (rb + 48 < r_end) t0 = load_tile(rb + 48);
-                if (rb + 16 < r_end) {
-                    process(t1, rb + 16);
-                    if (rb + 64 < r_end) t1 = load_tile(rb + 64);
-                }
-                if (rb + 32 < r_end) {
-                    process(t2, rb + 32);
-                    if (rb + 80 < r_end) t2 = load_tile(rb + 80);
-                }
+            Tile t0 = next_load(), t1 = next_load(), t2 = next_load();
+            for (int i = 0; i < n_tiles; i += 3) {
+                process(t0, cs, crb);
+                advance(cs, crb);
+                t0 = next_load();
+                if (i + 1 >= n_tiles) break;
+                process(t1, cs, crb);
+                advance(cs, crb);
+                t1 = next_load();
+                if (i + 2 >= n_tiles) break;
+                process(t2, cs, crb);
+                advance(cs, crb);
+                t2 = next_load();
             }
-            first_slice = false;
         }
         __syncthreads();
         // ------------------------------------------------ add the K slices in wave order, store fp16

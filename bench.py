@@ -32,7 +32,12 @@ SHAPES = {
 }
 
 
+CUSTOM = []  # filled by --matrices "ROWSxCOLS,..." (replaces the model's per-layer matrix list)
+
+
 def layer_matrices(model):
+    if CUSTOM:
+        return [(f"m{i}", r, c) for i, (r, c) in enumerate(CUSTOM)]
     h, q, kv, ffn, _ = SHAPES[model]
     return [("q_proj", q, h), ("k_proj", kv, h), ("v_proj", kv, h), ("o_proj", h, q),
             ("gate_proj", ffn, h), ("up_proj", ffn, h), ("down_proj", h, ffn)]
@@ -139,9 +144,13 @@ def main():
     ap.add_argument("--p-zero", type=float, default=0.42)
     ap.add_argument("--mode", default="plan", choices=["plan", "calls"],
                     help="plan: the whole sweep as one launch; calls: one operator call per matrix")
+    ap.add_argument("--matrices", default="", help='per-layer matrix list "ROWSxCOLS,..." instead of the model\'s')
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seed", type=int, default=20240611)
     args = ap.parse_args()
+    for item in filter(None, args.matrices.split(",")):
+        r, c = item.lower().split("x")
+        CUSTOM.append((int(r), int(c)))
     if args.gpus != 1:
         print("bench.py measures ONE GPU: this build has no multi-GPU path (--gpus must be 1).", file=sys.stderr)
         sys.exit(2)

@@ -65,6 +65,7 @@ struct PlanDevice {
     int max_batch = 0;
     // schedule of the MFMA kernel (use_mfma == false: the row-wave table kernel runs instead)
     bool use_mfma = false;
+    bool wide = false;  // 4 x 2048 tiles (every problem at batch 1) instead of 16 x 512
     int *task_prefix = nullptr;
     int *wg_first = nullptr;
     int grid = 0;

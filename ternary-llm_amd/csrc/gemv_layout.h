@@ -19,74 +19,81 @@
 
 namespace tllm {
 
-constexpr int kSliceCols = 512;   // columns whose activations one wave keeps in registers
-constexpr int kSliceWords = kSliceCols / 32;
-constexpr int kIterRows = 16;     // rows one MFMA tile covers
-constexpr int kMfmaPerSlice = 16; // 16 MFMAs of K=32 consume 16 rows x 512 columns
+constexpr int kChunkCols = 128;    // one scale group = the 16 bytes per plane one lane loads
+constexpr int kMfmaPerTile = 16;   // 16 MFMAs of K=32 consume the 64 lanes x 128 weights of a tile
 
-// Bit offset (inside an fp16 half) of the code of field slot m = 0..7. Only offsets >= 4 are used:
-// measured on gfx950, v_mfma_f32_16x16x32_f16 truncates products whose subnormal operand has its
-// significant bits at offsets 0..2 (relative error up to 5e-6 per product at offset 0, 1e-6 at 2),
-// while offsets 4..10 stay below fp32 rounding noise (1e-8). Offset 10 puts the code in the lowest
-// exponent bits: 0x0400 = 2^-14 and 0x0800 = 2^-13 continue the subnormal line c * 2^(10-24).
+// A 32-bit mask word holds 32 weights. Its even-numbered and odd-numbered weights are handled as two
+// "interleaved words" z = 0, 1; inside one, weight number f = 0..15 (bit 2f + z of the mask word)
+// owns the 2-bit field at bits (2f+1, 2f). Eight ANDs per interleaved word cut out eight operand
+// dwords m = 0..7, each holding one field in its low half and one in its high half, at bit offset
+// code_shift(m) inside the half. Fields 0..5 and 9..13 are taken in place; the others come from the
+// word rotated right by 6, which also brings field 0 into the high half and field 8 into the low one.
+//
+// Offsets 0 is never used: measured on gfx950, v_mfma_f32_16x16x32_f16 truncates products whose
+// subnormal operand has its significant bits at offset 0 (relative error up to 5e-6 per product);
+// offset 2 shows about 1e-7 and offsets 4..10 stay below fp32 rounding noise (1e-8). Offset 10 puts
+// the code in the lowest exponent bits: 0x0400 = 2^-14 and 0x0800 = 2^-13 continue the subnormal
+// line c * 2^(10-24).
 TLLM_HD constexpr int code_shift(int m) {
-    return m == 0 ? 4 : m == 1 ? 6 : m == 2 ? 4 : m == 3 ? 6 : m == 4 ? 8 : m == 5 ? 10 : m == 6 ? 6 : 8;
+    return m == 0 ? 10 : m == 1 ? 2 : m == 2 ? 4 : m == 3 ? 6 : m == 4 ? 8 : m == 5 ? 10 : m == 6 ? 6 : 8;
 }
+// Operand dword m and half (0 = low) that carry field f of an interleaved word.
+TLLM_HD constexpr int field_dword(int f) { return f & 7; }
+TLLM_HD constexpr int field_half(int f) { return (f & 7) == 0 ? 1 - (f >> 3) : f >> 3; }
 
-// 32 weights of one row -> 16 operand dwords. out[8*z + m] holds, in its low and high half, the
-// codes of the weights at bit (2*m + z) and bit (16 + 2*m + z) of the word, each shifted left by
-// code_shift(m) inside its half. Sign bits under clear nz bits are ignored (pos = nz & sg).
-// Cost: 7 operations to interleave the planes, 4 shifts and 16 ANDs per 32 weights.
+// 32 weights of one row -> 16 operand dwords out[8*z + m]. Sign bits under clear nz bits are
+// ignored (pos = nz & sg). Cost: 5 operations to interleave the planes, 2 rotates and 16 ANDs.
 TLLM_HD void decode_word(uint32_t nz, uint32_t sg, uint32_t out[16]) {
     const uint32_t pos = nz & sg;
-    const uint32_t nzn = ~nz;
-    // 2-bit code per weight, in place: bit 2i+1 = positive, bit 2i = not non-zero
+    // 2-bit code per weight, in place: bit 2f+1 = positive, bit 2f = not non-zero
     uint32_t q[2];
-    q[0] = ((pos << 1) & 0xAAAAAAAAu) | (nzn & 0x55555555u);  // weights at even bits
-    q[1] = (pos & 0xAAAAAAAAu) | ((nzn >> 1) & 0x55555555u);  // weights at odd bits
 #if defined(__HIP_DEVICE_COMPILE__)
+    // one three-input bit operation each: (a & c) | (~b & ~c), c = 0xAAAAAAAA
+    q[0] = __builtin_amdgcn_bitop3_b32(pos << 1, nz, 0xAAAAAAAAu, 0xB1);
+    q[1] = __builtin_amdgcn_bitop3_b32(pos, nz >> 1, 0xAAAAAAAAu, 0xB1);
     // keep the interleaved words materialised: otherwise the optimiser distributes the field
-    // masks over the OR and spends two operations per operand dword instead of one
+    // masks over them and spends two operations per operand dword instead of one
     asm volatile("" : "+v"(q[0]), "+v"(q[1]));
+#else
+    q[0] = ((pos << 1) & 0xAAAAAAAAu) | (~nz & 0x55555555u);
+    q[1] = (pos & 0xAAAAAAAAu) | (~(nz >> 1) & 0x55555555u);
 #endif
 #pragma unroll
     for (int z = 0; z < 2; z++) {
-        const uint32_t up = q[z] << 4;    // fields 0,1 (and 8,9 in the high half) move to offsets 4,6
-        const uint32_t down = q[z] >> 6;  // fields 6,7 (and 14,15) move to offsets 6,8
-        out[8 * z + 0] = up & 0x00300030u;
-        out[8 * z + 1] = up & 0x00C000C0u;
-        out[8 * z + 2] = q[z] & 0x00300030u;
-        out[8 * z + 3] = q[z] & 0x00C000C0u;
-        out[8 * z + 4] = q[z] & 0x03000300u;
-        out[8 * z + 5] = q[z] & 0x0C000C00u;
-        out[8 * z + 6] = down & 0x00C000C0u;
-        out[8 * z + 7] = down & 0x03000300u;
+        const uint32_t rot = (q[z] >> 6) | (q[z] << 26);
+        out[8 * z + 0] = rot & 0x0C000C00u;   // fields 8 (low half) and 0 (high half)
+        out[8 * z + 1] = q[z] & 0x000C000Cu;  // fields 1, 9
+        out[8 * z + 2] = q[z] & 0x00300030u;  // fields 2, 10
+        out[8 * z + 3] = q[z] & 0x00C000C0u;  // fields 3, 11
+        out[8 * z + 4] = q[z] & 0x03000300u;  // fields 4, 12
+        out[8 * z + 5] = q[z] & 0x0C000C00u;  // fields 5, 13
+        out[8 * z + 6] = rot & 0x00C000C0u;   // fields 6, 14
+        out[8 * z + 7] = rot & 0x03000300u;   // fields 7, 15
     }
 }
 
-// Where a slice-local column c (0..511) meets the MFMA: lane quarter q (which 128-column group of
-// the slice), MFMA index t (0..15), element e (0..7) of the 8-half operand, and the code shift p.
+// Where column cc (0..127) of a 128-column chunk (= one scale group) meets the MFMAs: MFMA index
+// t (0..15), element e (0..7) of the 8-half operand, and the code shift p of that element.
 // MFMA t = 4*word + 2*z + h consumes out[8*z + 4*h .. 8*z + 4*h + 3] of that word's decode.
 struct OperandSlot {
-    int q, t, e, p;
+    int t, e, p;
 };
-TLLM_HD OperandSlot column_slot(int c) {
-    const int bit = c & 31;
-    const int word = (c >> 5) & 3;
+TLLM_HD OperandSlot chunk_slot(int cc) {
+    const int bit = cc & 31;
+    const int word = (cc >> 5) & 3;
     const int z = bit & 1;
     const int field = bit >> 1;  // 0..15
-    const int half = field >> 3;
-    const int m = field & 7;
+    const int m = field_dword(field);
     const int h = m >> 2;
     OperandSlot s;
-    s.q = c >> 7;
     s.t = 4 * word + 2 * z + h;
-    s.e = 2 * (m & 3) + half;
+    s.e = 2 * (m & 3) + field_half(field);
     s.p = code_shift(m);
     return s;
 }
 
-// Index (in halfs) of operand element (t, q, e) inside the 512-half image of one slice.
-TLLM_HD int image_index(int t, int q, int e) { return (t * 4 + q) * 8 + e; }
+// Index (in halfs) of operand element (t, chunk, e) inside the activation image of one slice of
+// `chunks` 128-column chunks: the 16 bytes of one (t, chunk) are contiguous, chunks are adjacent.
+TLLM_HD int image_index(int t, int chunk, int e, int chunks) { return (t * chunks + chunk) * 8 + e; }
 
 }  // namespace tllm

@@ -1,17 +1,24 @@
-// Decode GEMV on the matrix cores (gfx950), group size 128, batch 1..4.
+// Decode GEMV on the matrix cores (gfx950), group size 128.
 //
 // Arithmetic (reference kernels/ternary_gemv.cu:47-86): y[r] = sum_g s[r,g] * sum_{k in g} w[r,k] x[k],
 // fp32 accumulation, fp16 store with round-to-nearest-even.
 //
-// Dataflow. A workgroup of 4 waves owns a range of rows of one matrix. Each wave owns 512-column
-// slices of K: it keeps the slice's activations in 64 VGPRs as ready-made MFMA B operands and
-// walks down the rows 16 at a time. Per iteration a lane loads 16 B of each mask plane (the 128
-// weights of one scale group of one row, so a 16-lane group reads 64 contiguous bytes per row),
-// turns them into 16 MFMA A operands with ~0.75 VALU ops per weight (see gemv_layout.h) and issues
-// 16 v_mfma_f32_16x16x32_f16. The B operand of lane (k-quarter q, column j) is non-zero only when
-// j % 4 == q, so output column j collects exactly one scale group (j % 4) of one batch column
-// (j / 4): the per-group fp32 scale is applied to a 16x16 tile once per 4 groups. Partial sums of
-// the K slices meet in LDS, one slot per wave, and are added in a fixed order (deterministic).
+// Dataflow. A workgroup of 4 waves owns a range of rows of one matrix; the activations of the matrix
+// are staged once in LDS as ready-made MFMA B operands (power-of-two normalised, see below). The
+// work of a range is cut into tiles of 64 (row, 128-column chunk) pairs: every lane loads 16 B of
+// each mask plane (one chunk = one scale group of one row), turns them into 16 MFMA A operands
+// with ~0.8 VALU operations per weight (gemv_layout.h) and the wave issues 16
+// v_mfma_f32_16x16x32_f16. Tiles are ordered slice-major (a slice = the columns whose activations
+// sit in the wave's 64 B-operand registers), split evenly over the waves, and loaded three tiles
+// ahead. The B operands are sparse by construction - lane (k-quarter q, column j) is non-zero for
+// one q only - so each output column of the 16x16 result collects exactly one scale group, and the
+// fp32 group scale is applied to whole result tiles, not to weights. Partial sums meet in LDS,
+// one slot per wave, and are added in a fixed order (deterministic).
+//
+// Two tile geometries:
+//   Wide (batch 1):   4 rows x 2048 columns. Lanes 4a..4a+3 read 64 contiguous bytes of row a, so
+//                     the loads coalesce; result column j is scale group j of the slice.
+//   Tall (batch 1-4): 16 rows x 512 columns. Result column j is group j % 4 of batch column j / 4.
 #include "common.h"
 #include "gemv_layout.h"
 
@@ -22,9 +29,31 @@ typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 
+// Weight streams are read through global-address-space pointers (pointers fetched from the
+// problem table would otherwise be treated as generic and use slower flat loads).
+typedef __attribute__((address_space(1))) const uint32_t GU32;
+typedef __attribute__((address_space(1))) const uint16_t GU16;
+typedef __attribute__((address_space(1))) const u4 GU4;
+#define GB __attribute__((address_space(1)))
+template <class T>
+__device__ __forceinline__ __attribute__((address_space(1))) const T *as_global(const T *p) {
+    return (__attribute__((address_space(1))) const T *)p;
+}
+
 constexpr int kNW = 4;  // waves per workgroup
 constexpr int kThreads = kNW * kWave;
 constexpr int kMaxBatch = TLLM_MAX_PLAN_BATCH;
+#ifndef TLLM_TILES_AHEAD
+#define TLLM_TILES_AHEAD 3
+#endif
+constexpr int kTilesAhead = TLLM_TILES_AHEAD;  // tile loads in flight per wave (register ring, unrolled)
+
+struct Wide {
+    static constexpr int kCols = 2048, kRows = 4, kChunks = 16, kScales = 1, kWgPerCu = 3;
+};
+struct Tall {
+    static constexpr int kCols = 512, kRows = 16, kChunks = 4, kScales = 4, kWgPerCu = 2;
+};
 
 struct Sched {
     const Problem *table;    // device table, or nullptr: use the by-value problem
@@ -35,28 +64,22 @@ struct Sched {
     int image_bytes;  // LDS bytes reserved for the activation image (the partial sums follow)
 };
 
+template <class G>
 struct Tile {
     u4 nz, sg;
-    uint16_t sc[4];
+    uint16_t sc[G::kScales];
 };
 
-// Weight streams are read through global-address-space pointers (pointers fetched from the
-// problem table would otherwise be treated as generic and use slower flat loads).
-typedef __attribute__((address_space(1))) const uint32_t GU32;
-typedef __attribute__((address_space(1))) const uint16_t GU16;
-typedef __attribute__((address_space(1))) const u4 GU4;
-template <class T>
-__device__ __forceinline__ __attribute__((address_space(1))) const T *as_global(const T *p) {
-    return (__attribute__((address_space(1))) const T *)p;
+template <int kCtrl>
+__device__ __forceinline__ float dpp_add(float v) {
+    // v + (v moved across lanes by the DPP control); all lanes and banks enabled
+    const int r = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), kCtrl, 0xF, 0xF, true);
+    return v + __builtin_bit_cast(float, r);
 }
-
-__device__ __forceinline__ float dpp_quad(float v, int ctrl_b1_or_4e) {
-    // quad_perm swaps inside groups of 4 lanes; 0xB1 = [1,0,3,2], 0x4E = [2,3,0,1]
-    int r = ctrl_b1_or_4e == 0xB1
-                ? __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true)
-                : __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true);
-    return __builtin_bit_cast(float, r);
-}
+constexpr int kQuadSwap1 = 0xB1;       // quad_perm [1,0,3,2]
+constexpr int kQuadSwap2 = 0x4E;       // quad_perm [2,3,0,1]
+constexpr int kRowHalfMirror = 0x141;  // lane k <-> 7-k inside each 8 lanes
+constexpr int kRowMirror = 0x140;      // lane k <-> 15-k inside each 16 lanes
 
 __device__ __forceinline__ f4 mfma16(const uint32_t *o, u4 b, f4 c) {
     const u4 a = {o[0], o[1], o[2], o[3]};
@@ -64,9 +87,8 @@ __device__ __forceinline__ f4 mfma16(const uint32_t *o, u4 b, f4 c) {
                                                   __builtin_bit_cast(h8, b), c, 0, 0, 0);
 }
 
-// 16 rows x 512 columns: D[i][j] = 2^-24 * sum over the 128 columns of group (j % 4) of
-// (w + 1) * x'' for row i and batch column j / 4.
-__device__ __forceinline__ f4 slice_product(const u4 nz, const u4 sg, const u4 (&B)[kMfmaPerSlice]) {
+// One tile: D[i][j] = 2^-24 * sum over the lanes' chunks that B lets through of (w + 1) * x''.
+__device__ __forceinline__ f4 tile_product(const u4 nz, const u4 sg, const u4 (&B)[kMfmaPerTile]) {
     f4 d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int w = 0; w < 4; w++) {
@@ -80,18 +102,23 @@ __device__ __forceinline__ f4 slice_product(const u4 nz, const u4 sg, const u4 (
     return d0 + d1;
 }
 
-__global__ __launch_bounds__(kThreads, 2) void gemv_mfma_kernel(Problem single, Sched sc) {
+template <class G>
+__global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Problem single, Sched sc) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     uint16_t *image = reinterpret_cast<uint16_t *>(lds);
     float *partial = reinterpret_cast<float *>(lds + sc.image_bytes);
     __shared__ uint32_t red_amax[kNW][kMaxBatch];
     __shared__ float fscale[kMaxBatch];
+    __shared__ u4 zero_operand;  // what the idle lanes of a B operand read
+    if (threadIdx.x == 0) zero_operand = u4{0u, 0u, 0u, 0u};
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
-    const int wave = tid >> 6;
-    const int li = lane & 15;  // A row / D column
-    const int lq = lane >> 4;  // k quarter / D row quad
+    // the wave index is uniform inside a wave: say so, or every loop counter and tile address that
+    // depends on it is computed per lane in vector registers
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 15;  // MFMA A row / D column
+    const int lq = lane >> 4;  // MFMA k quarter / D row quad
 
     int task_begin, task_end;
     if (sc.table) {
@@ -116,12 +143,13 @@ __global__ __launch_bounds__(kThreads, 2) void gemv_mfma_kernel(Problem single, 
         }
         if (pi != cur) {
             // ------------------------------------------------ stage the activations of problem pi
+            __syncthreads();  // every wave is done with the image of the problem before
             if (sc.table) p = sc.table[pi];
             cur = pi;
             words = p.cols / 32;
-            groups = p.cols / 128;
-            slices = (p.cols + kSliceCols - 1) / kSliceCols;
-            img_stride = slices * kSliceCols;
+            groups = p.cols / kChunkCols;
+            slices = (p.cols + G::kCols - 1) / G::kCols;
+            img_stride = slices * G::kCols;
             // (a) per batch column: largest magnitude -> power-of-two normalisation
             for (int b = 0; b < p.batch; b++) {
                 const uint4 *xv = reinterpret_cast<const uint4 *>(p.x + (size_t)b * p.cols);
@@ -145,24 +173,30 @@ __global__ __launch_bounds__(kThreads, 2) void gemv_mfma_kernel(Problem single, 
 #pragma unroll
                 for (int w = 0; w < kNW; w++) m = max(m, red_amax[w][b]);
                 // amax in [2^ex, 2^(ex+1)); x'' = x * 2^(14-ex) stays below 2^15
-                int ex = 0;  // all-zero activations: the image is zero whatever the exponent
+                int ex = 0;                 // all-zero activations: the image is zero whatever the exponent
                 if (m >= 0x7C00u) ex = 15;  // inf/nan present: they propagate to the outputs
                 else if (m) ex = (int)((__builtin_bit_cast(uint32_t, h2f((uint16_t)m)) >> 23) & 0xFF) - 127;
                 if (tid == 0) fscale[b] = m ? __builtin_bit_cast(float, (uint32_t)(127 + ex + 10) << 23) : 0.0f;
-                // (b) image: operand element (slice, t, q, e) = fp16(x[col] * 2^(14-ex-p))
+                // (b) image: operand element (slice, t, chunk, e) = fp16(x[col] * 2^(14-ex-p)). The last
+                // slice of a row that is not a whole number of slices is moved left so that it ends
+                // with the row; the chunks it then shares with the slice before it are zero here.
                 const uint4 *xv = reinterpret_cast<const uint4 *>(p.x + (size_t)b * p.cols);
                 uint16_t *img = image + (size_t)b * img_stride;
                 for (int c8 = tid; c8 < img_stride / 8; c8 += kThreads) {
+                    const int slice = (c8 * 8) / G::kCols;
+                    const int chunk = ((c8 * 8) % G::kCols) / kChunkCols;
+                    const int cc0 = (c8 * 8) % kChunkCols;
+                    const int g = min(slice * G::kChunks, groups - G::kChunks) + chunk;
                     uint4 v = {0u, 0u, 0u, 0u};
-                    if (c8 * 8 < p.cols && m) v = xv[c8];
+                    if (g >= slice * G::kChunks && m) v = xv[(g * kChunkCols + cc0) / 8];
                     const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
+                    uint16_t *dst = img + slice * G::kCols;
 #pragma unroll
                     for (int e = 0; e < 8; e++) {
-                        const int col = c8 * 8 + e;
-                        const OperandSlot s = column_slot(col & (kSliceCols - 1));
+                        const OperandSlot s = chunk_slot(cc0 + e);
                         const float mult = __builtin_bit_cast(float, (uint32_t)(127 + 14 - ex - s.p) << 23);
                         const uint16_t hx = (uint16_t)(w4[e >> 1] >> (16 * (e & 1)));
-                        img[(col / kSliceCols) * kSliceCols + image_index(s.t, s.q, s.e)] = f2h(h2f(hx) * mult);
+                        dst[image_index(s.t, chunk, s.e, G::kChunks)] = f2h(h2f(hx) * mult);
                     }
                 }
             }
@@ -171,122 +205,160 @@ __global__ __launch_bounds__(kThreads, 2) void gemv_mfma_kernel(Problem single, 
 
         const int r_begin = (task - first_task) * sc.range_rows;
         const int r_end = min(p.rows, r_begin + sc.range_rows);
-        const int nrows = r_end - r_begin;
-        const int bcol = li >> 2;               // batch column of this lane's D column
-        const bool b_active = (li & 3) == lq && bcol < p.batch;
-        float *my_part = partial + (size_t)wave * sc.range_rows * p.batch;
-        const bool part_lane = (li & 3) == 0 && bcol < p.batch;
+        // Each wave owns a quarter of the range's rows and walks them once per slice, so the B
+        // operands change only between such walks and no partial sum is shared between waves.
+        const int rows_per_wave = sc.range_rows / kNW;  // a multiple of kRows * kTilesAhead
+        const int w_begin = r_begin + wave * rows_per_wave;
+        const int w_rows = max(0, min(r_end - w_begin, rows_per_wave));
+        const int n_rb = (w_rows + G::kRows - 1) / G::kRows;        // live tiles per walk
+        const int n_slots = (n_rb + kTilesAhead - 1) / kTilesAhead * kTilesAhead;
+        float *my_part = partial + (size_t)wave * rows_per_wave * p.batch;
+        for (int k = lane; k < rows_per_wave * p.batch; k += kWave) my_part[k] = 0.0f;
 
-        // This wave's tiles: its slices (wave, wave + kNW, ...) times the 16-row blocks of the range,
-        // slice-major. Tile loads are issued three tiles ahead and never branch, so the hardware
-        // counters let two tiles stay in flight while one is being consumed.
-        const int n_rb = (nrows + kIterRows - 1) / kIterRows;
-        const int n_sl = slices > wave ? (slices - wave + kNW - 1) / kNW : 0;
-        const int n_tiles = n_sl * n_rb;
-        const GU32 *nz_g = as_global(p.nz);
-        const GU32 *sg_g = as_global(p.sg);
-        const GU16 *sc_g = as_global(p.scales);
+        // ---- which operand lanes are live, and what each lane loads
+        int bcol;       // batch column of this lane's D column
+        bool b_active;  // this lane's B operand is non-zero
+        int b_chunk;    // chunk (of the slice) the lane's B operand holds
+        int a_chunk;    // chunk (of the slice) whose weights the lane loads
+        int a_row;      // row (of the tile) whose weights the lane loads
+        if constexpr (G::kRows == 4) {
+            bcol = 0;
+            b_active = lq == (li >> 2);
+            b_chunk = li;
+            a_chunk = 4 * lq + (lane & 3);
+            a_row = (lane >> 2) & 3;
+        } else {
+            bcol = li >> 2;
+            b_active = (li & 3) == lq && bcol < p.batch;
+            b_chunk = lq;
+            a_chunk = lq;
+            a_row = li;
+        }
 
-        // Groups past the end of a row (last slice when cols % 512 != 0) are read from the row's last
-        // group instead: their activations in the image are zero, so they add nothing.
-        auto load_tile = [&](int slice, int rb) -> Tile {
-            Tile t;
-            const int ga = min(4 * slice + lq, groups - 1);
-            const int gs = min(4 * slice + (li & 3), groups - 1);
-            const int ra = min(rb + li, p.rows - 1);
-            const size_t off = (size_t)ra * words + 4 * ga;
-            t.nz = *reinterpret_cast<const GU4 *>(nz_g + off);
-            t.sg = *reinterpret_cast<const GU4 *>(sg_g + off);
+        // Tile addresses: a wave-uniform base (row block, slice) plus a per-lane offset that never
+        // changes, so the hot loop spends no vector operations on addressing. The last row block and
+        // the last slice are moved back to end exactly at the matrix edge (rows >= kRows and
+        // groups >= kChunks are guaranteed by the dispatcher); the rows such a block repeats are
+        // dropped again in the epilogue, the repeated columns are zero in the image.
+        const char GB *nz_g = reinterpret_cast<const char GB *>(as_global(p.nz));
+        const char GB *sg_g = reinterpret_cast<const char GB *>(as_global(p.sg));
+        const char GB *sc_g = reinterpret_cast<const char GB *>(as_global(p.scales));
+        const uint32_t lane_a = ((uint32_t)a_row * words + 4u * a_chunk) * 4u;
+        uint32_t lane_s[G::kScales];
+        if constexpr (G::kRows == 4) {
+            lane_s[0] = ((uint32_t)lq * groups + li) * 2u;
+        } else {
 #pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const int rs = min(rb + 4 * lq + v, p.rows - 1);
-                t.sc[v] = sc_g[(size_t)rs * groups + gs];
-            }
+            for (int v = 0; v < 4; v++) lane_s[v] = ((uint32_t)(4 * lq + v) * groups + (li & 3)) * 2u;
+        }
+
+        auto load_tile = [&](int slice, int rb) -> Tile<G> {
+            Tile<G> t;
+            const int rbe = min(rb, p.rows - G::kRows);
+            const int c0 = min(slice * G::kChunks, groups - G::kChunks);
+            const size_t base_a = ((size_t)rbe * words + (size_t)c0 * 4) * 4;
+            const size_t base_s = ((size_t)rbe * groups + c0) * 2;
+            t.nz = *reinterpret_cast<const GU4 *>(nz_g + base_a + lane_a);
+            t.sg = *reinterpret_cast<const GU4 *>(sg_g + base_a + lane_a);
+#pragma unroll
+            for (int v = 0; v < G::kScales; v++)
+                t.sc[v] = *reinterpret_cast<const GU16 *>(sc_g + base_s + lane_s[v]);
             return t;
         };
 
-        u4 B[kMfmaPerSlice];
-        f4 bias = {0.f, 0.f, 0.f, 0.f};
-        const u4 zero4 = {0u, 0u, 0u, 0u};
-#pragma unroll
-        for (int t = 0; t < kMfmaPerSlice; t++) B[t] = zero4;
-
-        auto process = [&](const Tile &t, int slice, int rb) {
-            if (rb == r_begin) {
-                // new slice: its activations become the B operands (zero outside the lane's own
-                // group / batch column), and an all-zero weight row gives the "+1" term of the code
-                const u4 *src = reinterpret_cast<const u4 *>(image + (size_t)bcol * img_stride +
-                                                             slice * kSliceCols) + lq;
-                if (b_active) {
-#pragma unroll
-                    for (int k = 0; k < kMfmaPerSlice; k++) B[k] = src[k * 4];
-                }
-                bias = slice_product(zero4, zero4, B);
-            }
-            const f4 d = slice_product(t.nz, t.sg, B);
-            float r[4];
-#pragma unroll
-            for (int v = 0; v < 4; v++) {
-                float x = h2f(t.sc[v]) * (d[v] - bias[v]);
-                x += dpp_quad(x, 0xB1);
-                x += dpp_quad(x, 0x4E);
-                r[v] = x;
-            }
-            if (part_lane) {
-                const bool first_slice = slice == wave;
-#pragma unroll
-                for (int v = 0; v < 4; v++) {
-                    float *dst = my_part + (size_t)(rb - r_begin + 4 * lq + v) * p.batch + bcol;
-                    *dst = first_slice ? r[v] : *dst + r[v];
-                }
-            }
-        };
-
-        if (n_tiles > 0) {
-            // load cursor (ls, lrb) runs three tiles ahead of the compute cursor (cs, crb)
-            int ls = wave, lrb = r_begin, cs = wave, crb = r_begin;
-            auto advance = [&](int &s_, int &rb_) {
-                rb_ += kIterRows;
-                if (rb_ >= r_end) { rb_ = r_begin; s_ += kNW; }
-            };
-            auto next_load = [&]() -> Tile {
-                // past the last tile the cursor is parked on it (a cached re-read, never out of range)
-                const Tile t = load_tile(ls < slices ? ls : cs, ls < slices ? lrb : crb);
-                if (ls < slices) advance(ls, lrb);
+        if (n_rb > 0) {
+            // Load cursor: slot j of a walk reads tile min(j, n_rb - 1) (slots past the live tiles
+            // re-read the last one; their results are dropped). It runs kTilesAhead slots ahead of
+            // the compute loop, across walks; past the last walk it parks.
+            int l_slice = 0, l_slot = 0;
+            auto next_load = [&]() -> Tile<G> {
+                const Tile<G> t = load_tile(min(l_slice, slices - 1),
+                                            w_begin + min(l_slot, n_rb - 1) * G::kRows);
+                if (++l_slot == n_slots) { l_slot = 0; l_slice++; }
                 return t;
             };
-            Tile t0 = next_load(), t1 = next_load(), t2 = next_load();
-            for (int i = 0; i < n_tiles; i += 3) {
-                process(t0, cs, crb);
-                advance(cs, crb);
-                t0 = next_load();
-                if (i + 1 >= n_tiles) break;
-                process(t1, cs, crb);
-                advance(cs, crb);
-                t1 = next_load();
-                if (i + 2 >= n_tiles) break;
-                process(t2, cs, crb);
-                advance(cs, crb);
-                t2 = next_load();
+            Tile<G> ring[kTilesAhead];
+#pragma unroll
+            for (int k = 0; k < kTilesAhead; k++) {
+                ring[k] = next_load();
+                __builtin_amdgcn_sched_barrier(0);  // same issue order as in the loop below
+            }
+
+            const u4 zero4 = {0u, 0u, 0u, 0u};
+            for (int slice = 0; slice < slices; slice++) {
+                // this slice's activations become the B operands. Every lane reads (no branch): the
+                // idle lanes read the zero operand with stride 0.
+                u4 B[kMfmaPerTile];
+                const u4 *src = b_active ? reinterpret_cast<const u4 *>(image + (size_t)bcol * img_stride +
+                                                                        slice * G::kCols) + b_chunk
+                                         : &zero_operand;
+                const int stride = b_active ? G::kChunks : 0;
+#pragma unroll
+                for (int k = 0; k < kMfmaPerTile; k++) B[k] = src[k * stride];
+                // an all-zero weight row gives the "+1" term of the code, to be subtracted
+                const f4 bias = tile_product(zero4, zero4, B);
+                float bias_sel = bias[0];  // wide tiles: the one bias entry this lane uses
+                if constexpr (G::kRows == 4) {
+                    const int v = li & 3;
+                    bias_sel = v == 0 ? bias[0] : v == 1 ? bias[1] : v == 2 ? bias[2] : bias[3];
+                }
+
+                auto process = [&](const Tile<G> &t, int rb, bool live) {
+                    const f4 d = tile_product(t.nz, t.sg, B);
+                    const int sh = rb - min(rb, p.rows - G::kRows);  // rows a moved-back block repeats
+                    if constexpr (G::kRows == 4) {
+                        // lane (row quad lq, column li): only D row 4*lq + (li & 3) pairs this column's
+                        // chunk with the row that loaded it; it is group li of row rb - sh + lq
+                        const int v = li & 3;
+                        const float dv = v == 0 ? d[0] : v == 1 ? d[1] : v == 2 ? d[2] : d[3];
+                        float x = h2f(t.sc[0]) * (dv - bias_sel);
+                        x = dpp_add<kQuadSwap1>(x);
+                        x = dpp_add<kQuadSwap2>(x);
+                        x = dpp_add<kRowHalfMirror>(x);
+                        x = dpp_add<kRowMirror>(x);
+                        if (li == 0 && lq >= sh && live) my_part[rb - sh - w_begin + lq] += x;
+                    } else {
+                        float r[4];
+#pragma unroll
+                        for (int v = 0; v < 4; v++) {
+                            float x = h2f(t.sc[v]) * (d[v] - bias[v]);
+                            x = dpp_add<kQuadSwap1>(x);
+                            x = dpp_add<kQuadSwap2>(x);
+                            r[v] = x;
+                        }
+                        if ((li & 3) == 0 && bcol < p.batch && live) {
+#pragma unroll
+                            for (int v = 0; v < 4; v++)
+                                if (4 * lq + v >= sh)
+                                    my_part[(size_t)(rb - sh - w_begin + 4 * lq + v) * p.batch + bcol] += r[v];
+                        }
+                    }
+                };
+
+                // No branch surrounds a load or an MFMA, so the wait counters stay exact and
+                // kTilesAhead - 1 tiles remain in flight while one is consumed.
+                for (int j = 0; j < n_slots; j += kTilesAhead) {
+#pragma unroll
+                    for (int k = 0; k < kTilesAhead; k++) {
+                        process(ring[k], w_begin + min(j + k, n_rb - 1) * G::kRows, j + k < n_rb);
+                        ring[k] = next_load();
+                        // keep the scheduler from interleaving whole tiles: that would need the
+                        // registers of several decodes at once and cost a resident wave per SIMD
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            }
+            // ------------------------------------------------ this wave's rows are complete: store fp16
+            for (int idx = lane; idx < w_rows * p.batch; idx += kWave) {
+                const int b = idx / w_rows, rl = idx - b * w_rows;
+                p.y[(size_t)b * p.rows + w_begin + rl] = f2h(my_part[(size_t)rl * p.batch + b] * fscale[b]);
             }
         }
-        __syncthreads();
-        // ------------------------------------------------ add the K slices in wave order, store fp16
-        const int live = min(kNW, slices);
-        for (int idx = tid; idx < nrows * p.batch; idx += kThreads) {
-            const int b = idx / nrows, rl = idx - b * nrows;
-            float sum = 0.0f;
-            for (int w = 0; w < live; w++)
-                sum += partial[((size_t)w * sc.range_rows + rl) * p.batch + b];
-            p.y[(size_t)b * p.rows + r_begin + rl] = f2h(sum * fscale[b]);
-        }
-        __syncthreads();
     }
 }
 
 struct DeviceInfo {
     int cus = 0;
-    bool attr_set = false;
 };
 
 DeviceInfo &device_info(int dev) {
@@ -294,57 +366,97 @@ DeviceInfo &device_info(int dev) {
     return info[dev < 0 || dev >= 64 ? 0 : dev];
 }
 
-constexpr int kLdsLimit = 80 * 1024;  // two workgroups per CU inside the 160 KB LDS
+constexpr int kLdsLimit = 64 * 1024;  // per workgroup; 160 KB per CU leaves room for two or three
 
 int round16(int v) { return (v + 15) / 16 * 16; }
 
-hipError_t prepare_device(int *cus) {
+template <class G>
+const void *kernel_ptr() {
+    return reinterpret_cast<const void *>(&gemv_mfma_kernel<G>);
+}
+
+hipError_t prepare_device(DeviceInfo **out) {
     int dev = 0;
     if (hipError_t e = hipGetDevice(&dev)) return e;
     DeviceInfo &di = device_info(dev);
     if (di.cus == 0) {
         int n = 0;
         if (hipError_t e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev)) return e;
+        if (hipError_t e = hipFuncSetAttribute(kernel_ptr<Wide>(), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit))
+            return e;
+        if (hipError_t e = hipFuncSetAttribute(kernel_ptr<Tall>(), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit))
+            return e;
         di.cus = n > 0 ? n : 256;
     }
-    if (!di.attr_set) {
-        if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_mfma_kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit))
-            return e;
-        di.attr_set = true;
-    }
-    *cus = di.cus;
+    *out = &di;
     return hipSuccess;
 }
 
-int image_bytes_of(int cols, int batch) {
-    return (cols + kSliceCols - 1) / kSliceCols * kSliceCols * 2 * batch;
+// Resident workgroups per CU for a given dynamic LDS size (asked from the runtime, capped at 4).
+template <class G>
+int resident_wgs(size_t lds_bytes) {
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gemv_mfma_kernel<G>, kThreads, lds_bytes) != hipSuccess || n < 1)
+        n = 1;
+    return n > 4 ? 4 : n;
 }
+
+template <class G>
+constexpr int range_unit() {  // rows: every wave walks whole groups of kTilesAhead tiles
+    return kNW * G::kRows * kTilesAhead;
+}
+
+template <class G>
+int image_bytes_of(int cols, int batch) {
+    return (cols + G::kCols - 1) / G::kCols * G::kCols * 2 * batch;
+}
+
+// Geometry limits: a tile must fit inside the matrix (edge tiles are moved back, not clipped).
+bool wide_ok(const Problem &p) {
+    return p.batch == 1 && p.rows >= 16 && p.cols >= Wide::kCols &&
+           image_bytes_of<Wide>(p.cols, 1) + range_unit<Wide>() * 4 <= kLdsLimit;
+}
+bool tall_ok(const Problem &p) {
+    return p.batch >= 1 && p.batch <= kMaxBatch && p.rows >= 16 && p.cols >= Tall::kCols &&
+           image_bytes_of<Tall>(p.cols, p.batch) + range_unit<Tall>() * p.batch * 4 <= kLdsLimit;
+}
+
+// rows per task: about `per_wg` tasks for each resident workgroup, a multiple of `unit` rows (each
+// wave walks whole groups of kTilesAhead tiles), inside what the partial sums allow
+int pick_range(int64_t total_rows, int wgs, int per_wg, int room, int unit) {
+    int64_t want = (total_rows + (int64_t)wgs * per_wg - 1) / ((int64_t)wgs * per_wg);
+    int range = (int)((want + unit - 1) / unit) * unit;
+    const int cap = (room < 768 ? room : 768) / unit * unit;
+    range = range > cap ? cap : range;
+    return range < unit ? unit : range;
+}
+
 
 }  // namespace
 
 bool gemv_mfma_supports(const Problem &p, int group) {
-    return group == 128 && p.batch >= 1 && p.batch <= kMaxBatch &&
-           image_bytes_of(p.cols, p.batch) + kNW * 16 * p.batch * 4 <= kLdsLimit;
+    return group == 128 && (size_t)p.rows * (p.cols / 8) < (size_t)1 << 32 && (wide_ok(p) || tall_ok(p));
 }
 
 hipError_t launch_gemv_mfma(const Problem &p, hipStream_t s) {
-    int cus = 0;
-    if (hipError_t e = prepare_device(&cus)) return e;
+    DeviceInfo *di = nullptr;
+    if (hipError_t e = prepare_device(&di)) return e;
     Sched sc{};
     sc.table = nullptr;
     sc.count = 1;
-    sc.image_bytes = image_bytes_of(p.cols, p.batch);
-    const int room = (kLdsLimit - sc.image_bytes) / (kNW * p.batch * 4) / 16 * 16;  // rows the partials can hold
-    int range = round16((p.rows + 2 * cus - 1) / (2 * cus));
-    range = range < 16 ? 16 : range;
-    range = range > 512 ? 512 : range;
-    range = range > room ? room : range;
-    sc.range_rows = range;
-    const int tasks = (p.rows + range - 1) / range;
-    const int grid = tasks < 2 * cus ? tasks : 2 * cus;
-    const size_t lds = (size_t)sc.image_bytes + (size_t)kNW * range * p.batch * 4;
-    gemv_mfma_kernel<<<grid, kThreads, lds, s>>>(p, sc);
+    const bool wide = wide_ok(p);
+    sc.image_bytes = wide ? image_bytes_of<Wide>(p.cols, 1) : image_bytes_of<Tall>(p.cols, p.batch);
+    const int room = (kLdsLimit - sc.image_bytes) / (p.batch * 4);  // rows the partial sums can hold
+    const int unit = wide ? range_unit<Wide>() : range_unit<Tall>();
+    const int wgs = (wide ? Wide::kWgPerCu : Tall::kWgPerCu) * di->cus;
+    sc.range_rows = pick_range(p.rows, wgs, 1, room, unit);
+    const int tasks = (p.rows + sc.range_rows - 1) / sc.range_rows;
+    const int grid = tasks < wgs ? tasks : wgs;
+    const size_t lds = (size_t)sc.image_bytes + (size_t)sc.range_rows * p.batch * 4;
+    if (wide)
+        gemv_mfma_kernel<Wide><<<grid, kThreads, lds, s>>>(p, sc);
+    else
+        gemv_mfma_kernel<Tall><<<grid, kThreads, lds, s>>>(p, sc);
     return hipGetLastError();
 }
 
@@ -353,31 +465,42 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
     PlanDevice d;
     d.count = (int)host.size();
     if (hipError_t e = hipGetDevice(&d.device)) return e;
-    int cus = 0;
-    if (hipError_t e = prepare_device(&cus)) return e;
+    DeviceInfo *di = nullptr;
+    if (hipError_t e = prepare_device(&di)) return e;
 
     int64_t total_rows = 0;
     int max_image = 0, max_batch = 1;
     for (const Problem &p : host) {
         total_rows += p.rows;
-        const int ib = image_bytes_of(p.cols, p.batch);
-        max_image = ib > max_image ? ib : max_image;
         max_batch = p.batch > max_batch ? p.batch : max_batch;
         d.max_rows = p.rows > d.max_rows ? p.rows : d.max_rows;
-        d.max_batch = max_batch;
     }
-    d.use_mfma = true;
-    for (const Problem &p : host) d.use_mfma = d.use_mfma && gemv_mfma_supports(p, 128);
-    const int room = (kLdsLimit - max_image) / (kNW * max_batch * 4) / 16 * 16;
-    if (room < 16) d.use_mfma = false;
+    d.max_batch = max_batch;
+    // one geometry per launch: wide tiles if every problem allows them, else tall ones
+    bool all_wide = true, all_tall = true;
+    for (const Problem &p : host) {
+        const bool addressable = (size_t)p.rows * (p.cols / 8) < (size_t)1 << 32;
+        all_wide = all_wide && addressable && wide_ok(p);
+        all_tall = all_tall && addressable && tall_ok(p);
+    }
+    d.wide = all_wide;
+    d.use_mfma = all_wide || all_tall;
+    for (const Problem &p : host) {
+        const int ib = d.wide ? image_bytes_of<Wide>(p.cols, 1) : image_bytes_of<Tall>(p.cols, p.batch);
+        max_image = ib > max_image ? ib : max_image;
+    }
+    const int unit = d.wide ? range_unit<Wide>() : range_unit<Tall>();
+    const int room = (kLdsLimit - max_image) / (max_batch * 4);  // rows the partial sums can hold
+    if (room < unit) d.use_mfma = false;
 
     std::vector<int> prefix(host.size() + 1, 0), wg_first;
     if (d.use_mfma) {
-        // about 8 tasks per workgroup, each a multiple of 16 rows that fits the partial-sum area
-        int range = round16((int)((total_rows + 16LL * cus - 1) / (16LL * cus)));
-        range = range < 16 ? 16 : range;
-        range = range > 512 ? 512 : range;
-        range = range > room ? room : range;
+        // size the grid for the workgroups that can be resident with a mid-sized partial-sum area,
+        // then cut the rows into about 8 tasks per workgroup
+        const size_t lds_guess = (size_t)max_image + (size_t)(room < 384 ? room : 384) * max_batch * 4;
+        const int per_cu = d.wide ? resident_wgs<Wide>(lds_guess) : resident_wgs<Tall>(lds_guess);
+        const int wgs = per_cu * di->cus;
+        const int range = pick_range(total_rows, wgs, 8, room, unit);
         std::vector<int64_t> weight;
         for (size_t i = 0; i < host.size(); i++) {
             const int n = (host[i].rows + range - 1) / range;
@@ -389,7 +512,7 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
             }
         }
         const int tasks = prefix.back();
-        const int grid = tasks < 2 * cus ? tasks : 2 * cus;
+        const int grid = tasks < wgs ? tasks : wgs;
         int64_t total_w = 0;
         for (int64_t w : weight) total_w += w;
         // contiguous shares of about equal weight; every workgroup gets at least one task
@@ -405,7 +528,7 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
         d.grid = grid;
         d.range_rows = range;
         d.image_bytes = max_image;
-        d.lds_bytes = max_image + kNW * range * max_batch * 4;
+        d.lds_bytes = max_image + range * max_batch * 4;
     }
 
     const size_t bytes_table = sizeof(Problem) * host.size();
@@ -438,7 +561,10 @@ hipError_t plan_device_launch(const PlanDevice &plan, hipStream_t s) {
     sc.range_rows = plan.range_rows;
     sc.image_bytes = plan.image_bytes;
     Problem none{};
-    gemv_mfma_kernel<<<plan.grid, kThreads, plan.lds_bytes, s>>>(none, sc);
+    if (plan.wide)
+        gemv_mfma_kernel<Wide><<<plan.grid, kThreads, plan.lds_bytes, s>>>(none, sc);
+    else
+        gemv_mfma_kernel<Tall><<<plan.grid, kThreads, plan.lds_bytes, s>>>(none, sc);
     return hipGetLastError();
 }
 

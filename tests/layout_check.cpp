@@ -27,12 +27,16 @@ int main() {
         // image[q][t][e] as the kernel builds it, with the 2^-p factor kept symbolic (double)
         double img[4][16][8];
         int seen[4][16][8] = {};
+        int used[512] = {};
         for (int c = 0; c < 512; c++) {
-            OperandSlot s = column_slot(c);
-            if (s.q != c / 128 || s.t < 0 || s.t > 15 || s.e < 0 || s.e > 7 || s.p < 4 || s.p > 10) bad++;
-            if (seen[s.q][s.t][s.e]++) bad++;                                // must be a bijection
-            img[s.q][s.t][s.e] = std::ldexp(x[c], -s.p);
-            if (image_index(s.t, s.q, s.e) != (s.t * 4 + s.q) * 8 + s.e) bad++;
+            const int q = c / 128;
+            OperandSlot s = chunk_slot(c % 128);
+            if (s.t < 0 || s.t > 15 || s.e < 0 || s.e > 7 || s.p < 2 || s.p > 10) bad++;
+            if (seen[q][s.t][s.e]++) bad++;                                  // must be a bijection
+            img[q][s.t][s.e] = std::ldexp(x[c], -s.p);
+            const int idx = image_index(s.t, q, s.e, 4);
+            if (idx < 0 || idx >= 512 || used[idx]++) bad++;                 // image slots are a bijection too
+            if (image_index(s.t, q, s.e, 16) != (s.t * 16 + q) * 8 + s.e) bad++;
         }
         for (int q = 0; q < 4; q++) {
             double mfma_sum = 0.0, plain = 0.0, bias = 0.0;

@@ -66,10 +66,10 @@ struct PlanDevice {
     // schedule of the MFMA kernel (use_mfma == false: the row-wave table kernel runs instead)
     bool use_mfma = false;
     bool wide = false;  // 4 x 2048 tiles (every problem at batch 1) instead of 16 x 512
-    int *task_prefix = nullptr;
+    int *unit_prefix = nullptr;
     int *wg_first = nullptr;
     int grid = 0;
-    int range_rows = 0;
+    int max_units = 0;
     int image_bytes = 0;
     int lds_bytes = 0;
 };

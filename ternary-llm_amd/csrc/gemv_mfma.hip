@@ -55,12 +55,16 @@ struct Tall {
     static constexpr int kCols = 512, kRows = 16, kChunks = 4, kScales = 4, kWgPerCu = 2;
 };
 
+// Work is counted in units of kNW * kRows * kTilesAhead rows of one matrix. A workgroup owns a
+// contiguous span of units (of about equal weight, cut by the host) and processes it in tasks of
+// up to max_units units that stay inside one matrix.
 struct Sched {
     const Problem *table;    // device table, or nullptr: use the by-value problem
-    const int *task_prefix;  // [count + 1] first task of each problem
-    const int *wg_first;     // [grid + 1] first task of each workgroup
+    const int *unit_prefix;  // [count + 1] first unit of each problem
+    const int *wg_first;     // [grid + 1] first unit of each workgroup
     int count;
-    int range_rows;   // rows per task, a multiple of 16
+    int max_units;    // units per task (bounds the partial-sum area)
+    int max_batch;    // largest batch of any problem (sizes the per-wave partial-sum areas)
     int image_bytes;  // LDS bytes reserved for the activation image (the partial sums follow)
 };
 
@@ -81,6 +85,14 @@ constexpr int kQuadSwap2 = 0x4E;       // quad_perm [2,3,0,1]
 constexpr int kRowHalfMirror = 0x141;  // lane k <-> 7-k inside each 8 lanes
 constexpr int kRowMirror = 0x140;      // lane k <-> 15-k inside each 16 lanes
 
+// dst = mask[lane] ? b : a, with the 64-bit lane mask held in scalar registers. Written out because
+// the compiler otherwise recomputes the lane compare in front of every select.
+__device__ __forceinline__ float lane_select(float a, float b, uint64_t mask) {
+    float r;
+    asm("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "s"(mask));
+    return r;
+}
+
 __device__ __forceinline__ f4 mfma16(const uint32_t *o, u4 b, f4 c) {
     const u4 a = {o[0], o[1], o[2], o[3]};
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a),
@@ -88,6 +100,22 @@ __device__ __forceinline__ f4 mfma16(const uint32_t *o, u4 b, f4 c) {
 }
 
 // One tile: D[i][j] = 2^-24 * sum over the lanes' chunks that B lets through of (w + 1) * x''.
+// Two accumulator chains keep dependent MFMAs apart; the caller adds them.
+__device__ __forceinline__ void tile_product2(const u4 nz, const u4 sg, const u4 (&B)[kMfmaPerTile],
+                                              f4 &d0, f4 &d1) {
+    d0 = f4{0.f, 0.f, 0.f, 0.f};
+    d1 = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+        uint32_t o[16];
+        decode_word(nz[w], sg[w], o);
+        d0 = mfma16(o + 0, B[4 * w + 0], d0);
+        d1 = mfma16(o + 4, B[4 * w + 1], d1);
+        d0 = mfma16(o + 8, B[4 * w + 2], d0);
+        d1 = mfma16(o + 12, B[4 * w + 3], d1);
+    }
+}
+
 __device__ __forceinline__ f4 tile_product(const u4 nz, const u4 sg, const u4 (&B)[kMfmaPerTile]) {
     f4 d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -120,14 +148,15 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
     const int li = lane & 15;  // MFMA A row / D column
     const int lq = lane >> 4;  // MFMA k quarter / D row quad
 
-    int task_begin, task_end;
+    constexpr int kUnitRows = kNW * G::kRows * kTilesAhead;
+    int u = 0, u_end = 0;
     if (sc.table) {
-        task_begin = sc.wg_first[blockIdx.x];
-        task_end = sc.wg_first[blockIdx.x + 1];
+        u = sc.wg_first[blockIdx.x];
+        u_end = sc.wg_first[blockIdx.x + 1];
     } else {
-        const int total = (single.rows + sc.range_rows - 1) / sc.range_rows;
-        task_begin = (int)((int64_t)total * blockIdx.x / gridDim.x);
-        task_end = (int)((int64_t)total * (blockIdx.x + 1) / gridDim.x);
+        const int total = (single.rows + kUnitRows - 1) / kUnitRows;
+        u = (int)((int64_t)total * blockIdx.x / gridDim.x);
+        u_end = (int)((int64_t)total * (blockIdx.x + 1) / gridDim.x);
     }
 
     int cur = -1;  // problem whose activations are staged
@@ -135,12 +164,17 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
     Problem p = single;
     int slices = 0, groups = 0, words = 0, img_stride = 0;
 
-    for (int task = task_begin; task < task_end; task++) {
-        int first_task = 0;
+    while (u < u_end) {
+        int first_unit = 0;
+        int p_units = (single.rows + kUnitRows - 1) / kUnitRows;
         if (sc.table) {
-            while (sc.task_prefix[pi + 1] <= task) pi++;
-            first_task = sc.task_prefix[pi];
+            while (sc.unit_prefix[pi + 1] <= u) pi++;
+            first_unit = sc.unit_prefix[pi];
+            p_units = sc.unit_prefix[pi + 1] - first_unit;
         }
+        const int n_units = min(min(u_end - u, first_unit + p_units - u), sc.max_units);
+        const int task_first_row = (u - first_unit) * kUnitRows;
+        u += n_units;
         if (pi != cur) {
             // ------------------------------------------------ stage the activations of problem pi
             __syncthreads();  // every wave is done with the image of the problem before
@@ -203,16 +237,17 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
             __syncthreads();
         }
 
-        const int r_begin = (task - first_task) * sc.range_rows;
-        const int r_end = min(p.rows, r_begin + sc.range_rows);
-        // Each wave owns a quarter of the range's rows and walks them once per slice, so the B
+        const int r_begin = task_first_row;
+        const int r_end = min(p.rows, r_begin + n_units * kUnitRows);
+        // Each wave owns a quarter of the task's rows and walks them once per slice, so the B
         // operands change only between such walks and no partial sum is shared between waves.
-        const int rows_per_wave = sc.range_rows / kNW;  // a multiple of kRows * kTilesAhead
+        const int rows_per_wave = n_units * (kUnitRows / kNW);  // a multiple of kRows * kTilesAhead
         const int w_begin = r_begin + wave * rows_per_wave;
         const int w_rows = max(0, min(r_end - w_begin, rows_per_wave));
         const int n_rb = (w_rows + G::kRows - 1) / G::kRows;        // live tiles per walk
         const int n_slots = (n_rb + kTilesAhead - 1) / kTilesAhead * kTilesAhead;
-        float *my_part = partial + (size_t)wave * rows_per_wave * p.batch;
+        // fixed per-wave area (sized for the longest task): waves run through tasks independently
+        float *my_part = partial + (size_t)wave * (sc.max_units * (kUnitRows / kNW)) * sc.max_batch;
         for (int k = lane; k < rows_per_wave * p.batch; k += kWave) my_part[k] = 0.0f;
 
         // ---- which operand lanes are live, and what each lane loads
@@ -285,6 +320,9 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
             }
 
             const u4 zero4 = {0u, 0u, 0u, 0u};
+            // lanes whose result row (li & 3) is odd / is 2 or 3 (wide tiles pick one of four D rows)
+            const uint64_t odd_lanes = __builtin_amdgcn_ballot_w64((li & 1) != 0);
+            const uint64_t hi_lanes = __builtin_amdgcn_ballot_w64((li & 2) != 0);
             for (int slice = 0; slice < slices; slice++) {
                 // this slice's activations become the B operands. Every lane reads (no branch): the
                 // idle lanes read the zero operand with stride 0.
@@ -297,20 +335,21 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
                 for (int k = 0; k < kMfmaPerTile; k++) B[k] = src[k * stride];
                 // an all-zero weight row gives the "+1" term of the code, to be subtracted
                 const f4 bias = tile_product(zero4, zero4, B);
-                float bias_sel = bias[0];  // wide tiles: the one bias entry this lane uses
-                if constexpr (G::kRows == 4) {
-                    const int v = li & 3;
-                    bias_sel = v == 0 ? bias[0] : v == 1 ? bias[1] : v == 2 ? bias[2] : bias[3];
-                }
+                // wide tiles: the one bias entry this lane uses
+                const float bias_sel = lane_select(lane_select(bias[0], bias[1], odd_lanes),
+                                                   lane_select(bias[2], bias[3], odd_lanes), hi_lanes);
 
                 auto process = [&](const Tile<G> &t, int rb, bool live) {
-                    const f4 d = tile_product(t.nz, t.sg, B);
+                    f4 d0, d1;
+                    tile_product2(t.nz, t.sg, B, d0, d1);
+                    const f4 d = d0 + d1;
                     const int sh = rb - min(rb, p.rows - G::kRows);  // rows a moved-back block repeats
                     if constexpr (G::kRows == 4) {
                         // lane (row quad lq, column li): only D row 4*lq + (li & 3) pairs this column's
-                        // chunk with the row that loaded it; it is group li of row rb - sh + lq
-                        const int v = li & 3;
-                        const float dv = v == 0 ? d[0] : v == 1 ? d[1] : v == 2 ? d[2] : d[3];
+                        // chunk with the row that loaded it; it is group li of row rb - sh + lq.
+                        // (bias_sel was formed the same way, so an all-zero row still gives exactly 0)
+                        const float dv = lane_select(lane_select(d[0], d[1], odd_lanes),
+                                                     lane_select(d[2], d[3], odd_lanes), hi_lanes);
                         float x = h2f(t.sc[0]) * (dv - bias_sel);
                         x = dpp_add<kQuadSwap1>(x);
                         x = dpp_add<kQuadSwap2>(x);
@@ -368,8 +407,6 @@ DeviceInfo &device_info(int dev) {
 
 constexpr int kLdsLimit = 64 * 1024;  // per workgroup; 160 KB per CU leaves room for two or three
 
-int round16(int v) { return (v + 15) / 16 * 16; }
-
 template <class G>
 const void *kernel_ptr() {
     return reinterpret_cast<const void *>(&gemv_mfma_kernel<G>);
@@ -421,16 +458,14 @@ bool tall_ok(const Problem &p) {
            image_bytes_of<Tall>(p.cols, p.batch) + range_unit<Tall>() * p.batch * 4 <= kLdsLimit;
 }
 
-// rows per task: about `per_wg` tasks for each resident workgroup, a multiple of `unit` rows (each
-// wave walks whole groups of kTilesAhead tiles), inside what the partial sums allow
-int pick_range(int64_t total_rows, int wgs, int per_wg, int room, int unit) {
-    int64_t want = (total_rows + (int64_t)wgs * per_wg - 1) / ((int64_t)wgs * per_wg);
-    int range = (int)((want + unit - 1) / unit) * unit;
-    const int cap = (room < 768 ? room : 768) / unit * unit;
-    range = range > cap ? cap : range;
-    return range < unit ? unit : range;
-}
+constexpr int kMaxTaskUnits = 10;  // longer tasks amortise the per-slice operand reload
 
+// units per task that the partial-sum area can hold
+int max_units_for(int image_bytes, int batch, int unit) {
+    const int room_rows = (kLdsLimit - image_bytes) / (batch * 4);
+    const int n = room_rows / unit;
+    return n > kMaxTaskUnits ? kMaxTaskUnits : n;
+}
 
 }  // namespace
 
@@ -446,13 +481,13 @@ hipError_t launch_gemv_mfma(const Problem &p, hipStream_t s) {
     sc.count = 1;
     const bool wide = wide_ok(p);
     sc.image_bytes = wide ? image_bytes_of<Wide>(p.cols, 1) : image_bytes_of<Tall>(p.cols, p.batch);
-    const int room = (kLdsLimit - sc.image_bytes) / (p.batch * 4);  // rows the partial sums can hold
     const int unit = wide ? range_unit<Wide>() : range_unit<Tall>();
+    sc.max_units = max_units_for(sc.image_bytes, p.batch, unit);
+    sc.max_batch = p.batch;
     const int wgs = (wide ? Wide::kWgPerCu : Tall::kWgPerCu) * di->cus;
-    sc.range_rows = pick_range(p.rows, wgs, 1, room, unit);
-    const int tasks = (p.rows + sc.range_rows - 1) / sc.range_rows;
-    const int grid = tasks < wgs ? tasks : wgs;
-    const size_t lds = (size_t)sc.image_bytes + (size_t)sc.range_rows * p.batch * 4;
+    const int units = (p.rows + unit - 1) / unit;
+    const int grid = units < wgs ? units : wgs;
+    const size_t lds = (size_t)sc.image_bytes + (size_t)sc.max_units * unit * p.batch * 4;
     if (wide)
         gemv_mfma_kernel<Wide><<<grid, kThreads, lds, s>>>(p, sc);
     else
@@ -468,10 +503,8 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
     DeviceInfo *di = nullptr;
     if (hipError_t e = prepare_device(&di)) return e;
 
-    int64_t total_rows = 0;
     int max_image = 0, max_batch = 1;
     for (const Problem &p : host) {
-        total_rows += p.rows;
         max_batch = p.batch > max_batch ? p.batch : max_batch;
         d.max_rows = p.rows > d.max_rows ? p.rows : d.max_rows;
     }
@@ -490,45 +523,41 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
         max_image = ib > max_image ? ib : max_image;
     }
     const int unit = d.wide ? range_unit<Wide>() : range_unit<Tall>();
-    const int room = (kLdsLimit - max_image) / (max_batch * 4);  // rows the partial sums can hold
-    if (room < unit) d.use_mfma = false;
+    const int max_units = max_units_for(max_image, max_batch, unit);
+    if (max_units < 1) d.use_mfma = false;
 
     std::vector<int> prefix(host.size() + 1, 0), wg_first;
     if (d.use_mfma) {
-        // size the grid for the workgroups that can be resident with a mid-sized partial-sum area,
-        // then cut the rows into about 8 tasks per workgroup
-        const size_t lds_guess = (size_t)max_image + (size_t)(room < 384 ? room : 384) * max_batch * 4;
-        const int per_cu = d.wide ? resident_wgs<Wide>(lds_guess) : resident_wgs<Tall>(lds_guess);
+        d.lds_bytes = max_image + max_units * unit * max_batch * 4;
+        const int per_cu = d.wide ? resident_wgs<Wide>(d.lds_bytes) : resident_wgs<Tall>(d.lds_bytes);
         const int wgs = per_cu * di->cus;
-        const int range = pick_range(total_rows, wgs, 8, room, unit);
+        // weight of every unit: its weights plus a fixed cost; then contiguous spans of about equal
+        // weight, at least one unit per workgroup
         std::vector<int64_t> weight;
         for (size_t i = 0; i < host.size(); i++) {
-            const int n = (host[i].rows + range - 1) / range;
+            const int n = (host[i].rows + unit - 1) / unit;
             prefix[i + 1] = prefix[i] + n;
             for (int t = 0; t < n; t++) {
-                const int r0 = t * range;
-                const int nr = host[i].rows - r0 < range ? host[i].rows - r0 : range;
-                weight.push_back((int64_t)nr * host[i].cols + 4096);  // + a fixed per-task cost
+                const int nr = host[i].rows - t * unit < unit ? host[i].rows - t * unit : unit;
+                weight.push_back((int64_t)nr * host[i].cols + 16384);
             }
         }
-        const int tasks = prefix.back();
-        const int grid = tasks < wgs ? tasks : wgs;
+        const int units = prefix.back();
+        const int grid = units < wgs ? units : wgs;
         int64_t total_w = 0;
         for (int64_t w : weight) total_w += w;
-        // contiguous shares of about equal weight; every workgroup gets at least one task
-        wg_first.assign(grid + 1, tasks);
+        wg_first.assign(grid + 1, units);
         wg_first[0] = 0;
-        int64_t acc = 0;  // weight of tasks [0, t)
+        int64_t acc = 0;  // weight of units [0, t)
         int t = 0;
         for (int g = 1; g < grid; g++) {
-            const int lo = wg_first[g - 1] + 1, hi = tasks - (grid - g);
+            const int lo = wg_first[g - 1] + 1, hi = units - (grid - g);
             while (t < hi && (t < lo || acc * grid < total_w * g)) acc += weight[t++];
             wg_first[g] = t;
         }
         d.grid = grid;
-        d.range_rows = range;
+        d.max_units = max_units;
         d.image_bytes = max_image;
-        d.lds_bytes = max_image + range * max_batch * 4;
     }
 
     const size_t bytes_table = sizeof(Problem) * host.size();
@@ -537,10 +566,10 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
     char *base = nullptr;
     if (hipError_t e = hipMalloc(&base, bytes_table + bytes_prefix + bytes_wg + 64)) return e;
     d.problems = reinterpret_cast<Problem *>(base);
-    d.task_prefix = reinterpret_cast<int *>(base + bytes_table);
+    d.unit_prefix = reinterpret_cast<int *>(base + bytes_table);
     d.wg_first = reinterpret_cast<int *>(base + bytes_table + bytes_prefix);
     hipError_t e = hipMemcpy(d.problems, host.data(), bytes_table, hipMemcpyHostToDevice);
-    if (!e) e = hipMemcpy(d.task_prefix, prefix.data(), bytes_prefix, hipMemcpyHostToDevice);
+    if (!e) e = hipMemcpy(d.unit_prefix, prefix.data(), bytes_prefix, hipMemcpyHostToDevice);
     if (!e && bytes_wg) e = hipMemcpy(d.wg_first, wg_first.data(), bytes_wg, hipMemcpyHostToDevice);
     if (e) {
         (void)hipFree(base);
@@ -555,10 +584,11 @@ hipError_t plan_device_launch(const PlanDevice &plan, hipStream_t s) {
         return launch_gemv_rowwave_f16_table(plan.problems, plan.count, plan.max_rows, plan.max_batch, 128, s);
     Sched sc{};
     sc.table = plan.problems;
-    sc.task_prefix = plan.task_prefix;
+    sc.unit_prefix = plan.unit_prefix;
     sc.wg_first = plan.wg_first;
     sc.count = plan.count;
-    sc.range_rows = plan.range_rows;
+    sc.max_units = plan.max_units;
+    sc.max_batch = plan.max_batch;
     sc.image_bytes = plan.image_bytes;
     Problem none{};
     if (plan.wide)

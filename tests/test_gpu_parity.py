@@ -281,6 +281,43 @@ def test_linear_plan_matches_single_calls(dev, oracle):
     plan.close()
 
 
+def test_linear_plan_model_sweep_every_row(dev, oracle):
+    """A LLaMA-1B-shaped sweep (8 layers x 7 matrices in one launch): every output row of every
+    problem must equal what the single-call operator gives for that matrix (same kernel, fixed
+    summation order: bit-identical), over several launches; layer 0 is checked against the oracle.
+    Workgroups cross matrix boundaries mid-span here, which small plans do not exercise."""
+    torch, tl = dev
+    shapes = [(2048, 2048), (512, 2048), (512, 2048), (2048, 2048), (8192, 2048), (8192, 2048), (2048, 8192)]
+    probs, host = [], []
+    for layer in range(8):
+        for k, (rows, cols) in enumerate(shapes):
+            nz, sg, s, x = synth.problem(7000 + 10 * layer + k, rows, cols, unit_rms=True)
+            y = torch.zeros((1, rows), dtype=torch.float16, device="cuda")
+            probs.append((up(torch, nz), up(torch, sg), up(torch, s), up(torch, x.reshape(1, -1)), y, rows, cols, 1))
+            host.append((nz, sg, s, x))
+    singles = []
+    for (dnz, dsg, ds, dx, _, rows, cols, _) in probs:
+        y1 = torch.zeros(rows, dtype=torch.float16, device="cuda")
+        tl.ternary_gemv(dnz, dsg, ds, dx, y1, rows, cols, 128)
+        singles.append(y1)
+    torch.cuda.synchronize()
+    for k in range(len(shapes)):
+        nz, sg, s, x = host[k]
+        ref = oracle.gemv_f64(nz, sg, s.view(np.uint16), x.view(np.uint16))
+        assert_close(oracle, singles[k].cpu().numpy().astype(np.float64), ref, what=f"layer0 matrix {k}")
+    plan = tl.LinearPlan(probs)
+    for launch in range(4):
+        for p in probs:
+            p[4].fill_(float("nan"))
+        plan.launch()
+        torch.cuda.synchronize()
+        for k, (p, y1) in enumerate(zip(probs, singles)):
+            got = p[4][0].cpu().numpy()
+            assert np.array_equal(got.view(np.uint16), y1.cpu().numpy().view(np.uint16)), \
+                f"launch {launch} problem {k}: plan and single call differ"
+    plan.close()
+
+
 # ---------------------------------------------- full-size, size-independent
 def test_full_size_properties_8b(dev, oracle):
     """LLaMA-3-8B gate_proj (14336 x 4096) at full size: sampled rows against the oracle, plus

@@ -146,6 +146,8 @@ def main():
                     help="plan: the whole sweep as one launch; calls: one operator call per matrix")
     ap.add_argument("--matrices", default="", help='per-layer matrix list "ROWSxCOLS,..." instead of the model\'s')
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a 1 GiB -> 1 GiB elementwise copy kernel (reference for HBM byte counters)")
     ap.add_argument("--seed", type=int, default=20240611)
     args = ap.parse_args()
     for item in filter(None, args.matrices.split(",")):
@@ -198,6 +200,14 @@ def main():
     dev_ms = ev0.elapsed_time(ev1)
     ms_per_step = dev_ms / args.steps
     gbps = sweep_bytes / (ms_per_step * 1e-3) / 1e9
+
+    if args.copy_calibration:
+        src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.mul(src, 1.0, out=dst)  # vectorized elementwise kernel: reads 2^30 B, writes 2^30 B
+        torch.cuda.synchronize()
+        del src, dst
 
     from oracle import oracle as orc
     if not os.path.exists(orc.LIB):

@@ -239,16 +239,17 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
 
         const int r_begin = task_first_row;
         const int r_end = min(p.rows, r_begin + n_units * kUnitRows);
-        // Each wave owns a quarter of the task's rows and walks them once per slice, so the B
-        // operands change only between such walks and no partial sum is shared between waves.
-        const int rows_per_wave = n_units * (kUnitRows / kNW);  // a multiple of kRows * kTilesAhead
-        const int w_begin = r_begin + wave * rows_per_wave;
-        const int w_rows = max(0, min(r_end - w_begin, rows_per_wave));
-        const int n_rb = (w_rows + G::kRows - 1) / G::kRows;        // live tiles per walk
-        const int n_slots = (n_rb + kTilesAhead - 1) / kTilesAhead * kTilesAhead;
-        // fixed per-wave area (sized for the longest task): waves run through tasks independently
-        float *my_part = partial + (size_t)wave * (sc.max_units * (kUnitRows / kNW)) * sc.max_batch;
-        for (int k = lane; k < rows_per_wave * p.batch; k += kWave) my_part[k] = 0.0f;
+        // The task's rows are cut into kNW chunks; a "walk" is one chunk under one slice (the B
+        // operands stay put during a walk). Walks are numbered chunk-major, slice-minor and dealt to
+        // the waves round-robin, so at any time the waves of a workgroup work on neighbouring
+        // slices of the same rows: the cache lines of a row (masks and, above all, the 2-byte
+        // scales) are fetched from HBM once and shared, not once per slice.
+        // chunk size: a quarter of the rows that exist, rounded up to whole groups of kTilesAhead tiles
+        const int chunk_rows = ((r_end - r_begin + kNW - 1) / kNW + kUnitRows / kNW - 1) / (kUnitRows / kNW) * (kUnitRows / kNW);
+        const int n_walks = kNW * slices;
+        const int my_walks = slices;  // walks wave, wave + kNW, ...
+        float *my_part = partial + (size_t)wave * (sc.max_units * kUnitRows) * sc.max_batch;
+        for (int k = lane; k < n_units * kUnitRows * p.batch; k += kWave) my_part[k] = 0.0f;
 
         // ---- which operand lanes are live, and what each lane loads
         int bcol;       // batch column of this lane's D column
@@ -301,15 +302,25 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
             return t;
         };
 
-        if (n_rb > 0) {
-            // Load cursor: slot j of a walk reads tile min(j, n_rb - 1) (slots past the live tiles
-            // re-read the last one; their results are dropped). It runs kTilesAhead slots ahead of
-            // the compute loop, across walks; past the last walk it parks.
-            int l_slice = 0, l_slot = 0;
+        // rows of chunk c that exist, as a number of tiles; slots round that up to whole groups of
+        // kTilesAhead (slots past the live tiles re-read the last one, their results are dropped)
+        auto chunk_tiles = [&](int c) -> int {
+            const int rows_c = max(0, min(r_end - (r_begin + c * chunk_rows), chunk_rows));
+            return (rows_c + G::kRows - 1) / G::kRows;
+        };
+        const int n_slots = chunk_rows / G::kRows;  // a multiple of kTilesAhead
+
+        {
+            // Load cursor over this wave's walks; it runs kTilesAhead slots ahead of the compute
+            // loop, across walks. Walks of chunks without rows are skipped by both cursors alike.
+            int l_walk = wave, l_slot = 0;
             auto next_load = [&]() -> Tile<G> {
-                const Tile<G> t = load_tile(min(l_slice, slices - 1),
-                                            w_begin + min(l_slot, n_rb - 1) * G::kRows);
-                if (++l_slot == n_slots) { l_slot = 0; l_slice++; }
+                // past the last walk the cursor parks on the wave's last tile
+                const int w_ = min(l_walk, n_walks - kNW + wave);
+                const int c = w_ / slices, sl = w_ - c * slices;
+                const int live_tiles = max(chunk_tiles(c), 1);
+                const Tile<G> t = load_tile(sl, r_begin + c * chunk_rows + min(l_slot, live_tiles - 1) * G::kRows);
+                if (++l_slot == n_slots) { l_slot = 0; l_walk += kNW; }
                 return t;
             };
             Tile<G> ring[kTilesAhead];
@@ -323,7 +334,11 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
             // lanes whose result row (li & 3) is odd / is 2 or 3 (wide tiles pick one of four D rows)
             const uint64_t odd_lanes = __builtin_amdgcn_ballot_w64((li & 1) != 0);
             const uint64_t hi_lanes = __builtin_amdgcn_ballot_w64((li & 2) != 0);
-            for (int slice = 0; slice < slices; slice++) {
+            for (int wi = 0; wi < my_walks; wi++) {
+                const int walk = wave + wi * kNW;
+                const int chunk = walk / slices, slice = walk - chunk * slices;
+                const int c_begin = r_begin + chunk * chunk_rows;
+                const int n_rb = chunk_tiles(chunk);  // live tiles of this walk (0: nothing to add)
                 // this slice's activations become the B operands. Every lane reads (no branch): the
                 // idle lanes read the zero operand with stride 0.
                 u4 B[kMfmaPerTile];
@@ -355,7 +370,7 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
                         x = dpp_add<kQuadSwap2>(x);
                         x = dpp_add<kRowHalfMirror>(x);
                         x = dpp_add<kRowMirror>(x);
-                        if (li == 0 && lq >= sh && live) my_part[rb - sh - w_begin + lq] += x;
+                        if (li == 0 && lq >= sh && live) my_part[rb - sh - r_begin + lq] += x;
                     } else {
                         float r[4];
 #pragma unroll
@@ -369,7 +384,7 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
 #pragma unroll
                             for (int v = 0; v < 4; v++)
                                 if (4 * lq + v >= sh)
-                                    my_part[(size_t)(rb - sh - w_begin + 4 * lq + v) * p.batch + bcol] += r[v];
+                                    my_part[(size_t)(rb - sh - r_begin + 4 * lq + v) * p.batch + bcol] += r[v];
                         }
                     }
                 };
@@ -379,7 +394,7 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
                 for (int j = 0; j < n_slots; j += kTilesAhead) {
 #pragma unroll
                     for (int k = 0; k < kTilesAhead; k++) {
-                        process(ring[k], w_begin + min(j + k, n_rb - 1) * G::kRows, j + k < n_rb);
+                        process(ring[k], c_begin + min(j + k, max(n_rb, 1) - 1) * G::kRows, j + k < n_rb);
                         ring[k] = next_load();
                         // keep the scheduler from interleaving whole tiles: that would need the
                         // registers of several decodes at once and cost a resident wave per SIMD
@@ -387,12 +402,21 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
                     }
                 }
             }
-            // ------------------------------------------------ this wave's rows are complete: store fp16
-            for (int idx = lane; idx < w_rows * p.batch; idx += kWave) {
-                const int b = idx / w_rows, rl = idx - b * w_rows;
-                p.y[(size_t)b * p.rows + w_begin + rl] = f2h(my_part[(size_t)rl * p.batch + b] * fscale[b]);
+        }
+        __syncthreads();
+        // ------------------------------------------------ add the waves' partial sums in wave order, store fp16
+        {
+            const int nrows = r_end - r_begin;
+            const size_t wave_stride = (size_t)(sc.max_units * kUnitRows) * sc.max_batch;
+            for (int idx = tid; idx < nrows * p.batch; idx += kThreads) {
+                const int b = idx / nrows, rl = idx - b * nrows;
+                float sum = 0.0f;
+#pragma unroll
+                for (int w = 0; w < kNW; w++) sum += partial[w * wave_stride + (size_t)rl * p.batch + b];
+                p.y[(size_t)b * p.rows + r_begin + rl] = f2h(sum * fscale[b]);
             }
         }
+        __syncthreads();
     }
 }
 
@@ -451,18 +475,18 @@ int image_bytes_of(int cols, int batch) {
 // Geometry limits: a tile must fit inside the matrix (edge tiles are moved back, not clipped).
 bool wide_ok(const Problem &p) {
     return p.batch == 1 && p.rows >= 16 && p.cols >= Wide::kCols &&
-           image_bytes_of<Wide>(p.cols, 1) + range_unit<Wide>() * 4 <= kLdsLimit;
+           image_bytes_of<Wide>(p.cols, 1) + kNW * range_unit<Wide>() * 4 <= kLdsLimit;
 }
 bool tall_ok(const Problem &p) {
     return p.batch >= 1 && p.batch <= kMaxBatch && p.rows >= 16 && p.cols >= Tall::kCols &&
-           image_bytes_of<Tall>(p.cols, p.batch) + range_unit<Tall>() * p.batch * 4 <= kLdsLimit;
+           image_bytes_of<Tall>(p.cols, p.batch) + kNW * range_unit<Tall>() * p.batch * 4 <= kLdsLimit;
 }
 
 constexpr int kMaxTaskUnits = 10;  // longer tasks amortise the per-slice operand reload
 
 // units per task that the partial-sum area can hold
 int max_units_for(int image_bytes, int batch, int unit) {
-    const int room_rows = (kLdsLimit - image_bytes) / (batch * 4);
+    const int room_rows = (kLdsLimit - image_bytes) / (kNW * batch * 4);  // one partial sum per wave and row
     const int n = room_rows / unit;
     return n > kMaxTaskUnits ? kMaxTaskUnits : n;
 }
@@ -487,7 +511,7 @@ hipError_t launch_gemv_mfma(const Problem &p, hipStream_t s) {
     const int wgs = (wide ? Wide::kWgPerCu : Tall::kWgPerCu) * di->cus;
     const int units = (p.rows + unit - 1) / unit;
     const int grid = units < wgs ? units : wgs;
-    const size_t lds = (size_t)sc.image_bytes + (size_t)sc.max_units * unit * p.batch * 4;
+    const size_t lds = (size_t)sc.image_bytes + (size_t)kNW * sc.max_units * unit * p.batch * 4;
     if (wide)
         gemv_mfma_kernel<Wide><<<grid, kThreads, lds, s>>>(p, sc);
     else
@@ -528,7 +552,7 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
 
     std::vector<int> prefix(host.size() + 1, 0), wg_first;
     if (d.use_mfma) {
-        d.lds_bytes = max_image + max_units * unit * max_batch * 4;
+        d.lds_bytes = max_image + kNW * max_units * unit * max_batch * 4;
         const int per_cu = d.wide ? resident_wgs<Wide>(d.lds_bytes) : resident_wgs<Tall>(d.lds_bytes);
         const int wgs = per_cu * di->cus;
         // weight of every unit: its weights plus a fixed cost; then contiguous spans of about equal

@@ -22,6 +22,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes one launch of the default workload moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by
+# a copy kernel of known size (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); valid for the default workload only.
+DEFAULT_WORKLOAD_TRAFFIC_BYTES = 1982129050
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 SHAPES = {
@@ -186,6 +189,8 @@ def main():
                     tl.ternary_gemm(x, nz, sg, sc, y, batch, rows, cols, 128)
         launches_per_step = len(problems)
 
+    default_workload = (args.model == "llama8b" and not CUSTOM and args.batch == 1 and args.mode == "plan"
+                        and layers == SHAPES["llama8b"][4] and args.p_zero == 0.42)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -232,7 +237,8 @@ def main():
         "parity_max_rel_sampled": parity,
         "roofline": {
             "bound": "hbm", "achieved": round(gbps, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(gbps / HBM_PEAK_GBS, 4), "traffic": None,
+            "frac": round(gbps / HBM_PEAK_GBS, 4),
+            "traffic": DEFAULT_WORKLOAD_TRAFFIC_BYTES if default_workload else None,
             "kernel": "tllm::gemv_mfma_kernel" if args.mode == "plan" else "per-matrix launches",
             "bytes_per_launch": sweep_bytes // launches_per_step,
         },

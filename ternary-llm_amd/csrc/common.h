@@ -53,6 +53,10 @@ hipError_t launch_quantize_absmax_i8(const uint16_t *x, int8_t *q, float *scale,
 bool gemv_mfma_supports(const Problem &p, int group);
 hipError_t launch_gemv_mfma(const Problem &p, hipStream_t s);
 
+// 128-group MFMA GEMM for M >= 16 (gemm_mfma.hip); Problem.batch is M, rows is N, cols is K.
+bool gemm_mfma_supports(const Problem &p, int group);
+hipError_t launch_gemm_mfma(const Problem &p, hipStream_t s);
+
 // Picks the kernel for one linear (fast 128-group paths when they apply, else the row-wave kernel).
 hipError_t dispatch_linear(const Problem &p, int group, hipStream_t s);
 

@@ -6,6 +6,7 @@ namespace tllm {
 hipError_t dispatch_linear(const Problem &p, int group, hipStream_t s) {
     if (group != 128) return launch_gemv_rowwave_f16(p, group, s);
     if (gemv_mfma_supports(p, group)) return launch_gemv_mfma(p, s);
+    if (gemm_mfma_supports(p, group)) return launch_gemm_mfma(p, s);
     // wider batches: four activation rows at a time through the same kernel
     for (int b0 = 0; b0 < p.batch; b0 += TLLM_MAX_PLAN_BATCH) {
         Problem q = p;

@@ -5,20 +5,26 @@
 // Here the product scale * w is formed exactly in fp16 (w in {-1,0,+1}), so the only difference to
 // the reference is the order of the fp32 additions.
 //
-// Tiling. A workgroup (4 waves, 2 x 2) computes BM activation rows x 128 weight rows. Per stage of
-// 64 columns of K:
-//   * activations: BM x 64 fp16 come from global memory into registers, are re-paired so that dword
-//     u of every 32-column block holds columns (u, u+16), and go to LDS;
-//   * weights: each thread decodes one 32-bit mask word pair of one weight row. One v_bitop3 puts the
-//     2-bit field (negative, non-zero) of every even/odd weight in place; shifted to the top of an
-//     fp16 half that field IS the number 0, +2.0 or -2.0 (bit 15 = sign, bit 14 = exponent MSB), so
-//     a packed shift, an AND and a packed fp16 multiply by the group scale give two elements
-//     +-2*scale: 1.6 vector operations per weight, once per workgroup. The factor 2 is undone on
-//     the fp32 accumulators at the end (exact);
-//   * each wave multiplies its 64 weight rows x BM/2 activation rows with v_mfma_f32_16x16x32_f16,
-//     operands read from LDS as 16-byte chunks (XOR-swizzled by row against bank conflicts).
-// Global loads for the next stage are issued before the MFMAs of the current one; LDS is double
-// buffered, one barrier per stage.
+// Tiling. A workgroup (4 waves) computes 128 weight rows x BM activation rows; every wave owns all
+// 128 weight rows and BM/4 activation rows of its own. Per stage of 64 columns of K:
+//   * weights: each thread decodes one 32-bit mask word pair of one weight row into LDS. One
+//     v_bitop3 puts the 2-bit field (negative, non-zero) of every even/odd weight in place, two
+//     v_perm gather the fields of weights (2f, 2f+1) into the two halves of one dword; shifted to
+//     the top of an fp16 half that field IS the number 0, +2.0 or -2.0 (bit 15 = sign, bit 14 =
+//     exponent MSB), so a packed shift, an AND and a packed fp16 multiply by the group scale give
+//     two elements +-2*scale: 1.7 vector operations per weight, once per workgroup. The factor 2
+//     is undone on the fp32 accumulators at the end (exact);
+//   * everything that comes from global memory (activations, mask words, scales) is written into
+//     LDS by the load instruction itself (global_load_lds), two to three stages ahead, without
+//     passing through registers. Activations are private to a wave: lane p of a load asks for the
+//     16-byte chunk that belongs at byte 16 p of the destination block under the row swizzle, so
+//     every load reads eight full 128-byte lines. (Loading the MFMA operand straight into
+//     registers instead needs 16 different rows per 16 lanes and was 2.5 times slower.)
+//   * each wave multiplies with v_mfma_f32_16x16x32_f16; inside a stage the MFMA with index ks
+//     sums columns 16q + 8ks .. + 7 for lane quad q (both operands use the same assignment, so the
+//     sum over the stage is complete); operands come from LDS as 16-byte chunks, XOR-swizzled by
+//     row against bank conflicts.
+// Three LDS buffers per operand, one barrier per stage; the loop body spells out the pipeline.
 #include "common.h"
 
 namespace tllm {
@@ -29,169 +35,243 @@ typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 typedef uint16_t us2 __attribute__((ext_vector_type(2)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(1))) const u4 GU4;
-typedef __attribute__((address_space(1))) const uint32_t GU32;
-typedef __attribute__((address_space(1))) const uint16_t GU16;
 
 constexpr int kBN = 128;     // weight rows per workgroup
 constexpr int kBK = 64;      // K columns per stage (two MFMA steps of 32)
 constexpr int kThreads = 256;
 constexpr int kRowBytes = kBK * 2;  // one LDS row: 64 fp16 = 8 chunks of 16 bytes
+constexpr int kNF = kBN / 16;       // MFMA row fragments per wave
+constexpr int kWBytes = kBN * kRowBytes;
 
-// byte offset of 16-byte chunk c (0..7) of row r inside a [rows][64] fp16 LDS tile
+// byte offset of 16-byte chunk c (0..7) of row r inside the [128][64] fp16 LDS tile
 __device__ __forceinline__ int chunk_off(int r, int c) { return r * kRowBytes + ((c ^ (r & 7)) << 4); }
 
-// 32 weights (one mask word pair) -> 16 dwords; dword u holds weights (u, u + 16) as +-2*scale / 0.
-__device__ __forceinline__ void decode_scaled(uint32_t nz, uint32_t sg, uint32_t scale_pair, uint32_t out[16]) {
-    const uint32_t neg = nz & ~sg;
+// Decoder of 32 weights (one mask word pair) into 16 dwords; dword d holds weights (2d, 2d + 1) as
+// +-2*scale / 0. Split in steps so that the caller can spread the work between MFMAs.
+struct Decoder {
     uint32_t q[2];
-    // field (negative, non-zero) of weight 2f+z at bits (2f+1, 2f) of q[z]:  (a & c) | (b & ~c), c = 0xAAAAAAAA
-    q[0] = __builtin_amdgcn_bitop3_b32(neg << 1, nz, 0xAAAAAAAAu, 0xE4);
-    q[1] = __builtin_amdgcn_bitop3_b32(neg, nz >> 1, 0xAAAAAAAAu, 0xE4);
-    const h2 sp = __builtin_bit_cast(h2, scale_pair);
-#pragma unroll
-    for (int z = 0; z < 2; z++) {
-#pragma unroll
-        for (int f = 0; f < 8; f++) {
-            us2 v = __builtin_bit_cast(us2, q[z]);
-            v = v << (uint16_t)(14 - 2 * f);  // both halves: field f (and f + 8) to bits 15:14
-            const uint32_t top = __builtin_bit_cast(uint32_t, v) & 0xC000C000u;  // 0, +2.0 or -2.0
-            out[2 * f + z] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, top) * sp);
-        }
+    h2 sp;
+    __device__ __forceinline__ void begin(uint32_t nz, uint32_t sg, uint32_t scale) {
+        const uint32_t neg = nz & ~sg;
+        // field (negative, non-zero) of weight 2f+z at bits (2f+1, 2f) of t[z]:  (a & c) | (b & ~c), c = 0xAAAAAAAA
+        const uint32_t t0 = __builtin_amdgcn_bitop3_b32(neg << 1, nz, 0xAAAAAAAAu, 0xE4);
+        const uint32_t t1 = __builtin_amdgcn_bitop3_b32(neg, nz >> 1, 0xAAAAAAAAu, 0xE4);
+        q[0] = __builtin_amdgcn_perm(t1, t0, 0x05040100u);  // low half: weights 0,2,..,14; high half: 1,3,..,15
+        q[1] = __builtin_amdgcn_perm(t1, t0, 0x07060302u);  // the same for weights 16..31
+        sp = __builtin_bit_cast(h2, scale | (scale << 16));
     }
-}
+    // dword d (0..15)
+    __device__ __forceinline__ uint32_t dword(int d) const {
+        us2 v = __builtin_bit_cast(us2, q[d >> 3]);
+        v = v << (uint16_t)(14 - 2 * (d & 7));  // field of both halves to bits 15:14
+        const uint32_t top = __builtin_bit_cast(uint32_t, v) & 0xC000C000u;  // 0, +2.0 or -2.0
+        return __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, top) * sp);
+    }
+};
 
-template <int BM>
+constexpr int kBufs = 3;  // LDS buffers per operand (stages in flight)
+
+template <int MF>  // MFMA column fragments (16 activation rows each) per wave
 __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
     const uint16_t *__restrict__ A, const uint32_t *__restrict__ nzB, const uint32_t *__restrict__ sgB,
     const uint16_t *__restrict__ scB, uint16_t *__restrict__ C, int M, int N, int K) {
-    constexpr int kWM = BM / 2;          // activation rows per wave
-    constexpr int kMF = kWM / 16;        // MFMA column fragments per wave
-    constexpr int kNF = 4;               // MFMA row fragments per wave (64 weight rows)
-    constexpr int kAUnits = BM * 4 / kThreads;  // (row, k-unit) pairs of the activation tile per thread
+    constexpr int kWM = MF * 16;             // activation rows per wave
+    constexpr int BM = 4 * kWM;
+    constexpr int kActWave = kWM * kRowBytes;  // bytes of one wave's activation tile per stage
+    constexpr int kActBytes = 4 * kActWave;
+    constexpr int kActBase = kBufs * kWBytes;  // weights buffers first, activation buffers behind them
+    constexpr int kMaskBase = kActBase + kBufs * kActBytes;  // raw mask words and scales: 3 planes of 1 KB per buffer
+    constexpr int kMaskBytes = 3 * 1024;
+    constexpr int kDma = kWM / 8;              // direct-to-LDS loads per wave and stage (8 rows of 128 bytes each)
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    constexpr int kABytes = BM * kRowBytes, kWBytes = kBN * kRowBytes;
-    // buffer b: activations at b * (kABytes + kWBytes), weights right behind them
+    typedef __attribute__((address_space(3))) unsigned char LB;
+    LB *lds_dma = (LB *)lds;  // the same memory as a local-address-space pointer, for the direct loads
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lq = lane >> 4;
-    const int wn = wave & 1, wm = wave >> 1;  // wave position: weight-row half, activation-row half
 
     // tile coordinates: consecutive workgroups share the weight tile (same n0), so it stays in L2
     const int m_tiles = (M + BM - 1) / BM;
     const int n0 = (blockIdx.x / m_tiles) * kBN;
-    const int m0 = (blockIdx.x % m_tiles) * BM;
+    const int m0 = (blockIdx.x % m_tiles) * BM + wave * kWM;
     const int words = K / 32, groups = K / 128;
+    const int last = K / kBK - 1;  // index of the last stage
 
-    // ---- what this thread stages per 64-column stage
-    // activations: unit (row r, u4 pair p): global chunks (p&1) + 4*(p>>1) and that + 2 of row r
-    //   p = 0: columns 0-7 & 16-23 -> LDS chunks 0,1;  p = 1: 8-15 & 24-31 -> chunks 2,3;  p = 2,3: same in the second 32
-    int a_row[kAUnits], a_p[kAUnits];
-    const GU4 *a_src[kAUnits];
-    bool a_ok[kAUnits];
+    // activations: load t of a stage brings rows 8t .. 8t+7 of the wave's tile, 128 bytes each, straight
+    // into LDS. The hardware puts lane p's 16 bytes at byte 16 p of the 1 KB block, so lane p asks for
+    // the chunk that belongs there under the row swizzle: row p / 8, chunk (p % 8) ^ (p / 8).
+    // Rows past M re-read row M-1; their results are not stored.
+    typedef __attribute__((address_space(1))) const unsigned char GB;
+    GB *a_src[kDma];
 #pragma unroll
-    for (int i = 0; i < kAUnits; i++) {
-        const int unit = tid + i * kThreads;
-        a_row[i] = unit >> 2;
-        a_p[i] = unit & 3;
-        const int gm = m0 + a_row[i];
-        a_ok[i] = gm < M;
-        const int col = (a_p[i] >> 1) * 32 + (a_p[i] & 1) * 8;
-        a_src[i] = reinterpret_cast<const GU4 *>((__attribute__((address_space(1))) const uint16_t *)A +
-                                                 (size_t)(a_ok[i] ? gm : 0) * K + col);
+    for (int t = 0; t < kDma; t++) {
+        const int gm = min(m0 + 8 * t + (lane >> 3), M - 1);
+        a_src[t] = (GB *)A + ((size_t)gm * K + 8 * ((lane & 7) ^ (lane >> 3))) * 2;
     }
     // weights: row w_row, 32-column word w_word of the stage
     const int w_row = tid >> 1, w_word = tid & 1;
     const int gn = min(n0 + w_row, N - 1);
-    const GU32 *nz_src = (GU32 *)nzB + (size_t)gn * words + w_word;
-    const GU32 *sg_src = (GU32 *)sgB + (size_t)gn * words + w_word;
-    const GU16 *sc_src = (GU16 *)scB + (size_t)gn * groups;
+    GB *nz_src = (GB *)nzB + ((size_t)gn * words + w_word) * 4;
+    GB *sg_src = (GB *)sgB + ((size_t)gn * words + w_word) * 4;
+    // the scale of group g travels as the aligned dword that contains it; sc_half picks the half
+    GB *sc_src = (GB *)scB + (size_t)gn * groups * 2;
+    const int w_off = chunk_off(w_row, w_word * 4);      // chunk c of the word: w_off ^ (c << 4)
+    const int fr_off = chunk_off(li, 2 * lq);            // fragment i, step ks: (fr_off ^ (ks << 4)) + i * 16 rows
 
-    u4 a_lo[kAUnits], a_hi[kAUnits];
-    uint32_t w_nz, w_sg, w_sc;
-    auto fetch = [&](int k0) {
-#pragma unroll
-        for (int i = 0; i < kAUnits; i++) {
-            const u4 z = {0u, 0u, 0u, 0u};
-            a_lo[i] = a_ok[i] ? a_src[i][k0 / 8] : z;
-            a_hi[i] = a_ok[i] ? a_src[i][k0 / 8 + 2] : z;
-        }
-        w_nz = nz_src[k0 / 32];
-        w_sg = sg_src[k0 / 32];
-        w_sc = sc_src[(k0 + 32 * w_word) / 128];
+    struct Masks {
+        uint32_t nz, sg, sc;
     };
-    auto stage = [&](int buf) {
-        unsigned char *As = lds + buf * (kABytes + kWBytes);
-        unsigned char *Ws = As + kABytes;
+    // Mask words and scales also come through LDS: thread t asks for its own three dwords, which the
+    // hardware puts at byte 4 t of each 1 KB plane, and reads them back itself (no barrier involved).
+    auto dma_masks = [&](int buf, int stage) {
+        const int k0 = min(stage, last) * kBK;
+        LB *dst = lds_dma + kMaskBase + buf * kMaskBytes + wave * 256;
+        __builtin_amdgcn_global_load_lds((__attribute__((address_space(1))) const void *)(nz_src + k0 / 8),
+                                         (__attribute__((address_space(3))) void *)dst, 4, 0, 0);
+        __builtin_amdgcn_global_load_lds((__attribute__((address_space(1))) const void *)(sg_src + k0 / 8),
+                                         (__attribute__((address_space(3))) void *)(dst + 1024), 4, 0, 0);
+        const uintptr_t sc_addr = reinterpret_cast<uintptr_t>(sc_src) + (k0 / 128) * 2;
+        __builtin_amdgcn_global_load_lds((__attribute__((address_space(1))) const void *)(sc_addr & ~(uintptr_t)3),
+                                         (__attribute__((address_space(3))) void *)(dst + 2048), 4, 0, 0);
+    };
+    auto read_masks = [&](Masks &w, int buf, int stage) {
+        const unsigned char *src = lds + kMaskBase + buf * kMaskBytes + tid * 4;
+        w.nz = *reinterpret_cast<const uint32_t *>(src);
+        w.sg = *reinterpret_cast<const uint32_t *>(src + 1024);
+        const uint32_t pair = *reinterpret_cast<const uint32_t *>(src + 2048);
+        const uintptr_t sc_addr = reinterpret_cast<uintptr_t>(sc_src) + (min(stage, last) * kBK / 128) * 2;
+        w.sc = (sc_addr & 2) ? pair >> 16 : pair & 0xFFFFu;
+    };
+    auto dma_acts = [&](int buf, int stage) {
+        const int k0 = min(stage, last) * kBK;
 #pragma unroll
-        for (int i = 0; i < kAUnits; i++) {
-            // dwords (a[u], a[u+16]): low halves of (lo, hi) -> even u, high halves -> odd u
-            uint32_t o[8];
+        for (int t = 0; t < kDma; t++)
+            __builtin_amdgcn_global_load_lds(
+                (__attribute__((address_space(1))) const void *)(a_src[t] + k0 * 2),
+                (__attribute__((address_space(3))) void *)(lds_dma + kActBase + buf * kActBytes + wave * kActWave + t * 1024),
+                16, 0, 0);
+    };
+    auto read_w = [&](u4 (&af)[kNF], int buf, int ks) {
+        const unsigned char *Ws = lds + buf * kWBytes + (fr_off ^ (ks << 4));
 #pragma unroll
-            for (int d = 0; d < 4; d++) {
-                o[2 * d] = __builtin_amdgcn_perm(a_hi[i][d], a_lo[i][d], 0x05040100u);
-                o[2 * d + 1] = __builtin_amdgcn_perm(a_hi[i][d], a_lo[i][d], 0x07060302u);
-            }
-            const int c = (a_p[i] >> 1) * 4 + (a_p[i] & 1) * 2;
-            *reinterpret_cast<u4 *>(As + chunk_off(a_row[i], c)) = u4{o[0], o[1], o[2], o[3]};
-            *reinterpret_cast<u4 *>(As + chunk_off(a_row[i], c + 1)) = u4{o[4], o[5], o[6], o[7]};
-        }
-        uint32_t o[16];
-        decode_scaled(w_nz, w_sg, w_sc | (w_sc << 16), o);
+        for (int i = 0; i < kNF; i++) af[i] = *reinterpret_cast<const u4 *>(Ws + i * 16 * kRowBytes);
+    };
+    auto read_a = [&](u4 (&bf)[MF], int buf, int ks) {
+        const unsigned char *As = lds + kActBase + buf * kActBytes + wave * kActWave + (fr_off ^ (ks << 4));
 #pragma unroll
-        for (int c = 0; c < 4; c++)
-            *reinterpret_cast<u4 *>(Ws + chunk_off(w_row, w_word * 4 + c)) =
-                u4{o[4 * c], o[4 * c + 1], o[4 * c + 2], o[4 * c + 3]};
+        for (int j = 0; j < MF; j++) bf[j] = *reinterpret_cast<const u4 *>(As + j * 16 * kRowBytes);
     };
 
-    f4 acc[kNF][kMF];
+    f4 acc[kNF][MF];
 #pragma unroll
     for (int i = 0; i < kNF; i++)
 #pragma unroll
-        for (int j = 0; j < kMF; j++) acc[i][j] = f4{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < MF; j++) acc[i][j] = f4{0.f, 0.f, 0.f, 0.f};
+    auto mfma_row = [&](const u4 &a, const u4 (&bf)[MF], int i) {
+#pragma unroll
+        for (int j = 0; j < MF; j++)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a), __builtin_bit_cast(h8, bf[j]),
+                                                               acc[i][j], 0, 0, 0);
+    };
+    auto decode_all = [&](const Masks &w, int buf) {
+        Decoder d;
+        d.begin(w.nz, w.sg, w.sc);
+        unsigned char *Ws = lds + buf * kWBytes;
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+            *reinterpret_cast<u4 *>(Ws + (w_off ^ (c << 4))) =
+                u4{d.dword(4 * c), d.dword(4 * c + 1), d.dword(4 * c + 2), d.dword(4 * c + 3)};
+    };
 
-    fetch(0);
-    stage(0);
+    // Software pipeline, per stage s (buffer indices modulo 3). Everything that comes from global
+    // memory is written into LDS by the load itself; such loads complete in order, so "at most n
+    // still in flight" is the test for the older ones.
+    //   top:    activations of stage s+2 are requested; the masks of stage s+2 (requested in stage s-3)
+    //           and the fragments of the second half of stage s are read from LDS;
+    //   half 1: MFMAs of the first half; between them the masks are decoded into weight buffer s+2,
+    //           then the masks of stage s+5 are requested into the mask buffer just read;
+    //   middle: fragments of the first half of stage s+1 are read from LDS;
+    //   half 2: MFMAs of the second half; barrier.
+    // The barrier at the end of stage s publishes weight buffer s+2 before its first read (middle of
+    // stage s+1); that buffer was last read at the top of stage s-1. Activation and mask buffers are
+    // private to a wave, ordered by the wave's own waits.
+    Masks w;
+    u4 af0[kNF], af1[kNF], bf0[MF], bf1[MF];
+    dma_acts(0, 0);
+    dma_acts(1, 1);
+#pragma unroll
+    for (int u = 0; u < kBufs; u++) dma_masks(u, u);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    read_masks(w, 0, 0);
+    decode_all(w, 0);
+    read_masks(w, 1, 1);
+    decode_all(w, 1);
+    dma_masks(0, 3);
+    dma_masks(1, 4);
     __syncthreads();
-    const int stages = K / kBK;
-    for (int s = 0; s < stages; s++) {
-        const int buf = s & 1;
-        if (s + 1 < stages) fetch((s + 1) * kBK);
-        const unsigned char *As = lds + buf * (kABytes + kWBytes);
-        const unsigned char *Ws = As + kABytes;
+    read_w(af0, 0, 0);
+    read_a(bf0, 0, 0);
+    for (int s0 = 0; s0 <= last; s0 += kBufs) {
 #pragma unroll
-        for (int ks = 0; ks < 2; ks++) {
-            u4 af[kNF], bf[kMF];
+        for (int u = 0; u < kBufs; u++) {
+            const int s = s0 + u;
+            if (s > last) break;
+            dma_acts((u + 2) % kBufs, s + 2);
+            // masks of stage s+2: requested in stage s-3; newer requests: 2 stages of (kDma + 3), this stage's kDma
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * kDma + 6) : "memory");
+            read_masks(w, (u + 2) % kBufs, s + 2);
+            read_w(af1, u, 1);
+            read_a(bf1, u, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            {
+                // group 0 only multiplies (its operands arrived during the previous stage); groups 1..7
+                // also decode 3,2,2,3,2,2,2 dwords and store every finished 16-byte chunk
+                Decoder d;
+                unsigned char *Ws = lds + ((u + 2) % kBufs) * kWBytes;
+                uint32_t o[16];
+                mfma_row(af0[0], bf0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                d.begin(w.nz, w.sg, w.sc);
 #pragma unroll
-            for (int i = 0; i < kNF; i++)
-                af[i] = *reinterpret_cast<const u4 *>(Ws + chunk_off(wn * 64 + i * 16 + li, ks * 4 + lq));
+                for (int i = 1; i < kNF; i++) {
+                    constexpr int kEnd[kNF] = {0, 3, 5, 7, 10, 12, 14, 16};
+                    mfma_row(af0[i], bf0, i);
 #pragma unroll
-            for (int j = 0; j < kMF; j++)
-                bf[j] = *reinterpret_cast<const u4 *>(As + chunk_off(wm * kWM + j * 16 + li, ks * 4 + lq));
+                    for (int dw = kEnd[i - 1]; dw < kEnd[i]; dw++) o[dw] = d.dword(dw);
 #pragma unroll
-            for (int i = 0; i < kNF; i++)
+                    for (int c = 0; c < 4; c++)
+                        if (kEnd[i - 1] < 4 * c + 4 && 4 * c + 4 <= kEnd[i])
+                            *reinterpret_cast<u4 *>(Ws + (w_off ^ (c << 4))) = u4{o[4 * c], o[4 * c + 1], o[4 * c + 2], o[4 * c + 3]};
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                dma_masks((u + 2) % kBufs, s + 5);
+            }
+            read_w(af0, (u + 1) % kBufs, 0);
+            // the activations of stage s+1 were requested at the top of stage s-1; newer requests: the
+            // masks of that stage (3), this stage's activations (kDma) and masks (3)
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kDma + 6) : "memory");
+            read_a(bf0, (u + 1) % kBufs, 0);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int j = 0; j < kMF; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, af[i]),
-                                                                       __builtin_bit_cast(h8, bf[j]),
-                                                                       acc[i][j], 0, 0, 0);
+            for (int i = 0; i < kNF; i++) mfma_row(af1[i], bf1, i);
+            __builtin_amdgcn_sched_barrier(0);
+            // plain barrier: a fence here would also wait for the requests in flight
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         }
-        if (s + 1 < stages) stage(buf ^ 1);
-        __syncthreads();
     }
 
     // ---- store: lane (lq, li) of fragment (i, j) holds weight rows n .. n+3 for activation row m
     uint16_t *Cg = C;
     const bool vec_store = (N & 3) == 0 && (reinterpret_cast<uintptr_t>(C) & 7) == 0;
 #pragma unroll
-    for (int j = 0; j < kMF; j++) {
-        const int m = m0 + wm * kWM + j * 16 + li;
+    for (int j = 0; j < MF; j++) {
+        const int m = m0 + j * 16 + li;
         if (m >= M) continue;
 #pragma unroll
         for (int i = 0; i < kNF; i++) {
-            const int n = n0 + wn * 64 + i * 16 + 4 * lq;
+            const int n = n0 + i * 16 + 4 * lq;
             uint16_t h[4];
 #pragma unroll
             for (int v = 0; v < 4; v++) h[v] = f2h(acc[i][j][v] * 0.5f);
@@ -208,33 +288,38 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
     }
 }
 
-template <int BM>
+template <int MF>
 hipError_t launch(const Problem &p, hipStream_t s) {
+    constexpr int BM = 64 * MF;
     static bool attr_set[64] = {};
     int dev = 0;
     if (hipError_t e = hipGetDevice(&dev)) return e;
-    const size_t lds = 2 * (size_t)(BM + kBN) * kRowBytes;
+    const size_t lds = kBufs * (size_t)(kWBytes + BM * kRowBytes + 3 * 1024);
     if (dev >= 0 && dev < 64 && !attr_set[dev]) {
-        if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_mfma_kernel<BM>),
+        if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_mfma_kernel<MF>),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
             return e;
         attr_set[dev] = true;
     }
     const int m_tiles = (p.batch + BM - 1) / BM, n_tiles = (p.rows + kBN - 1) / kBN;
-    gemm_mfma_kernel<BM><<<m_tiles * n_tiles, kThreads, lds, s>>>(p.x, p.nz, p.sg, p.scales, p.y, p.batch,
-                                                                  p.rows, p.cols);
+    gemm_mfma_kernel<MF><<<m_tiles * n_tiles, kThreads, lds, s>>>(p.x, p.nz, p.sg, p.scales, p.y, p.batch, p.rows,
+                                                                  p.cols);
     return hipGetLastError();
 }
 
 }  // namespace
 
 bool gemm_mfma_supports(const Problem &p, int group) {
+    // scales are fetched as aligned dwords: the array must start on one and hold an even count
+    if ((reinterpret_cast<uintptr_t>(p.scales) & 3) || (((size_t)p.rows * (p.cols / 128)) & 1)) return false;
     return group == 128 && p.batch >= 16 && p.cols % 128 == 0 && (size_t)p.rows * (p.cols / 32) < ((size_t)1 << 31) &&
            (size_t)p.batch * p.cols < ((size_t)1 << 31);
 }
 
 hipError_t launch_gemm_mfma(const Problem &p, hipStream_t s) {
-    return p.batch > 128 ? launch<256>(p, s) : launch<128>(p, s);
+    if (p.batch > 128) return launch<4>(p, s);
+    if (p.batch > 64) return launch<2>(p, s);
+    return launch<1>(p, s);
 }
 
 }  // namespace tllm

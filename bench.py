@@ -136,6 +136,58 @@ def cpu_baseline(oracle, problems, n_layer_mats, threads, mt_layers=8):
     }
 
 
+MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense FP16 matrix peak
+
+
+def gemm_report(torch, tl, orc, seed, m_list, p_zero=0.42, calls=20):
+    """Prefill GEMM (cfg4): LLaMA-3-8B gate/up 14336x4096 and down 4096x14336, M tokens each.
+    Times `calls` back-to-back launches with events on the launch stream, checks sampled outputs
+    against the FP64 oracle, and reports dense-equivalent 2*M*N*K flops."""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(seed + 4)
+    cases = []
+    for (n, k) in ((14336, 4096), (4096, 14336)):
+        nz, sg = gen_masks(torch, n, k, p_zero, gen)
+        sc = (torch.rand((n, k // 128), device="cuda", generator=gen) * 0.02 + 0.01).to(torch.float16)
+        for m in m_list:
+            a = torch.randn((m, k), device="cuda", generator=gen).to(torch.float16)
+            c = torch.zeros((m, n), dtype=torch.float16, device="cuda")
+            for _ in range(3):
+                tl.ternary_gemm(a, nz, sg, sc, c, m, n, k, 128)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(calls):
+                tl.ternary_gemm(a, nz, sg, sc, c, m, n, k, 128)
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) / calls * 1e3
+            rng = np.random.default_rng(m + n)
+            ms_ = np.unique(rng.integers(0, m, 4))
+            ns_ = np.unique(rng.integers(0, n, 96))
+            ref = orc.gemm_f64(a[ms_].cpu().numpy().view(np.uint16), nz[ns_].cpu().numpy().view(np.uint32),
+                               sg[ns_].cpu().numpy().view(np.uint32), sc[ns_].cpu().numpy().view(np.uint16))
+            full = c.float()
+            tau = float(torch.sqrt(torch.mean(full * full)).item()) / 64.0
+            got = full.cpu().numpy().astype(np.float64)[np.ix_(ms_, ns_)]
+            rel = float((np.abs(got - ref) / np.maximum(np.abs(ref), tau)).max())
+            tflops = 2.0 * m * n * k / us / 1e6
+            cases.append({"M": m, "N": n, "K": k, "us": round(us, 2), "tflops": round(tflops, 1),
+                          "frac_mfma_peak": round(tflops / MFMA_F16_PEAK_TFLOPS, 4), "max_rel_sampled": rel})
+            del a, c, full
+        del nz, sg, sc
+    m512 = [c for c in cases if c["M"] == 512]
+    agg = None
+    if m512:
+        agg = sum(2.0 * c["M"] * c["N"] * c["K"] for c in m512) / sum(c["us"] for c in m512) / 1e6
+    return {"workload": "cfg4: prefill GEMM, LLaMA-3-8B gate/up 14336x4096 and down 4096x14336",
+            "unit": "TFLOP/s (2*M*N*K)", "bound": "mfma", "peak": MFMA_F16_PEAK_TFLOPS,
+            "kernel": "tllm::gemm_mfma_kernel", "calls_timed": calls,
+            "m512_tflops": round(agg, 1) if agg else None,
+            "m512_frac": round(agg / MFMA_F16_PEAK_TFLOPS, 4) if agg else None,
+            "cases": cases}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -151,6 +203,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a 1 GiB -> 1 GiB elementwise copy kernel (reference for HBM byte counters)")
+    ap.add_argument("--gemm-m", default="512", help='token counts M of the prefill GEMM report, e.g. "16,128,512,2048"; "" skips it')
     ap.add_argument("--seed", type=int, default=20240611)
     args = ap.parse_args()
     for item in filter(None, args.matrices.split(",")):
@@ -243,6 +296,9 @@ def main():
             "bytes_per_launch": sweep_bytes // launches_per_step,
         },
     }
+    gemm_m = [int(v) for v in args.gemm_m.split(",") if v.strip()]
+    if gemm_m:
+        out["gemm"] = gemm_report(torch, tl, orc, args.seed, gemm_m, args.p_zero)
     if not args.no_cpu_baseline:
         threads = min(os.cpu_count() or 1, 16)
         out["cpu_baseline"] = cpu_baseline(orc, problems, n_mats, threads)

@@ -317,8 +317,31 @@ bool gemm_mfma_supports(const Problem &p, int group) {
 }
 
 hipError_t launch_gemm_mfma(const Problem &p, hipStream_t s) {
-    if (p.batch > 128) return launch<4>(p, s);
-    if (p.batch > 64) return launch<2>(p, s);
+    // One workgroup occupies a CU (LDS). Taller tiles do more per stage, shorter tiles fill the chip
+    // when there are few of them: pick the height with the smallest (rounds of workgroups over the
+    // CUs) x (time of one stage, measured: 1.2 / 0.83 / 0.65 us for 256 / 128 / 64 activation rows).
+    static int cus[64] = {};
+    int dev = 0;
+    if (hipError_t e = hipGetDevice(&dev)) return e;
+    int n_cu = 256;
+    if (dev >= 0 && dev < 64) {
+        if (!cus[dev]) {
+            if (hipError_t e = hipDeviceGetAttribute(&cus[dev], hipDeviceAttributeMultiprocessorCount, dev)) return e;
+        }
+        n_cu = cus[dev] > 0 ? cus[dev] : 256;
+    }
+    const int n_tiles = (p.rows + kBN - 1) / kBN;
+    const float stage_us[3] = {0.65f, 0.83f, 1.2f};
+    int best = 0;
+    float best_cost = 0.f;
+    for (int c = 0; c < 3; c++) {
+        const int bm = 64 << c;
+        const long wgs = (long)n_tiles * ((p.batch + bm - 1) / bm);
+        const float cost = (float)((wgs + n_cu - 1) / n_cu) * stage_us[c];
+        if (c == 0 || cost < best_cost) best = c, best_cost = cost;
+    }
+    if (best == 2) return launch<4>(p, s);
+    if (best == 1) return launch<2>(p, s);
     return launch<1>(p, s);
 }
 

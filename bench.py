@@ -292,7 +292,8 @@ def main():
             "bound": "hbm", "achieved": round(gbps, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(gbps / HBM_PEAK_GBS, 4),
             "traffic": DEFAULT_WORKLOAD_TRAFFIC_BYTES if default_workload else None,
-            "kernel": "tllm::gemv_mfma_kernel" if args.mode == "plan" else "per-matrix launches",
+            "kernel": ("tllm::gemv_mfma_kernel" if args.batch == 1 else "tllm::gemv_batch_kernel")
+                      if args.mode == "plan" else "per-matrix launches",
             "bytes_per_launch": sweep_bytes // launches_per_step,
         },
     }

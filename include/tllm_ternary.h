@@ -112,7 +112,7 @@ typedef struct tllm_linear_problem {
     int32_t reserved;
 } tllm_linear_problem;
 
-enum { TLLM_MAX_PLAN_BATCH = 4 };
+enum { TLLM_MAX_PLAN_BATCH = 16 };
 
 typedef struct tllm_linear_plan tllm_linear_plan;
 

@@ -53,9 +53,17 @@ hipError_t launch_quantize_absmax_i8(const uint16_t *x, int8_t *q, float *scale,
 bool gemv_mfma_supports(const Problem &p, int group);
 hipError_t launch_gemv_mfma(const Problem &p, hipStream_t s);
 
+// 128-group MFMA kernel for 2..16 activation rows, K a multiple of 512 (gemv_batch.hip).
+bool gemv_batch_supports(const Problem &p, int group);
+hipError_t launch_gemv_batch(const Problem &p, hipStream_t s);
+int gemv_batch_block_rows();
+hipError_t launch_gemv_batch_table(const Problem *table, const int *unit_prefix, const int *wg_first, int grid,
+                                   hipStream_t s);
+
 // 128-group MFMA GEMM for M >= 16 (gemm_mfma.hip); Problem.batch is M, rows is N, cols is K.
 bool gemm_mfma_supports(const Problem &p, int group);
 hipError_t launch_gemm_mfma(const Problem &p, hipStream_t s);
+float gemm_mfma_cost_us(const Problem &p);  // rough time of launch_gemm_mfma, to choose between kernels
 
 // Picks the kernel for one linear (fast 128-group paths when they apply, else the row-wave kernel).
 hipError_t dispatch_linear(const Problem &p, int group, hipStream_t s);
@@ -70,6 +78,7 @@ struct PlanDevice {
     // schedule of the MFMA kernel (use_mfma == false: the row-wave table kernel runs instead)
     bool use_mfma = false;
     bool wide = false;  // 4 x 2048 tiles (every problem at batch 1) instead of 16 x 512
+    bool batch_kernel = false;  // the 2..16-row kernel runs (its blocks are the units below)
     int *unit_prefix = nullptr;
     int *wg_first = nullptr;
     int grid = 0;

@@ -316,19 +316,17 @@ bool gemm_mfma_supports(const Problem &p, int group) {
            (size_t)p.batch * p.cols < ((size_t)1 << 31);
 }
 
-hipError_t launch_gemm_mfma(const Problem &p, hipStream_t s) {
-    // One workgroup occupies a CU (LDS). Taller tiles do more per stage, shorter tiles fill the chip
-    // when there are few of them: pick the height with the smallest (rounds of workgroups over the
-    // CUs) x (time of one stage, measured: 1.2 / 0.83 / 0.65 us for 256 / 128 / 64 activation rows).
+namespace {
+// One workgroup occupies a CU (LDS). Taller tiles do more per stage, shorter tiles fill the chip
+// when there are few of them: take the height with the smallest (rounds of workgroups over the
+// CUs) x (time of one stage, measured: 1.2 / 0.83 / 0.65 us for 256 / 128 / 64 activation rows).
+int choose_height(const Problem &p, float *stage_rounds_us) {
     static int cus[64] = {};
-    int dev = 0;
-    if (hipError_t e = hipGetDevice(&dev)) return e;
-    int n_cu = 256;
-    if (dev >= 0 && dev < 64) {
-        if (!cus[dev]) {
-            if (hipError_t e = hipDeviceGetAttribute(&cus[dev], hipDeviceAttributeMultiprocessorCount, dev)) return e;
-        }
-        n_cu = cus[dev] > 0 ? cus[dev] : 256;
+    int dev = 0, n_cu = 256;
+    if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64) {
+        if (!cus[dev] && hipDeviceGetAttribute(&cus[dev], hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+            cus[dev] = 0;
+        if (cus[dev] > 0) n_cu = cus[dev];
     }
     const int n_tiles = (p.rows + kBN - 1) / kBN;
     const float stage_us[3] = {0.65f, 0.83f, 1.2f};
@@ -340,6 +338,19 @@ hipError_t launch_gemm_mfma(const Problem &p, hipStream_t s) {
         const float cost = (float)((wgs + n_cu - 1) / n_cu) * stage_us[c];
         if (c == 0 || cost < best_cost) best = c, best_cost = cost;
     }
+    if (stage_rounds_us) *stage_rounds_us = best_cost;
+    return best;
+}
+}  // namespace
+
+float gemm_mfma_cost_us(const Problem &p) {
+    float per_stage = 0.f;
+    (void)choose_height(p, &per_stage);
+    return per_stage * (float)(p.cols / kBK) + 5.0f;
+}
+
+hipError_t launch_gemm_mfma(const Problem &p, hipStream_t s) {
+    const int best = choose_height(p, nullptr);
     if (best == 2) return launch<4>(p, s);
     if (best == 1) return launch<2>(p, s);
     return launch<1>(p, s);

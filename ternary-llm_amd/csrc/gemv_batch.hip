@@ -1,0 +1,376 @@
+// Batched decode (2..16 activation rows) on the matrix cores (gfx950), group size 128, K % 512 == 0.
+//
+// Arithmetic (reference kernels/ternary_gemm.cu:106-175 at small M, kernels/ternary_gemv.cu:47-86 per
+// row): y[b, r] = sum_g s[r,g] * sum_{k in g} w[r,k] x[b,k], fp32 accumulation, fp16 store (RNE).
+// The weights are streamed once for all activation rows: HBM-bound like the batch-1 kernel.
+//
+// Dataflow. A workgroup of 4 waves owns a block of up to 256 weight rows and walks K in slices of
+// 512 columns. Per slice the workgroup turns x[0..16, slice] into ready-made MFMA B operands in LDS
+// (power-of-two normalised per activation row and slice, laid out in the element order of the
+// decode below), every wave copies them into 64 registers, and then each wave streams its own tiles
+// of 16 rows x 512 columns: lane (row i, chunk q) loads 16 bytes of each mask plane (one scale group
+// of one row), four lane-row swaps transpose the 4 x 4 (chunk, word) block held by lanes i, i+16,
+// i+32, i+48 so that in each of the four registers all four k-quarters of an MFMA belong to ONE scale
+// group, the 2-bit codes are cut out with one AND per two weights (gemv_layout.h) and 4 x 4
+// v_mfma_f32_16x16x32_f16 give one 16 x 16 result per scale group: rows x activation rows. The fp32
+// group scales multiply whole result tiles; results stay in registers over all slices (every wave
+// owns its rows for the whole of K), so there is no reduction between waves and no atomics.
+// The "+1" of the code c = w + 1 is removed by subtracting the product of an all-zero weight row,
+// computed once per slice with the same instructions (exact zeros stay exact).
+#include "common.h"
+#include "gemv_layout.h"
+
+namespace tllm {
+namespace {
+
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+typedef uint16_t us2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(1))) const u4 GU4;
+typedef __attribute__((address_space(1))) const u2 GU2;
+#define GB __attribute__((address_space(1)))
+
+constexpr int kNW = 8;                          // waves: 4 tile quarters x 2 slice parities
+constexpr int kThreads = kNW * kWave;
+constexpr int kSliceCols = 512;                 // 4 scale groups
+constexpr int kTileRows = 16;
+constexpr int kTilesPerWave = 4;                // tiles of one wave per slice = loads in flight
+constexpr int kBlockRows = 4 * kTilesPerWave * kTileRows;    // 256
+constexpr int kImageBytes = 16 * kSliceCols * 2;             // operands of one slice, 16 activation rows
+
+struct BatchSched {
+    const Problem *table;    // device table, or nullptr: use the by-value problem
+    const int *unit_prefix;  // [count + 1] first block of each problem
+    const int *wg_first;     // [grid + 1] first block of each workgroup
+};
+
+struct Tile {
+    u4 nz, sg;
+};
+struct Scales {
+    u2 sc[4];  // scales of rows 4*lq + v, groups 4*slice .. +3 (fp16 x 4)
+};
+
+__device__ __forceinline__ f4 mfma16(const uint32_t *o, u4 b, f4 c) {
+    const u4 a = {o[0], o[1], o[2], o[3]};
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a), __builtin_bit_cast(h8, b), c, 0, 0, 0);
+}
+
+// Lanes i, i+16, i+32, i+48 hold row q of a 4 x 4 matrix in a[0..3]; afterwards they hold column q.
+__device__ __forceinline__ void transpose4(u4 &a) {
+    auto s0 = __builtin_amdgcn_permlane32_swap(a[0], a[2], false, false);
+    auto s1 = __builtin_amdgcn_permlane32_swap(a[1], a[3], false, false);
+    auto t0 = __builtin_amdgcn_permlane16_swap(s0[0], s1[0], false, false);
+    auto t1 = __builtin_amdgcn_permlane16_swap(s0[1], s1[1], false, false);
+    a = u4{t0[0], t0[1], t1[0], t1[1]};
+}
+
+__global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single, BatchSched sc) {
+    // [buffer][slice parity]: the operands of two neighbouring slices are built per step
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    unsigned char (*image)[2][kImageBytes] = reinterpret_cast<unsigned char (*)[2][kImageBytes]>(lds_raw);
+    // per activation row: 2^(ex + 10) of the slice, 0 for an all-zero slice
+    float (*pow2)[2][16] = reinterpret_cast<float (*)[2][16]>(lds_raw + 4 * kImageBytes);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    // Wave w works on tile quarter w % 4 under the slices of parity w / 4. The two waves that share
+    // their tiles read the two 64-byte halves of every 128-byte line of the mask planes at about the
+    // same time, so each line comes from HBM once (one wave walking all slices fetched it twice).
+    const int wave8 = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave = wave8 & 3;
+    const int parity = wave8 >> 2;
+    const int li = lane & 15;  // MFMA A row / D column (activation row)
+    const int lq = lane >> 4;  // MFMA k quarter / D row quad
+
+    int u = 0, u_end = 0;
+    if (sc.table) {
+        u = sc.wg_first[blockIdx.x];
+        u_end = sc.wg_first[blockIdx.x + 1];
+    } else {
+        const int total = (single.rows + kBlockRows - 1) / kBlockRows;
+        u = (int)((int64_t)total * blockIdx.x / gridDim.x);
+        u_end = (int)((int64_t)total * (blockIdx.x + 1) / gridDim.x);
+    }
+
+    // operands of an all-zero weight row (every code = 1)
+    uint32_t zero_o[16];
+    decode_word(0u, 0u, zero_o);
+
+    int pi = 0;
+    Problem p = single;
+    for (; u < u_end; u++) {
+        int first_unit = 0;
+        if (sc.table) {
+            while (sc.unit_prefix[pi + 1] <= u) pi++;
+            first_unit = sc.unit_prefix[pi];
+            p = sc.table[pi];
+        }
+        const int r0 = (u - first_unit) * kBlockRows;
+        const int n_tiles = (min(kBlockRows, p.rows - r0) + kTileRows - 1) / kTileRows;
+        const int words = p.cols / 32, groups = p.cols / kChunkCols, slices = p.cols / kSliceCols;
+
+        // ---- this wave's tiles: k-th tile is tile number 4k + wave of the block. Tiles past the end
+        // of the block re-read its last tile (not stored); a tile that would pass the end of the
+        // matrix is moved back to end with it, the rows it repeats are not stored.
+        const char GB *nz_g = (const char GB *)p.nz;
+        const char GB *sg_g = (const char GB *)p.sg;
+        const char GB *sc_g = (const char GB *)p.scales;
+        // Addresses: a wave-uniform part per tile (first row) plus one per-lane offset for all tiles.
+        auto tile_first_row = [&](int k, int *skip) -> int {
+            const int rb = r0 + min(4 * k + wave, n_tiles - 1) * kTileRows;
+            const int rbe = min(rb, p.rows - kTileRows);
+            if (skip) *skip = rb - rbe;
+            return rbe;
+        };
+        const uint32_t lane_mask_off = ((uint32_t)li * words + 4u * lq) * 4u;
+        const uint32_t lane_scale_off = (uint32_t)(4 * lq) * groups * 2u;
+        auto load_tile = [&](int k, int slice) -> Tile {
+            Tile t;
+            const size_t base = (size_t)tile_first_row(k, nullptr) * words * 4 + (size_t)slice * 64;
+            t.nz = *reinterpret_cast<const GU4 *>(nz_g + base + lane_mask_off);
+            t.sg = *reinterpret_cast<const GU4 *>(sg_g + base + lane_mask_off);
+            return t;
+        };
+        // the scales (8 bytes per row and slice, mostly cache hits) are asked for one tile ahead only
+        auto load_scales = [&](int k, int slice) -> Scales {
+            Scales t;
+            const size_t base = (size_t)tile_first_row(k, nullptr) * groups * 2 + (size_t)slice * 8;
+#pragma unroll
+            for (int v = 0; v < 4; v++)
+                t.sc[v] = *reinterpret_cast<const GU2 *>(sc_g + base + (size_t)(v * groups) * 2 + lane_scale_off);
+            return t;
+        };
+
+        // ---- activations: thread (row j = tid / 16, segment = tid % 16) owns 32 columns of a slice
+        const int xpar = tid >> 8, xj = (tid >> 4) & 15, xseg = tid & 15;
+        const bool x_live = xj < p.batch;
+        const GU4 *x_src = (const GU4 *)(p.x + (size_t)(x_live ? xj : 0) * p.cols) + xseg * 4;
+        // a slice past the end of an odd number of slices is built as zeros
+        auto load_x = [&](u4 (&xr)[4], int slice) {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                xr[i] = x_live && slice < slices ? x_src[slice * (kSliceCols / 8) + i] : u4{0u, 0u, 0u, 0u};
+        };
+        // builds the operands of one slice: element (chunk c, word q, step t, row j, e) at
+        // ((c*4 + t)*64 + q*16 + j)*16 + 2e bytes: lane (j, q) of MFMA (c, t) reads 16 contiguous bytes
+        auto build_image = [&](const u4 (&xr)[4], int buf) {
+            // largest magnitude of the activation row inside the slice: packed unsigned maximum of the
+            // sign-stripped halves, then across the 16 threads of the row (one DPP row rotation each)
+            us2 m2 = {0, 0};
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    m2 = __builtin_elementwise_max(m2, __builtin_bit_cast(us2, xr[i][e] & 0x7FFF7FFFu));
+            uint32_t m = max((uint32_t)m2[0], (uint32_t)m2[1]);
+            m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x128, 0xF, 0xF, true));  // row_ror:8
+            m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x124, 0xF, 0xF, true));  // row_ror:4
+            m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x122, 0xF, 0xF, true));  // row_ror:2
+            m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x121, 0xF, 0xF, true));  // row_ror:1
+            // amax in [2^ex, 2^(ex+1)); x'' = x * 2^(14-ex) stays below 2^15
+            int ex = 0;
+            if (m >= 0x7C00u) ex = 15;  // inf/nan present: they propagate to the outputs
+            else if (m) ex = (int)((__builtin_bit_cast(uint32_t, h2f((uint16_t)m)) >> 23) & 0xFF) - 127;
+            // The multipliers 2^(14-ex-p), p = 2..10, must be normal fp16 numbers: ex >= -3. Rows with
+            // a smaller maximum are normalised as if it were 2^-3: their multipliers are then >= 2^7,
+            // and multiplying an fp16 number by a power of two >= 1 is exact (no overflow: |x| < 2^-2).
+            const int exl = max(ex, -3);
+            if (xseg == 0) pow2[buf][xpar][xj] = m ? __builtin_bit_cast(float, (uint32_t)(127 + exl + 10) << 23) : 0.0f;
+            uint32_t src[16];
+#pragma unroll
+            for (int d = 0; d < 16; d++) src[d] = xr[d >> 2][d & 3];
+            const int c = xseg >> 2, q = xseg & 3;
+            // Operand t = 2z + h, dword d' holds the elements of decode dword m = 4h + d' (gemv_layout.h):
+            // column 2m + z in its low half, column 2(m + 8) + z in its high half (m = 0: the other
+            // way round); both sit in half z of source dwords m and m + 8. One byte permute and one
+            // packed multiply by 2^(14-ex-p(m)) per dword; the product of an fp16 number and a power of
+            // two is exact or rounded once to nearest even, as in the fp32 route.
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const int z = t >> 1, h = t & 1;
+                u4 v;
+#pragma unroll
+                for (int dq = 0; dq < 4; dq++) {
+                    const int mm = 4 * h + dq;
+                    const uint32_t lo = mm == 0 ? src[8] : src[mm], hi = mm == 0 ? src[0] : src[mm + 8];
+                    const uint32_t pair = __builtin_amdgcn_perm(hi, lo, z ? 0x07060302u : 0x05040100u);
+                    const uint16_t cbits = (uint16_t)((29 - exl - code_shift(mm)) << 10);
+                    const h2 mult = __builtin_bit_cast(h2, (uint32_t)cbits | ((uint32_t)cbits << 16));
+                    v[dq] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, pair) * mult);
+                }
+                *reinterpret_cast<u4 *>(&image[buf][xpar][(((c * 4 + t) * 64) + q * 16 + xj) * 16]) = v;
+            }
+        };
+
+        f4 acc[kTilesPerWave];
+#pragma unroll
+        for (int k = 0; k < kTilesPerWave; k++) acc[k] = f4{0.f, 0.f, 0.f, 0.f};
+
+        const int steps = (slices + 1) / 2;
+        auto my_slice = [&](int step) -> int { return min(2 * step + parity, slices - 1); };  // weights: clamped
+        u4 xr[4];
+        load_x(xr, xpar);
+        Tile ring[kTilesPerWave];
+#pragma unroll
+        for (int k = 0; k < kTilesPerWave; k++) ring[k] = load_tile(k, my_slice(0));
+        Scales sc_next = load_scales(0, my_slice(0));
+
+        for (int st = 0; st < steps; st++) {
+            const int buf = st & 1;
+            const int s = my_slice(st);
+            build_image(xr, buf);
+            if (st + 1 < steps) load_x(xr, 2 * (st + 1) + xpar);
+            // one barrier per step: it publishes buffer `buf`; the other buffer is rewritten only in
+            // the next iteration, after every wave has passed this barrier and so has finished
+            // reading it into registers.
+            __syncthreads();
+            u4 B[16];
+#pragma unroll
+            for (int k = 0; k < 16; k++) B[k] = *reinterpret_cast<const u4 *>(&image[buf][parity][(k * 64 + lane) * 16]);
+            const float scale_j = pow2[buf][parity][li];
+            // the product of an all-zero weight row (the "+1" of every code), formed exactly like a
+            // tile's own product, so that subtracting it leaves exact zeros where the weights are zero
+            f4 bias[4];
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                f4 d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
+                d0 = mfma16(zero_o + 0, B[4 * c + 0], d0);
+                d1 = mfma16(zero_o + 4, B[4 * c + 1], d1);
+                d0 = mfma16(zero_o + 8, B[4 * c + 2], d0);
+                d1 = mfma16(zero_o + 12, B[4 * c + 3], d1);
+                bias[c] = d0 + d1;
+            }
+            const int s_next = my_slice(min(st + 1, steps - 1));
+#pragma unroll
+            for (int k = 0; k < kTilesPerWave; k++) {
+                Tile t = ring[k];
+                const Scales ts = sc_next;
+                // order matters: loads return in order, so the scales (needed by the next tile) are
+                // asked for before the masks of the next slice (needed four tiles from now)
+                sc_next = k + 1 < kTilesPerWave ? load_scales(k + 1, s) : load_scales(0, s_next);
+                ring[k] = load_tile(k, s_next);
+                transpose4(t.nz);
+                transpose4(t.sg);
+                f4 r = {0.f, 0.f, 0.f, 0.f};
+                // the MFMAs of chunk c + 1 are issued before the results of chunk c are touched
+                f4 da[2], db[2];
+                auto issue = [&](int c) {
+                    uint32_t o[16];
+                    decode_word(t.nz[c], t.sg[c], o);
+                    da[c & 1] = mfma16(o + 0, B[4 * c + 0], f4{0.f, 0.f, 0.f, 0.f});
+                    db[c & 1] = mfma16(o + 4, B[4 * c + 1], f4{0.f, 0.f, 0.f, 0.f});
+                    da[c & 1] = mfma16(o + 8, B[4 * c + 2], da[c & 1]);
+                    db[c & 1] = mfma16(o + 12, B[4 * c + 3], db[c & 1]);
+                };
+                auto retire = [&](int c) {
+                    const f4 d = da[c & 1] + db[c & 1] - bias[c];
+#pragma unroll
+                    for (int v = 0; v < 4; v++) {
+                        const uint16_t sbits = (uint16_t)(ts.sc[v][c >> 1] >> (16 * (c & 1)));
+                        r[v] += h2f(sbits) * d[v];
+                    }
+                };
+                issue(0);
+                __builtin_amdgcn_sched_barrier(0);
+                issue(1);
+                __builtin_amdgcn_sched_barrier(0);
+                retire(0);
+                issue(2);
+                __builtin_amdgcn_sched_barrier(0);
+                retire(1);
+                issue(3);
+                __builtin_amdgcn_sched_barrier(0);
+                retire(2);
+                retire(3);
+                acc[k] += r * scale_j;
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+
+        // ---- the odd-slice waves hand their sums to their even-slice partners through LDS (the image
+        // buffers are free once every wave is past its last step), which add and store
+        __syncthreads();
+        float *hand = reinterpret_cast<float *>(&image[0][0][0]) + (size_t)wave * (kTilesPerWave * 4 * kWave);
+        if (parity == 1) {
+#pragma unroll
+            for (int k = 0; k < kTilesPerWave; k++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) hand[(k * 4 + v) * kWave + lane] = acc[k][v];
+        }
+        __syncthreads();
+        // lane (lq, li) holds rows first + 4*lq + v of activation row li
+        if (parity == 0 && li < p.batch) {
+#pragma unroll
+            for (int k = 0; k < kTilesPerWave; k++) {
+                if (4 * k + wave >= n_tiles) continue;
+                int skip = 0;
+                const int first = tile_first_row(k, &skip);
+#pragma unroll
+                for (int v = 0; v < 4; v++)
+                    if (4 * lq + v >= skip)
+                        p.y[(size_t)li * p.rows + first + 4 * lq + v] = f2h(acc[k][v] + hand[(k * 4 + v) * kWave + lane]);
+            }
+        }
+        __syncthreads();  // the next block rewrites the image buffers
+    }
+}
+
+int device_cus() {
+    static int cus[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (!cus[dev]) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) n = 256;
+        cus[dev] = n;
+    }
+    return cus[dev];
+}
+
+}  // namespace
+
+bool gemv_batch_supports(const Problem &p, int group) {
+    return group == 128 && p.batch >= 1 && p.batch <= 16 && p.rows >= kTileRows && p.cols >= kSliceCols &&
+           p.cols % kSliceCols == 0 && (reinterpret_cast<uintptr_t>(p.scales) & 7) == 0 && (size_t)p.rows * (p.cols / 8) < ((size_t)1 << 32) &&
+           (size_t)p.rows * (p.cols / 128) * 2 < ((size_t)1 << 32);
+}
+
+constexpr size_t kLdsBytes = 4 * kImageBytes + 2 * 2 * 16 * sizeof(float);
+
+static hipError_t prepare_kernel() {
+    static bool done[64] = {};
+    int dev = 0;
+    if (hipError_t e = hipGetDevice(&dev)) return e;
+    if (dev < 0 || dev >= 64 || done[dev]) return hipSuccess;
+    if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_batch_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes))
+        return e;
+    done[dev] = true;
+    return hipSuccess;
+}
+
+hipError_t launch_gemv_batch(const Problem &p, hipStream_t s) {
+    if (hipError_t e = prepare_kernel()) return e;
+    const int blocks = (p.rows + kBlockRows - 1) / kBlockRows;
+    const int wgs = device_cus();  // one workgroup of 8 waves per CU
+    BatchSched sc{nullptr, nullptr, nullptr};
+    gemv_batch_kernel<<<blocks < wgs ? blocks : wgs, kThreads, kLdsBytes, s>>>(p, sc);
+    return hipGetLastError();
+}
+
+int gemv_batch_block_rows() { return kBlockRows; }
+
+hipError_t launch_gemv_batch_table(const Problem *table, const int *unit_prefix, const int *wg_first, int grid,
+                                   hipStream_t s) {
+    if (hipError_t e = prepare_kernel()) return e;
+    BatchSched sc{table, unit_prefix, wg_first};
+    Problem none{};
+    gemv_batch_kernel<<<grid, kThreads, kLdsBytes, s>>>(none, sc);
+    return hipGetLastError();
+}
+
+}  // namespace tllm

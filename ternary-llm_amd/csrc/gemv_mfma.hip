@@ -42,7 +42,7 @@ __device__ __forceinline__ __attribute__((address_space(1))) const T *as_global(
 
 constexpr int kNW = 4;  // waves per workgroup
 constexpr int kThreads = kNW * kWave;
-constexpr int kMaxBatch = TLLM_MAX_PLAN_BATCH;
+constexpr int kMaxBatch = 4;  // activation rows the tall tiles carry
 #ifndef TLLM_TILES_AHEAD
 #define TLLM_TILES_AHEAD 3
 #endif
@@ -533,30 +533,10 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
         d.max_rows = p.rows > d.max_rows ? p.rows : d.max_rows;
     }
     d.max_batch = max_batch;
-    // one geometry per launch: wide tiles if every problem allows them, else tall ones
-    bool all_wide = true, all_tall = true;
-    for (const Problem &p : host) {
-        const bool addressable = (size_t)p.rows * (p.cols / 8) < (size_t)1 << 32;
-        all_wide = all_wide && addressable && wide_ok(p);
-        all_tall = all_tall && addressable && tall_ok(p);
-    }
-    d.wide = all_wide;
-    d.use_mfma = all_wide || all_tall;
-    for (const Problem &p : host) {
-        const int ib = d.wide ? image_bytes_of<Wide>(p.cols, 1) : image_bytes_of<Tall>(p.cols, p.batch);
-        max_image = ib > max_image ? ib : max_image;
-    }
-    const int unit = d.wide ? range_unit<Wide>() : range_unit<Tall>();
-    const int max_units = max_units_for(max_image, max_batch, unit);
-    if (max_units < 1) d.use_mfma = false;
-
+    // contiguous spans of units of about equal weight (a unit's weights plus a fixed cost), at least
+    // one unit per workgroup
     std::vector<int> prefix(host.size() + 1, 0), wg_first;
-    if (d.use_mfma) {
-        d.lds_bytes = max_image + kNW * max_units * unit * max_batch * 4;
-        const int per_cu = d.wide ? resident_wgs<Wide>(d.lds_bytes) : resident_wgs<Tall>(d.lds_bytes);
-        const int wgs = per_cu * di->cus;
-        // weight of every unit: its weights plus a fixed cost; then contiguous spans of about equal
-        // weight, at least one unit per workgroup
+    auto partition = [&](int unit, int wgs) {
         std::vector<int64_t> weight;
         for (size_t i = 0; i < host.size(); i++) {
             const int n = (host[i].rows + unit - 1) / unit;
@@ -580,8 +560,38 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
             wg_first[g] = t;
         }
         d.grid = grid;
-        d.max_units = max_units;
-        d.image_bytes = max_image;
+    };
+
+    // several activation rows: the batched kernel if every problem fits it
+    bool all_batch = max_batch >= 2;
+    for (const Problem &p : host) all_batch = all_batch && gemv_batch_supports(p, 128);
+    // one geometry per launch otherwise: wide tiles if every problem allows them, else tall ones
+    bool all_wide = true, all_tall = true;
+    for (const Problem &p : host) {
+        const bool addressable = (size_t)p.rows * (p.cols / 8) < (size_t)1 << 32;
+        all_wide = all_wide && addressable && wide_ok(p);
+        all_tall = all_tall && addressable && tall_ok(p);
+    }
+    if (all_batch) {
+        d.batch_kernel = true;
+        partition(gemv_batch_block_rows(), di->cus);
+    } else {
+        d.wide = all_wide;
+        d.use_mfma = all_wide || all_tall;
+        for (const Problem &p : host) {
+            const int ib = d.wide ? image_bytes_of<Wide>(p.cols, 1) : image_bytes_of<Tall>(p.cols, p.batch);
+            max_image = ib > max_image ? ib : max_image;
+        }
+        const int unit = d.wide ? range_unit<Wide>() : range_unit<Tall>();
+        const int max_units = max_units_for(max_image, max_batch, unit);
+        if (max_units < 1) d.use_mfma = false;
+        if (d.use_mfma) {
+            d.lds_bytes = max_image + kNW * max_units * unit * max_batch * 4;
+            const int per_cu = d.wide ? resident_wgs<Wide>(d.lds_bytes) : resident_wgs<Tall>(d.lds_bytes);
+            partition(unit, per_cu * di->cus);
+            d.max_units = max_units;
+            d.image_bytes = max_image;
+        }
     }
 
     const size_t bytes_table = sizeof(Problem) * host.size();
@@ -604,6 +614,8 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
 }
 
 hipError_t plan_device_launch(const PlanDevice &plan, hipStream_t s) {
+    if (plan.batch_kernel)
+        return launch_gemv_batch_table(plan.problems, plan.unit_prefix, plan.wg_first, plan.grid, s);
     if (!plan.use_mfma)
         return launch_gemv_rowwave_f16_table(plan.problems, plan.count, plan.max_rows, plan.max_batch, 128, s);
     Sched sc{};

@@ -50,7 +50,7 @@ def test_validation_codes():
     assert L.tllm_ternary_gemv_i8_dscale(0x1000, 0x2000, 0x3000, 0x4000, None, 0x5000, 4, 256, 128, None) == -1
     h = C.c_void_p(0)
     assert L.tllm_linear_plan_create(C.byref(h), None, 1, 128) == -1
-    arr = (ops._Problem * 1)(ops._Problem(0x1000, 0x2000, 0x3000, 0x4000, 0x9000, 4, 256, 9, 0))
+    arr = (ops._Problem * 1)(ops._Problem(0x1000, 0x2000, 0x3000, 0x4000, 0x9000, 4, 256, 17, 0))
     assert L.tllm_linear_plan_create(C.byref(h), arr, 1, 128) == -6   # batch > TLLM_MAX_PLAN_BATCH
     assert L.tllm_linear_plan_create(C.byref(h), arr, 0, 128) == -6
     assert L.tllm_linear_plan_create(C.byref(h), arr, 1, 64) == -3

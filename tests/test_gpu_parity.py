@@ -207,6 +207,77 @@ def test_gemm_rows_equal_gemv(dev, oracle):
         assert_close(oracle, yv, ref, what=f"gemv row {m}")
 
 
+# ---------------------------------------------------------- batched decode
+@pytest.mark.parametrize("M,N,K", [(2, 16, 512), (3, 17, 512), (4, 4096, 14336 // 7), (4, 1000, 1536),
+                                   (8, 300, 4096), (13, 255, 1024), (16, 256, 512), (16, 1031, 2048),
+                                   (16, 64, 28672), (4, 512, 14336), (20, 272, 1024), (48, 100, 512)])
+def test_batched_decode_vs_oracle(dev, oracle, M, N, K):
+    """2..16 activation rows (and passes of 16 above that) on K a multiple of 512: block edges
+    (N not a multiple of 16 or 256), long K, unused activation rows."""
+    nz, sg, s, _ = synth.problem(M * 977 + N, N, K, dontcare_sign=True)
+    A = synth.acts_f16(np.random.default_rng(M + K), M, K)
+    ref = oracle.gemm_f64(A.view(np.uint16), nz, sg, s.view(np.uint16))
+    assert_close(oracle, run_gemm(dev, A, nz, sg, s), ref, what=f"batched {M}x{N}x{K}")
+
+
+def test_batched_decode_special_cases(dev, oracle):
+    """Exact zeros for empty rows, rows of one kind, per-row activation ranges that differ by many
+    orders of magnitude (every activation row and slice is normalised on its own), zero activation rows."""
+    rng = np.random.default_rng(31)
+    N, K, M = 96, 1024, 6
+    w = synth.ternary_matrix(rng, N, K)
+    w[0] = 0
+    w[1] = 1
+    w[2] = -1
+    w[3, :] = 0
+    w[3, 700] = -1
+    nz, sg = synth.pack_np(w)
+    s = synth.scales_f16(rng, N, K // 128, lo=1.0, hi=3.0)  # large scales: tiny activations still give normal fp16 outputs
+    A = synth.acts_f16(rng, M, K).astype(np.float64)
+    A[1] *= 1e-3
+    A[2] *= 200.0
+    A[3] = 0.0
+    A[4, :512] = 0.0          # one all-zero slice
+    A[5, 512:] *= 2.0 ** -10  # slices of very different magnitude in one row
+    A = A.astype(np.float16)
+    ref = oracle.gemm_f64(A.view(np.uint16), nz, sg, s.view(np.uint16))
+    got = run_gemm(dev, A, nz, sg, s)
+    assert np.all(got[:, 0] == 0.0) and np.all(got[3] == 0.0)
+    for m in range(M):
+        if m == 3:
+            continue
+        assert_close(oracle, got[m], ref[m], what=f"batched special row {m}")
+
+
+def test_batched_plan_8b_layer_batch4_and_16(dev, oracle):
+    """One LLaMA-3-8B-shaped layer (7 projections, rows cut to keep the oracle fast) as a plan at
+    batch 4 and batch 16: plan output == single-call output bit for bit, sampled rows == oracle."""
+    torch, tl = dev
+    shapes = [(512, 4096), (128, 4096), (128, 4096), (512, 4096), (1800, 4096), (1800, 4096), (520, 14336)]
+    for batch in (4, 16):
+        probs, host = [], []
+        for k, (rows, cols) in enumerate(shapes):
+            nz, sg, s, _ = synth.problem(8100 + k, rows, cols)
+            x = synth.acts_f16(np.random.default_rng(8200 + k + batch), batch, cols)
+            y = torch.full((batch, rows), float("nan"), dtype=torch.float16, device="cuda")
+            probs.append((up(torch, nz), up(torch, sg), up(torch, s), up(torch, x), y, rows, cols, batch))
+            host.append((nz, sg, s, x))
+        plan = tl.LinearPlan(probs)
+        for launch in range(2):
+            for pr in probs:
+                pr[4].fill_(float("nan"))
+            plan.launch()
+            torch.cuda.synchronize()
+            for k, (pr, (nz, sg, s, x)) in enumerate(zip(probs, host)):
+                got = pr[4].cpu().numpy()
+                single = run_gemm(dev, x, nz, sg, s)
+                assert np.array_equal(got.astype(np.float64), single), f"batch {batch} problem {k}: plan != single call"
+                rows_s = np.unique(np.random.default_rng(k).integers(0, nz.shape[0], 64))
+                ref = oracle.gemm_f64(x.view(np.uint16), nz[rows_s], sg[rows_s], s[rows_s].view(np.uint16))
+                assert_close(oracle, got.astype(np.float64)[:, rows_s], ref, what=f"batch {batch} problem {k}")
+        plan.close()
+
+
 # --------------------------------------------------------------- INT8 pair
 @pytest.mark.parametrize("n", [1, 63, 2048, 4096, 14336, 28672])
 def test_quantize_bit_exact(dev, oracle, n):

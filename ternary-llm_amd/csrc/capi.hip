@@ -92,6 +92,11 @@ static int gemv_i8_common(const uint32_t *nz, const uint32_t *sg, const uint16_t
     if (!xq || !y) return TLLM_ERR_NULL_POINTER;
     if (tllm::misaligned(xq, 16) || tllm::misaligned(y, 2)) return TLLM_ERR_MISALIGNED;
     if (tllm::overlaps(xq, (size_t)cols, y, (size_t)rows * 2)) return TLLM_ERR_ALIAS;
+    // int8 values are exact in fp16 and the group sums stay exact in the fp32 accumulators, so the
+    // fp16 matrix-core kernel computes the reference's integer arithmetic on them
+    Problem p{nz, sg, scales, reinterpret_cast<const uint16_t *>(xq), y, rows, cols, 1, 0};
+    if (group == 128 && tllm::gemv_mfma_supports(p, group))
+        return (int)tllm::launch_gemv_mfma_i8(p, scale_value, scale_dev, (hipStream_t)stream);
     return (int)tllm::launch_gemv_rowwave_i8(nz, sg, scales, xq, scale_value, scale_dev, y, rows,
                                              cols, group, (hipStream_t)stream);
 }

@@ -52,6 +52,8 @@ hipError_t launch_quantize_absmax_i8(const uint16_t *x, int8_t *q, float *scale,
 // 128-group MFMA GEMV, batch 1..4 (gemv_mfma.hip).
 bool gemv_mfma_supports(const Problem &p, int group);
 hipError_t launch_gemv_mfma(const Problem &p, hipStream_t s);
+// The same kernel on INT8 activations (p.x is an int8 pointer, batch 1): y = scale * sum_g s_g * (integer sum).
+hipError_t launch_gemv_mfma_i8(const Problem &p, float scale_value, const float *scale_dev, hipStream_t s);
 
 // 128-group MFMA kernel for 2..16 activation rows, K a multiple of 512 (gemv_batch.hip).
 bool gemv_batch_supports(const Problem &p, int group);

@@ -66,6 +66,12 @@ struct Sched {
     int max_units;    // units per task (bounds the partial-sum area)
     int max_batch;    // largest batch of any problem (sizes the per-wave partial-sum areas)
     int image_bytes;  // LDS bytes reserved for the activation image (the partial sums follow)
+    // INT8 activations (single problem, batch 1): x points at int8 values; every output is multiplied
+    // by the activation scale, given by value or read from device memory (reference
+    // kernels/ternary_gemv.cu:116-216: exact integer group sums, fp32 scales).
+    int x_is_i8;
+    float i8_scale;
+    const float *i8_scale_dev;
 };
 
 template <class G>
@@ -184,12 +190,21 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
             groups = p.cols / kChunkCols;
             slices = (p.cols + G::kCols - 1) / G::kCols;
             img_stride = slices * G::kCols;
+            // eight consecutive activations as fp16 bits; int8 values convert exactly
+            auto load8 = [&](int b, int c8) -> uint4 {
+                if (!sc.x_is_i8) return reinterpret_cast<const uint4 *>(p.x + (size_t)b * p.cols)[c8];
+                const uint2 q = reinterpret_cast<const uint2 *>(p.x)[c8];
+                const uint32_t w2[2] = {q.x, q.y};
+                uint32_t h[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) h[e] = f2h((float)(int8_t)(w2[e >> 2] >> (8 * (e & 3))));
+                return uint4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
+            };
             // (a) per batch column: largest magnitude -> power-of-two normalisation
             for (int b = 0; b < p.batch; b++) {
-                const uint4 *xv = reinterpret_cast<const uint4 *>(p.x + (size_t)b * p.cols);
                 uint32_t m = 0;
                 for (int c8 = tid; c8 < p.cols / 8; c8 += kThreads) {
-                    const uint4 v = xv[c8];
+                    const uint4 v = load8(b, c8);
                     const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
@@ -210,11 +225,14 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
                 int ex = 0;                 // all-zero activations: the image is zero whatever the exponent
                 if (m >= 0x7C00u) ex = 15;  // inf/nan present: they propagate to the outputs
                 else if (m) ex = (int)((__builtin_bit_cast(uint32_t, h2f((uint16_t)m)) >> 23) & 0xFF) - 127;
-                if (tid == 0) fscale[b] = m ? __builtin_bit_cast(float, (uint32_t)(127 + ex + 10) << 23) : 0.0f;
+                if (tid == 0) {
+                    float f = m ? __builtin_bit_cast(float, (uint32_t)(127 + ex + 10) << 23) : 0.0f;
+                    if (sc.x_is_i8) f *= sc.i8_scale_dev ? *sc.i8_scale_dev : sc.i8_scale;
+                    fscale[b] = f;
+                }
                 // (b) image: operand element (slice, t, chunk, e) = fp16(x[col] * 2^(14-ex-p)). The last
                 // slice of a row that is not a whole number of slices is moved left so that it ends
                 // with the row; the chunks it then shares with the slice before it are zero here.
-                const uint4 *xv = reinterpret_cast<const uint4 *>(p.x + (size_t)b * p.cols);
                 uint16_t *img = image + (size_t)b * img_stride;
                 for (int c8 = tid; c8 < img_stride / 8; c8 += kThreads) {
                     const int slice = (c8 * 8) / G::kCols;
@@ -222,7 +240,7 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
                     const int cc0 = (c8 * 8) % kChunkCols;
                     const int g = min(slice * G::kChunks, groups - G::kChunks) + chunk;
                     uint4 v = {0u, 0u, 0u, 0u};
-                    if (g >= slice * G::kChunks && m) v = xv[(g * kChunkCols + cc0) / 8];
+                    if (g >= slice * G::kChunks && m) v = load8(b, (g * kChunkCols + cc0) / 8);
                     const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
                     uint16_t *dst = img + slice * G::kCols;
 #pragma unroll
@@ -497,10 +515,14 @@ bool gemv_mfma_supports(const Problem &p, int group) {
     return group == 128 && (size_t)p.rows * (p.cols / 8) < (size_t)1 << 32 && (wide_ok(p) || tall_ok(p));
 }
 
-hipError_t launch_gemv_mfma(const Problem &p, hipStream_t s) {
+static hipError_t launch_single(const Problem &p, bool x_is_i8, float i8_scale, const float *i8_scale_dev,
+                                hipStream_t s) {
     DeviceInfo *di = nullptr;
     if (hipError_t e = prepare_device(&di)) return e;
     Sched sc{};
+    sc.x_is_i8 = x_is_i8 ? 1 : 0;
+    sc.i8_scale = i8_scale;
+    sc.i8_scale_dev = i8_scale_dev;
     sc.table = nullptr;
     sc.count = 1;
     const bool wide = wide_ok(p);
@@ -517,6 +539,13 @@ hipError_t launch_gemv_mfma(const Problem &p, hipStream_t s) {
     else
         gemv_mfma_kernel<Tall><<<grid, kThreads, lds, s>>>(p, sc);
     return hipGetLastError();
+}
+
+hipError_t launch_gemv_mfma(const Problem &p, hipStream_t s) { return launch_single(p, false, 0.0f, nullptr, s); }
+
+// p.x points at int8 activations (batch 1, 8-byte aligned)
+hipError_t launch_gemv_mfma_i8(const Problem &p, float scale_value, const float *scale_dev, hipStream_t s) {
+    return launch_single(p, true, scale_value, scale_dev, s);
 }
 
 // ------------------------------------------------------------------ multi-problem plan

@@ -59,6 +59,7 @@ hipError_t launch_gemv_mfma_i8(const Problem &p, float scale_value, const float 
 bool gemv_batch_supports(const Problem &p, int group);
 hipError_t launch_gemv_batch(const Problem &p, hipStream_t s);
 int gemv_batch_block_rows();
+float gemv_batch_cost_us(const Problem &p);  // rough time of one launch_gemv_batch
 hipError_t launch_gemv_batch_table(const Problem *table, const int *unit_prefix, const int *wg_first, int grid,
                                    hipStream_t s);
 

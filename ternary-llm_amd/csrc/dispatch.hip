@@ -1,4 +1,6 @@
 // Kernel selection for one linear.
+#include <stdlib.h>
+
 #include "common.h"
 
 namespace tllm {
@@ -7,10 +9,15 @@ namespace {
 constexpr int kTallBatch = 4;    // activation rows per pass of the batch-1 family's tall tiles
 constexpr int kBatchRows = 16;   // activation rows per pass of the batched decode kernel
 
-// rough time of `passes` sweeps over the packed weights at the rate the streaming kernels sustain
-float stream_cost_us(const Problem &p, int passes) {
-    const float bytes = 0.265625f * (float)p.rows * (float)p.cols;
-    return (float)passes * (bytes / 4.0e6f + 3.0f);
+// TLLM_GEMM_PATH=mfma|stream forces the choice between the prefill GEMM and passes of the batched
+// decode kernel for M > 16 (a tuning aid; unset: the cost model decides)
+int forced_path() {
+    static int v = -1;
+    if (v < 0) {
+        const char *e = getenv("TLLM_GEMM_PATH");
+        v = !e ? 0 : (e[0] == 'm' ? 1 : e[0] == 's' ? 2 : 0);
+    }
+    return v;
 }
 }  // namespace
 
@@ -22,7 +29,9 @@ hipError_t dispatch_linear(const Problem &p, int group, hipStream_t s) {
     if (p.batch > 1 && gemv_batch_supports(probe, group)) {
         const int passes = (p.batch + kBatchRows - 1) / kBatchRows;
         const bool gemm_ok = gemm_mfma_supports(p, group);
-        if (passes == 1 || !gemm_ok || stream_cost_us(p, passes) < gemm_mfma_cost_us(p)) {
+        bool stream = passes == 1 || !gemm_ok || (float)passes * gemv_batch_cost_us(probe) < gemm_mfma_cost_us(p);
+        if (passes > 1 && gemm_ok && forced_path()) stream = forced_path() == 2;
+        if (stream) {
             for (int b0 = 0; b0 < p.batch; b0 += kBatchRows) {
                 Problem q = p;
                 q.batch = p.batch - b0 < kBatchRows ? p.batch - b0 : kBatchRows;

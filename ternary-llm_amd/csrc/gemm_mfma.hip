@@ -34,13 +34,14 @@ typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 typedef uint16_t us2 __attribute__((ext_vector_type(2)));
 typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float f16v __attribute__((ext_vector_type(16)));
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 
 constexpr int kBN = 128;     // weight rows per workgroup
 constexpr int kBK = 64;      // K columns per stage (two MFMA steps of 32)
 constexpr int kThreads = 256;
 constexpr int kRowBytes = kBK * 2;  // one LDS row: 64 fp16 = 8 chunks of 16 bytes
-constexpr int kNF = kBN / 16;       // MFMA row fragments per wave
+constexpr int kNF = kBN / 32;       // MFMA row fragments (32 weight rows each) per wave
 constexpr int kWBytes = kBN * kRowBytes;
 
 // byte offset of 16-byte chunk c (0..7) of row r inside the [128][64] fp16 LDS tile
@@ -71,11 +72,11 @@ struct Decoder {
 
 constexpr int kBufs = 3;  // LDS buffers per operand (stages in flight)
 
-template <int MF>  // MFMA column fragments (16 activation rows each) per wave
+template <int MF>  // MFMA column fragments (32 activation rows each) per wave
 __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
     const uint16_t *__restrict__ A, const uint32_t *__restrict__ nzB, const uint32_t *__restrict__ sgB,
     const uint16_t *__restrict__ scB, uint16_t *__restrict__ C, int M, int N, int K) {
-    constexpr int kWM = MF * 16;             // activation rows per wave
+    constexpr int kWM = MF * 32;             // activation rows per wave
     constexpr int BM = 4 * kWM;
     constexpr int kActWave = kWM * kRowBytes;  // bytes of one wave's activation tile per stage
     constexpr int kActBytes = 4 * kActWave;
@@ -90,7 +91,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int li = lane & 15, lq = lane >> 4;
+    const int li = lane & 31, lq = lane >> 5;  // MFMA 32x32x16: operand row / column, k half
 
     // tile coordinates: consecutive workgroups share the weight tile (same n0), so it stays in L2
     const int m_tiles = (M + BM - 1) / BM;
@@ -118,7 +119,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
     // the scale of group g travels as the aligned dword that contains it; sc_half picks the half
     GB *sc_src = (GB *)scB + (size_t)gn * groups * 2;
     const int w_off = chunk_off(w_row, w_word * 4);      // chunk c of the word: w_off ^ (c << 4)
-    const int fr_off = chunk_off(li, 2 * lq);            // fragment i, step ks: (fr_off ^ (ks << 4)) + i * 16 rows
+    const int fr_off = chunk_off(li, lq);                // fragment i, step ks: (fr_off ^ (ks << 5)) + i * 32 rows
 
     struct Masks {
         uint32_t nz, sg, sc;
@@ -154,25 +155,27 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
                 16, 0, 0);
     };
     auto read_w = [&](u4 (&af)[kNF], int buf, int ks) {
-        const unsigned char *Ws = lds + buf * kWBytes + (fr_off ^ (ks << 4));
+        const unsigned char *Ws = lds + buf * kWBytes + (fr_off ^ (ks << 5));
 #pragma unroll
-        for (int i = 0; i < kNF; i++) af[i] = *reinterpret_cast<const u4 *>(Ws + i * 16 * kRowBytes);
+        for (int i = 0; i < kNF; i++) af[i] = *reinterpret_cast<const u4 *>(Ws + i * 32 * kRowBytes);
     };
     auto read_a = [&](u4 (&bf)[MF], int buf, int ks) {
-        const unsigned char *As = lds + kActBase + buf * kActBytes + wave * kActWave + (fr_off ^ (ks << 4));
+        const unsigned char *As = lds + kActBase + buf * kActBytes + wave * kActWave + (fr_off ^ (ks << 5));
 #pragma unroll
-        for (int j = 0; j < MF; j++) bf[j] = *reinterpret_cast<const u4 *>(As + j * 16 * kRowBytes);
+        for (int j = 0; j < MF; j++) bf[j] = *reinterpret_cast<const u4 *>(As + j * 32 * kRowBytes);
     };
 
-    f4 acc[kNF][MF];
+    f16v acc[kNF][MF];
 #pragma unroll
     for (int i = 0; i < kNF; i++)
 #pragma unroll
-        for (int j = 0; j < MF; j++) acc[i][j] = f4{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < MF; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
     auto mfma_row = [&](const u4 &a, const u4 (&bf)[MF], int i) {
 #pragma unroll
         for (int j = 0; j < MF; j++)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a), __builtin_bit_cast(h8, bf[j]),
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, a), __builtin_bit_cast(h8, bf[j]),
                                                                acc[i][j], 0, 0, 0);
     };
     auto decode_all = [&](const Masks &w, int buf) {
@@ -187,15 +190,15 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
 
     // Software pipeline, per stage s (buffer indices modulo 3). Everything that comes from global
     // memory is written into LDS by the load itself; such loads complete in order, so "at most n
-    // still in flight" is the test for the older ones.
-    //   top:    activations of stage s+2 are requested; the masks of stage s+2 (requested in stage s-3)
-    //           and the fragments of the second half of stage s are read from LDS;
-    //   half 1: MFMAs of the first half; between them the masks are decoded into weight buffer s+2,
-    //           then the masks of stage s+5 are requested into the mask buffer just read;
-    //   middle: fragments of the first half of stage s+1 are read from LDS;
-    //   half 2: MFMAs of the second half; barrier.
-    // The barrier at the end of stage s publishes weight buffer s+2 before its first read (middle of
-    // stage s+1); that buffer was last read at the top of stage s-1. Activation and mask buffers are
+    // still in flight" is the test for the older ones. A stage is four MFMA steps of 16 columns;
+    // the fragments of a step are read from LDS while the MFMAs of the step before run.
+    //   step 0: activations of stage s+2 are requested; the masks of stage s+2 (requested in stage
+    //           s-3) are read from LDS; fragments of step 1 are read; MFMAs of step 0;
+    //   steps 0-2: between the MFMAs the masks are decoded into weight buffer s+2; then the masks of
+    //           stage s+5 are requested into the mask buffer just read;
+    //   step 3: fragments of step 0 of stage s+1 are read; MFMAs of step 3; barrier.
+    // The barrier at the end of stage s publishes weight buffer s+2 before its first read (step 3 of
+    // stage s+1); that buffer was last read in step 2 of stage s-1. Activation and mask buffers are
     // private to a wave, ordered by the wave's own waits.
     Masks w;
     u4 af0[kNF], af1[kNF], bf0[MF], bf1[MF];
@@ -222,32 +225,52 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
             // masks of stage s+2: requested in stage s-3; newer requests: 2 stages of (kDma + 3), this stage's kDma
             asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * kDma + 6) : "memory");
             read_masks(w, (u + 2) % kBufs, s + 2);
+            Decoder d;
+            unsigned char *Ws = lds + ((u + 2) % kBufs) * kWBytes;
+            uint32_t o[16];
+            // ---- step 0 (fragments af0/bf0), fragments of step 1 on their way
             read_w(af1, u, 1);
             read_a(bf1, u, 1);
             __builtin_amdgcn_sched_barrier(0);
-            {
-                // group 0 only multiplies (its operands arrived during the previous stage); groups 1..7
-                // also decode 3,2,2,3,2,2,2 dwords and store every finished 16-byte chunk
-                Decoder d;
-                unsigned char *Ws = lds + ((u + 2) % kBufs) * kWBytes;
-                uint32_t o[16];
-                mfma_row(af0[0], bf0, 0);
+            mfma_row(af0[0], bf0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            d.begin(w.nz, w.sg, w.sc);
+#pragma unroll
+            for (int i = 1; i < kNF; i++) {
+                mfma_row(af0[i], bf0, i);
+#pragma unroll
+                for (int dw = 2 * (i - 1); dw < 2 * i; dw++) o[dw] = d.dword(dw);
                 __builtin_amdgcn_sched_barrier(0);
-                d.begin(w.nz, w.sg, w.sc);
-#pragma unroll
-                for (int i = 1; i < kNF; i++) {
-                    constexpr int kEnd[kNF] = {0, 3, 5, 7, 10, 12, 14, 16};
-                    mfma_row(af0[i], bf0, i);
-#pragma unroll
-                    for (int dw = kEnd[i - 1]; dw < kEnd[i]; dw++) o[dw] = d.dword(dw);
-#pragma unroll
-                    for (int c = 0; c < 4; c++)
-                        if (kEnd[i - 1] < 4 * c + 4 && 4 * c + 4 <= kEnd[i])
-                            *reinterpret_cast<u4 *>(Ws + (w_off ^ (c << 4))) = u4{o[4 * c], o[4 * c + 1], o[4 * c + 2], o[4 * c + 3]};
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-                dma_masks((u + 2) % kBufs, s + 5);
             }
+            // ---- step 1 (af1/bf1), fragments of step 2 into af0/bf0
+            read_w(af0, u, 2);
+            read_a(bf0, u, 2);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < kNF; i++) {
+                mfma_row(af1[i], bf1, i);
+#pragma unroll
+                for (int dw = 6 + 2 * i; dw < 8 + 2 * i; dw++) o[dw] = d.dword(dw);
+                if (i == 0) *reinterpret_cast<u4 *>(Ws + (w_off ^ (0 << 4))) = u4{o[0], o[1], o[2], o[3]};
+                if (i == 1) *reinterpret_cast<u4 *>(Ws + (w_off ^ (1 << 4))) = u4{o[4], o[5], o[6], o[7]};
+                if (i == 3) *reinterpret_cast<u4 *>(Ws + (w_off ^ (2 << 4))) = u4{o[8], o[9], o[10], o[11]};
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // ---- step 2 (af0/bf0), fragments of step 3 into af1/bf1
+            read_w(af1, u, 3);
+            read_a(bf1, u, 3);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < kNF; i++) {
+                mfma_row(af0[i], bf0, i);
+                if (i < 2) {
+                    o[14 + i] = d.dword(14 + i);
+                }
+                if (i == 1) *reinterpret_cast<u4 *>(Ws + (w_off ^ (3 << 4))) = u4{o[12], o[13], o[14], o[15]};
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            dma_masks((u + 2) % kBufs, s + 5);
+            // ---- step 3 (af1/bf1), fragments of step 0 of the next stage into af0/bf0
             read_w(af0, (u + 1) % kBufs, 0);
             // the activations of stage s+1 were requested at the top of stage s-1; newer requests: the
             // masks of that stage (3), this stage's activations (kDma) and masks (3)
@@ -262,27 +285,31 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
         }
     }
 
-    // ---- store: lane (lq, li) of fragment (i, j) holds weight rows n .. n+3 for activation row m
+    // ---- store: lane (k half lq, column li) of fragment (i, j) holds, for activation row m, the weight
+    // rows n0 + 32 i + 8 g + 4 lq + v in register 4 g + v (g, v = 0..3)
     uint16_t *Cg = C;
     const bool vec_store = (N & 3) == 0 && (reinterpret_cast<uintptr_t>(C) & 7) == 0;
 #pragma unroll
     for (int j = 0; j < MF; j++) {
-        const int m = m0 + j * 16 + li;
+        const int m = m0 + j * 32 + li;
         if (m >= M) continue;
 #pragma unroll
         for (int i = 0; i < kNF; i++) {
-            const int n = n0 + i * 16 + 4 * lq;
-            uint16_t h[4];
 #pragma unroll
-            for (int v = 0; v < 4; v++) h[v] = f2h(acc[i][j][v] * 0.5f);
-            uint16_t *dst = Cg + (size_t)m * N + n;
-            if (n + 3 < N && vec_store) {
-                *reinterpret_cast<uint2 *>(dst) = uint2{(uint32_t)h[0] | ((uint32_t)h[1] << 16),
-                                                        (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
-            } else {
+            for (int g = 0; g < 4; g++) {
+                const int n = n0 + i * 32 + 8 * g + 4 * lq;
+                uint16_t h[4];
 #pragma unroll
-                for (int v = 0; v < 4; v++)
-                    if (n + v < N) dst[v] = h[v];
+                for (int v = 0; v < 4; v++) h[v] = f2h(acc[i][j][4 * g + v] * 0.5f);
+                uint16_t *dst = Cg + (size_t)m * N + n;
+                if (n + 3 < N && vec_store) {
+                    *reinterpret_cast<uint2 *>(dst) = uint2{(uint32_t)h[0] | ((uint32_t)h[1] << 16),
+                                                            (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 4; v++)
+                        if (n + v < N) dst[v] = h[v];
+                }
             }
         }
     }
@@ -290,7 +317,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
 
 template <int MF>
 hipError_t launch(const Problem &p, hipStream_t s) {
-    constexpr int BM = 64 * MF;
+    constexpr int BM = 128 * MF;
     static bool attr_set[64] = {};
     int dev = 0;
     if (hipError_t e = hipGetDevice(&dev)) return e;
@@ -319,7 +346,7 @@ bool gemm_mfma_supports(const Problem &p, int group) {
 namespace {
 // One workgroup occupies a CU (LDS). Taller tiles do more per stage, shorter tiles fill the chip
 // when there are few of them: take the height with the smallest (rounds of workgroups over the
-// CUs) x (time of one stage, measured: 1.2 / 0.83 / 0.65 us for 256 / 128 / 64 activation rows).
+// CUs) x (time of one stage, measured: 1.19 / 0.70 us for 256 / 128 activation rows).
 int choose_height(const Problem &p, float *stage_rounds_us) {
     static int cus[64] = {};
     int dev = 0, n_cu = 256;
@@ -329,11 +356,11 @@ int choose_height(const Problem &p, float *stage_rounds_us) {
         if (cus[dev] > 0) n_cu = cus[dev];
     }
     const int n_tiles = (p.rows + kBN - 1) / kBN;
-    const float stage_us[3] = {0.65f, 0.83f, 1.2f};
+    const float stage_us[2] = {0.70f, 1.19f};
     int best = 0;
     float best_cost = 0.f;
-    for (int c = 0; c < 3; c++) {
-        const int bm = 64 << c;
+    for (int c = 0; c < 2; c++) {
+        const int bm = 128 << c;
         const long wgs = (long)n_tiles * ((p.batch + bm - 1) / bm);
         const float cost = (float)((wgs + n_cu - 1) / n_cu) * stage_us[c];
         if (c == 0 || cost < best_cost) best = c, best_cost = cost;
@@ -351,7 +378,6 @@ float gemm_mfma_cost_us(const Problem &p) {
 
 hipError_t launch_gemm_mfma(const Problem &p, hipStream_t s) {
     const int best = choose_height(p, nullptr);
-    if (best == 2) return launch<4>(p, s);
     if (best == 1) return launch<2>(p, s);
     return launch<1>(p, s);
 }

@@ -37,8 +37,7 @@ constexpr int kNW = 8;                          // waves: 4 tile quarters x 2 sl
 constexpr int kThreads = kNW * kWave;
 constexpr int kSliceCols = 512;                 // 4 scale groups
 constexpr int kTileRows = 16;
-constexpr int kTilesPerWave = 4;                // tiles of one wave per slice = loads in flight
-constexpr int kBlockRows = 4 * kTilesPerWave * kTileRows;    // 256
+constexpr int kMaxTilesPerWave = 4;             // tiles of one wave per slice = loads in flight
 constexpr int kImageBytes = 16 * kSliceCols * 2;             // operands of one slice, 16 activation rows
 
 struct BatchSched {
@@ -68,7 +67,11 @@ __device__ __forceinline__ void transpose4(u4 &a) {
     a = u4{t0[0], t0[1], t1[0], t1[1]};
 }
 
+// kTilesPerWave: 4 for long streams (256-row blocks amortise the per-slice operand build best);
+// 2 or 1 when one matrix alone must fill the chip (128- and 64-row blocks).
+template <int kTilesPerWave>
 __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single, BatchSched sc) {
+    constexpr int kBlockRows = 4 * kTilesPerWave * kTileRows;
     // [buffer][slice parity]: the operands of two neighbouring slices are built per step
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     unsigned char (*image)[2][kImageBytes] = reinterpret_cast<unsigned char (*)[2][kImageBytes]>(lds_raw);
@@ -335,41 +338,71 @@ int device_cus() {
 
 bool gemv_batch_supports(const Problem &p, int group) {
     return group == 128 && p.batch >= 1 && p.batch <= 16 && p.rows >= kTileRows && p.cols >= kSliceCols &&
-           p.cols % kSliceCols == 0 && (reinterpret_cast<uintptr_t>(p.scales) & 7) == 0 && (size_t)p.rows * (p.cols / 8) < ((size_t)1 << 32) &&
-           (size_t)p.rows * (p.cols / 128) * 2 < ((size_t)1 << 32);
+           p.cols % kSliceCols == 0 && (reinterpret_cast<uintptr_t>(p.scales) & 7) == 0 &&
+           (size_t)p.rows * (p.cols / 8) < ((size_t)1 << 32) && (size_t)p.rows * (p.cols / 128) * 2 < ((size_t)1 << 32);
 }
 
 constexpr size_t kLdsBytes = 4 * kImageBytes + 2 * 2 * 16 * sizeof(float);
 
+template <int T>
 static hipError_t prepare_kernel() {
     static bool done[64] = {};
     int dev = 0;
     if (hipError_t e = hipGetDevice(&dev)) return e;
     if (dev < 0 || dev >= 64 || done[dev]) return hipSuccess;
-    if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_batch_kernel),
+    if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_batch_kernel<T>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes))
         return e;
     done[dev] = true;
     return hipSuccess;
 }
 
-hipError_t launch_gemv_batch(const Problem &p, hipStream_t s) {
-    if (hipError_t e = prepare_kernel()) return e;
-    const int blocks = (p.rows + kBlockRows - 1) / kBlockRows;
-    const int wgs = device_cus();  // one workgroup of 8 waves per CU
+template <int T>
+static hipError_t launch_single(const Problem &p, int wgs, hipStream_t s) {
+    if (hipError_t e = prepare_kernel<T>()) return e;
+    const int blocks = (p.rows + 64 * T - 1) / (64 * T);
     BatchSched sc{nullptr, nullptr, nullptr};
-    gemv_batch_kernel<<<blocks < wgs ? blocks : wgs, kThreads, kLdsBytes, s>>>(p, sc);
+    gemv_batch_kernel<T><<<blocks < wgs ? blocks : wgs, kThreads, kLdsBytes, s>>>(p, sc);
     return hipGetLastError();
 }
 
-int gemv_batch_block_rows() { return kBlockRows; }
+// tiles per wave for one matrix alone: the largest block size that still gives every CU a block
+static int single_tiles(const Problem &p, int cus) {
+    for (int t = kMaxTilesPerWave; t > 1; t /= 2)
+        if ((p.rows + 64 * t - 1) / (64 * t) >= cus) return t;
+    return 1;
+}
+
+hipError_t launch_gemv_batch(const Problem &p, hipStream_t s) {
+    const int cus = device_cus();  // one workgroup of 8 waves per CU
+    switch (single_tiles(p, cus)) {
+        case 4: return launch_single<4>(p, cus, s);
+        case 2: return launch_single<2>(p, cus, s);
+        default: return launch_single<1>(p, cus, s);
+    }
+}
+
+float gemv_batch_cost_us(const Problem &p) {
+    // measured on single matrices: 3 us of launch and ramp, then the larger of the streaming time
+    // (a workgroup moves about 17 bytes of packed weights per ns with 256-row blocks, 13 with 64-row
+    // blocks) and the latency chain of the K loop (1.8 us per step of 1024 columns)
+    const int cus = device_cus();
+    const int t = single_tiles(p, cus);
+    const int blocks = (p.rows + 64 * t - 1) / (64 * t);
+    const float rate = (t == 4 ? 17.0e3f : t == 2 ? 15.0e3f : 13.0e3f) * (float)(blocks < cus ? blocks : cus);
+    const float stream = 0.265625f * (float)p.rows * (float)p.cols / rate;
+    const float chain = 1.8f * (float)((p.cols / kSliceCols + 1) / 2);
+    return 3.0f + (stream > chain ? stream : chain);
+}
+
+int gemv_batch_block_rows() { return 64 * kMaxTilesPerWave; }
 
 hipError_t launch_gemv_batch_table(const Problem *table, const int *unit_prefix, const int *wg_first, int grid,
                                    hipStream_t s) {
-    if (hipError_t e = prepare_kernel()) return e;
+    if (hipError_t e = prepare_kernel<kMaxTilesPerWave>()) return e;
     BatchSched sc{table, unit_prefix, wg_first};
     Problem none{};
-    gemv_batch_kernel<<<grid, kThreads, kLdsBytes, s>>>(none, sc);
+    gemv_batch_kernel<kMaxTilesPerWave><<<grid, kThreads, kLdsBytes, s>>>(none, sc);
     return hipGetLastError();
 }
 

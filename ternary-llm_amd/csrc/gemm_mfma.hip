@@ -123,6 +123,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
 
     struct Masks {
         uint32_t nz, sg, sc;
+        bool hi;  // the scale is the high half of sc
     };
     // Mask words and scales also come through LDS: thread t asks for its own three dwords, which the
     // hardware puts at byte 4 t of each 1 KB plane, and reads them back itself (no barrier involved).
@@ -141,10 +142,11 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
         const unsigned char *src = lds + kMaskBase + buf * kMaskBytes + tid * 4;
         w.nz = *reinterpret_cast<const uint32_t *>(src);
         w.sg = *reinterpret_cast<const uint32_t *>(src + 1024);
-        const uint32_t pair = *reinterpret_cast<const uint32_t *>(src + 2048);
+        w.sc = *reinterpret_cast<const uint32_t *>(src + 2048);  // the dword that holds the scale
         const uintptr_t sc_addr = reinterpret_cast<uintptr_t>(sc_src) + (min(stage, last) * kBK / 128) * 2;
-        w.sc = (sc_addr & 2) ? pair >> 16 : pair & 0xFFFFu;
+        w.hi = (sc_addr & 2) != 0;
     };
+    auto scale_of = [](const Masks &w) -> uint32_t { return w.hi ? w.sc >> 16 : w.sc & 0xFFFFu; };
     auto dma_acts = [&](int buf, int stage) {
         const int k0 = min(stage, last) * kBK;
 #pragma unroll
@@ -180,7 +182,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
     };
     auto decode_all = [&](const Masks &w, int buf) {
         Decoder d;
-        d.begin(w.nz, w.sg, w.sc);
+        d.begin(w.nz, w.sg, scale_of(w));
         unsigned char *Ws = lds + buf * kWBytes;
 #pragma unroll
         for (int c = 0; c < 4; c++)
@@ -191,12 +193,12 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
     // Software pipeline, per stage s (buffer indices modulo 3). Everything that comes from global
     // memory is written into LDS by the load itself; such loads complete in order, so "at most n
     // still in flight" is the test for the older ones. A stage is four MFMA steps of 16 columns;
-    // the fragments of a step are read from LDS while the MFMAs of the step before run.
-    //   step 0: activations of stage s+2 are requested; the masks of stage s+2 (requested in stage
-    //           s-3) are read from LDS; fragments of step 1 are read; MFMAs of step 0;
-    //   steps 0-2: between the MFMAs the masks are decoded into weight buffer s+2; then the masks of
-    //           stage s+5 are requested into the mask buffer just read;
-    //   step 3: fragments of step 0 of stage s+1 are read; MFMAs of step 3; barrier.
+    // the fragments of a step are read from LDS during the step before, after its first MFMAs.
+    //   top:    activations of stage s+2 are requested;
+    //   step 0: the masks of stage s+2 (requested in stage s-3) are read from LDS;
+    //   steps 1-3: between the MFMAs the masks are decoded into weight buffer s+2;
+    //   step 3: fragments of step 0 of stage s+1 are read; at the end the masks of stage s+5 are
+    //           requested into the mask buffer just read; barrier.
     // The barrier at the end of stage s publishes weight buffer s+2 before its first read (step 3 of
     // stage s+1); that buffer was last read in step 2 of stage s-1. Activation and mask buffers are
     // private to a wave, ordered by the wave's own waits.
@@ -213,6 +215,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
     decode_all(w, 1);
     dma_masks(0, 3);
     dma_masks(1, 4);
+    // everything requested so far has landed: the in-loop waits count only requests made in the loop
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     read_w(af0, 0, 0);
     read_a(bf0, 0, 0);
@@ -221,65 +225,73 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
         for (int u = 0; u < kBufs; u++) {
             const int s = s0 + u;
             if (s > last) break;
-            dma_acts((u + 2) % kBufs, s + 2);
-            // masks of stage s+2: requested in stage s-3; newer requests: 2 stages of (kDma + 3), this stage's kDma
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * kDma + 6) : "memory");
-            read_masks(w, (u + 2) % kBufs, s + 2);
+            // Every LDS read is issued right AFTER the first MFMAs of a step, one step before its
+            // data is used: the wait in front of a step's first MFMA then finds nothing younger in
+            // the LDS queue and costs nothing.
             Decoder d;
             unsigned char *Ws = lds + ((u + 2) % kBufs) * kWBytes;
             uint32_t o[16];
-            // ---- step 0 (fragments af0/bf0), fragments of step 1 on their way
+            dma_acts((u + 2) % kBufs, s + 2);
+            // ---- step 0 (af0/bf0)
+            mfma_row(af0[0], bf0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            // masks of stage s+2: requested in stage s-3; newer requests: 2 stages of (kDma + 3), this stage's kDma
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * kDma + 6) : "memory");
+            read_masks(w, (u + 2) % kBufs, s + 2);
             read_w(af1, u, 1);
             read_a(bf1, u, 1);
             __builtin_amdgcn_sched_barrier(0);
-            mfma_row(af0[0], bf0, 0);
+#pragma unroll
+            for (int i = 1; i < kNF; i++) mfma_row(af0[i], bf0, i);
             __builtin_amdgcn_sched_barrier(0);
-            d.begin(w.nz, w.sg, w.sc);
+            // ---- step 1 (af1/bf1): decode starts
+            mfma_row(af1[0], bf1, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            read_w(af0, u, 2);
+            read_a(bf0, u, 2);
+            d.begin(w.nz, w.sg, scale_of(w));
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 1; i < kNF; i++) {
-                mfma_row(af0[i], bf0, i);
+                mfma_row(af1[i], bf1, i);
 #pragma unroll
                 for (int dw = 2 * (i - 1); dw < 2 * i; dw++) o[dw] = d.dword(dw);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            // ---- step 1 (af1/bf1), fragments of step 2 into af0/bf0
-            read_w(af0, u, 2);
-            read_a(bf0, u, 2);
+            // ---- step 2 (af0/bf0)
+            mfma_row(af0[0], bf0, 0);
+            o[6] = d.dword(6);
+            o[7] = d.dword(7);
             __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int i = 0; i < kNF; i++) {
-                mfma_row(af1[i], bf1, i);
-#pragma unroll
-                for (int dw = 6 + 2 * i; dw < 8 + 2 * i; dw++) o[dw] = d.dword(dw);
-                if (i == 0) *reinterpret_cast<u4 *>(Ws + (w_off ^ (0 << 4))) = u4{o[0], o[1], o[2], o[3]};
-                if (i == 1) *reinterpret_cast<u4 *>(Ws + (w_off ^ (1 << 4))) = u4{o[4], o[5], o[6], o[7]};
-                if (i == 3) *reinterpret_cast<u4 *>(Ws + (w_off ^ (2 << 4))) = u4{o[8], o[9], o[10], o[11]};
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            // ---- step 2 (af0/bf0), fragments of step 3 into af1/bf1
             read_w(af1, u, 3);
             read_a(bf1, u, 3);
+            *reinterpret_cast<u4 *>(Ws + (w_off ^ (0 << 4))) = u4{o[0], o[1], o[2], o[3]};
+            *reinterpret_cast<u4 *>(Ws + (w_off ^ (1 << 4))) = u4{o[4], o[5], o[6], o[7]};
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int i = 0; i < kNF; i++) {
+            for (int i = 1; i < kNF; i++) {
                 mfma_row(af0[i], bf0, i);
-                if (i < 2) {
-                    o[14 + i] = d.dword(14 + i);
-                }
-                if (i == 1) *reinterpret_cast<u4 *>(Ws + (w_off ^ (3 << 4))) = u4{o[12], o[13], o[14], o[15]};
+#pragma unroll
+                for (int dw = 6 + 2 * i; dw < 8 + 2 * i; dw++) o[dw] = d.dword(dw);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            dma_masks((u + 2) % kBufs, s + 5);
-            // ---- step 3 (af1/bf1), fragments of step 0 of the next stage into af0/bf0
+            // ---- step 3 (af1/bf1): fragments of step 0 of the next stage
+            mfma_row(af1[0], bf1, 0);
+            o[14] = d.dword(14);
+            o[15] = d.dword(15);
+            __builtin_amdgcn_sched_barrier(0);
+            *reinterpret_cast<u4 *>(Ws + (w_off ^ (2 << 4))) = u4{o[8], o[9], o[10], o[11]};
+            *reinterpret_cast<u4 *>(Ws + (w_off ^ (3 << 4))) = u4{o[12], o[13], o[14], o[15]};
             read_w(af0, (u + 1) % kBufs, 0);
             // the activations of stage s+1 were requested at the top of stage s-1; newer requests: the
-            // masks of that stage (3), this stage's activations (kDma) and masks (3)
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kDma + 6) : "memory");
+            // masks of that stage (3) and this stage's activations (kDma)
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kDma + 3) : "memory");
             read_a(bf0, (u + 1) % kBufs, 0);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int i = 0; i < kNF; i++) mfma_row(af1[i], bf1, i);
+            for (int i = 1; i < kNF; i++) mfma_row(af1[i], bf1, i);
             __builtin_amdgcn_sched_barrier(0);
+            dma_masks((u + 2) % kBufs, s + 5);
             // plain barrier: a fence here would also wait for the requests in flight
             asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         }

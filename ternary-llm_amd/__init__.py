@@ -2,7 +2,9 @@
 `lib/libtllm_ternary.so` (hand-written HIP, gfx950). There is no CPU or PyTorch fallback:
 every operator raises if the library is missing or a call is rejected."""
 from .ops import (  # noqa: F401
+    FileHeader,
     LinearPlan,
+    ModelFile,
     TllmError,
     lib,
     lib_path,
@@ -10,4 +12,6 @@ from .ops import (  # noqa: F401
     ternary_gemm,
     ternary_gemv,
     ternary_gemv_int8,
+    ternarize_pack,
+    write_synthetic_model,
 )

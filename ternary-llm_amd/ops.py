@@ -18,6 +18,12 @@ ABI_SYMBOLS = (
     "tllm_linear_plan_create", "tllm_linear_plan_launch", "tllm_linear_plan_weight_bytes",
     "tllm_linear_plan_destroy",
 )
+# include/tllm_model_file.h
+FILE_ABI_SYMBOLS = (
+    "tllm_ternarize_pack_f32", "tllm_model_file_open", "tllm_model_file_close", "tllm_model_file_header",
+    "tllm_model_file_linear_count", "tllm_model_file_linear", "tllm_model_file_pool_bytes",
+    "tllm_model_file_upload", "tllm_model_file_problem", "tllm_model_file_write_synthetic",
+)
 
 
 class TllmError(RuntimeError):
@@ -30,6 +36,20 @@ class _Problem(C.Structure):
     _fields_ = [("nonzero_masks", C.c_void_p), ("sign_masks", C.c_void_p), ("scales", C.c_void_p),
                 ("input", C.c_void_p), ("output", C.c_void_p), ("rows", C.c_int32),
                 ("cols", C.c_int32), ("batch", C.c_int32), ("reserved", C.c_int32)]
+
+
+class FileHeader(C.Structure):
+    """The 256-byte .tllm header (include/tllm_model_file.h, reference include/format.h:20-37)."""
+    _fields_ = [(n, C.c_uint32) for n in (
+        "magic", "version", "arch", "vocab_size", "hidden_dim", "intermediate_dim", "n_layers", "n_heads",
+        "n_kv_heads", "max_seq_len", "head_dim", "rope_theta_bits", "group_size", "rms_norm_eps_bits", "flags")] + \
+        [("reserved", C.c_uint8 * (256 - 15 * 4))]
+
+
+class FileLinear(C.Structure):
+    _fields_ = [(n, C.c_uint64) for n in ("nonzero_file", "sign_file", "scales_file",
+                                           "nonzero_pool", "sign_pool", "scales_pool")] + \
+        [(n, C.c_int32) for n in ("rows", "cols", "layer", "kind")]
 
 
 def lib_path():
@@ -60,6 +80,18 @@ def lib():
     L.tllm_linear_plan_weight_bytes.restype = C.c_int64
     L.tllm_linear_plan_destroy.argtypes = [vp]
     L.tllm_linear_plan_destroy.restype = None
+    L.tllm_ternarize_pack_f32.argtypes = [vp, i, i, i, f, vp, vp, vp]
+    L.tllm_model_file_open.argtypes = [C.c_char_p, C.POINTER(vp)]
+    L.tllm_model_file_close.argtypes = [vp]
+    L.tllm_model_file_close.restype = None
+    L.tllm_model_file_header.argtypes = [vp, C.POINTER(FileHeader)]
+    L.tllm_model_file_linear_count.argtypes = [vp]
+    L.tllm_model_file_linear.argtypes = [vp, i, C.POINTER(FileLinear)]
+    L.tllm_model_file_pool_bytes.argtypes = [vp]
+    L.tllm_model_file_pool_bytes.restype = C.c_uint64
+    L.tllm_model_file_upload.argtypes = [vp, vp, C.c_uint64, vp]
+    L.tllm_model_file_problem.argtypes = [vp, i, vp, C.POINTER(_Problem)]
+    L.tllm_model_file_write_synthetic.argtypes = [C.c_char_p, C.POINTER(FileHeader), C.c_uint64]
     _lib = L
     return L
 
@@ -140,6 +172,65 @@ class LinearPlan:
     def close(self):
         if self._h:
             lib().tllm_linear_plan_destroy(self._h)
+            self._h = C.c_void_p(0)
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def ternarize_pack(weight, group_size=128, threshold_factor=0.7):
+    """Host: fp32 matrix [rows, cols] -> (nonzero uint32 [rows, cols/32], sign uint32, scales fp16
+    [rows, cols/group]) as numpy arrays (reference ternarize/pack.py:41-101, 120-169)."""
+    import numpy as np
+    w = np.ascontiguousarray(weight, dtype=np.float32)
+    rows, cols = w.shape
+    nz = np.zeros((rows, max(cols // 32, 1)), np.uint32)
+    sg = np.zeros_like(nz)
+    sc = np.zeros((rows, max(cols // max(group_size, 1), 1)), np.uint16)
+    check(lib().tllm_ternarize_pack_f32(w.ctypes.data, rows, cols, group_size, threshold_factor,
+                                        nz.ctypes.data, sg.ctypes.data, sc.ctypes.data))
+    return nz, sg, sc.view(np.float16)
+
+
+def write_synthetic_model(path, seed=0, **dims):
+    """Writes a synthetic .tllm file; dims are FileHeader fields (vocab_size, hidden_dim, ...)."""
+    h = FileHeader()
+    for k, v in dims.items():
+        setattr(h, k, v)
+    check(lib().tllm_model_file_write_synthetic(os.fsencode(path), C.byref(h), seed))
+
+
+class ModelFile:
+    """A .tllm file: header, the layout of its ternary linears, upload into one device pool."""
+
+    def __init__(self, path):
+        self._h = C.c_void_p(0)
+        check(lib().tllm_model_file_open(os.fsencode(path), C.byref(self._h)))
+        self.header = FileHeader()
+        check(lib().tllm_model_file_header(self._h, C.byref(self.header)))
+        self.linears = []
+        for k in range(lib().tllm_model_file_linear_count(self._h)):
+            fl = FileLinear()
+            check(lib().tllm_model_file_linear(self._h, k, C.byref(fl)))
+            self.linears.append(fl)
+        self.pool_bytes = int(lib().tllm_model_file_pool_bytes(self._h))
+
+    def upload(self, pool, stream=None):
+        """pool: a uint8 device tensor of at least pool_bytes."""
+        check(lib().tllm_model_file_upload(self._h, _ptr(pool), pool.numel(), _stream(stream)))
+
+    def problem(self, index, pool):
+        """(nz_ptr, sign_ptr, scales_ptr, rows, cols) of linear `index` inside `pool`."""
+        pr = _Problem()
+        check(lib().tllm_model_file_problem(self._h, index, _ptr(pool), C.byref(pr)))
+        return pr.nonzero_masks, pr.sign_masks, pr.scales, pr.rows, pr.cols
+
+    def close(self):
+        if self._h:
+            lib().tllm_model_file_close(self._h)
             self._h = C.c_void_p(0)
 
     def __del__(self):

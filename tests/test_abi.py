@@ -22,6 +22,11 @@ def test_header_symbols_exported():
     for name in declared:
         assert hasattr(L, name), name
     assert L.tllm_abi_version() == 1
+    text = open(os.path.join(ROOT, "include", "tllm_model_file.h")).read()
+    declared = set(re.findall(r"\b(tllm_[a-z0-9_]+)\s*\(", text))
+    assert declared == set(ops.FILE_ABI_SYMBOLS)
+    for name in declared:
+        assert hasattr(L, name), name
 
 
 def test_missing_library_fails_loudly(monkeypatch):

@@ -25,6 +25,8 @@
 //     sum over the stage is complete); operands come from LDS as 16-byte chunks, XOR-swizzled by
 //     row against bank conflicts.
 // Three LDS buffers per operand, one barrier per stage; the loop body spells out the pipeline.
+#include <mutex>
+
 #include "common.h"
 
 namespace tllm {
@@ -75,7 +77,8 @@ constexpr int kBufs = 3;  // LDS buffers per operand (stages in flight)
 template <int MF>  // MFMA column fragments (32 activation rows each) per wave
 __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
     const uint16_t *__restrict__ A, const uint32_t *__restrict__ nzB, const uint32_t *__restrict__ sgB,
-    const uint16_t *__restrict__ scB, uint16_t *__restrict__ C, int M, int N, int K) {
+    const uint16_t *__restrict__ scB, uint16_t *__restrict__ C, int M, int N, int K, int splits,
+    float *__restrict__ partial, unsigned *__restrict__ arrivals) {
     constexpr int kWM = MF * 32;             // activation rows per wave
     constexpr int BM = 4 * kWM;
     constexpr int kActWave = kWM * kRowBytes;  // bytes of one wave's activation tile per stage
@@ -94,11 +97,16 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
     const int li = lane & 31, lq = lane >> 5;  // MFMA 32x32x16: operand row / column, k half
 
     // tile coordinates: consecutive workgroups share the weight tile (same n0), so it stays in L2
+    // With splits > 1, `splits` consecutive workgroups share a tile and take consecutive ranges of
+    // whole scale groups of K; the last of them to finish adds the partial sums (below).
     const int m_tiles = (M + BM - 1) / BM;
-    const int n0 = (blockIdx.x / m_tiles) * kBN;
-    const int m0 = (blockIdx.x % m_tiles) * BM + wave * kWM;
+    const int tile = blockIdx.x / splits, split = blockIdx.x - tile * splits;
+    const int n0 = (tile / m_tiles) * kBN;
+    const int m0 = (tile % m_tiles) * BM + wave * kWM;
     const int words = K / 32, groups = K / 128;
-    const int last = K / kBK - 1;  // index of the last stage
+    const int g_begin = (int)((long)groups * split / splits), g_end = (int)((long)groups * (split + 1) / splits);
+    const int k_begin = g_begin * 128;
+    const int last = (g_end - g_begin) * 128 / kBK - 1;  // index of this workgroup's last stage
 
     // activations: load t of a stage brings rows 8t .. 8t+7 of the wave's tile, 128 bytes each, straight
     // into LDS. The hardware puts lane p's 16 bytes at byte 16 p of the 1 KB block, so lane p asks for
@@ -109,15 +117,15 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
 #pragma unroll
     for (int t = 0; t < kDma; t++) {
         const int gm = min(m0 + 8 * t + (lane >> 3), M - 1);
-        a_src[t] = (GB *)A + ((size_t)gm * K + 8 * ((lane & 7) ^ (lane >> 3))) * 2;
+        a_src[t] = (GB *)A + ((size_t)gm * K + k_begin + 8 * ((lane & 7) ^ (lane >> 3))) * 2;
     }
     // weights: row w_row, 32-column word w_word of the stage
     const int w_row = tid >> 1, w_word = tid & 1;
     const int gn = min(n0 + w_row, N - 1);
-    GB *nz_src = (GB *)nzB + ((size_t)gn * words + w_word) * 4;
-    GB *sg_src = (GB *)sgB + ((size_t)gn * words + w_word) * 4;
+    GB *nz_src = (GB *)nzB + ((size_t)gn * words + k_begin / 32 + w_word) * 4;
+    GB *sg_src = (GB *)sgB + ((size_t)gn * words + k_begin / 32 + w_word) * 4;
     // the scale of group g travels as the aligned dword that contains it; sc_half picks the half
-    GB *sc_src = (GB *)scB + (size_t)gn * groups * 2;
+    GB *sc_src = (GB *)scB + ((size_t)gn * groups + g_begin) * 2;
     const int w_off = chunk_off(w_row, w_word * 4);      // chunk c of the word: w_off ^ (c << 4)
     const int fr_off = chunk_off(li, lq);                // fragment i, step ks: (fr_off ^ (ks << 5)) + i * 32 rows
 
@@ -297,6 +305,59 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
         }
     }
 
+    // ---- split K: every workgroup of a tile leaves its fp32 sums in its own slot; the one that
+    // arrives last adds all slots in split order (its own included, read back: the result does not
+    // depend on who is last) and stores. The slots are written with stores that go through to memory
+    // (sc1) and are acknowledged (s_waitcnt vmcnt(0)) before the workgroup counts as arrived; the
+    // reader drops what its L2 may still hold of the slots (acquire fence = invalidate, cheap) and
+    // then reads them with ordinary 16-byte loads. A release fence instead of the write-through
+    // stores would write back the whole L2 of the XCD and cost more than the GEMM.
+    if (splits > 1) {
+        constexpr int kSlot = BM * kBN;  // floats; element (c, tid, e) of a slot at (c * kThreads + tid) * 4 + e
+        float *mine = partial + ((size_t)tile * splits + split) * kSlot + tid * 4;
+#pragma unroll
+        for (int i = 0; i < kNF; i++)
+#pragma unroll
+            for (int j = 0; j < MF; j++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const f4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                    float *dst = mine + (size_t)((i * MF + j) * 4 + g) * kThreads * 4;
+                    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(dst), "v"(v) : "memory");
+                }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __shared__ unsigned last_arrival;
+        __syncthreads();
+        if (tid == 0) {
+            const unsigned before = __hip_atomic_fetch_add(&arrivals[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            last_arrival = before == (unsigned)splits - 1;
+            if (last_arrival) __hip_atomic_store(&arrivals[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+        }
+        __syncthreads();
+        if (!last_arrival) return;
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        const float *slots = partial + (size_t)tile * splits * kSlot + tid * 4;
+#pragma unroll
+        for (int i = 0; i < kNF; i++)
+#pragma unroll
+            for (int j = 0; j < MF; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+        for (int q = 0; q < splits; q++) {
+            const float *slot = slots + (size_t)q * kSlot;
+#pragma unroll
+            for (int i = 0; i < kNF; i++)
+#pragma unroll
+                for (int j = 0; j < MF; j++)
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        const f4 v = *reinterpret_cast<const f4 *>(slot + (size_t)((i * MF + j) * 4 + g) * kThreads * 4);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) acc[i][j][4 * g + e] += v[e];
+                    }
+        }
+    }
+
     // ---- store: lane (k half lq, column li) of fragment (i, j) holds, for activation row m, the weight
     // rows n0 + 32 i + 8 g + 4 lq + v in register 4 g + v (g, v = 0..3)
     uint16_t *Cg = C;
@@ -327,8 +388,54 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
     }
 }
 
+// Split-K workspace: fp32 slots and arrival counters, one set per (device, stream), created on the
+// first call that needs it and grown on demand (the only allocation this file makes; never during
+// a call that does not split). Calls on one stream run in order and so may share a set.
+struct SplitWorkspace {
+    int device = -1;
+    hipStream_t stream = nullptr;
+    float *partial = nullptr;
+    size_t floats = 0;
+    unsigned *arrivals = nullptr;
+    size_t tiles = 0;
+};
+std::mutex g_ws_mutex;
+std::vector<SplitWorkspace> g_ws;
+
+hipError_t split_workspace(hipStream_t s, size_t floats, size_t tiles, float **partial, unsigned **arrivals) {
+    int dev = 0;
+    if (hipError_t e = hipGetDevice(&dev)) return e;
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    SplitWorkspace *w = nullptr;
+    for (SplitWorkspace &c : g_ws)
+        if (c.device == dev && c.stream == s) w = &c;
+    if (!w) {
+        g_ws.push_back(SplitWorkspace{});
+        w = &g_ws.back();
+        w->device = dev;
+        w->stream = s;
+    }
+    if (w->floats < floats || w->tiles < tiles) {
+        if (hipError_t e = hipStreamSynchronize(s)) return e;  // earlier launches may still use the old buffers
+        if (w->partial) (void)hipFree(w->partial);
+        if (w->arrivals) (void)hipFree(w->arrivals);
+        w->partial = nullptr;
+        w->arrivals = nullptr;
+        w->floats = w->tiles = 0;
+        const size_t nf = floats > w->floats ? floats : w->floats, nt = tiles > 1024 ? tiles : 1024;
+        if (hipError_t e = hipMalloc(reinterpret_cast<void **>(&w->partial), nf * sizeof(float))) return e;
+        if (hipError_t e = hipMalloc(reinterpret_cast<void **>(&w->arrivals), nt * sizeof(unsigned))) return e;
+        if (hipError_t e = hipMemset(w->arrivals, 0, nt * sizeof(unsigned))) return e;
+        w->floats = nf;
+        w->tiles = nt;
+    }
+    *partial = w->partial;
+    *arrivals = w->arrivals;
+    return hipSuccess;
+}
+
 template <int MF>
-hipError_t launch(const Problem &p, hipStream_t s) {
+hipError_t launch(const Problem &p, int splits, hipStream_t s) {
     constexpr int BM = 128 * MF;
     static bool attr_set[64] = {};
     int dev = 0;
@@ -341,8 +448,13 @@ hipError_t launch(const Problem &p, hipStream_t s) {
         attr_set[dev] = true;
     }
     const int m_tiles = (p.batch + BM - 1) / BM, n_tiles = (p.rows + kBN - 1) / kBN;
-    gemm_mfma_kernel<MF><<<m_tiles * n_tiles, kThreads, lds, s>>>(p.x, p.nz, p.sg, p.scales, p.y, p.batch, p.rows,
-                                                                  p.cols);
+    const int tiles = m_tiles * n_tiles;
+    float *partial = nullptr;
+    unsigned *arrivals = nullptr;
+    if (splits > 1)
+        if (hipError_t e = split_workspace(s, (size_t)tiles * splits * BM * kBN, (size_t)tiles, &partial, &arrivals)) return e;
+    gemm_mfma_kernel<MF><<<tiles * splits, kThreads, lds, s>>>(p.x, p.nz, p.sg, p.scales, p.y, p.batch, p.rows, p.cols,
+                                                              splits, partial, arrivals);
     return hipGetLastError();
 }
 
@@ -356,10 +468,17 @@ bool gemm_mfma_supports(const Problem &p, int group) {
 }
 
 namespace {
+struct GemmConfig {
+    int height;  // 0: 128 activation rows per workgroup, 1: 256
+    int splits;  // workgroups per tile along K
+    float us;    // estimated time
+};
+
 // One workgroup occupies a CU (LDS). Taller tiles do more per stage, shorter tiles fill the chip
-// when there are few of them: take the height with the smallest (rounds of workgroups over the
-// CUs) x (time of one stage, measured: 1.19 / 0.70 us for 256 / 128 activation rows).
-int choose_height(const Problem &p, float *stage_rounds_us) {
+// when there are few of them, and when even those leave CUs idle K is split across workgroups.
+// Estimate: (rounds of workgroups over the CUs) x (stages per workgroup) x (time of one stage,
+// measured: 1.19 / 0.70 us for 256 / 128 activation rows) + 5 us + the traffic of a split's exchange.
+GemmConfig choose_config(const Problem &p) {
     static int cus[64] = {};
     int dev = 0, n_cu = 256;
     if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64) {
@@ -367,31 +486,32 @@ int choose_height(const Problem &p, float *stage_rounds_us) {
             cus[dev] = 0;
         if (cus[dev] > 0) n_cu = cus[dev];
     }
-    const int n_tiles = (p.rows + kBN - 1) / kBN;
+    const int n_tiles = (p.rows + kBN - 1) / kBN, groups = p.cols / 128;
     const float stage_us[2] = {0.70f, 1.19f};
-    int best = 0;
-    float best_cost = 0.f;
+    GemmConfig best{0, 1, 0.f};
     for (int c = 0; c < 2; c++) {
         const int bm = 128 << c;
-        const long wgs = (long)n_tiles * ((p.batch + bm - 1) / bm);
-        const float cost = (float)((wgs + n_cu - 1) / n_cu) * stage_us[c];
-        if (c == 0 || cost < best_cost) best = c, best_cost = cost;
+        const long tiles = (long)n_tiles * ((p.batch + bm - 1) / bm);
+        for (int splits = 1; splits <= 8; splits *= 2) {
+            if (splits > 1 && (tiles * splits > n_cu || groups / splits < 4)) break;  // only to fill idle CUs
+            const long wgs = tiles * splits;
+            const float stages = (float)((groups + splits - 1) / splits * 2);
+            // the exchange writes and reads every fp32 partial tile once, at about 1.5 TB/s
+            const float exchange = splits > 1 ? 2.0f * (float)wgs * (float)(bm * kBN * 4) / 1.5e6f : 0.0f;
+            const float us = (float)((wgs + n_cu - 1) / n_cu) * stages * stage_us[c] + 5.0f + exchange;
+            if (best.us == 0.f || us < best.us) best = GemmConfig{c, splits, us};
+        }
     }
-    if (stage_rounds_us) *stage_rounds_us = best_cost;
     return best;
 }
 }  // namespace
 
-float gemm_mfma_cost_us(const Problem &p) {
-    float per_stage = 0.f;
-    (void)choose_height(p, &per_stage);
-    return per_stage * (float)(p.cols / kBK) + 5.0f;
-}
+float gemm_mfma_cost_us(const Problem &p) { return choose_config(p).us; }
 
 hipError_t launch_gemm_mfma(const Problem &p, hipStream_t s) {
-    const int best = choose_height(p, nullptr);
-    if (best == 1) return launch<2>(p, s);
-    return launch<1>(p, s);
+    const GemmConfig c = choose_config(p);
+    if (c.height == 1) return launch<2>(p, c.splits, s);
+    return launch<1>(p, c.splits, s);
 }
 
 }  // namespace tllm

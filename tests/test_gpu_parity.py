@@ -207,6 +207,44 @@ def test_gemm_rows_equal_gemv(dev, oracle):
         assert_close(oracle, yv, ref, what=f"gemv row {m}")
 
 
+def test_gemm_split_k_repeatable_and_streams(dev, oracle):
+    """Shapes with few weight tiles split K across workgroups (fp32 partial tiles exchanged through a
+    per-stream workspace, summed in a fixed order): every repetition must give the same bits, the
+    workspace must survive a change of shape, and two streams must not disturb each other."""
+    torch, tl = dev
+    cases = []
+    for k, (M, N, K) in enumerate([(512, 1024, 4096), (130, 512, 2048), (512, 1024, 4096), (256, 256, 8192)]):
+        nz, sg, s, _ = synth.problem(4000 + k, N, K)
+        A = synth.acts_f16(np.random.default_rng(4100 + k), M, K)
+        ref_rows = np.unique(np.random.default_rng(k).integers(0, M, 5))
+        ref = oracle.gemm_f64(A[ref_rows].view(np.uint16), nz, sg, s.view(np.uint16))
+        cases.append((M, N, K, up(torch, A), up(torch, nz), up(torch, sg), up(torch, s), ref_rows, ref))
+    first = {}
+    for rep in range(3):
+        for k, (M, N, K, dA, dnz, dsg, ds, rows, ref) in enumerate(cases):
+            Cm = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+            tl.ternary_gemm(dA, dnz, dsg, ds, Cm, M, N, K, 128)
+            torch.cuda.synchronize()
+            got = Cm.cpu().numpy()
+            assert_close(oracle, got.astype(np.float64)[rows], ref, what=f"split-K {M}x{N}x{K} rep {rep}")
+            if k in first:
+                assert np.array_equal(got.view(np.uint16), first[k]), f"case {k} rep {rep}: bits changed"
+            else:
+                first[k] = got.view(np.uint16).copy()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    outs = []
+    for rep in range(4):
+        for st, k in ((s1, 0), (s2, 3)):
+            M, N, K, dA, dnz, dsg, ds, rows, ref = cases[k]
+            Cm = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+            with torch.cuda.stream(st):
+                tl.ternary_gemm(dA, dnz, dsg, ds, Cm, M, N, K, 128, stream=st)
+            outs.append((k, Cm))
+    torch.cuda.synchronize()
+    for k, Cm in outs:
+        assert np.array_equal(Cm.cpu().numpy().view(np.uint16), first[k]), f"two streams: case {k} differs"
+
+
 # ---------------------------------------------------------- batched decode
 @pytest.mark.parametrize("M,N,K", [(2, 16, 512), (3, 17, 512), (4, 4096, 14336 // 7), (4, 1000, 1536),
                                    (8, 300, 4096), (13, 255, 1024), (16, 256, 512), (16, 1031, 2048),

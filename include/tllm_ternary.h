@@ -88,7 +88,7 @@ int tllm_quantize_absmax_i8(const uint16_t *input, int8_t *output, float *scale,
  * A fp16 [M,K] row-major, packed weight [N,K], C fp16 [M,N] row-major.
  * Replaces ternary::ternary_gemm, reference include/kernels.cuh:37-40
  * (kernels/ternary_gemm.cu:33-195). Any M >= 1 is accepted.
-  * Allocation: none per call, except that the first call on a stream whose shape leaves CUs idle
+ * Allocation: none per call, except that the first call on a stream whose shape leaves CUs idle
  * (few weight tiles) creates a per-stream fp32 workspace for splitting K, grown on demand.
  */
 int tllm_ternary_gemm_f16(const uint16_t *A, const uint32_t *nz_B, const uint32_t *sign_B,

@@ -155,10 +155,10 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
         w.hi = (sc_addr & 2) != 0;
     };
     auto scale_of = [](const Masks &w) -> uint32_t { return w.hi ? w.sc >> 16 : w.sc & 0xFFFFu; };
-    auto dma_acts = [&](int buf, int stage) {
+    auto dma_acts = [&](int buf, int stage, int t_begin, int t_end) {
         const int k0 = min(stage, last) * kBK;
 #pragma unroll
-        for (int t = 0; t < kDma; t++)
+        for (int t = t_begin; t < t_end; t++)
             __builtin_amdgcn_global_load_lds(
                 (__attribute__((address_space(1))) const void *)(a_src[t] + k0 * 2),
                 (__attribute__((address_space(3))) void *)(lds_dma + kActBase + buf * kActBytes + wave * kActWave + t * 1024),
@@ -212,8 +212,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
     // private to a wave, ordered by the wave's own waits.
     Masks w;
     u4 af0[kNF], af1[kNF], bf0[MF], bf1[MF];
-    dma_acts(0, 0);
-    dma_acts(1, 1);
+    dma_acts(0, 0, 0, kDma);
+    dma_acts(1, 1, 0, kDma);
 #pragma unroll
     for (int u = 0; u < kBufs; u++) dma_masks(u, u);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -239,15 +239,18 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
             Decoder d;
             unsigned char *Ws = lds + ((u + 2) % kBufs) * kWBytes;
             uint32_t o[16];
-            dma_acts((u + 2) % kBufs, s + 2);
+            // the activation requests of stage s+2 are spread over the four steps (a quarter each, behind
+            // the step's first MFMAs): issued back to back they hold the wave up
+            constexpr int kQ = kDma / 4;
             // ---- step 0 (af0/bf0)
             mfma_row(af0[0], bf0, 0);
             __builtin_amdgcn_sched_barrier(0);
-            // masks of stage s+2: requested in stage s-3; newer requests: 2 stages of (kDma + 3), this stage's kDma
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * kDma + 6) : "memory");
+            // masks of stage s+2: requested in stage s-3; newer requests: 2 stages of (kDma + 3)
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kDma + 6) : "memory");
             read_masks(w, (u + 2) % kBufs, s + 2);
             read_w(af1, u, 1);
             read_a(bf1, u, 1);
+            dma_acts((u + 2) % kBufs, s + 2, 0, kQ);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 1; i < kNF; i++) mfma_row(af0[i], bf0, i);
@@ -257,6 +260,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
             __builtin_amdgcn_sched_barrier(0);
             read_w(af0, u, 2);
             read_a(bf0, u, 2);
+            dma_acts((u + 2) % kBufs, s + 2, kQ, 2 * kQ);
             d.begin(w.nz, w.sg, scale_of(w));
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -273,6 +277,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
             __builtin_amdgcn_sched_barrier(0);
             read_w(af1, u, 3);
             read_a(bf1, u, 3);
+            dma_acts((u + 2) % kBufs, s + 2, 2 * kQ, 3 * kQ);
             *reinterpret_cast<u4 *>(Ws + (w_off ^ (0 << 4))) = u4{o[0], o[1], o[2], o[3]};
             *reinterpret_cast<u4 *>(Ws + (w_off ^ (1 << 4))) = u4{o[4], o[5], o[6], o[7]};
             __builtin_amdgcn_sched_barrier(0);
@@ -291,8 +296,9 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
             *reinterpret_cast<u4 *>(Ws + (w_off ^ (2 << 4))) = u4{o[8], o[9], o[10], o[11]};
             *reinterpret_cast<u4 *>(Ws + (w_off ^ (3 << 4))) = u4{o[12], o[13], o[14], o[15]};
             read_w(af0, (u + 1) % kBufs, 0);
-            // the activations of stage s+1 were requested at the top of stage s-1; newer requests: the
-            // masks of that stage (3) and this stage's activations (kDma)
+            dma_acts((u + 2) % kBufs, s + 2, 3 * kQ, kDma);
+            // the activations of stage s+1 were requested during stage s-1; newer requests: the masks
+            // of that stage (3) and this stage's activations (kDma)
             asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kDma + 3) : "memory");
             read_a(bf0, (u + 1) % kBufs, 0);
             __builtin_amdgcn_sched_barrier(0);

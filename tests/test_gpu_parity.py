@@ -179,6 +179,15 @@ def test_gemm_vs_oracle(dev, oracle, M, N, K):
     assert_close(oracle, run_gemm(dev, A, nz, sg, s), ref, what=f"gemm {M}x{N}x{K}")
 
 
+@pytest.mark.parametrize("group,M", [(32, 3), (64, 20), (256, 5)])
+def test_gemm_other_group_sizes(dev, oracle, group, M):
+    """Group sizes the .tllm files do not use still give the reference's result (general kernel)."""
+    nz, sg, s, _ = synth.problem(group + M, 72, 1024, group=group)
+    A = synth.acts_f16(np.random.default_rng(group), M, 1024)
+    ref = oracle.gemm_f64(A.view(np.uint16), nz, sg, s.view(np.uint16), group)
+    assert_close(oracle, run_gemm(dev, A, nz, sg, s, group), ref, what=f"gemm group {group}")
+
+
 def test_gemm_prefill_shapes_sampled(dev, oracle):
     """8B gate/up and down shapes at M=16 and M=512; the oracle is evaluated on sampled output
     rows/columns (the full fp64 product would take minutes), every output is checked finite."""

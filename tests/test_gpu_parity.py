@@ -171,7 +171,8 @@ def test_golden_fixtures_on_gpu(dev, oracle):
 
 # -------------------------------------------------------------------- GEMM
 @pytest.mark.parametrize("M,N,K", [(2, 64, 256), (4, 1024, 4096), (5, 100, 1152), (16, 512, 2048),
-                                   (33, 130, 640), (64, 256, 1024), (128, 384, 2048), (130, 200, 896)])
+                                   (33, 130, 640), (64, 256, 1024), (128, 384, 2048), (130, 200, 896),
+                                   (130, 200, 2688), (300, 100, 3072), (257, 129, 5248)])  # K split unevenly
 def test_gemm_vs_oracle(dev, oracle, M, N, K):
     nz, sg, s, _ = synth.problem(M * 1000 + N, N, K, dontcare_sign=True)
     A = synth.acts_f16(np.random.default_rng(M + K), M, K)

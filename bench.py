@@ -280,7 +280,8 @@ def main():
         "metric": "ternary GEMV packed-weight GB/s (% HBM peak) at B=1; GEMM TOPS at M=512",
         "value": round(gbps, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f16 activations x 2-bit ternary weights, f32 accumulation",
+        "vs_baseline": None, "dtype": "f16",
+        "dtype_detail": "fp16 activations x 2-bit ternary weights (fp16 group scales), fp32 accumulation, fp16 outputs",
         "data": "synthetic (seeded; P(0)=%.2f, fp16 scales U[%.3f,%.3f], x ~ N(0,1))" % (args.p_zero, lo, hi),
         "config": {
             "workload": f"cfg3: {args.model} {layers}-layer decode projection sweep "

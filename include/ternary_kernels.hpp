@@ -1,9 +1,10 @@
 // Drop-in C++ operator interface over the C ABI (include/tllm_ternary.h).
 //
 // Re-declares the four ternary operators of the reference's `namespace ternary`
-// (include/kernels.cuh:11-40) with the same names, argument order and default stream,
-// so the call expressions in src/transformer.cpp:107-116, 132-142, 201-217, 266-278
-// compile unchanged against this header. `half` is HIP's __half (hip/hip_fp16.h) and the
+// (include/kernels.cuh:11-40) and the two element-wise operators next to them
+// (include/kernels.cuh:45-48, 60-62) with the same names, argument order and default stream,
+// so the call expressions in src/transformer.cpp:107-116, 132-142, 193-196, 201-217, 258-261,
+// 266-278, 285-286 compile unchanged against this header. `half` is HIP's __half (hip/hip_fp16.h) and the
 // stream is a hipStream_t. Like the reference these return void; a rejected call is
 // reported through the optional handler below instead of being silently dropped.
 #pragma once
@@ -70,6 +71,22 @@ inline void ternary_gemm(const half *A, const uint32_t *nz_B, const uint32_t *si
            tllm_ternary_gemm_f16(reinterpret_cast<const uint16_t *>(A), nz_B, sign_B,
                                  reinterpret_cast<const uint16_t *>(scales_B),
                                  reinterpret_cast<uint16_t *>(C), M, N, K, group_size, stream));
+}
+
+// Reference include/kernels.cuh:45-48.
+inline void rmsnorm_forward(const half *input, const half *weight, half *output, const half *residual,
+                            half *residual_out, int batch, int dim, float eps, hipStream_t stream = 0) {
+    report("rmsnorm_forward",
+           tllm_rmsnorm_f16(reinterpret_cast<const uint16_t *>(input), reinterpret_cast<const uint16_t *>(weight),
+                            reinterpret_cast<uint16_t *>(output), reinterpret_cast<const uint16_t *>(residual),
+                            reinterpret_cast<uint16_t *>(residual_out), batch, dim, eps, stream));
+}
+
+// Reference include/kernels.cuh:60-62.
+inline void silu_mul_forward(const half *gate, const half *up, half *output, int size, hipStream_t stream = 0) {
+    report("silu_mul_forward",
+           tllm_silu_mul_f16(reinterpret_cast<const uint16_t *>(gate), reinterpret_cast<const uint16_t *>(up),
+                             reinterpret_cast<uint16_t *>(output), size, stream));
 }
 
 }  // namespace ternary

@@ -96,6 +96,25 @@ int tllm_ternary_gemm_f16(const uint16_t *A, const uint32_t *nz_B, const uint32_
                           int group_size, tllm_stream_t stream);
 
 /*
+ * output[b, i] = fp16( t[b, i] / sqrt(mean_i t[b, i]^2 + eps) * weight[i] ),  t = input (+ residual), fp32.
+ * residual may be NULL; residual_out, when given (with a residual), receives fp16(t) and the
+ * normalised output is then computed from that rounded value, as the reference does.
+ * Replaces ternary::rmsnorm_forward, reference include/kernels.cuh:45-48 (kernels/rmsnorm.cu:20-127):
+ * the operator in front of every projection group (src/transformer.cpp:193-196, 258-261).
+ */
+int tllm_rmsnorm_f16(const uint16_t *input, const uint16_t *weight, uint16_t *output,
+                     const uint16_t *residual, uint16_t *residual_out, int batch, int dim, float eps,
+                     tllm_stream_t stream);
+
+/*
+ * output[i] = fp16( gate[i] / (1 + exp(-gate[i])) * up[i] ), fp32 arithmetic.
+ * Replaces ternary::silu_mul_forward, reference include/kernels.cuh:60-62
+ * (kernels/activations.cu:18-74): the operator between the gate/up and the down projection.
+ */
+int tllm_silu_mul_f16(const uint16_t *gate, const uint16_t *up, uint16_t *output, int size,
+                      tllm_stream_t stream);
+
+/*
  * Several independent ternary linears in ONE launch (e.g. q/k/v, gate/up, or a whole
  * back-to-back projection sweep). Each problem is what one tllm_ternary_gemv_f16 /
  * small-M tllm_ternary_gemm_f16 call would take: input fp16 [batch, cols],

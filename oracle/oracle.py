@@ -60,7 +60,10 @@ def load():
     L.tllm_oracle_gemv_i8_f64.argtypes = [_u32p, _u32p, _u16p, _i8p, C.c_float, _f64p, C.c_int,
                                           C.c_int, C.c_int]
     L.tllm_oracle_ternarize.argtypes = [_f32p, C.c_int64, C.c_int, C.c_float, _i8p, _u16p]
-    for f in ("pack", "unpack", "gemv_f64", "gemv_hostloop", "gemv_hostloop_mt", "gemm_f64",
+    L.tllm_oracle_rmsnorm_f64.argtypes = [_u16p, _u16p, C.c_void_p, C.c_void_p, _f64p, C.c_int, C.c_int,
+                                          C.c_float]
+    L.tllm_oracle_silu_mul_f64.argtypes = [_u16p, _u16p, _f64p, C.c_int]
+    for f in ("rmsnorm_f64", "silu_mul_f64", "pack", "unpack", "gemv_f64", "gemv_hostloop", "gemv_hostloop_mt", "gemm_f64",
               "gemm_f32_elem", "quantize_i8", "gemv_i8_f64", "ternarize"):
         getattr(L, "tllm_oracle_" + f).restype = None
     _lib = L
@@ -151,6 +154,25 @@ def gemv_i8_f64(nz, sg, scales, xq, input_scale, group=128):
     load().tllm_oracle_gemv_i8_f64(nz, sg, _c(scales, np.uint16), _c(xq, np.int8),
                                    float(input_scale), y, rows, words * 32, group)
     return y
+
+
+def rmsnorm_f64(x, w, eps, residual=None, store_residual=False):
+    """x, residual: fp16 bits [batch, dim]; w: fp16 bits [dim]. Returns (out f64, residual_out bits or None)."""
+    x, w = _c(x, np.uint16), _c(w, np.uint16)
+    batch, dim = x.shape
+    out = np.empty((batch, dim), np.float64)
+    res = _c(residual, np.uint16) if residual is not None else None
+    ro = np.empty((batch, dim), np.uint16) if (store_residual and res is not None) else None
+    load().tllm_oracle_rmsnorm_f64(x, w, res.ctypes.data if res is not None else None,
+                                   ro.ctypes.data if ro is not None else None, out, batch, dim, float(eps))
+    return out, ro
+
+
+def silu_mul_f64(gate, up):
+    gate, up = _c(gate, np.uint16).reshape(-1), _c(up, np.uint16).reshape(-1)
+    out = np.empty(gate.size, np.float64)
+    load().tllm_oracle_silu_mul_f64(gate, up, out, gate.size)
+    return out
 
 
 def ternarize(w, group=128, factor=0.7):

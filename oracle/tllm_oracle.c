@@ -16,6 +16,8 @@
  *   tllm_oracle_quantize_i8 ..... kernels/activations.cu:100-141
  *   tllm_oracle_gemv_i8_f64 ..... kernels/ternary_gemv.cu:148-198
  *   tllm_oracle_ternarize ....... ternarize/pack.py:41-101
+ *   tllm_oracle_rmsnorm_f64 ..... kernels/rmsnorm.cu:20-106
+ *   tllm_oracle_silu_mul_f64 .... kernels/activations.cu:18-59
  *
  * Pinning status (what each function is checked against in tests/test_oracle.py):
  *   pack/unpack ........ the known-answer words of tests/test_packing.py:55-81
@@ -35,6 +37,13 @@
  *                        would produce for its torch seeds 42/123 are parity unpinned
  *                        (they depend on torch's random stream; only shape/dtype/value-set
  *                        properties are asserted by the reference for those seeds).
+ *   rmsnorm_f64 ........ the reference holds no test or fixture for it; pinned by closed
+ *                        forms (constant row -> c/sqrt(c^2+eps); unit RMS of the output at
+ *                        eps=0, w=1; invariance under x -> a*x at eps=0; linearity in w;
+ *                        residual path == plain path on the pre-added fp16 sum) and a numpy
+ *                        restatement through np.linalg.norm.
+ *   silu_mul_f64 ....... closed forms (silu(0)=0, silu(g)-silu(-g)=g, g>>0 -> g*u) and
+ *                        scipy.special.expit.
  */
 #include <math.h>
 #include <pthread.h>
@@ -310,6 +319,48 @@ void tllm_oracle_gemv_i8_f64(const uint32_t *nz, const uint32_t *sg, const uint1
             acc += (double)tllm_oracle_half_to_float(scales[(size_t)r * groups + g]) * (double)gs;
         }
         y[r] = (double)input_scale * acc;
+    }
+}
+
+/* ----------------------------------------------------------- element-wise */
+
+/* RMSNorm with the optional residual add. t = x (+ r), the sum formed in fp32 as the kernel does;
+ * res_out (may be NULL) receives fp16(t) and, when given, the normalised value is taken from that
+ * rounded copy. The mean square always uses the unrounded t. Everything else in fp64; out is left
+ * unrounded. */
+void tllm_oracle_rmsnorm_f64(const uint16_t *x, const uint16_t *w, const uint16_t *res,
+                             uint16_t *res_out, double *out, int batch, int dim, float eps) {
+    for (int b = 0; b < batch; b++) {
+        size_t o = (size_t)b * dim;
+        double ss = 0.0;
+        for (int i = 0; i < dim; i++) {
+            float t = tllm_oracle_half_to_float(x[o + i]);
+            if (res) {
+                t += tllm_oracle_half_to_float(res[o + i]);
+                if (res_out) res_out[o + i] = tllm_oracle_float_to_half(t);
+            }
+            ss += (double)t * (double)t;
+        }
+        double inv = 1.0 / sqrt(ss / (double)dim + (double)eps);
+        for (int i = 0; i < dim; i++) {
+            double t;
+            if (res && res_out)
+                t = (double)tllm_oracle_half_to_float(res_out[o + i]);
+            else if (res)
+                t = (double)(tllm_oracle_half_to_float(x[o + i]) + tllm_oracle_half_to_float(res[o + i]));
+            else
+                t = (double)tllm_oracle_half_to_float(x[o + i]);
+            out[o + i] = t * inv * (double)tllm_oracle_half_to_float(w[i]);
+        }
+    }
+}
+
+/* out = gate / (1 + exp(-gate)) * up, fp64, unrounded. */
+void tllm_oracle_silu_mul_f64(const uint16_t *gate, const uint16_t *up, double *out, int n) {
+    for (int i = 0; i < n; i++) {
+        double g = (double)tllm_oracle_half_to_float(gate[i]);
+        double u = (double)tllm_oracle_half_to_float(up[i]);
+        out[i] = g / (1.0 + exp(-g)) * u;
     }
 }
 

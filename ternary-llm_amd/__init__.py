@@ -9,6 +9,8 @@ from .ops import (  # noqa: F401
     lib,
     lib_path,
     quantize_absmax_int8,
+    rmsnorm,
+    silu_mul,
     ternary_gemm,
     ternary_gemv,
     ternary_gemv_int8,

@@ -7,7 +7,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libtllm_ternary.so")
-SOURCES = ["capi.hip", "dispatch.hip", "rowwave.hip", "gemv_mfma.hip", "gemv_batch.hip", "gemm_mfma.hip", "model_file.hip"]
+SOURCES = ["capi.hip", "dispatch.hip", "rowwave.hip", "gemv_mfma.hip", "gemv_batch.hip", "gemm_mfma.hip", "elementwise.hip", "model_file.hip"]
 # packed fp32 VALU forms are disabled on purpose for every device compile.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-command-line-argument",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

@@ -128,6 +128,21 @@ int tllm_quantize_absmax_i8(const uint16_t *input, int8_t *output, float *scale,
     return (int)tllm::launch_quantize_absmax_i8(input, output, scale, n, (hipStream_t)stream);
 }
 
+int tllm_rmsnorm_f16(const uint16_t *input, const uint16_t *weight, uint16_t *output, const uint16_t *residual,
+                     uint16_t *residual_out, int batch, int dim, float eps, tllm_stream_t stream) {
+    if (!input || !weight || !output) return TLLM_ERR_NULL_POINTER;
+    if (batch < 1 || dim < 1) return TLLM_ERR_BAD_SHAPE;
+    if ((int64_t)batch * dim > INT32_MAX) return TLLM_ERR_TOO_LARGE;
+    if (residual_out && !residual) return TLLM_ERR_NULL_POINTER;
+    return (int)tllm::launch_rmsnorm(input, weight, output, residual, residual_out, batch, dim, eps, (hipStream_t)stream);
+}
+
+int tllm_silu_mul_f16(const uint16_t *gate, const uint16_t *up, uint16_t *output, int size, tllm_stream_t stream) {
+    if (!gate || !up || !output) return TLLM_ERR_NULL_POINTER;
+    if (size < 1) return TLLM_ERR_BAD_SHAPE;
+    return (int)tllm::launch_silu_mul(gate, up, output, size, (hipStream_t)stream);
+}
+
 int tllm_linear_plan_create(tllm_linear_plan **plan, const tllm_linear_problem *problems,
                             int count, int group_size) {
     if (!plan || !problems) return TLLM_ERR_NULL_POINTER;

@@ -49,6 +49,11 @@ hipError_t launch_gemv_rowwave_i8(const uint32_t *nz, const uint32_t *sg, const 
 hipError_t launch_quantize_absmax_i8(const uint16_t *x, int8_t *q, float *scale, int n,
                                      hipStream_t s);
 
+// Element-wise neighbours of the linears (elementwise.hip).
+hipError_t launch_rmsnorm(const uint16_t *input, const uint16_t *weight, uint16_t *output, const uint16_t *residual,
+                          uint16_t *residual_out, int batch, int dim, float eps, hipStream_t s);
+hipError_t launch_silu_mul(const uint16_t *gate, const uint16_t *up, uint16_t *output, int size, hipStream_t s);
+
 // 128-group MFMA GEMV, batch 1..4 (gemv_mfma.hip).
 bool gemv_mfma_supports(const Problem &p, int group);
 hipError_t launch_gemv_mfma(const Problem &p, hipStream_t s);

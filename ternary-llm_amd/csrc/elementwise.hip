@@ -1,0 +1,173 @@
+// The two decode-step element-wise operators that sit directly around the ternary linears: RMSNorm
+// (with the optional fused residual add) in front of every projection group and SiLU(gate) * up
+// between the FFN projections. Both are bandwidth-trivial (a few KB per token); fp32 arithmetic,
+// fp16 in and out, as the reference's kernels.
+#include "common.h"
+
+namespace tllm {
+namespace {
+
+constexpr int kNormThreads = 256;
+
+// Reference kernels/rmsnorm.cu:20-106. One workgroup per token row. With a residual the sum
+// t = x + r is formed in fp32; the mean square uses that fp32 value, while the normalised output is
+// computed from the fp16-rounded t when it is also stored to residual_out (the reference re-reads
+// what it stored), else from the fp32 t. Every element is read and written by the same lane in both
+// passes, so output may be input and residual_out may be residual.
+__global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(const uint16_t *input, const uint16_t *__restrict__ weight,
+                                                               uint16_t *output, const uint16_t *residual,
+                                                               uint16_t *residual_out, int dim, float eps) {
+    __shared__ float partial[kNormThreads / kWave];
+    const size_t row = (size_t)blockIdx.x * dim;
+    const uint16_t *x = input + row, *r = residual ? residual + row : nullptr;
+    uint16_t *ro = residual_out ? residual_out + row : nullptr;
+    float ss = 0.0f;
+    for (int i = threadIdx.x; i < dim; i += kNormThreads) {
+        float v = h2f(x[i]);
+        if (r) {
+            v += h2f(r[i]);
+            if (ro) ro[i] = f2h(v);
+        }
+        ss += v * v;
+    }
+    ss = wave_sum(ss);
+    if ((threadIdx.x & (kWave - 1)) == 0) partial[threadIdx.x / kWave] = ss;
+    __syncthreads();
+    float total = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kNormThreads / kWave; w++) total += partial[w];
+    const float inv = 1.0f / sqrtf(total / (float)dim + eps);
+    for (int i = threadIdx.x; i < dim; i += kNormThreads) {
+        float v;
+        if (r) v = ro ? h2f(ro[i]) : h2f(x[i]) + h2f(r[i]);
+        else v = h2f(x[i]);
+        output[row + i] = f2h(v * inv * h2f(weight[i]));
+    }
+}
+
+// The same operator for rows of up to 2048 * kChunks elements whose pointers are 16-byte aligned and
+// whose length is a multiple of 8: every lane keeps its 8-element chunks in registers between the
+// two passes, so the row is read once, through 16-byte loads.
+template <int kChunks>
+__global__ __launch_bounds__(kNormThreads) void rmsnorm_rows_kernel(const uint16_t *input,
+                                                                    const uint16_t *__restrict__ weight,
+                                                                    uint16_t *output, const uint16_t *residual,
+                                                                    uint16_t *residual_out, int dim, float eps) {
+    __shared__ float partial[kNormThreads / kWave];
+    const size_t row = (size_t)blockIdx.x * dim;
+    const int chunks = dim >> 3;
+    float v[kChunks][8];
+    float ss = 0.0f;
+#pragma unroll
+    for (int c = 0; c < kChunks; c++) {
+        const int chunk = c * kNormThreads + threadIdx.x;
+        if (chunk >= chunks) break;
+        const size_t at = row + (size_t)chunk * 8;
+        const uint4 xq = *(const uint4 *)(input + at);
+        const uint32_t xw[4] = {xq.x, xq.y, xq.z, xq.w};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            v[c][2 * j] = h2f((uint16_t)xw[j]);
+            v[c][2 * j + 1] = h2f((uint16_t)(xw[j] >> 16));
+        }
+        if (residual) {
+            const uint4 rq = *(const uint4 *)(residual + at);
+            const uint32_t rw[4] = {rq.x, rq.y, rq.z, rq.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                v[c][2 * j] += h2f((uint16_t)rw[j]);
+                v[c][2 * j + 1] += h2f((uint16_t)(rw[j] >> 16));
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) ss += v[c][j] * v[c][j];
+        if (residual && residual_out) {
+            uint32_t o[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint16_t lo = f2h(v[c][2 * j]), hi = f2h(v[c][2 * j + 1]);
+                o[j] = (uint32_t)lo | (uint32_t)hi << 16;
+                v[c][2 * j] = h2f(lo);  // the normalised value is taken from the rounded copy
+                v[c][2 * j + 1] = h2f(hi);
+            }
+            *(uint4 *)(residual_out + at) = make_uint4(o[0], o[1], o[2], o[3]);
+        }
+    }
+    ss = wave_sum(ss);
+    if ((threadIdx.x & (kWave - 1)) == 0) partial[threadIdx.x / kWave] = ss;
+    __syncthreads();
+    float total = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kNormThreads / kWave; w++) total += partial[w];
+    const float inv = 1.0f / sqrtf(total / (float)dim + eps);
+#pragma unroll
+    for (int c = 0; c < kChunks; c++) {
+        const int chunk = c * kNormThreads + threadIdx.x;
+        if (chunk >= chunks) break;
+        const uint4 wq = *(const uint4 *)(weight + (size_t)chunk * 8);
+        const uint32_t ww[4] = {wq.x, wq.y, wq.z, wq.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            o[j] = (uint32_t)f2h(v[c][2 * j] * inv * h2f((uint16_t)ww[j])) |
+                   (uint32_t)f2h(v[c][2 * j + 1] * inv * h2f((uint16_t)(ww[j] >> 16))) << 16;
+        *(uint4 *)(output + row + (size_t)chunk * 8) = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+}
+
+// Reference kernels/activations.cu:18-59: out = gate / (1 + exp(-gate)) * up. The reference calls it
+// in place (output == gate, src/transformer.cpp:285), so neither pointer is declared restrict.
+__device__ __forceinline__ uint16_t silu_mul_one(uint16_t gate, uint16_t up) {
+    const float g = h2f(gate);
+    return f2h(g / (1.0f + expf(-g)) * h2f(up));
+}
+
+// Eight elements per lane through 16-byte loads; `vec8` counts the full groups, the remaining
+// size - 8*vec8 elements are handled one per lane by the workgroups past the vector part.
+__global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t *gate, const uint16_t *up, uint16_t *output,
+                                                       int size, int vec8) {
+    const int t = blockIdx.x * 256 + threadIdx.x;
+    if (t < vec8) {
+        const uint4 g = ((const uint4 *)gate)[t], u = ((const uint4 *)up)[t];
+        const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, uw[4] = {u.x, u.y, u.z, u.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            o[j] = (uint32_t)silu_mul_one((uint16_t)gw[j], (uint16_t)uw[j]) |
+                   (uint32_t)silu_mul_one((uint16_t)(gw[j] >> 16), (uint16_t)(uw[j] >> 16)) << 16;
+        ((uint4 *)output)[t] = make_uint4(o[0], o[1], o[2], o[3]);
+        return;
+    }
+    const int i = vec8 * 8 + (t - vec8);
+    if (i < size) output[i] = silu_mul_one(gate[i], up[i]);
+}
+
+}  // namespace
+
+hipError_t launch_rmsnorm(const uint16_t *input, const uint16_t *weight, uint16_t *output, const uint16_t *residual,
+                          uint16_t *residual_out, int batch, int dim, float eps, hipStream_t s) {
+    const uintptr_t all = (uintptr_t)input | (uintptr_t)weight | (uintptr_t)output | (uintptr_t)residual |
+                          (uintptr_t)residual_out;
+    const int per_pass = kNormThreads * 8;
+    if ((all & 15) == 0 && dim % 8 == 0 && dim <= 4 * per_pass) {
+        if (dim <= per_pass)
+            rmsnorm_rows_kernel<1><<<batch, kNormThreads, 0, s>>>(input, weight, output, residual, residual_out, dim, eps);
+        else if (dim <= 2 * per_pass)
+            rmsnorm_rows_kernel<2><<<batch, kNormThreads, 0, s>>>(input, weight, output, residual, residual_out, dim, eps);
+        else
+            rmsnorm_rows_kernel<4><<<batch, kNormThreads, 0, s>>>(input, weight, output, residual, residual_out, dim, eps);
+    } else {
+        rmsnorm_kernel<<<batch, kNormThreads, 0, s>>>(input, weight, output, residual, residual_out, dim, eps);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_silu_mul(const uint16_t *gate, const uint16_t *up, uint16_t *output, int size, hipStream_t s) {
+    const bool aligned = (((uintptr_t)gate | (uintptr_t)up | (uintptr_t)output) & 15) == 0;
+    const int vec8 = aligned ? size / 8 : 0;
+    const int lanes = vec8 + (size - vec8 * 8);
+    silu_mul_kernel<<<(lanes + 255) / 256, 256, 0, s>>>(gate, up, output, size, vec8);
+    return hipGetLastError();
+}
+
+}  // namespace tllm

@@ -16,7 +16,7 @@ ABI_SYMBOLS = (
     "tllm_error_string", "tllm_abi_version", "tllm_ternary_gemv_f16", "tllm_ternary_gemv_i8",
     "tllm_ternary_gemv_i8_dscale", "tllm_quantize_absmax_i8", "tllm_ternary_gemm_f16",
     "tllm_linear_plan_create", "tllm_linear_plan_launch", "tllm_linear_plan_weight_bytes",
-    "tllm_linear_plan_destroy",
+    "tllm_linear_plan_destroy", "tllm_rmsnorm_f16", "tllm_silu_mul_f16",
 )
 # include/tllm_model_file.h
 FILE_ABI_SYMBOLS = (
@@ -80,6 +80,8 @@ def lib():
     L.tllm_linear_plan_weight_bytes.restype = C.c_int64
     L.tllm_linear_plan_destroy.argtypes = [vp]
     L.tllm_linear_plan_destroy.restype = None
+    L.tllm_rmsnorm_f16.argtypes = [vp, vp, vp, vp, vp, i, i, f, vp]
+    L.tllm_silu_mul_f16.argtypes = [vp, vp, vp, i, vp]
     L.tllm_ternarize_pack_f32.argtypes = [vp, i, i, i, f, vp, vp, vp]
     L.tllm_model_file_open.argtypes = [C.c_char_p, C.POINTER(vp)]
     L.tllm_model_file_close.argtypes = [vp]
@@ -146,6 +148,17 @@ def ternary_gemm(A, nz_B, sign_B, scales_B, Cout, M, N, K, group_size=128, strea
     """C[M,N] = A[M,K] @ W[N,K]^T (reference include/kernels.cuh:37-40)."""
     check(lib().tllm_ternary_gemm_f16(_ptr(A), _ptr(nz_B), _ptr(sign_B), _ptr(scales_B), _ptr(Cout),
                                       M, N, K, group_size, _stream(stream)))
+
+
+def rmsnorm(input, weight, output, residual, residual_out, batch, dim, eps, stream=None):
+    """RMSNorm with optional fused residual add (reference include/kernels.cuh:45-48)."""
+    check(lib().tllm_rmsnorm_f16(_ptr(input), _ptr(weight), _ptr(output), _ptr(residual), _ptr(residual_out),
+                                 batch, dim, float(eps), _stream(stream)))
+
+
+def silu_mul(gate, up, output, size, stream=None):
+    """SiLU(gate) * up (reference include/kernels.cuh:60-62)."""
+    check(lib().tllm_silu_mul_f16(_ptr(gate), _ptr(up), _ptr(output), size, _stream(stream)))
 
 
 class LinearPlan:

@@ -1,6 +1,6 @@
 // Compile-and-run check of the C++ drop-in interface: the call expressions below have
 // the shapes of the reference's callers (src/transformer.cpp:107-116 ternary_linear,
-// :132-142 ternary_linear_int8). With null pointers every call must be rejected by the
+// :132-142 ternary_linear_int8, :193-196 rmsnorm_forward, :285-286 silu_mul_forward). With null pointers every call must be rejected by the
 // argument validation before any GPU work, so this runs on a host without a GPU.
 #include <cstdio>
 #include <cstdlib>
@@ -37,6 +37,13 @@ int main() {
     ternary::quantize_absmax_int8(input, int8_buf_, int8_scale_, dim);
     ternary::ternary_gemv_int8(w.nonzero_masks, w.sign_masks, w.scales, int8_buf_, h_scale, output,
                                w.out_features, w.in_features, gs);
+    half *residual_buf_ = nullptr, *hidden_buf_ = nullptr, *gate_buf_ = nullptr, *up_buf_ = nullptr;
+    const half *attn_norm_weight = nullptr;
+    int hidden = 2048, inter = 5632;
+    float rms_norm_eps = 1e-5f;
+    ternary::rmsnorm_forward(residual_buf_, attn_norm_weight, hidden_buf_, nullptr, nullptr, n_tokens, hidden,
+                             rms_norm_eps);
+    ternary::silu_mul_forward(gate_buf_, up_buf_, gate_buf_, n_tokens * inter);
     std::printf("rejected=%d\n", rejected);
-    return rejected == 4 ? 0 : 1;
+    return rejected == 6 ? 0 : 1;
 }

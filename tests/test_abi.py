@@ -53,6 +53,12 @@ def test_validation_codes():
     assert L.tllm_quantize_absmax_i8(0x10, 0x20, 0x40, 0, None) == -2
     assert L.tllm_ternary_gemv_i8(0x1000, 0x2000, 0x3000, None, 1.0, 0x5000, 4, 256, 128, None) == -1
     assert L.tllm_ternary_gemv_i8_dscale(0x1000, 0x2000, 0x3000, 0x4000, None, 0x5000, 4, 256, 128, None) == -1
+    assert L.tllm_rmsnorm_f16(None, 0x20, 0x30, None, None, 1, 8, 1e-5, None) == -1
+    assert L.tllm_rmsnorm_f16(0x10, 0x20, 0x30, None, 0x40, 1, 8, 1e-5, None) == -1   # residual_out without residual
+    assert L.tllm_rmsnorm_f16(0x10, 0x20, 0x30, None, None, 0, 8, 1e-5, None) == -2
+    assert L.tllm_rmsnorm_f16(0x10, 0x20, 0x30, None, None, 1 << 20, 1 << 12, 1e-5, None) == -4
+    assert L.tllm_silu_mul_f16(0x10, None, 0x30, 4, None) == -1
+    assert L.tllm_silu_mul_f16(0x10, 0x20, 0x30, 0, None) == -2
     h = C.c_void_p(0)
     assert L.tllm_linear_plan_create(C.byref(h), None, 1, 128) == -1
     arr = (ops._Problem * 1)(ops._Problem(0x1000, 0x2000, 0x3000, 0x4000, 0x9000, 4, 256, 17, 0))
@@ -76,4 +82,4 @@ def test_cpp_dropin_call_shapes(tmp_path):
     subprocess.run(cmd, check=True, capture_output=True, text=True)
     out = subprocess.run([str(exe)], capture_output=True, text=True)
     assert out.returncode == 0, out.stdout + out.stderr
-    assert "rejected=4" in out.stdout
+    assert "rejected=6" in out.stdout

@@ -326,6 +326,99 @@ def test_batched_plan_8b_layer_batch4_and_16(dev, oracle):
         plan.close()
 
 
+
+# ------------------------------------------------------------- element-wise
+def _half_out(oracle, ref):
+    """fp16 rounding of an fp64 reference, as float64 (for a 1-ulp comparison)."""
+    return np.asarray(ref, np.float64).astype(np.float16).astype(np.float64)
+
+
+@pytest.mark.parametrize("batch,dim", [(1, 4096), (1, 2048), (3, 8192), (512, 4096), (2, 100), (1, 1), (5, 257),
+                                       (2, 8), (3, 5120), (2, 8200)])
+def test_rmsnorm_vs_oracle(dev, oracle, batch, dim):
+    torch, tl = dev
+    rng = np.random.default_rng(batch * 131 + dim)
+    x = oracle.half_bits(rng.normal(0, 1.5, (batch, dim)))
+    w = oracle.half_bits(rng.normal(1, 0.3, dim))
+    eps = 1e-5
+    ref, _ = oracle.rmsnorm_f64(x, w, eps)
+    y = torch.full((batch, dim), float("nan"), dtype=torch.float16, device="cuda")
+    tl.rmsnorm(up(torch, x), up(torch, w), y, None, None, batch, dim, eps)
+    torch.cuda.synchronize()
+    assert_close(oracle, y.cpu().numpy().astype(np.float64), ref, what=f"rmsnorm {batch}x{dim}")
+    # in place, as a caller that normalises its own buffer would
+    xin = up(torch, x)
+    tl.rmsnorm(xin, up(torch, w), xin, None, None, batch, dim, eps)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(xin.cpu().numpy(), y.cpu().numpy())
+
+
+@pytest.mark.parametrize("dim", [264, 2048, 4096, 6144, 16384])
+@pytest.mark.parametrize("store", [False, True])
+def test_rmsnorm_residual_vs_oracle(dev, oracle, store, dim):
+    torch, tl = dev
+    batch, eps = 7, 1e-6
+    rng = np.random.default_rng(99 + dim)
+    x = oracle.half_bits(rng.normal(0, 1, (batch, dim)))
+    r = oracle.half_bits(rng.normal(0, 2, (batch, dim)))
+    w = oracle.half_bits(rng.normal(1, 0.3, dim))
+    ref, ro_ref = oracle.rmsnorm_f64(x, w, eps, residual=r, store_residual=store)
+    y = torch.full((batch, dim), float("nan"), dtype=torch.float16, device="cuda")
+    ro = torch.full((batch, dim), float("nan"), dtype=torch.float16, device="cuda") if store else None
+    tl.rmsnorm(up(torch, x), up(torch, w), y, up(torch, r), ro, batch, dim, eps)
+    torch.cuda.synchronize()
+    assert_close(oracle, y.cpu().numpy().astype(np.float64), ref, what="rmsnorm+residual")
+    if store:   # fp32 add then one fp16 rounding: bit-exact
+        np.testing.assert_array_equal(ro.cpu().numpy().view(np.uint16), ro_ref)
+
+
+def test_rmsnorm_closed_form_on_gpu(dev, oracle):
+    torch, tl = dev
+    dim = 4096
+    x = torch.full((2, dim), 3.0, dtype=torch.float16, device="cuda")
+    w = torch.ones(dim, dtype=torch.float16, device="cuda")
+    y = torch.empty_like(x)
+    tl.rmsnorm(x, w, y, None, None, 2, dim, 0.0)
+    torch.cuda.synchronize()
+    assert (y.cpu().numpy() == np.float16(1.0)).all()
+
+
+@pytest.mark.parametrize("n", [1, 2, 255, 14336, 512 * 14336 + 1])
+def test_silu_mul_vs_oracle(dev, oracle, n):
+    torch, tl = dev
+    rng = np.random.default_rng(n)
+    g = oracle.half_bits(rng.normal(0, 3, n))
+    u = oracle.half_bits(rng.normal(0, 1, n))
+    ref = oracle.silu_mul_f64(g, u)
+    gd, ud = up(torch, g), up(torch, u)
+    out = torch.full((n,), float("nan"), dtype=torch.float16, device="cuda")
+    tl.silu_mul(gd, ud, out, n)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy().astype(np.float64)
+    assert_close(oracle, got, ref, what=f"silu_mul {n}")
+    # the reference calls it in place on the gate buffer (src/transformer.cpp:285)
+    tl.silu_mul(gd, ud, gd, n)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(gd.cpu().numpy(), out.cpu().numpy())
+    if n > 2:   # buffers that start on an odd element (2-byte alignment only)
+        gd = up(torch, g)
+        out2 = torch.full((n,), float("nan"), dtype=torch.float16, device="cuda")
+        tl.silu_mul(gd[1:], ud[1:], out2[1:], n - 1)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(out2.cpu().numpy()[1:], out.cpu().numpy()[1:])
+
+
+def test_silu_mul_tails(dev, oracle):
+    torch, tl = dev
+    g = np.array([0.0, -0.0, 40.0, -40.0, 65504.0, -65504.0, 1.0], np.float16)
+    u = np.array([5.0, 5.0, 2.0, 2.0, 1.0, 1.0, 1.0], np.float16)
+    out = torch.full((7,), float("nan"), dtype=torch.float16, device="cuda")
+    tl.silu_mul(up(torch, g), up(torch, u), out, 7)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy().astype(np.float64)
+    assert got[0] == 0 and got[1] == 0 and got[2] == 80.0 and got[3] == 0 and got[4] == 65504.0 and got[5] == 0
+    assert got[6] == np.float64(np.float16(1.0 / (1.0 + np.exp(-1.0))))
+
 # --------------------------------------------------------------- INT8 pair
 @pytest.mark.parametrize("n", [1, 63, 2048, 4096, 14336, 28672])
 def test_quantize_bit_exact(dev, oracle, n):

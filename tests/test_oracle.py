@@ -271,3 +271,77 @@ def test_golden_fixtures(oracle):
             np.testing.assert_allclose(got, y[b], rtol=1e-12, atol=1e-14)
         got = oracle.gemm_f64(x, nz, sg, s, fx["group"])
         np.testing.assert_allclose(got, y, rtol=1e-12, atol=1e-14)
+
+
+# ------------------------------------------------------------ element-wise
+def test_rmsnorm_closed_forms(oracle):
+    dim, eps = 384, float(np.float32(1e-5))   # eps travels as a C float
+    ones = oracle.half_bits(np.ones(dim))
+    # constant row c: every output is c / sqrt(c^2 + eps)
+    for c in (0.5, -2.0, 3.0):
+        out, _ = oracle.rmsnorm_f64(oracle.half_bits(np.full((1, dim), c)), ones, eps)
+        np.testing.assert_allclose(out, c / np.sqrt(c * c + eps), rtol=1e-14)
+    rng = np.random.default_rng(5)
+    x = oracle.half_bits(rng.normal(0, 1.3, (3, dim)))
+    # eps = 0, w = 1: the output has unit RMS; and scaling x by a power of two changes nothing
+    out, _ = oracle.rmsnorm_f64(x, ones, 0.0)
+    np.testing.assert_allclose(np.sqrt((out ** 2).mean(axis=1)), 1.0, rtol=1e-13)
+    x4 = oracle.half_bits(oracle.half_values(x) * 4.0)
+    out4, _ = oracle.rmsnorm_f64(x4, ones, 0.0)
+    np.testing.assert_allclose(out4, out, rtol=1e-13)
+    # the weight multiplies element-wise and is shared by the rows (not indexed by row)
+    w = oracle.half_bits(rng.normal(1, 0.2, dim))
+    outw, _ = oracle.rmsnorm_f64(x, w, eps)
+    out1, _ = oracle.rmsnorm_f64(x, ones, eps)
+    np.testing.assert_allclose(outw, out1 * oracle.half_values(w)[None, :], rtol=1e-13)
+    # numpy restatement through the 2-norm: x * sqrt(dim) / sqrt(|x|^2 + dim*eps)
+    xv = oracle.half_values(x)
+    ref = xv * np.sqrt(dim) / np.sqrt(np.linalg.norm(xv, axis=1, keepdims=True) ** 2 + dim * eps)
+    np.testing.assert_allclose(out1, ref, rtol=1e-13)
+
+
+def test_rmsnorm_residual_path(oracle):
+    dim, eps = 256, float(np.float32(1e-5))
+    rng = np.random.default_rng(6)
+    # values on a coarse grid: x + r is exact in fp16, so all three variants must coincide
+    x = oracle.half_bits(rng.integers(-64, 64, (2, dim)) / 8.0)
+    r = oracle.half_bits(rng.integers(-64, 64, (2, dim)) / 8.0)
+    w = oracle.half_bits(rng.normal(1, 0.2, dim))
+    summed = oracle.half_bits(oracle.half_values(x) + oracle.half_values(r))
+    plain, _ = oracle.rmsnorm_f64(summed, w, eps)
+    fused, ro = oracle.rmsnorm_f64(x, w, eps, residual=r, store_residual=True)
+    nostore, none = oracle.rmsnorm_f64(x, w, eps, residual=r)
+    assert none is None
+    np.testing.assert_array_equal(ro, summed)
+    np.testing.assert_allclose(fused, plain, rtol=1e-14)
+    np.testing.assert_allclose(nostore, plain, rtol=1e-14)
+    # inexact sums: the stored residual is the RNE fp16 of the fp32 sum; the statistic uses the
+    # unrounded sum, the normalised value the rounded one
+    x = oracle.half_bits(rng.normal(0, 1, (2, dim)))
+    r = oracle.half_bits(rng.normal(0, 1, (2, dim)))
+    t32 = oracle.half_values(x).astype(np.float32) + oracle.half_values(r).astype(np.float32)
+    fused, ro = oracle.rmsnorm_f64(x, w, eps, residual=r, store_residual=True)
+    np.testing.assert_array_equal(ro, t32.astype(np.float16).view(np.uint16))
+    inv = 1.0 / np.sqrt((t32.astype(np.float64) ** 2).mean(axis=1, keepdims=True) + eps)
+    np.testing.assert_allclose(fused, oracle.half_values(ro) * inv * oracle.half_values(w), rtol=1e-13)
+    nostore, _ = oracle.rmsnorm_f64(x, w, eps, residual=r)
+    np.testing.assert_allclose(nostore, t32.astype(np.float64) * inv * oracle.half_values(w), rtol=1e-13)
+
+
+def test_silu_mul_closed_forms(oracle):
+    from scipy.special import expit
+    rng = np.random.default_rng(7)
+    g = rng.normal(0, 3, 1001).astype(np.float16)
+    u = rng.normal(0, 1, 1001).astype(np.float16)
+    one = np.ones_like(g)
+    out = oracle.silu_mul_f64(g.view(np.uint16), u.view(np.uint16))
+    gv, uv = g.astype(np.float64), u.astype(np.float64)
+    np.testing.assert_allclose(out, gv * expit(gv) * uv, rtol=1e-13, atol=1e-300)
+    # silu(0) = 0; silu(g) - silu(-g) = g; far right tail is the identity, far left tail vanishes
+    assert oracle.silu_mul_f64(np.zeros(4, np.uint16), one[:4].view(np.uint16)).tolist() == [0.0] * 4
+    sp = oracle.silu_mul_f64(g.view(np.uint16), one.view(np.uint16))
+    sm = oracle.silu_mul_f64((-g).view(np.uint16), one.view(np.uint16))
+    np.testing.assert_allclose(sp - sm, gv, rtol=1e-13, atol=1e-15)
+    tail = oracle.silu_mul_f64(np.array([40.0, -40.0], np.float16).view(np.uint16),
+                               np.array([2.0, 2.0], np.float16).view(np.uint16))
+    assert tail[0] == pytest.approx(80.0, rel=1e-15) and abs(tail[1]) < 1e-15

@@ -43,7 +43,7 @@ constexpr int kImageBytes = 16 * kSliceCols * 2;             // operands of one 
 struct BatchSched {
     const Problem *table;    // device table, or nullptr: use the by-value problem
     const int *unit_prefix;  // [count + 1] first block of each problem
-    const int *wg_first;     // [grid + 1] first block of each workgroup
+    const int *wg_first;     // [grid + 1] first block of each workgroup, then [grid] the problem that block is in
 };
 
 struct Tile {
@@ -89,10 +89,11 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
     const int li = lane & 15;  // MFMA A row / D column (activation row)
     const int lq = lane >> 4;  // MFMA k quarter / D row quad
 
-    int u = 0, u_end = 0;
+    int u = 0, u_end = 0, pi = 0;
     if (sc.table) {
         u = sc.wg_first[blockIdx.x];
         u_end = sc.wg_first[blockIdx.x + 1];
+        pi = sc.wg_first[gridDim.x + 1 + blockIdx.x];  // no scan over the problems before this span
     } else {
         const int total = (single.rows + kBlockRows - 1) / kBlockRows;
         u = (int)((int64_t)total * blockIdx.x / gridDim.x);
@@ -103,7 +104,6 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
     uint32_t zero_o[16];
     decode_word(0u, 0u, zero_o);
 
-    int pi = 0;
     Problem p = single;
     for (; u < u_end; u++) {
         int first_unit = 0;

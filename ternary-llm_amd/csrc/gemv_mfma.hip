@@ -19,6 +19,8 @@
 //   Wide (batch 1):   4 rows x 2048 columns. Lanes 4a..4a+3 read 64 contiguous bytes of row a, so
 //                     the loads coalesce; result column j is scale group j of the slice.
 //   Tall (batch 1-4): 16 rows x 512 columns. Result column j is group j % 4 of batch column j / 4.
+#include <cstdio>
+#include <cstdlib>
 #include "common.h"
 #include "gemv_layout.h"
 
@@ -61,7 +63,7 @@ struct Tall {
 struct Sched {
     const Problem *table;    // device table, or nullptr: use the by-value problem
     const int *unit_prefix;  // [count + 1] first unit of each problem
-    const int *wg_first;     // [grid + 1] first unit of each workgroup
+    const int *wg_first;     // [grid + 1] first unit of each workgroup, then [grid] the problem that unit is in
     int count;
     int max_units;    // units per task (bounds the partial-sum area)
     int max_batch;    // largest batch of any problem (sizes the per-wave partial-sum areas)
@@ -155,10 +157,11 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
     const int lq = lane >> 4;  // MFMA k quarter / D row quad
 
     constexpr int kUnitRows = kNW * G::kRows * kTilesAhead;
-    int u = 0, u_end = 0;
+    int u = 0, u_end = 0, pi = 0;
     if (sc.table) {
         u = sc.wg_first[blockIdx.x];
         u_end = sc.wg_first[blockIdx.x + 1];
+        pi = sc.wg_first[gridDim.x + 1 + blockIdx.x];  // no scan over the problems before this span
     } else {
         const int total = (single.rows + kUnitRows - 1) / kUnitRows;
         u = (int)((int64_t)total * blockIdx.x / gridDim.x);
@@ -166,7 +169,6 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
     }
 
     int cur = -1;  // problem whose activations are staged
-    int pi = 0;
     Problem p = single;
     int slices = 0, groups = 0, words = 0, img_stride = 0;
 
@@ -200,24 +202,44 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
                 for (int e = 0; e < 8; e++) h[e] = f2h((float)(int8_t)(w2[e >> 2] >> (8 * (e & 3))));
                 return uint4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
             };
-            // (a) per batch column: largest magnitude -> power-of-two normalisation
-            for (int b = 0; b < p.batch; b++) {
-                uint32_t m = 0;
-                for (int c8 = tid; c8 < p.cols / 8; c8 += kThreads) {
-                    const uint4 v = load8(b, c8);
-                    const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
+            // Image element (slice, t, chunk, e) = fp16(x[col] * 2^(14-ex-p)), where 2^ex is the power
+            // of two at or below the largest magnitude of the batch column. The last slice of a row
+            // that is not a whole number of slices is moved left so that it ends with the row; the
+            // chunks it then shares with the slice before it are zero in the image. Eight-element
+            // pieces are numbered in image order; piece_of() loads the activations of one.
+            const int pieces = img_stride / 8;
+            auto piece_of = [&](int b, int c8) -> uint4 {
+                const int slice = (c8 * 8) / G::kCols;
+                const int chunk = ((c8 * 8) % G::kCols) / kChunkCols;
+                const int g = min(slice * G::kChunks, groups - G::kChunks) + chunk;
+                if (g < slice * G::kChunks) return uint4{0u, 0u, 0u, 0u};
+                return load8(b, (g * kChunkCols + (c8 * 8) % kChunkCols) / 8);
+            };
+            auto magnitude = [](uint32_t m, const uint4 &v) -> uint32_t {
+                const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        m = max(m, w4[e] & 0x7FFFu);
-                        m = max(m, (w4[e] >> 16) & 0x7FFFu);
-                    }
+                for (int e = 0; e < 4; e++) {
+                    m = max(m, w4[e] & 0x7FFFu);
+                    m = max(m, (w4[e] >> 16) & 0x7FFFu);
                 }
+                return m;
+            };
+            auto write_piece = [&](uint16_t *img, int c8, const uint4 &v, int ex) {
+                const int slice = (c8 * 8) / G::kCols;
+                const int chunk = ((c8 * 8) % G::kCols) / kChunkCols;
+                const int cc0 = (c8 * 8) % kChunkCols;
+                const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
+                uint16_t *dst = img + slice * G::kCols;
 #pragma unroll
-                for (int off = 32; off > 0; off >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, off, kWave));
-                if (lane == 0) red_amax[wave][b] = m;
-            }
-            __syncthreads();
-            for (int b = 0; b < p.batch; b++) {
+                for (int e = 0; e < 8; e++) {
+                    const OperandSlot s = chunk_slot(cc0 + e);
+                    const float mult = __builtin_bit_cast(float, (uint32_t)(127 + 14 - ex - s.p) << 23);
+                    const uint16_t hx = (uint16_t)(w4[e >> 1] >> (16 * (e & 1)));
+                    dst[image_index(s.t, chunk, s.e, G::kChunks)] = f2h(h2f(hx) * mult);
+                }
+            };
+            // amax bits -> exponent; also sets the output scale of the column
+            auto exponent_of = [&](int b) -> int {
                 uint32_t m = 0;
 #pragma unroll
                 for (int w = 0; w < kNW; w++) m = max(m, red_amax[w][b]);
@@ -230,26 +252,49 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
                     if (sc.x_is_i8) f *= sc.i8_scale_dev ? *sc.i8_scale_dev : sc.i8_scale;
                     fscale[b] = f;
                 }
-                // (b) image: operand element (slice, t, chunk, e) = fp16(x[col] * 2^(14-ex-p)). The last
-                // slice of a row that is not a whole number of slices is moved left so that it ends
-                // with the row; the chunks it then shares with the slice before it are zero here.
-                uint16_t *img = image + (size_t)b * img_stride;
-                for (int c8 = tid; c8 < img_stride / 8; c8 += kThreads) {
-                    const int slice = (c8 * 8) / G::kCols;
-                    const int chunk = ((c8 * 8) % G::kCols) / kChunkCols;
-                    const int cc0 = (c8 * 8) % kChunkCols;
-                    const int g = min(slice * G::kChunks, groups - G::kChunks) + chunk;
-                    uint4 v = {0u, 0u, 0u, 0u};
-                    if (g >= slice * G::kChunks && m) v = load8(b, (g * kChunkCols + cc0) / 8);
-                    const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
-                    uint16_t *dst = img + slice * G::kCols;
+                return ex;
+            };
+            // The piece addresses depend on the thread index only; hidden behind an empty asm they are
+            // worked out here, each time, instead of living in registers across the whole kernel.
+            int stid = tid;
+            asm volatile("" : "+v"(stid));
+            constexpr int kKeep = 8;  // pieces per thread that stay in registers between the two steps
+            if (p.batch == 1 && pieces <= kKeep * kThreads) {
+                // one pass over x: all loads are issued together and kept for the image
+                uint4 keep[kKeep];
+                uint32_t m = 0;
 #pragma unroll
-                    for (int e = 0; e < 8; e++) {
-                        const OperandSlot s = chunk_slot(cc0 + e);
-                        const float mult = __builtin_bit_cast(float, (uint32_t)(127 + 14 - ex - s.p) << 23);
-                        const uint16_t hx = (uint16_t)(w4[e >> 1] >> (16 * (e & 1)));
-                        dst[image_index(s.t, chunk, s.e, G::kChunks)] = f2h(h2f(hx) * mult);
-                    }
+                for (int k = 0; k < kKeep; k++) {
+                    const int c8 = stid + k * kThreads;
+                    keep[k] = c8 < pieces ? piece_of(0, c8) : uint4{0u, 0u, 0u, 0u};
+                }
+#pragma unroll
+                for (int k = 0; k < kKeep; k++) m = magnitude(m, keep[k]);
+#pragma unroll
+                for (int off = 32; off > 0; off >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, off, kWave));
+                if (lane == 0) red_amax[wave][0] = m;
+                __syncthreads();
+                const int ex = exponent_of(0);
+#pragma unroll
+                for (int k = 0; k < kKeep; k++) {
+                    const int c8 = stid + k * kThreads;
+                    if (c8 < pieces) write_piece(image, c8, keep[k], ex);
+                    __builtin_amdgcn_sched_barrier(0);  // one piece at a time: keeps the register need low
+                }
+            } else {
+                // long rows or several batch columns: one pass for the magnitudes, one for the image
+                for (int b = 0; b < p.batch; b++) {
+                    uint32_t m = 0;
+                    for (int c8 = stid; c8 < pieces; c8 += kThreads) m = magnitude(m, piece_of(b, c8));
+#pragma unroll
+                    for (int off = 32; off > 0; off >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, off, kWave));
+                    if (lane == 0) red_amax[wave][b] = m;
+                }
+                __syncthreads();
+                for (int b = 0; b < p.batch; b++) {
+                    const int ex = exponent_of(b);
+                    for (int c8 = stid; c8 < pieces; c8 += kThreads)
+                        write_piece(image + (size_t)b * img_stride, c8, piece_of(b, c8), ex);
                 }
             }
             __syncthreads();
@@ -500,7 +545,39 @@ bool tall_ok(const Problem &p) {
            image_bytes_of<Tall>(p.cols, p.batch) + kNW * range_unit<Tall>() * p.batch * 4 <= kLdsLimit;
 }
 
-constexpr int kMaxTaskUnits = 10;  // longer tasks amortise the per-slice operand reload
+#ifndef TLLM_MAX_TASK_UNITS
+#define TLLM_MAX_TASK_UNITS 20
+#endif
+constexpr int kMaxTaskUnits = TLLM_MAX_TASK_UNITS;  // longer tasks amortise the per-slice operand reload
+
+// The workgroups of one launch all start together, three per CU, and the CU serves its oldest
+// waves first: measured on the 8B sweep with equal spans, the first 256 workgroups (one per CU)
+// finished after 233 us, the second 256 after 280 us and the last after 333 us; the odd XCDs
+// (workgroup index % 8) ran 8 % slower than the even ones, and what is left after these two effects
+// is +-2 %. Spans are therefore cut in proportion to the speed of the place a workgroup will run in,
+// so that they end together. TLLM_SPAN_SHARES="s0,s1,s2,odd" overrides the four factors.
+struct SpanShares {
+    double slot[3] = {1.38, 1.0, 0.68};
+    double odd_xcd = 0.92;
+};
+const SpanShares &span_shares() {
+    static const SpanShares shares = [] {
+        SpanShares v;
+        if (const char *e = getenv("TLLM_SPAN_SHARES")) {
+            SpanShares w;
+            if (sscanf(e, "%lf,%lf,%lf,%lf", &w.slot[0], &w.slot[1], &w.slot[2], &w.odd_xcd) == 4 && w.slot[0] > 0 &&
+                w.slot[1] > 0 && w.slot[2] > 0 && w.odd_xcd > 0)
+                v = w;
+        }
+        return v;
+    }();
+    return shares;
+}
+double span_share(int wg, int cus, int grid) {
+    if (grid != 3 * cus) return 1.0;  // measured for three full rounds of workgroups only
+    const SpanShares &v = span_shares();
+    return v.slot[wg / cus] * ((wg & 1) ? v.odd_xcd : 1.0);
+}
 
 // units per task that the partial-sum area can hold
 int max_units_for(int image_bytes, int batch, int unit) {
@@ -562,10 +639,10 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
         d.max_rows = p.rows > d.max_rows ? p.rows : d.max_rows;
     }
     d.max_batch = max_batch;
-    // contiguous spans of units of about equal weight (a unit's weights plus a fixed cost), at least
-    // one unit per workgroup
+    // Contiguous spans of units, one per workgroup, cut by weight (a unit's weights plus a fixed
+    // cost) in proportion to the workgroup's share; at least one unit per workgroup.
     std::vector<int> prefix(host.size() + 1, 0), wg_first;
-    auto partition = [&](int unit, int wgs) {
+    auto partition = [&](int unit, int wgs, bool shares) {
         std::vector<int64_t> weight;
         for (size_t i = 0; i < host.size(); i++) {
             const int n = (host[i].rows + unit - 1) / unit;
@@ -579,14 +656,22 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
         const int grid = units < wgs ? units : wgs;
         int64_t total_w = 0;
         for (int64_t w : weight) total_w += w;
+        std::vector<double> upto(grid + 1, 0.0);  // shares of the workgroups before g
+        for (int g = 0; g < grid; g++) upto[g + 1] = upto[g] + (shares ? span_share(g, di->cus, grid) : 1.0);
         wg_first.assign(grid + 1, units);
         wg_first[0] = 0;
         int64_t acc = 0;  // weight of units [0, t)
         int t = 0;
         for (int g = 1; g < grid; g++) {
             const int lo = wg_first[g - 1] + 1, hi = units - (grid - g);
-            while (t < hi && (t < lo || acc * grid < total_w * g)) acc += weight[t++];
+            const double want = (double)total_w * upto[g] / upto[grid];
+            while (t < hi && (t < lo || (double)acc < want)) acc += weight[t++];
             wg_first[g] = t;
+        }
+        // the problem each span starts in, so that a workgroup does not scan the prefix from 0
+        for (int g = 0, pr = 0; g < grid; g++) {
+            while (prefix[pr + 1] <= wg_first[g]) pr++;
+            wg_first.push_back(pr);
         }
         d.grid = grid;
     };
@@ -603,7 +688,7 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
     }
     if (all_batch) {
         d.batch_kernel = true;
-        partition(gemv_batch_block_rows(), di->cus);
+        partition(gemv_batch_block_rows(), di->cus, false);
     } else {
         d.wide = all_wide;
         d.use_mfma = all_wide || all_tall;
@@ -617,23 +702,26 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
         if (d.use_mfma) {
             d.lds_bytes = max_image + kNW * max_units * unit * max_batch * 4;
             const int per_cu = d.wide ? resident_wgs<Wide>(d.lds_bytes) : resident_wgs<Tall>(d.lds_bytes);
-            partition(unit, per_cu * di->cus);
+            partition(unit, per_cu * di->cus, true);
             d.max_units = max_units;
             d.image_bytes = max_image;
         }
     }
 
-    const size_t bytes_table = sizeof(Problem) * host.size();
-    const size_t bytes_prefix = sizeof(int) * prefix.size();
-    const size_t bytes_wg = sizeof(int) * wg_first.size();
+    // one allocation: table | unit prefix | spans
+    auto round16 = [](size_t v) { return (v + 15) / 16 * 16; };
+    const size_t bytes_table = round16(sizeof(Problem) * host.size());
+    const size_t bytes_prefix = round16(sizeof(int) * prefix.size());
+    const size_t bytes_wg = round16(sizeof(int) * wg_first.size());
     char *base = nullptr;
-    if (hipError_t e = hipMalloc(&base, bytes_table + bytes_prefix + bytes_wg + 64)) return e;
+    if (hipError_t e = hipMalloc(&base, bytes_table + bytes_prefix + bytes_wg + 16)) return e;
     d.problems = reinterpret_cast<Problem *>(base);
     d.unit_prefix = reinterpret_cast<int *>(base + bytes_table);
     d.wg_first = reinterpret_cast<int *>(base + bytes_table + bytes_prefix);
-    hipError_t e = hipMemcpy(d.problems, host.data(), bytes_table, hipMemcpyHostToDevice);
-    if (!e) e = hipMemcpy(d.unit_prefix, prefix.data(), bytes_prefix, hipMemcpyHostToDevice);
-    if (!e && bytes_wg) e = hipMemcpy(d.wg_first, wg_first.data(), bytes_wg, hipMemcpyHostToDevice);
+    hipError_t e = hipMemcpy(d.problems, host.data(), sizeof(Problem) * host.size(), hipMemcpyHostToDevice);
+    if (!e) e = hipMemcpy(d.unit_prefix, prefix.data(), sizeof(int) * prefix.size(), hipMemcpyHostToDevice);
+    if (!e && !wg_first.empty())
+        e = hipMemcpy(d.wg_first, wg_first.data(), sizeof(int) * wg_first.size(), hipMemcpyHostToDevice);
     if (e) {
         (void)hipFree(base);
         return e;

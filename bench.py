@@ -139,7 +139,7 @@ def cpu_baseline(oracle, problems, n_layer_mats, threads, mt_layers=8):
 MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense FP16 matrix peak
 
 
-def gemm_report(torch, tl, orc, seed, m_list, p_zero=0.42, calls=20):
+def gemm_report(torch, tl, orc, seed, m_list, p_zero=0.42, calls=200, warm=20):
     """Prefill GEMM (cfg4): LLaMA-3-8B gate/up 14336x4096 and down 4096x14336, M tokens each.
     Times `calls` back-to-back launches with events on the launch stream, checks sampled outputs
     against the FP64 oracle, and reports dense-equivalent 2*M*N*K flops."""
@@ -152,7 +152,7 @@ def gemm_report(torch, tl, orc, seed, m_list, p_zero=0.42, calls=20):
         for m in m_list:
             a = torch.randn((m, k), device="cuda", generator=gen).to(torch.float16)
             c = torch.zeros((m, n), dtype=torch.float16, device="cuda")
-            for _ in range(3):
+            for _ in range(warm):
                 tl.ternary_gemm(a, nz, sg, sc, c, m, n, k, 128)
             torch.cuda.synchronize()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -191,8 +191,10 @@ def gemm_report(torch, tl, orc, seed, m_list, p_zero=0.42, calls=20):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    # A step is 0.35 ms. The GPU idles at ~100 MHz and takes tens of milliseconds of load to settle at
+    # its working clocks: 5 warm-up steps give 0.367 ms per step over the next 20, 500 give 0.345.
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--model", default="llama8b", choices=sorted(SHAPES))
     ap.add_argument("--layers", type=int, default=0, help="0 = the model's own layer count")
     ap.add_argument("--batch", type=int, default=1)

@@ -89,6 +89,9 @@ struct PlanDevice {
     bool batch_kernel = false;  // the 2..16-row kernel runs (its blocks are the units below)
     int *unit_prefix = nullptr;
     int *wg_first = nullptr;
+    int *pool_first = nullptr;  // shared pool of small tasks (MFMA kernel, large plans)
+    int pool_count = 0;
+    int *counters = nullptr;
     int grid = 0;
     int max_units = 0;
     int image_bytes = 0;

@@ -64,6 +64,13 @@ struct Sched {
     const Problem *table;    // device table, or nullptr: use the by-value problem
     const int *unit_prefix;  // [count + 1] first unit of each problem
     const int *wg_first;     // [grid + 1] first unit of each workgroup, then [grid] the problem that unit is in
+    // Shared pool (large plans): tasks that belong to no span. A workgroup that has finished its
+    // span takes them one at a time through counters[0]; counters[1] counts the workgroups that
+    // have left, and the last one to leave sets both back to zero for the next launch. Launches of
+    // one plan must therefore not overlap (they would also race on the outputs).
+    const int *pool_first;  // [pool_count + 1] first unit of each pool task, then [pool_count] its problem
+    int pool_count;
+    int *counters;
     int count;
     int max_units;    // units per task (bounds the partial-sum area)
     int max_batch;    // largest batch of any problem (sizes the per-wave partial-sum areas)
@@ -172,7 +179,19 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
     Problem p = single;
     int slices = 0, groups = 0, words = 0, img_stride = 0;
 
-    while (u < u_end) {
+    __shared__ int pool_task;
+    for (;;) {
+        if (u >= u_end) {
+            // The span (or pool task) is done: go on with the pool task that was asked for when the
+            // walks of the task before ended. The two barriers that end a task lie between the write
+            // of pool_task and this read, and between this read and the next write.
+            if (sc.pool_count == 0) break;
+            const int t = __builtin_amdgcn_readfirstlane(pool_task);
+            if (t >= sc.pool_count) break;
+            u = sc.pool_first[t];
+            u_end = sc.pool_first[t + 1];
+            pi = sc.pool_first[sc.pool_count + 1 + t];
+        }
         int first_unit = 0;
         int p_units = (single.rows + kUnitRows - 1) / kUnitRows;
         if (sc.table) {
@@ -466,6 +485,12 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
                 }
             }
         }
+        // last task of the span, or a pool task: ask for the next pool task now (not earlier: a
+        // request is a claim, and a workgroup must not claim work long before it can start it); the
+        // answer arrives while the partial sums are added up
+        const bool request = sc.pool_count != 0 && u >= u_end && tid == 0;
+        int requested = 0;
+        if (request) requested = __hip_atomic_fetch_add(sc.counters, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         // ------------------------------------------------ add the waves' partial sums in wave order, store fp16
         {
@@ -479,7 +504,15 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
                 p.y[(size_t)b * p.rows + r_begin + rl] = f2h(sum * fscale[b]);
             }
         }
+        if (request) pool_task = requested;
         __syncthreads();
+    }
+    if (sc.pool_count != 0 && tid == 0) {
+        const int left = __hip_atomic_fetch_add(sc.counters + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (left == (int)gridDim.x - 1) {  // every other workgroup has made its last request
+            __hip_atomic_store(sc.counters, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(sc.counters + 1, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
 }
 
@@ -557,7 +590,7 @@ constexpr int kMaxTaskUnits = TLLM_MAX_TASK_UNITS;  // longer tasks amortise the
 // is +-2 %. Spans are therefore cut in proportion to the speed of the place a workgroup will run in,
 // so that they end together. TLLM_SPAN_SHARES="s0,s1,s2,odd" overrides the four factors.
 struct SpanShares {
-    double slot[3] = {1.38, 1.0, 0.68};
+    double slot[3] = {1.4, 1.0, 0.65};
     double odd_xcd = 0.92;
 };
 const SpanShares &span_shares() {
@@ -578,6 +611,22 @@ double span_share(int wg, int cus, int grid) {
     const SpanShares &v = span_shares();
     return v.slot[wg / cus] * ((wg & 1) ? v.odd_xcd : 1.0);
 }
+
+// Part of a large plan's weights that is kept out of the spans and dealt out at run time in pieces
+// of about kPoolTaskWeights weights: spans of the right average size still do not end together
+// (+-4 % from workgroup to workgroup and launch to launch), and the last workgroup sets the time.
+// Measured on the 8B sweep in steady state: 0 -> 5375 GB/s, 0.10 -> 5495, 0.15 -> 5517, 0.30 slower
+// again (a pool task of 768 K weights spends a quarter of its 25 us on staging and hand-over).
+// TLLM_POOL_FRACTION overrides it (0 switches the pool off).
+double pool_fraction() {
+    static const double f = [] {
+        const char *e = getenv("TLLM_POOL_FRACTION");
+        const double v = e ? atof(e) : 0.15;
+        return v < 0.0 ? 0.0 : v > 0.5 ? 0.5 : v;
+    }();
+    return f;
+}
+constexpr int64_t kPoolTaskWeights = 768 * 1024;
 
 // units per task that the partial-sum area can hold
 int max_units_for(int image_bytes, int batch, int unit) {
@@ -639,25 +688,60 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
         d.max_rows = p.rows > d.max_rows ? p.rows : d.max_rows;
     }
     d.max_batch = max_batch;
+    // Device table order: the problems whose units are dealt out as spans, then those of the shared
+    // pool; `prefix` counts units in that order.
+    std::vector<Problem> ordered = host;
+    std::vector<int> prefix(host.size() + 1, 0), wg_first, pool_first;
     // Contiguous spans of units, one per workgroup, cut by weight (a unit's weights plus a fixed
-    // cost) in proportion to the workgroup's share; at least one unit per workgroup.
-    std::vector<int> prefix(host.size() + 1, 0), wg_first;
-    auto partition = [&](int unit, int wgs, bool shares) {
+    // cost) in proportion to the workgroup's share; at least one unit per workgroup. With
+    // max_task_units > 0 and enough work, the last problems with short rows (staging x is cheap
+    // there) go to the shared pool instead, cut into small tasks inside one problem each.
+    auto partition = [&](int unit, int wgs, int max_task_units) {
+        const int n = (int)host.size();
+        auto units_of = [&](const Problem &p) { return (p.rows + unit - 1) / unit; };
+        std::vector<char> pooled(n, 0);
+        int64_t all_w = 0;
+        int all_units = 0, min_cols = host[0].cols;
+        for (const Problem &p : host) {
+            all_w += (int64_t)p.rows * p.cols;
+            all_units += units_of(p);
+            min_cols = p.cols < min_cols ? p.cols : min_cols;
+        }
+        if (max_task_units > 0 && all_units >= 8 * wgs) {
+            const int64_t want = (int64_t)((double)all_w * pool_fraction());
+            int64_t got = 0;
+            int left_units = all_units;
+            for (int pass = 0; pass < 2 && got < want; pass++)
+                for (int i = n - 1; i >= 0 && got < want; i--) {
+                    if (pooled[i] || (pass == 0 && host[i].cols > 2 * min_cols)) continue;
+                    if (left_units - units_of(host[i]) < 4 * wgs) continue;
+                    pooled[i] = 1;
+                    got += (int64_t)host[i].rows * host[i].cols;
+                    left_units -= units_of(host[i]);
+                }
+        }
+        int k = 0, n_static = 0;
+        for (int pass = 0; pass < 2; pass++) {
+            for (int i = 0; i < n; i++)
+                if (pooled[i] == pass) ordered[k++] = host[i];
+            if (pass == 0) n_static = k;
+        }
         std::vector<int64_t> weight;
-        for (size_t i = 0; i < host.size(); i++) {
-            const int n = (host[i].rows + unit - 1) / unit;
-            prefix[i + 1] = prefix[i] + n;
-            for (int t = 0; t < n; t++) {
-                const int nr = host[i].rows - t * unit < unit ? host[i].rows - t * unit : unit;
-                weight.push_back((int64_t)nr * host[i].cols + 16384);
+        for (int i = 0; i < n; i++) {
+            const int nu = units_of(ordered[i]);
+            prefix[i + 1] = prefix[i] + nu;
+            for (int t = 0; t < nu && i < n_static; t++) {
+                const int nr = ordered[i].rows - t * unit < unit ? ordered[i].rows - t * unit : unit;
+                weight.push_back((int64_t)nr * ordered[i].cols + 16384);
             }
         }
-        const int units = prefix.back();
+        const int units = prefix[n_static];
         const int grid = units < wgs ? units : wgs;
         int64_t total_w = 0;
         for (int64_t w : weight) total_w += w;
         std::vector<double> upto(grid + 1, 0.0);  // shares of the workgroups before g
-        for (int g = 0; g < grid; g++) upto[g + 1] = upto[g] + (shares ? span_share(g, di->cus, grid) : 1.0);
+        for (int g = 0; g < grid; g++)
+            upto[g + 1] = upto[g] + (max_task_units > 0 ? span_share(g, di->cus, grid) : 1.0);
         wg_first.assign(grid + 1, units);
         wg_first[0] = 0;
         int64_t acc = 0;  // weight of units [0, t)
@@ -672,6 +756,21 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
         for (int g = 0, pr = 0; g < grid; g++) {
             while (prefix[pr + 1] <= wg_first[g]) pr++;
             wg_first.push_back(pr);
+        }
+        std::vector<int> pool_problem;
+        for (int i = n_static; i < n; i++) {
+            const int64_t unit_w = (int64_t)unit * ordered[i].cols;
+            int64_t per = (kPoolTaskWeights + unit_w / 2) / unit_w;
+            per = per < 1 ? 1 : per > max_task_units ? max_task_units : per;
+            for (int u0 = prefix[i]; u0 < prefix[i + 1]; u0 += (int)per) {
+                pool_first.push_back(u0);
+                pool_problem.push_back(i);
+            }
+        }
+        d.pool_count = (int)pool_problem.size();
+        if (d.pool_count) {
+            pool_first.push_back(prefix[n]);
+            pool_first.insert(pool_first.end(), pool_problem.begin(), pool_problem.end());
         }
         d.grid = grid;
     };
@@ -688,7 +787,7 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
     }
     if (all_batch) {
         d.batch_kernel = true;
-        partition(gemv_batch_block_rows(), di->cus, false);
+        partition(gemv_batch_block_rows(), di->cus, 0);
     } else {
         d.wide = all_wide;
         d.use_mfma = all_wide || all_tall;
@@ -702,26 +801,32 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
         if (d.use_mfma) {
             d.lds_bytes = max_image + kNW * max_units * unit * max_batch * 4;
             const int per_cu = d.wide ? resident_wgs<Wide>(d.lds_bytes) : resident_wgs<Tall>(d.lds_bytes);
-            partition(unit, per_cu * di->cus, true);
+            partition(unit, per_cu * di->cus, max_units);
             d.max_units = max_units;
             d.image_bytes = max_image;
         }
     }
 
-    // one allocation: table | unit prefix | spans
+    // one allocation: table | unit prefix | spans | pool tasks | the two counters
     auto round16 = [](size_t v) { return (v + 15) / 16 * 16; };
-    const size_t bytes_table = round16(sizeof(Problem) * host.size());
+    const size_t bytes_table = round16(sizeof(Problem) * ordered.size());
     const size_t bytes_prefix = round16(sizeof(int) * prefix.size());
     const size_t bytes_wg = round16(sizeof(int) * wg_first.size());
+    const size_t bytes_pool = round16(sizeof(int) * pool_first.size());
     char *base = nullptr;
-    if (hipError_t e = hipMalloc(&base, bytes_table + bytes_prefix + bytes_wg + 16)) return e;
+    if (hipError_t e = hipMalloc(&base, bytes_table + bytes_prefix + bytes_wg + bytes_pool + 16)) return e;
     d.problems = reinterpret_cast<Problem *>(base);
     d.unit_prefix = reinterpret_cast<int *>(base + bytes_table);
     d.wg_first = reinterpret_cast<int *>(base + bytes_table + bytes_prefix);
-    hipError_t e = hipMemcpy(d.problems, host.data(), sizeof(Problem) * host.size(), hipMemcpyHostToDevice);
+    d.pool_first = reinterpret_cast<int *>(base + bytes_table + bytes_prefix + bytes_wg);
+    d.counters = reinterpret_cast<int *>(base + bytes_table + bytes_prefix + bytes_wg + bytes_pool);
+    hipError_t e = hipMemcpy(d.problems, ordered.data(), sizeof(Problem) * ordered.size(), hipMemcpyHostToDevice);
     if (!e) e = hipMemcpy(d.unit_prefix, prefix.data(), sizeof(int) * prefix.size(), hipMemcpyHostToDevice);
     if (!e && !wg_first.empty())
         e = hipMemcpy(d.wg_first, wg_first.data(), sizeof(int) * wg_first.size(), hipMemcpyHostToDevice);
+    if (!e && !pool_first.empty())
+        e = hipMemcpy(d.pool_first, pool_first.data(), sizeof(int) * pool_first.size(), hipMemcpyHostToDevice);
+    if (!e) e = hipMemset(d.counters, 0, 16);
     if (e) {
         (void)hipFree(base);
         return e;
@@ -739,6 +844,9 @@ hipError_t plan_device_launch(const PlanDevice &plan, hipStream_t s) {
     sc.table = plan.problems;
     sc.unit_prefix = plan.unit_prefix;
     sc.wg_first = plan.wg_first;
+    sc.pool_first = plan.pool_first;
+    sc.pool_count = plan.pool_count;
+    sc.counters = plan.counters;
     sc.count = plan.count;
     sc.max_units = plan.max_units;
     sc.max_batch = plan.max_batch;

@@ -530,6 +530,47 @@ def test_linear_plan_model_sweep_every_row(dev, oracle):
     plan.close()
 
 
+def test_linear_plan_large_sweep_shared_pool(dev, oracle):
+    """A plan big enough (16 LLaMA-1B layers, 112 matrices) that part of it is dealt out at run time
+    instead of belonging to a fixed span: whichever workgroup takes a piece, every output must equal
+    the single-call result bit for bit, on every launch (the hand-out counters reset themselves)."""
+    torch, tl = dev
+    shapes = [(2048, 2048), (512, 2048), (512, 2048), (2048, 2048), (8192, 2048), (8192, 2048), (2048, 8192)]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(4242)
+    probs = []
+    for layer in range(16):
+        for rows, cols in shapes:
+            nz = torch.randint(-2**31, 2**31 - 1, (rows, cols // 32), dtype=torch.int32, device="cuda", generator=gen)
+            sg = torch.randint(-2**31, 2**31 - 1, (rows, cols // 32), dtype=torch.int32, device="cuda", generator=gen)
+            sc = (torch.rand((rows, cols // 128), device="cuda", generator=gen) * 0.02 + 0.01).to(torch.float16)
+            x = torch.randn((1, cols), device="cuda", generator=gen).to(torch.float16)
+            y = torch.zeros((1, rows), dtype=torch.float16, device="cuda")
+            probs.append((nz, sg, sc, x, y, rows, cols, 1))
+    singles = []
+    for (nz, sg, sc, x, _, rows, cols, _) in probs:
+        y1 = torch.zeros(rows, dtype=torch.float16, device="cuda")
+        tl.ternary_gemv(nz, sg, sc, x, y1, rows, cols, 128)
+        singles.append(y1)
+    torch.cuda.synchronize()
+    for k in (0, 55, 111):   # the single calls themselves, sampled rows against the oracle
+        nz, sg, sc, x, _, rows, cols, _ = probs[k]
+        pick = np.random.default_rng(k).integers(0, rows, 96)
+        ref = oracle.gemv_f64(nz[pick].cpu().numpy().view(np.uint32), sg[pick].cpu().numpy().view(np.uint32),
+                              sc[pick].cpu().numpy().view(np.uint16), x[0].cpu().numpy().view(np.uint16))
+        assert_close(oracle, singles[k][pick].cpu().numpy().astype(np.float64), ref, what=f"single call {k}")
+    plan = tl.LinearPlan(probs)
+    for launch in range(3):
+        for p in probs:
+            p[4].fill_(float("nan"))
+        plan.launch()
+        torch.cuda.synchronize()
+        for k, (p, y1) in enumerate(zip(probs, singles)):
+            assert torch.equal(p[4][0].view(torch.int16), y1.view(torch.int16)), \
+                f"launch {launch} problem {k}: plan and single call differ"
+    plan.close()
+
+
 # ---------------------------------------------- full-size, size-independent
 def test_full_size_properties_8b(dev, oracle):
     """LLaMA-3-8B gate_proj (14336 x 4096) at full size: sampled rows against the oracle, plus

@@ -24,7 +24,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 # HBM bytes one launch of the default workload moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by
 # a copy kernel of known size (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); valid for the default workload only.
-DEFAULT_WORKLOAD_TRAFFIC_BYTES = 1982129050
+DEFAULT_WORKLOAD_TRAFFIC_BYTES = 1980595008
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 SHAPES = {
@@ -208,6 +208,8 @@ def main():
     ap.add_argument("--also-batch", default="4", help='extra activation-row counts measured on the same weights '
                     '(cfg3 asks for batch 1 and 4), e.g. "4,16"; "" skips')
     ap.add_argument("--gemm-m", default="512", help='token counts M of the prefill GEMM report, e.g. "16,128,512,2048"; "" skips it')
+    ap.add_argument("--gemm-calls", type=int, default=200, help="timed launches per GEMM case")
+    ap.add_argument("--gemm-warm", type=int, default=20, help="untimed launches before them")
     ap.add_argument("--seed", type=int, default=20240611)
     args = ap.parse_args()
     for item in filter(None, args.matrices.split(",")):
@@ -334,7 +336,7 @@ def main():
         del probs_b
     gemm_m = [int(v) for v in args.gemm_m.split(",") if v.strip()]
     if gemm_m:
-        out["gemm"] = gemm_report(torch, tl, orc, args.seed, gemm_m, args.p_zero)
+        out["gemm"] = gemm_report(torch, tl, orc, args.seed, gemm_m, args.p_zero, args.gemm_calls, args.gemm_warm)
     if not args.no_cpu_baseline:
         threads = min(os.cpu_count() or 1, 16)
         out["cpu_baseline"] = cpu_baseline(orc, problems, n_mats, threads)

@@ -66,6 +66,7 @@ hipError_t launch_gemv_batch(const Problem &p, hipStream_t s);
 int gemv_batch_block_rows();
 float gemv_batch_cost_us(const Problem &p);  // rough time of one launch_gemv_batch
 hipError_t launch_gemv_batch_table(const Problem *table, const int *unit_prefix, const int *wg_first, int grid,
+                                   int pool_begin, int pool_end, const int *pool_problem, int *counters,
                                    hipStream_t s);
 
 // 128-group MFMA GEMM for M >= 16 (gemm_mfma.hip); Problem.batch is M, rows is N, cols is K.
@@ -91,6 +92,7 @@ struct PlanDevice {
     int *wg_first = nullptr;
     int *pool_first = nullptr;  // shared pool of small tasks (MFMA kernel, large plans)
     int pool_count = 0;
+    int pool_begin = 0, pool_end = 0;  // batched kernel: blocks handed out at run time, their problems in pool_first
     int *counters = nullptr;
     int grid = 0;
     int max_units = 0;

@@ -44,6 +44,12 @@ struct BatchSched {
     const Problem *table;    // device table, or nullptr: use the by-value problem
     const int *unit_prefix;  // [count + 1] first block of each problem
     const int *wg_first;     // [grid + 1] first block of each workgroup, then [grid] the problem that block is in
+    // Blocks [pool_begin, pool_end) belong to no workgroup: whoever has finished its own blocks takes
+    // them one at a time through counters[0]. counters[1] counts the workgroups that have left; the
+    // last one sets both back to zero for the next launch (launches of one plan must not overlap).
+    int pool_begin, pool_end;
+    const int *pool_problem;  // [pool_end - pool_begin] the problem each pool block is in
+    int *counters;            // nullptr: no pool
 };
 
 struct Tile {
@@ -105,7 +111,23 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
     decode_word(0u, 0u, zero_o);
 
     Problem p = single;
-    for (; u < u_end; u++) {
+    __shared__ int pool_block;
+    for (;; u++) {
+        if (u >= u_end) {
+            // own blocks done: go on with the pool block asked for while the last block was running
+            // (the barriers that end a block separate the write of pool_block, this read, and the
+            // next write)
+            if (!sc.counters) break;
+            const int t = __builtin_amdgcn_readfirstlane(pool_block);
+            if (t >= sc.pool_end - sc.pool_begin) break;
+            u = sc.pool_begin + t;
+            u_end = u + 1;
+            pi = sc.pool_problem[t];
+        }
+        // the last block of the span, or a pool block: ask for the next pool block
+        const bool request = sc.counters != nullptr && u + 1 >= u_end && tid == 0;
+        int requested = 0;
+        if (request) requested = __hip_atomic_fetch_add(sc.counters, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         int first_unit = 0;
         if (sc.table) {
             while (sc.unit_prefix[pi + 1] <= u) pi++;
@@ -318,7 +340,15 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
                         p.y[(size_t)li * p.rows + first + 4 * lq + v] = f2h(acc[k][v] + hand[(k * 4 + v) * kWave + lane]);
             }
         }
+        if (request) pool_block = requested;
         __syncthreads();  // the next block rewrites the image buffers
+    }
+    if (sc.counters && tid == 0) {
+        const int left = __hip_atomic_fetch_add(sc.counters + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (left == (int)gridDim.x - 1) {  // every other workgroup has made its last request
+            __hip_atomic_store(sc.counters, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(sc.counters + 1, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
 }
 
@@ -398,9 +428,11 @@ float gemv_batch_cost_us(const Problem &p) {
 int gemv_batch_block_rows() { return 64 * kMaxTilesPerWave; }
 
 hipError_t launch_gemv_batch_table(const Problem *table, const int *unit_prefix, const int *wg_first, int grid,
+                                   int pool_begin, int pool_end, const int *pool_problem, int *counters,
                                    hipStream_t s) {
     if (hipError_t e = prepare_kernel<kMaxTilesPerWave>()) return e;
-    BatchSched sc{table, unit_prefix, wg_first};
+    BatchSched sc{table, unit_prefix, wg_first, pool_begin, pool_end, pool_problem,
+                  pool_end > pool_begin ? counters : nullptr};
     Problem none{};
     gemv_batch_kernel<kMaxTilesPerWave><<<grid, kThreads, kLdsBytes, s>>>(none, sc);
     return hipGetLastError();

@@ -627,6 +627,15 @@ double pool_fraction() {
     return f;
 }
 constexpr int64_t kPoolTaskWeights = 768 * 1024;
+// The same for the batched kernel, whose blocks are all independent (TLLM_BLOCK_POOL_FRACTION).
+double block_pool_fraction() {
+    static const double f = [] {
+        const char *e = getenv("TLLM_BLOCK_POOL_FRACTION");
+        const double v = e ? atof(e) : 0.25;
+        return v < 0.0 ? 0.0 : v > 0.9 ? 0.9 : v;
+    }();
+    return f;
+}
 
 // units per task that the partial-sum area can hold
 int max_units_for(int image_bytes, int batch, int unit) {
@@ -775,6 +784,50 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
         d.grid = grid;
     };
 
+    // The batched kernel works in blocks of rows that need nothing from the block before: equal
+    // spans of blocks over the first part of the list, the blocks of the last part handed out one by
+    // one at run time (the XCDs of one box differed by 15 % in speed under this kernel).
+    auto partition_blocks = [&](int unit, int wgs) {
+        std::vector<int64_t> weight;
+        std::vector<int> block_problem;
+        for (size_t i = 0; i < host.size(); i++) {
+            const int n = (host[i].rows + unit - 1) / unit;
+            prefix[i + 1] = prefix[i] + n;
+            for (int t = 0; t < n; t++) {
+                const int nr = host[i].rows - t * unit < unit ? host[i].rows - t * unit : unit;
+                weight.push_back((int64_t)nr * host[i].cols + 16384);
+                block_problem.push_back((int)i);
+            }
+        }
+        const int all_units = prefix.back();
+        int64_t all_w = 0;
+        for (int64_t w : weight) all_w += w;
+        int units = all_units;  // blocks that belong to spans
+        if (all_units >= 8 * wgs) {
+            int64_t acc = 0;
+            units = 0;
+            while (units < all_units && (double)acc < (double)all_w * (1.0 - block_pool_fraction())) acc += weight[units++];
+            units = units < 4 * wgs ? 4 * wgs : units;
+        }
+        const int grid = units < wgs ? units : wgs;
+        int64_t total_w = 0;
+        for (int t = 0; t < units; t++) total_w += weight[t];
+        wg_first.assign(grid + 1, units);
+        wg_first[0] = 0;
+        int64_t acc = 0;  // weight of blocks [0, t)
+        int t = 0;
+        for (int g = 1; g < grid; g++) {
+            const int lo = wg_first[g - 1] + 1, hi = units - (grid - g);
+            while (t < hi && (t < lo || acc * grid < total_w * g)) acc += weight[t++];
+            wg_first[g] = t;
+        }
+        for (int g = 0; g < grid; g++) wg_first.push_back(block_problem[wg_first[g]]);
+        pool_first.assign(block_problem.begin() + units, block_problem.end());
+        d.pool_begin = units;
+        d.pool_end = all_units;
+        d.grid = grid;
+    };
+
     // several activation rows: the batched kernel if every problem fits it
     bool all_batch = max_batch >= 2;
     for (const Problem &p : host) all_batch = all_batch && gemv_batch_supports(p, 128);
@@ -787,7 +840,7 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
     }
     if (all_batch) {
         d.batch_kernel = true;
-        partition(gemv_batch_block_rows(), di->cus, 0);
+        partition_blocks(gemv_batch_block_rows(), di->cus);
     } else {
         d.wide = all_wide;
         d.use_mfma = all_wide || all_tall;
@@ -837,7 +890,8 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
 
 hipError_t plan_device_launch(const PlanDevice &plan, hipStream_t s) {
     if (plan.batch_kernel)
-        return launch_gemv_batch_table(plan.problems, plan.unit_prefix, plan.wg_first, plan.grid, s);
+        return launch_gemv_batch_table(plan.problems, plan.unit_prefix, plan.wg_first, plan.grid, plan.pool_begin,
+                                       plan.pool_end, plan.pool_first, plan.counters, s);
     if (!plan.use_mfma)
         return launch_gemv_rowwave_f16_table(plan.problems, plan.count, plan.max_rows, plan.max_batch, 128, s);
     Sched sc{};

@@ -262,12 +262,12 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
             f4 bias[4];
 #pragma unroll
             for (int c = 0; c < 4; c++) {
-                f4 d0 = {0.f, 0.f, 0.f, 0.f}, d1 = {0.f, 0.f, 0.f, 0.f};
+                f4 d0 = {0.f, 0.f, 0.f, 0.f};
                 d0 = mfma16(zero_o + 0, B[4 * c + 0], d0);
-                d1 = mfma16(zero_o + 4, B[4 * c + 1], d1);
+                d0 = mfma16(zero_o + 4, B[4 * c + 1], d0);
                 d0 = mfma16(zero_o + 8, B[4 * c + 2], d0);
-                d1 = mfma16(zero_o + 12, B[4 * c + 3], d1);
-                bias[c] = d0 + d1;
+                d0 = mfma16(zero_o + 12, B[4 * c + 3], d0);
+                bias[c] = d0;
             }
             const int s_next = my_slice(min(st + 1, steps - 1));
 #pragma unroll
@@ -282,17 +282,17 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
                 transpose4(t.sg);
                 f4 r = {0.f, 0.f, 0.f, 0.f};
                 // the MFMAs of chunk c + 1 are issued before the results of chunk c are touched
-                f4 da[2], db[2];
+                f4 da[2];  // one chain of four MFMAs per scale group; two groups in flight
                 auto issue = [&](int c) {
                     uint32_t o[16];
                     decode_word(t.nz[c], t.sg[c], o);
                     da[c & 1] = mfma16(o + 0, B[4 * c + 0], f4{0.f, 0.f, 0.f, 0.f});
-                    db[c & 1] = mfma16(o + 4, B[4 * c + 1], f4{0.f, 0.f, 0.f, 0.f});
+                    da[c & 1] = mfma16(o + 4, B[4 * c + 1], da[c & 1]);
                     da[c & 1] = mfma16(o + 8, B[4 * c + 2], da[c & 1]);
-                    db[c & 1] = mfma16(o + 12, B[4 * c + 3], db[c & 1]);
+                    da[c & 1] = mfma16(o + 12, B[4 * c + 3], da[c & 1]);
                 };
                 auto retire = [&](int c) {
-                    const f4 d = da[c & 1] + db[c & 1] - bias[c];
+                    const f4 d = da[c & 1] - bias[c];
 #pragma unroll
                     for (int v = 0; v < 4; v++) {
                         const uint16_t sbits = (uint16_t)(ts.sc[v][c >> 1] >> (16 * (c & 1)));

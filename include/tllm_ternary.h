@@ -141,7 +141,10 @@ typedef struct tllm_linear_plan tllm_linear_plan;
  * Allocates device memory; not for the per-token path. group_size must be 128. */
 int tllm_linear_plan_create(tllm_linear_plan **plan, const tllm_linear_problem *problems,
                             int count, int group_size);
-/* One launch over every problem of the plan. Allocation-free. */
+/* One launch over every problem of the plan. Allocation-free. Launches of ONE plan must not overlap in
+ * time (two streams, or two graph branches): besides the outputs they share two device counters that
+ * deal the tail of a large plan out to the workgroups; the kernel resets them when it ends, so
+ * launches that follow each other on a stream, or replays of a captured graph, need no clearing. */
 int tllm_linear_plan_launch(const tllm_linear_plan *plan, tllm_stream_t stream);
 /* Algorithmic weight-stream bytes (masks + scales) one launch reads. */
 int64_t tllm_linear_plan_weight_bytes(const tllm_linear_plan *plan);

@@ -571,6 +571,50 @@ def test_linear_plan_large_sweep_shared_pool(dev, oracle):
     plan.close()
 
 
+def test_large_plan_in_a_captured_graph(dev, oracle):
+    """The same kind of plan recorded into a HIP graph: every replay (with eager work and
+    synchronisation between replays) must reproduce the eager launch bit for bit. The kernel's own
+    hand-out counters are reset by the kernel, not by a memset node."""
+    torch, tl = dev
+    shapes = [(2048, 2048), (512, 2048), (512, 2048), (2048, 2048), (8192, 2048), (8192, 2048), (2048, 8192)]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(777)
+    probs = []
+    for layer in range(16):
+        for rows, cols in shapes:
+            nz = torch.randint(-2**31, 2**31 - 1, (rows, cols // 32), dtype=torch.int32, device="cuda", generator=gen)
+            sg = torch.randint(-2**31, 2**31 - 1, (rows, cols // 32), dtype=torch.int32, device="cuda", generator=gen)
+            sc = (torch.rand((rows, cols // 128), device="cuda", generator=gen) * 0.02 + 0.01).to(torch.float16)
+            x = torch.randn((1, cols), device="cuda", generator=gen).to(torch.float16)
+            y = torch.zeros((1, rows), dtype=torch.float16, device="cuda")
+            probs.append((nz, sg, sc, x, y, rows, cols, 1))
+    plan = tl.LinearPlan(probs)
+    plan.launch()
+    torch.cuda.synchronize()
+    eager = [p[4].clone() for p in probs]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        plan.launch()          # warm-up on the capture stream
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            plan.launch()
+    torch.cuda.synchronize()
+    for replay in range(4):
+        for p in probs:
+            p[4].fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for k, (p, e) in enumerate(zip(probs, eager)):
+            assert torch.equal(p[4].view(torch.int16), e.view(torch.int16)), f"replay {replay} problem {k}"
+        if replay == 1:   # an eager launch between replays must not disturb the next replay
+            plan.launch()
+            torch.cuda.synchronize()
+    plan.close()
+
+
 # ---------------------------------------------- full-size, size-independent
 def test_full_size_properties_8b(dev, oracle):
     """LLaMA-3-8B gate_proj (14336 x 4096) at full size: sampled rows against the oracle, plus

@@ -130,10 +130,21 @@ typedef struct tllm_linear_problem {
     int32_t rows;
     int32_t cols;
     int32_t batch; /* 1..TLLM_MAX_PLAN_BATCH */
-    int32_t reserved;
+    int32_t flags; /* 0, or TLLM_PROBLEM_SWIGLU_GATE */
 } tllm_linear_problem;
 
 enum { TLLM_MAX_PLAN_BATCH = 16 };
+
+/*
+ * Flag of a problem that is the GATE projection of a SwiGLU pair. The next problem of the array must
+ * then be the UP projection: same rows, cols, batch (1 only) and input. The pair is computed together
+ * and ONE result is stored, in the gate problem's output:
+ *   output[b, r] = fp16( silu(g) * u ),  g = fp16(gate row r . x_b),  u = fp16(up row r . x_b),
+ * i.e. exactly what the two projections followed by tllm_silu_mul_f16 store (the up problem's output
+ * pointer is not written and may be NULL). Replaces the three launches of the reference's FFN front
+ * half, src/transformer.cpp:266-286 (gate GEMV, up GEMV, silu_mul_forward).
+ */
+enum { TLLM_PROBLEM_SWIGLU_GATE = 1 };
 
 typedef struct tllm_linear_plan tllm_linear_plan;
 

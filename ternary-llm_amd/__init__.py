@@ -4,6 +4,7 @@ every operator raises if the library is missing or a call is rejected."""
 from .ops import (  # noqa: F401
     FileHeader,
     LinearPlan,
+    SWIGLU_GATE,
     ModelFile,
     TllmError,
     lib,

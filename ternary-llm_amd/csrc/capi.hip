@@ -154,8 +154,20 @@ int tllm_linear_plan_create(tllm_linear_plan **plan, const tllm_linear_problem *
     for (int i = 0; i < count; i++) {
         const tllm_linear_problem &q = problems[i];
         host[i] = Problem{q.nonzero_masks, q.sign_masks, q.scales, q.input, q.output,
-                          q.rows, q.cols, q.batch, 0};
+                          q.rows, q.cols, q.batch, q.flags};
         if (q.batch < 1 || q.batch > TLLM_MAX_PLAN_BATCH) return TLLM_ERR_BAD_PLAN;
+        if (q.flags & ~TLLM_PROBLEM_SWIGLU_GATE) return TLLM_ERR_BAD_PLAN;
+        const bool is_up = i > 0 && (problems[i - 1].flags & TLLM_PROBLEM_SWIGLU_GATE);
+        if (is_up) {
+            // the up half of a SwiGLU pair: same shape and activations as its gate, no output of its own
+            const tllm_linear_problem &g = problems[i - 1];
+            if (q.flags || q.rows != g.rows || q.cols != g.cols || q.batch != g.batch || q.input != g.input)
+                return TLLM_ERR_BAD_PLAN;
+            host[i].y = host[i - 1].y;
+        }
+        if (q.flags & TLLM_PROBLEM_SWIGLU_GATE) {
+            if (i + 1 >= count || q.batch != 1) return TLLM_ERR_BAD_PLAN;
+        }
         if (int e = tllm::check_linear(host[i], group_size)) return e;
         bytes += (int64_t)q.rows * (q.cols / 32) * 8 + (int64_t)q.rows * (q.cols / group_size) * 2;
     }
@@ -164,6 +176,13 @@ int tllm_linear_plan_create(tllm_linear_plan **plan, const tllm_linear_problem *
     if (hipError_t e = tllm::plan_device_create(pl->host, &pl->dev)) {
         delete pl;
         return (int)e;
+    }
+    bool has_pairs = false;
+    for (const Problem &p : pl->host) has_pairs = has_pairs || (p.flags & TLLM_PROBLEM_SWIGLU_GATE);
+    if (has_pairs && !pl->dev.use_mfma) {  // a shape that only the general kernel serves: no fused pairs
+        tllm::plan_device_destroy(&pl->dev);
+        delete pl;
+        return TLLM_ERR_BAD_PLAN;
     }
     *plan = pl;
     return TLLM_OK;

@@ -21,9 +21,10 @@ struct Problem {
     int32_t rows;
     int32_t cols;
     int32_t batch;
-    int32_t reserved;
+    int32_t flags;  // kProblemSwigluGate
 };
 static_assert(sizeof(Problem) == sizeof(tllm_linear_problem), "ABI struct mirrors Problem");
+constexpr int kProblemSwigluGate = TLLM_PROBLEM_SWIGLU_GATE;
 
 __device__ __forceinline__ float h2f(uint16_t bits) {
     return (float)__builtin_bit_cast(_Float16, bits);
@@ -96,6 +97,7 @@ struct PlanDevice {
     int *counters = nullptr;
     int grid = 0;
     int max_units = 0;
+    int pair_stride = 0;  // floats between the two partial-sum areas of a SwiGLU pair (0: no pairs)
     int image_bytes = 0;
     int lds_bytes = 0;
 };

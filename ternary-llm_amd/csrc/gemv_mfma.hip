@@ -72,6 +72,7 @@ struct Sched {
     int pool_count;
     int *counters;
     int count;
+    int pair_stride;  // floats between the partial sums of a gate matrix and of its up matrix; 0: no pairs
     int max_units;    // units per task (bounds the partial-sum area)
     int max_batch;    // largest batch of any problem (sizes the per-wave partial-sum areas)
     int image_bytes;  // LDS bytes reserved for the activation image (the partial sums follow)
@@ -145,7 +146,9 @@ __device__ __forceinline__ f4 tile_product(const u4 nz, const u4 sg, const u4 (&
     return d0 + d1;
 }
 
-template <class G>
+// kPairs: the table may hold SwiGLU pairs (a separate instance, so that plans without them keep the
+// register allocation of the plain kernel).
+template <class G, bool kPairs = false>
 __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Problem single, Sched sc) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     uint16_t *image = reinterpret_cast<uint16_t *>(lds);
@@ -330,7 +333,19 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
         const int chunk_rows = ((r_end - r_begin + kNW - 1) / kNW + kUnitRows / kNW - 1) / (kUnitRows / kNW) * (kUnitRows / kNW);
         const int n_walks = kNW * slices;
         const int my_walks = slices;  // walks wave, wave + kNW, ...
-        float *my_part = partial + (size_t)wave * (sc.max_units * kUnitRows) * sc.max_batch;
+        // A SwiGLU pair (flag on the gate problem; the up problem follows it in the table, same shape
+        // and activations, no units of its own) runs the walks twice over the same rows, with the same
+        // operand image, into two partial-sum areas; the epilogue below joins them.
+        const bool pair = kPairs && (p.flags & kProblemSwigluGate) != 0;
+        for (int mat = 0; mat < (pair ? 2 : 1); mat++) {
+        const uint32_t *w_nz = p.nz, *w_sg = p.sg;
+        const uint16_t *w_sc = p.scales;
+        if (mat == 1) {
+            w_nz = sc.table[pi + 1].nz;
+            w_sg = sc.table[pi + 1].sg;
+            w_sc = sc.table[pi + 1].scales;
+        }
+        float *my_part = partial + (size_t)mat * sc.pair_stride + (size_t)wave * (sc.max_units * kUnitRows) * sc.max_batch;
         for (int k = lane; k < n_units * kUnitRows * p.batch; k += kWave) my_part[k] = 0.0f;
 
         // ---- which operand lanes are live, and what each lane loads
@@ -358,9 +373,9 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
         // the last slice are moved back to end exactly at the matrix edge (rows >= kRows and
         // groups >= kChunks are guaranteed by the dispatcher); the rows such a block repeats are
         // dropped again in the epilogue, the repeated columns are zero in the image.
-        const char GB *nz_g = reinterpret_cast<const char GB *>(as_global(p.nz));
-        const char GB *sg_g = reinterpret_cast<const char GB *>(as_global(p.sg));
-        const char GB *sc_g = reinterpret_cast<const char GB *>(as_global(p.scales));
+        const char GB *nz_g = reinterpret_cast<const char GB *>(as_global(w_nz));
+        const char GB *sg_g = reinterpret_cast<const char GB *>(as_global(w_sg));
+        const char GB *sc_g = reinterpret_cast<const char GB *>(as_global(w_sc));
         const uint32_t lane_a = ((uint32_t)a_row * words + 4u * a_chunk) * 4u;
         uint32_t lane_s[G::kScales];
         if constexpr (G::kRows == 4) {
@@ -485,6 +500,7 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
                 }
             }
         }
+        }  // matrices of the task
         // last task of the span, or a pool task: ask for the next pool task now (not earlier: a
         // request is a claim, and a workgroup must not claim work long before it can start it); the
         // answer arrives while the partial sums are added up
@@ -501,7 +517,18 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
                 float sum = 0.0f;
 #pragma unroll
                 for (int w = 0; w < kNW; w++) sum += partial[w * wave_stride + (size_t)rl * p.batch + b];
-                p.y[(size_t)b * p.rows + r_begin + rl] = f2h(sum * fscale[b]);
+                uint16_t out = f2h(sum * fscale[b]);
+                if (pair) {
+                    // out = silu(gate) * up on the fp16-rounded projections, in fp32: what the two
+                    // launches and the element-wise kernel after them would store
+                    float sum_up = 0.0f;
+#pragma unroll
+                    for (int w = 0; w < kNW; w++)
+                        sum_up += partial[sc.pair_stride + w * wave_stride + (size_t)rl * p.batch + b];
+                    const float g = h2f(out), up = h2f(f2h(sum_up * fscale[b]));
+                    out = f2h(g / (1.0f + expf(-g)) * up);
+                }
+                p.y[(size_t)b * p.rows + r_begin + rl] = out;
             }
         }
         if (request) pool_task = requested;
@@ -527,9 +554,9 @@ DeviceInfo &device_info(int dev) {
 
 constexpr int kLdsLimit = 64 * 1024;  // per workgroup; 160 KB per CU leaves room for two or three
 
-template <class G>
+template <class G, bool kPairs = false>
 const void *kernel_ptr() {
-    return reinterpret_cast<const void *>(&gemv_mfma_kernel<G>);
+    return reinterpret_cast<const void *>(&gemv_mfma_kernel<G, kPairs>);
 }
 
 hipError_t prepare_device(DeviceInfo **out) {
@@ -543,6 +570,8 @@ hipError_t prepare_device(DeviceInfo **out) {
             return e;
         if (hipError_t e = hipFuncSetAttribute(kernel_ptr<Tall>(), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit))
             return e;
+        if (hipError_t e = hipFuncSetAttribute(kernel_ptr<Wide, true>(), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit))
+            return e;
         di.cus = n > 0 ? n : 256;
     }
     *out = &di;
@@ -550,10 +579,10 @@ hipError_t prepare_device(DeviceInfo **out) {
 }
 
 // Resident workgroups per CU for a given dynamic LDS size (asked from the runtime, capped at 4).
-template <class G>
+template <class G, bool kPairs = false>
 int resident_wgs(size_t lds_bytes) {
     int n = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gemv_mfma_kernel<G>, kThreads, lds_bytes) != hipSuccess || n < 1)
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gemv_mfma_kernel<G, kPairs>, kThreads, lds_bytes) != hipSuccess || n < 1)
         n = 1;
     return n > 4 ? 4 : n;
 }
@@ -638,8 +667,9 @@ double block_pool_fraction() {
 }
 
 // units per task that the partial-sum area can hold
-int max_units_for(int image_bytes, int batch, int unit) {
-    const int room_rows = (kLdsLimit - image_bytes) / (kNW * batch * 4);  // one partial sum per wave and row
+int max_units_for(int image_bytes, int batch, int unit, int mats = 1) {
+    // one partial sum per wave, row and matrix of the task (two for a SwiGLU pair)
+    const int room_rows = (kLdsLimit - image_bytes) / (kNW * batch * 4 * mats);
     const int n = room_rows / unit;
     return n > kMaxTaskUnits ? kMaxTaskUnits : n;
 }
@@ -707,14 +737,17 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
     // there) go to the shared pool instead, cut into small tasks inside one problem each.
     auto partition = [&](int unit, int wgs, int max_task_units) {
         const int n = (int)host.size();
-        auto units_of = [&](const Problem &p) { return (p.rows + unit - 1) / unit; };
+        // the up half of a SwiGLU pair has no units: its rows are done with the gate's
+        auto is_up = [&](const std::vector<Problem> &v, int i) { return i > 0 && (v[i - 1].flags & kProblemSwigluGate); };
+        auto mats = [&](const Problem &p) { return (p.flags & kProblemSwigluGate) ? 2 : 1; };
+        auto units_in = [&](const std::vector<Problem> &v, int i) { return is_up(v, i) ? 0 : (v[i].rows + unit - 1) / unit; };
         std::vector<char> pooled(n, 0);
         int64_t all_w = 0;
         int all_units = 0, min_cols = host[0].cols;
-        for (const Problem &p : host) {
-            all_w += (int64_t)p.rows * p.cols;
-            all_units += units_of(p);
-            min_cols = p.cols < min_cols ? p.cols : min_cols;
+        for (int i = 0; i < n; i++) {
+            all_w += (int64_t)host[i].rows * host[i].cols;
+            all_units += units_in(host, i);
+            min_cols = host[i].cols < min_cols ? host[i].cols : min_cols;
         }
         if (max_task_units > 0 && all_units >= 8 * wgs) {
             const int64_t want = (int64_t)((double)all_w * pool_fraction());
@@ -722,11 +755,12 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
             int left_units = all_units;
             for (int pass = 0; pass < 2 && got < want; pass++)
                 for (int i = n - 1; i >= 0 && got < want; i--) {
-                    if (pooled[i] || (pass == 0 && host[i].cols > 2 * min_cols)) continue;
-                    if (left_units - units_of(host[i]) < 4 * wgs) continue;
+                    if (pooled[i] || is_up(host, i) || (pass == 0 && host[i].cols > 2 * min_cols)) continue;
+                    if (left_units - units_in(host, i) < 4 * wgs) continue;
                     pooled[i] = 1;
-                    got += (int64_t)host[i].rows * host[i].cols;
-                    left_units -= units_of(host[i]);
+                    got += (int64_t)host[i].rows * host[i].cols * mats(host[i]);
+                    left_units -= units_in(host, i);
+                    if (mats(host[i]) == 2) pooled[i + 1] = 1;  // a pair stays together
                 }
         }
         int k = 0, n_static = 0;
@@ -737,11 +771,11 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
         }
         std::vector<int64_t> weight;
         for (int i = 0; i < n; i++) {
-            const int nu = units_of(ordered[i]);
+            const int nu = units_in(ordered, i);
             prefix[i + 1] = prefix[i] + nu;
             for (int t = 0; t < nu && i < n_static; t++) {
                 const int nr = ordered[i].rows - t * unit < unit ? ordered[i].rows - t * unit : unit;
-                weight.push_back((int64_t)nr * ordered[i].cols + 16384);
+                weight.push_back((int64_t)nr * ordered[i].cols * mats(ordered[i]) + 16384);
             }
         }
         const int units = prefix[n_static];
@@ -768,7 +802,7 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
         }
         std::vector<int> pool_problem;
         for (int i = n_static; i < n; i++) {
-            const int64_t unit_w = (int64_t)unit * ordered[i].cols;
+            const int64_t unit_w = (int64_t)unit * ordered[i].cols * mats(ordered[i]);
             int64_t per = (kPoolTaskWeights + unit_w / 2) / unit_w;
             per = per < 1 ? 1 : per > max_task_units ? max_task_units : per;
             for (int u0 = prefix[i]; u0 < prefix[i + 1]; u0 += (int)per) {
@@ -829,7 +863,9 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
     };
 
     // several activation rows: the batched kernel if every problem fits it
-    bool all_batch = max_batch >= 2;
+    bool has_pairs = false;
+    for (const Problem &p : host) has_pairs = has_pairs || (p.flags & kProblemSwigluGate);
+    bool all_batch = max_batch >= 2 && !has_pairs;  // pairs are joined in the MFMA GEMV kernel only
     for (const Problem &p : host) all_batch = all_batch && gemv_batch_supports(p, 128);
     // one geometry per launch otherwise: wide tiles if every problem allows them, else tall ones
     bool all_wide = true, all_tall = true;
@@ -843,17 +879,21 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
         partition_blocks(gemv_batch_block_rows(), di->cus);
     } else {
         d.wide = all_wide;
-        d.use_mfma = all_wide || all_tall;
+        d.use_mfma = has_pairs ? all_wide : all_wide || all_tall;  // pairs: batch 1, wide tiles only
         for (const Problem &p : host) {
             const int ib = d.wide ? image_bytes_of<Wide>(p.cols, 1) : image_bytes_of<Tall>(p.cols, p.batch);
             max_image = ib > max_image ? ib : max_image;
         }
         const int unit = d.wide ? range_unit<Wide>() : range_unit<Tall>();
-        const int max_units = max_units_for(max_image, max_batch, unit);
+        const int mats = has_pairs ? 2 : 1;
+        const int max_units = max_units_for(max_image, max_batch, unit, mats);
         if (max_units < 1) d.use_mfma = false;
         if (d.use_mfma) {
-            d.lds_bytes = max_image + kNW * max_units * unit * max_batch * 4;
-            const int per_cu = d.wide ? resident_wgs<Wide>(d.lds_bytes) : resident_wgs<Tall>(d.lds_bytes);
+            d.pair_stride = has_pairs ? kNW * max_units * unit * max_batch : 0;
+            d.lds_bytes = max_image + kNW * max_units * unit * max_batch * 4 * mats;
+            const int per_cu = has_pairs ? resident_wgs<Wide, true>(d.lds_bytes)
+                               : d.wide  ? resident_wgs<Wide>(d.lds_bytes)
+                                         : resident_wgs<Tall>(d.lds_bytes);
             partition(unit, per_cu * di->cus, max_units);
             d.max_units = max_units;
             d.image_bytes = max_image;
@@ -902,11 +942,14 @@ hipError_t plan_device_launch(const PlanDevice &plan, hipStream_t s) {
     sc.pool_count = plan.pool_count;
     sc.counters = plan.counters;
     sc.count = plan.count;
+    sc.pair_stride = plan.pair_stride;
     sc.max_units = plan.max_units;
     sc.max_batch = plan.max_batch;
     sc.image_bytes = plan.image_bytes;
     Problem none{};
-    if (plan.wide)
+    if (plan.pair_stride)
+        gemv_mfma_kernel<Wide, true><<<plan.grid, kThreads, plan.lds_bytes, s>>>(none, sc);
+    else if (plan.wide)
         gemv_mfma_kernel<Wide><<<plan.grid, kThreads, plan.lds_bytes, s>>>(none, sc);
     else
         gemv_mfma_kernel<Tall><<<plan.grid, kThreads, plan.lds_bytes, s>>>(none, sc);

@@ -35,7 +35,7 @@ class TllmError(RuntimeError):
 class _Problem(C.Structure):
     _fields_ = [("nonzero_masks", C.c_void_p), ("sign_masks", C.c_void_p), ("scales", C.c_void_p),
                 ("input", C.c_void_p), ("output", C.c_void_p), ("rows", C.c_int32),
-                ("cols", C.c_int32), ("batch", C.c_int32), ("reserved", C.c_int32)]
+                ("cols", C.c_int32), ("batch", C.c_int32), ("flags", C.c_int32)]
 
 
 class FileHeader(C.Structure):
@@ -161,17 +161,24 @@ def silu_mul(gate, up, output, size, stream=None):
     check(lib().tllm_silu_mul_f16(_ptr(gate), _ptr(up), _ptr(output), size, _stream(stream)))
 
 
+SWIGLU_GATE = 1  # TLLM_PROBLEM_SWIGLU_GATE
+
+
 class LinearPlan:
     """Several independent ternary linears issued as one launch."""
 
     def __init__(self, problems, group_size=128):
-        """problems: iterable of (nz, sign, scales, input, output, rows, cols, batch)."""
+        """problems: iterable of (nz, sign, scales, input, output, rows, cols, batch[, flags]);
+        flags = SWIGLU_GATE marks the gate of a pair whose up projection is the next problem
+        (output may be None there): the pair stores silu(gate) * up in the gate's output."""
         problems = list(problems)
         arr = (_Problem * max(len(problems), 1))()
         self._keep = problems  # keep the tensors alive as long as the plan
-        for k, (nz, sg, sc, x, y, rows, cols, batch) in enumerate(problems):
+        for k, prob in enumerate(problems):
+            nz, sg, sc, x, y, rows, cols, batch = prob[:8]
+            flags = prob[8] if len(prob) > 8 else 0
             arr[k] = _Problem(nz.data_ptr(), sg.data_ptr(), sc.data_ptr(), x.data_ptr(),
-                              y.data_ptr(), rows, cols, batch, 0)
+                              y.data_ptr() if y is not None else 0, rows, cols, batch, flags)
         self._h = C.c_void_p(0)
         check(lib().tllm_linear_plan_create(C.byref(self._h), arr, len(problems), group_size))
 

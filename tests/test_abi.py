@@ -65,6 +65,18 @@ def test_validation_codes():
     assert L.tllm_linear_plan_create(C.byref(h), arr, 1, 128) == -6   # batch > TLLM_MAX_PLAN_BATCH
     assert L.tllm_linear_plan_create(C.byref(h), arr, 0, 128) == -6
     assert L.tllm_linear_plan_create(C.byref(h), arr, 1, 64) == -3
+    # SwiGLU pairs: the flagged gate needs an up problem right after it, same shape and input, batch 1
+    P, GATE = ops._Problem, ops.SWIGLU_GATE
+    gate = P(0x1000, 0x2000, 0x3000, 0x4000, 0x9000, 64, 2048, 1, GATE)
+    for bad in ([gate],                                                             # nothing follows
+                [gate, P(0x1000, 0x2000, 0x3000, 0x4000, 0, 32, 2048, 1, 0)],         # other shape
+                [gate, P(0x1000, 0x2000, 0x3000, 0x5000, 0, 64, 2048, 1, 0)],         # other input
+                [gate, P(0x1000, 0x2000, 0x3000, 0x4000, 0, 64, 2048, 1, GATE)],      # up flagged too
+                [P(0x1000, 0x2000, 0x3000, 0x4000, 0x9000, 64, 2048, 2, GATE),
+                 P(0x1000, 0x2000, 0x3000, 0x4000, 0, 64, 2048, 2, 0)],               # batch 2
+                [P(0x1000, 0x2000, 0x3000, 0x4000, 0x9000, 64, 2048, 1, 2)]):         # unknown flag
+        arr = (P * len(bad))(*bad)
+        assert L.tllm_linear_plan_create(C.byref(h), arr, len(bad), 128) == -6
     assert L.tllm_linear_plan_launch(None, None) == -6
     for code in range(-7, 1):
         assert L.tllm_error_string(code)

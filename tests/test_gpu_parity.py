@@ -530,6 +530,103 @@ def test_linear_plan_model_sweep_every_row(dev, oracle):
     plan.close()
 
 
+def _rand_weight(torch, gen, rows, cols):
+    nz = torch.randint(-2**31, 2**31 - 1, (rows, cols // 32), dtype=torch.int32, device="cuda", generator=gen)
+    sg = torch.randint(-2**31, 2**31 - 1, (rows, cols // 32), dtype=torch.int32, device="cuda", generator=gen)
+    sc = (torch.rand((rows, cols // 128), device="cuda", generator=gen) * 0.02 + 0.01).to(torch.float16)
+    return nz, sg, sc
+
+
+@pytest.mark.parametrize("rows,cols", [(14336, 4096), (8192, 2048), (100, 2048), (28672, 8192)])
+def test_swiglu_pair_vs_oracle_and_unfused(dev, oracle, rows, cols):
+    """gate/up pair in one launch with the SiLU*mul epilogue: equal, bit for bit, to the two
+    projections followed by the element-wise operator, and within tolerance of the fp64 evaluation
+    silu(fp16(gate.x)) * fp16(up.x)."""
+    torch, tl = dev
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(rows + cols)
+    g_w, u_w = _rand_weight(torch, gen, rows, cols), _rand_weight(torch, gen, rows, cols)
+    x = torch.randn((1, cols), device="cuda", generator=gen).to(torch.float16)
+    fused = torch.full((1, rows), float("nan"), dtype=torch.float16, device="cuda")
+    plan = tl.LinearPlan([(*g_w, x, fused, rows, cols, 1, tl.SWIGLU_GATE), (*u_w, x, None, rows, cols, 1)])
+    plan.launch()
+    torch.cuda.synchronize()
+    g = torch.zeros(rows, dtype=torch.float16, device="cuda")
+    u = torch.zeros(rows, dtype=torch.float16, device="cuda")
+    tl.ternary_gemv(*g_w, x, g, rows, cols, 128)
+    tl.ternary_gemv(*u_w, x, u, rows, cols, 128)
+    unfused = torch.empty_like(g)
+    tl.silu_mul(g, u, unfused, rows)
+    torch.cuda.synchronize()
+    assert torch.equal(fused[0].view(torch.int16), unfused.view(torch.int16))
+    pick = np.random.default_rng(1).integers(0, rows, 128)
+    xs = x[0].cpu().numpy().view(np.uint16)
+    ref_g = oracle.gemv_f64(g_w[0][pick].cpu().numpy().view(np.uint32), g_w[1][pick].cpu().numpy().view(np.uint32),
+                            g_w[2][pick].cpu().numpy().view(np.uint16), xs)
+    ref_u = oracle.gemv_f64(u_w[0][pick].cpu().numpy().view(np.uint32), u_w[1][pick].cpu().numpy().view(np.uint32),
+                            u_w[2][pick].cpu().numpy().view(np.uint16), xs)
+    # the operator is defined on the fp16-rounded projections, as the reference's three launches are
+    ref = oracle.silu_mul_f64(oracle.half_bits(ref_g), oracle.half_bits(ref_u))
+    got = fused[0][pick].cpu().numpy().astype(np.float64)
+    # a projection that lands on the other side of an fp16 rounding boundary moves the product by one
+    # fp16 ulp of that factor: 2^-10 relative
+    assert_close(oracle, got, ref, tol=2.5e-3, what=f"swiglu pair {rows}x{cols}")
+    plan.close()
+
+
+def test_swiglu_pairs_in_a_layer_sweep(dev, oracle):
+    """Twelve 8B-shaped layers as one plan (q, k, v, o, the gate/up pair, down): large enough for the
+    run-time pool, pairs in spans and in the pool alike; every output equals the separate calls."""
+    torch, tl = dev
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(99)
+    h, kv, ffn = 4096, 1024, 14336
+    probs, expect = [], []
+    for layer in range(12):
+        x = torch.randn((1, h), device="cuda", generator=gen).to(torch.float16)
+        xf = torch.randn((1, ffn), device="cuda", generator=gen).to(torch.float16)
+        for rows, cols, xin in ((h, h, x), (kv, h, x), (kv, h, x), (h, h, x)):
+            w = _rand_weight(torch, gen, rows, cols)
+            y = torch.zeros((1, rows), dtype=torch.float16, device="cuda")
+            probs.append((*w, xin, y, rows, cols, 1))
+            e = torch.zeros(rows, dtype=torch.float16, device="cuda")
+            tl.ternary_gemv(*w, xin, e, rows, cols, 128)
+            expect.append((y, e))
+        g_w, u_w = _rand_weight(torch, gen, ffn, h), _rand_weight(torch, gen, ffn, h)
+        y = torch.zeros((1, ffn), dtype=torch.float16, device="cuda")
+        probs.append((*g_w, x, y, ffn, h, 1, tl.SWIGLU_GATE))
+        probs.append((*u_w, x, None, ffn, h, 1))
+        g = torch.zeros(ffn, dtype=torch.float16, device="cuda")
+        u = torch.zeros(ffn, dtype=torch.float16, device="cuda")
+        tl.ternary_gemv(*g_w, x, g, ffn, h, 128)
+        tl.ternary_gemv(*u_w, x, u, ffn, h, 128)
+        e = torch.empty_like(g)
+        tl.silu_mul(g, u, e, ffn)
+        expect.append((y, e))
+        w = _rand_weight(torch, gen, h, ffn)
+        y = torch.zeros((1, h), dtype=torch.float16, device="cuda")
+        probs.append((*w, xf, y, h, ffn, 1))
+        e = torch.zeros(h, dtype=torch.float16, device="cuda")
+        tl.ternary_gemv(*w, xf, e, h, ffn, 128)
+        expect.append((y, e))
+    torch.cuda.synchronize()
+    plan = tl.LinearPlan(probs)
+    for launch in range(3):
+        for y, _ in expect:
+            y.fill_(float("nan"))
+        plan.launch()
+        torch.cuda.synchronize()
+        for k, (y, e) in enumerate(expect):
+            got, want = y[0].float(), e.float()
+            # K = 14336: plan and single call may add a row's fp32 partial sums in a different
+            # order; everything else is bit-identical
+            if y.shape[1] == h and k % 6 == 5:
+                assert torch.allclose(got, want, rtol=2e-3, atol=1e-4), f"launch {launch} output {k}"
+            else:
+                assert torch.equal(y[0].view(torch.int16), e.view(torch.int16)), f"launch {launch} output {k}"
+    plan.close()
+
+
 def test_linear_plan_large_sweep_shared_pool(dev, oracle):
     """A plan big enough (16 LLaMA-1B layers, 112 matrices) that part of it is dealt out at run time
     instead of belonging to a fixed span: whichever workgroup takes a piece, every output must equal

@@ -152,6 +152,18 @@ typedef struct tllm_linear_plan tllm_linear_plan;
  * Allocates device memory; not for the per-token path. group_size must be 128. */
 int tllm_linear_plan_create(tllm_linear_plan **plan, const tllm_linear_problem *problems,
                             int count, int group_size);
+/*
+ * The same with an RMSNorm prologue: where norm_weights[i] is not NULL, problem i reads its input
+ * through   x' = fp16( x / sqrt(mean(x^2) + eps) * norm_weights[i] )   (fp32 arithmetic, the sums taken
+ * in the order of tllm_rmsnorm_f16, whose output it reproduces bit for bit when cols is a multiple of
+ * 2048), so the normalised vector is never written to memory. Such problems need batch 1 and
+ * cols <= 16384; both halves of a SwiGLU pair carry the same weights. norm_weights is a HOST array of
+ * `count` DEVICE pointers (fp16 [cols], 16-byte aligned). Replaces the rmsnorm_forward launch in
+ * front of each projection group, reference src/transformer.cpp:193-196, 258-261.
+ */
+int tllm_linear_plan_create_normed(tllm_linear_plan **plan, const tllm_linear_problem *problems,
+                                   const uint16_t *const *norm_weights, float eps, int count,
+                                   int group_size);
 /* One launch over every problem of the plan. Allocation-free. Launches of ONE plan must not overlap in
  * time (two streams, or two graph branches): besides the outputs they share two device counters that
  * deal the tail of a large plan out to the workgroups; the kernel resets them when it ends, so

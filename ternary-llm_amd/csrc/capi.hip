@@ -143,8 +143,8 @@ int tllm_silu_mul_f16(const uint16_t *gate, const uint16_t *up, uint16_t *output
     return (int)tllm::launch_silu_mul(gate, up, output, size, (hipStream_t)stream);
 }
 
-int tllm_linear_plan_create(tllm_linear_plan **plan, const tllm_linear_problem *problems,
-                            int count, int group_size) {
+static int create_plan(tllm_linear_plan **plan, const tllm_linear_problem *problems,
+                       const uint16_t *const *norm_weights, float eps, int count, int group_size) {
     if (!plan || !problems) return TLLM_ERR_NULL_POINTER;
     *plan = nullptr;
     if (count < 1) return TLLM_ERR_BAD_PLAN;
@@ -169,6 +169,16 @@ int tllm_linear_plan_create(tllm_linear_plan **plan, const tllm_linear_problem *
             if (i + 1 >= count || q.batch != 1) return TLLM_ERR_BAD_PLAN;
         }
         if (int e = tllm::check_linear(host[i], group_size)) return e;
+        if (norm_weights && norm_weights[i]) {
+            // RMSNorm prologue: batch 1, a row that the one-pass staging holds, 16-byte aligned weights
+            if (q.batch != 1 || q.cols > 16384 || !(eps >= 0.0f)) return TLLM_ERR_BAD_PLAN;
+            if (tllm::misaligned(norm_weights[i], 16)) return TLLM_ERR_MISALIGNED;
+            if (is_up && norm_weights[i] != norm_weights[i - 1]) return TLLM_ERR_BAD_PLAN;
+            host[i].norm_w = norm_weights[i];
+            host[i].eps = eps;
+        } else if (is_up && norm_weights && norm_weights[i - 1]) {
+            return TLLM_ERR_BAD_PLAN;  // the halves of a pair see the same activations
+        }
         bytes += (int64_t)q.rows * (q.cols / 32) * 8 + (int64_t)q.rows * (q.cols / group_size) * 2;
     }
     tllm_linear_plan *pl = new (std::nothrow) tllm_linear_plan{std::move(host), {}, group_size, bytes};
@@ -177,15 +187,25 @@ int tllm_linear_plan_create(tllm_linear_plan **plan, const tllm_linear_problem *
         delete pl;
         return (int)e;
     }
-    bool has_pairs = false;
-    for (const Problem &p : pl->host) has_pairs = has_pairs || (p.flags & TLLM_PROBLEM_SWIGLU_GATE);
-    if (has_pairs && !pl->dev.use_mfma) {  // a shape that only the general kernel serves: no fused pairs
+    if (pl->dev.extras && !pl->dev.use_mfma) {  // a shape that only the general kernel serves: no pairs, no prologue
         tllm::plan_device_destroy(&pl->dev);
         delete pl;
         return TLLM_ERR_BAD_PLAN;
     }
     *plan = pl;
     return TLLM_OK;
+}
+
+int tllm_linear_plan_create(tllm_linear_plan **plan, const tllm_linear_problem *problems,
+                            int count, int group_size) {
+    return create_plan(plan, problems, nullptr, 0.0f, count, group_size);
+}
+
+int tllm_linear_plan_create_normed(tllm_linear_plan **plan, const tllm_linear_problem *problems,
+                                   const uint16_t *const *norm_weights, float eps, int count,
+                                   int group_size) {
+    if (!norm_weights) return TLLM_ERR_NULL_POINTER;
+    return create_plan(plan, problems, norm_weights, eps, count, group_size);
 }
 
 int tllm_linear_plan_launch(const tllm_linear_plan *plan, tllm_stream_t stream) {

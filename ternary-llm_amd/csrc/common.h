@@ -22,8 +22,12 @@ struct Problem {
     int32_t cols;
     int32_t batch;
     int32_t flags;  // kProblemSwigluGate
+    // optional prologue (plans only): x is RMS-normalised with these weights before it is used
+    const uint16_t *norm_w;
+    float eps;
+    int32_t pad;
 };
-static_assert(sizeof(Problem) == sizeof(tllm_linear_problem), "ABI struct mirrors Problem");
+static_assert(sizeof(Problem) == sizeof(tllm_linear_problem) + 16, "tllm_linear_problem, then the prologue");
 constexpr int kProblemSwigluGate = TLLM_PROBLEM_SWIGLU_GATE;
 
 __device__ __forceinline__ float h2f(uint16_t bits) {
@@ -98,6 +102,7 @@ struct PlanDevice {
     int grid = 0;
     int max_units = 0;
     int pair_stride = 0;  // floats between the two partial-sum areas of a SwiGLU pair (0: no pairs)
+    bool extras = false;  // SwiGLU pairs or RMSNorm prologues present: the kernel instance that knows them
     int image_bytes = 0;
     int lds_bytes = 0;
 };

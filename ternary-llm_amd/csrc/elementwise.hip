@@ -45,7 +45,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(const uint16_t *i
     }
 }
 
-// The same operator for rows of up to 2048 * kChunks elements whose pointers are 16-byte aligned and
+// The same operator for rows of up to 2048 * kChunks elements (kChunks 1, 2, 4, 8) whose pointers are 16-byte aligned and
 // whose length is a multiple of 8: every lane keeps its 8-element chunks in registers between the
 // two passes, so the row is read once, through 16-byte loads.
 template <int kChunks>
@@ -149,13 +149,15 @@ hipError_t launch_rmsnorm(const uint16_t *input, const uint16_t *weight, uint16_
     const uintptr_t all = (uintptr_t)input | (uintptr_t)weight | (uintptr_t)output | (uintptr_t)residual |
                           (uintptr_t)residual_out;
     const int per_pass = kNormThreads * 8;
-    if ((all & 15) == 0 && dim % 8 == 0 && dim <= 4 * per_pass) {
+    if ((all & 15) == 0 && dim % 8 == 0 && dim <= 8 * per_pass) {
         if (dim <= per_pass)
             rmsnorm_rows_kernel<1><<<batch, kNormThreads, 0, s>>>(input, weight, output, residual, residual_out, dim, eps);
         else if (dim <= 2 * per_pass)
             rmsnorm_rows_kernel<2><<<batch, kNormThreads, 0, s>>>(input, weight, output, residual, residual_out, dim, eps);
-        else
+        else if (dim <= 4 * per_pass)
             rmsnorm_rows_kernel<4><<<batch, kNormThreads, 0, s>>>(input, weight, output, residual, residual_out, dim, eps);
+        else
+            rmsnorm_rows_kernel<8><<<batch, kNormThreads, 0, s>>>(input, weight, output, residual, residual_out, dim, eps);
     } else {
         rmsnorm_kernel<<<batch, kNormThreads, 0, s>>>(input, weight, output, residual, residual_out, dim, eps);
     }

@@ -146,14 +146,15 @@ __device__ __forceinline__ f4 tile_product(const u4 nz, const u4 sg, const u4 (&
     return d0 + d1;
 }
 
-// kPairs: the table may hold SwiGLU pairs (a separate instance, so that plans without them keep the
-// register allocation of the plain kernel).
-template <class G, bool kPairs = false>
+// kExtras: the table may hold SwiGLU pairs and RMSNorm prologues (a separate instance, so that plans
+// without them keep the register allocation of the plain kernel).
+template <class G, bool kExtras = false>
 __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Problem single, Sched sc) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     uint16_t *image = reinterpret_cast<uint16_t *>(lds);
     float *partial = reinterpret_cast<float *>(lds + sc.image_bytes);
     __shared__ uint32_t red_amax[kNW][kMaxBatch];
+    __shared__ float red_ss[kNW];
     __shared__ float fscale[kMaxBatch];
     __shared__ u4 zero_operand;  // what the idle lanes of a B operand read
     if (threadIdx.x == 0) zero_operand = u4{0u, 0u, 0u, 0u};
@@ -237,6 +238,14 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
                 if (g < slice * G::kChunks) return uint4{0u, 0u, 0u, 0u};
                 return load8(b, (g * kChunkCols + (c8 * 8) % kChunkCols) / 8);
             };
+            // the RMSNorm weights of the columns of piece c8 (zero where the piece is a duplicate)
+            auto norm_piece = [&](int c8) -> uint4 {
+                const int slice = (c8 * 8) / G::kCols;
+                const int chunk = ((c8 * 8) % G::kCols) / kChunkCols;
+                const int g = min(slice * G::kChunks, groups - G::kChunks) + chunk;
+                if (g < slice * G::kChunks) return uint4{0u, 0u, 0u, 0u};
+                return reinterpret_cast<const uint4 *>(p.norm_w)[(g * kChunkCols + (c8 * 8) % kChunkCols) / 8];
+            };
             auto magnitude = [](uint32_t m, const uint4 &v) -> uint32_t {
                 const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
@@ -290,6 +299,54 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
                     const int c8 = stid + k * kThreads;
                     keep[k] = c8 < pieces ? piece_of(0, c8) : uint4{0u, 0u, 0u, 0u};
                 }
+                if (kExtras && p.norm_w) {
+                    // RMSNorm prologue, reference kernels/rmsnorm.cu:20-106 without residual: the kept
+                    // pieces become fp16(x * rsqrt(mean x^2 + eps) * w). Same sums in the same order as
+                    // the stand-alone operator (elementwise.hip), so both give the same bits.
+                    float ss = 0.0f;
+#pragma unroll
+                    for (int k = 0; k < kKeep; k++) {
+                        const uint32_t w4[4] = {keep[k].x, keep[k].y, keep[k].z, keep[k].w};
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const float lo = h2f((uint16_t)w4[e]), hi = h2f((uint16_t)(w4[e] >> 16));
+                            ss += lo * lo;
+                            ss += hi * hi;
+                        }
+                        __builtin_amdgcn_sched_barrier(0);  // piece by piece: few registers
+                    }
+                    ss = wave_sum(ss);
+                    if (lane == 0) red_ss[wave] = ss;
+                    __syncthreads();
+                    float total = 0.0f;
+#pragma unroll
+                    for (int w = 0; w < kNW; w++) total += red_ss[w];
+                    const float inv = 1.0f / sqrtf(total / (float)p.cols + p.eps);
+                    // the weights come in two batches of loads, to keep the register need of this
+                    // rarely run code below that of the tile loop
+#pragma unroll
+                    for (int half = 0; half < 2; half++) {
+                        uint4 wk[kKeep / 2];
+#pragma unroll
+                        for (int k = 0; k < kKeep / 2; k++) {
+                            const int c8 = stid + (half * (kKeep / 2) + k) * kThreads;
+                            wk[k] = c8 < pieces ? norm_piece(c8) : uint4{0u, 0u, 0u, 0u};
+                        }
+#pragma unroll
+                        for (int k = 0; k < kKeep / 2; k++) {
+                            uint4 &x = keep[half * (kKeep / 2) + k];
+                            const uint32_t x4[4] = {x.x, x.y, x.z, x.w};
+                            const uint32_t n4[4] = {wk[k].x, wk[k].y, wk[k].z, wk[k].w};
+                            uint32_t o[4];
+#pragma unroll
+                            for (int e = 0; e < 4; e++)
+                                o[e] = (uint32_t)f2h(h2f((uint16_t)x4[e]) * inv * h2f((uint16_t)n4[e])) |
+                                       (uint32_t)f2h(h2f((uint16_t)(x4[e] >> 16)) * inv * h2f((uint16_t)(n4[e] >> 16))) << 16;
+                            x = uint4{o[0], o[1], o[2], o[3]};
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    }
+                }
 #pragma unroll
                 for (int k = 0; k < kKeep; k++) m = magnitude(m, keep[k]);
 #pragma unroll
@@ -336,7 +393,7 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
         // A SwiGLU pair (flag on the gate problem; the up problem follows it in the table, same shape
         // and activations, no units of its own) runs the walks twice over the same rows, with the same
         // operand image, into two partial-sum areas; the epilogue below joins them.
-        const bool pair = kPairs && (p.flags & kProblemSwigluGate) != 0;
+        const bool pair = kExtras && (p.flags & kProblemSwigluGate) != 0;
         for (int mat = 0; mat < (pair ? 2 : 1); mat++) {
         const uint32_t *w_nz = p.nz, *w_sg = p.sg;
         const uint16_t *w_sc = p.scales;
@@ -554,9 +611,9 @@ DeviceInfo &device_info(int dev) {
 
 constexpr int kLdsLimit = 64 * 1024;  // per workgroup; 160 KB per CU leaves room for two or three
 
-template <class G, bool kPairs = false>
+template <class G, bool kExtras = false>
 const void *kernel_ptr() {
-    return reinterpret_cast<const void *>(&gemv_mfma_kernel<G, kPairs>);
+    return reinterpret_cast<const void *>(&gemv_mfma_kernel<G, kExtras>);
 }
 
 hipError_t prepare_device(DeviceInfo **out) {
@@ -579,10 +636,10 @@ hipError_t prepare_device(DeviceInfo **out) {
 }
 
 // Resident workgroups per CU for a given dynamic LDS size (asked from the runtime, capped at 4).
-template <class G, bool kPairs = false>
+template <class G, bool kExtras = false>
 int resident_wgs(size_t lds_bytes) {
     int n = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gemv_mfma_kernel<G, kPairs>, kThreads, lds_bytes) != hipSuccess || n < 1)
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gemv_mfma_kernel<G, kExtras>, kThreads, lds_bytes) != hipSuccess || n < 1)
         n = 1;
     return n > 4 ? 4 : n;
 }
@@ -863,9 +920,14 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
     };
 
     // several activation rows: the batched kernel if every problem fits it
-    bool has_pairs = false;
-    for (const Problem &p : host) has_pairs = has_pairs || (p.flags & kProblemSwigluGate);
-    bool all_batch = max_batch >= 2 && !has_pairs;  // pairs are joined in the MFMA GEMV kernel only
+    bool has_pairs = false, has_norm = false;
+    for (const Problem &p : host) {
+        has_pairs = has_pairs || (p.flags & kProblemSwigluGate);
+        has_norm = has_norm || p.norm_w != nullptr;
+    }
+    // SwiGLU pairs and RMSNorm prologues exist in the wide-tile MFMA GEMV kernel only (batch 1)
+    d.extras = has_pairs || has_norm;
+    bool all_batch = max_batch >= 2 && !d.extras;
     for (const Problem &p : host) all_batch = all_batch && gemv_batch_supports(p, 128);
     // one geometry per launch otherwise: wide tiles if every problem allows them, else tall ones
     bool all_wide = true, all_tall = true;
@@ -879,7 +941,7 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
         partition_blocks(gemv_batch_block_rows(), di->cus);
     } else {
         d.wide = all_wide;
-        d.use_mfma = has_pairs ? all_wide : all_wide || all_tall;  // pairs: batch 1, wide tiles only
+        d.use_mfma = d.extras ? all_wide : all_wide || all_tall;
         for (const Problem &p : host) {
             const int ib = d.wide ? image_bytes_of<Wide>(p.cols, 1) : image_bytes_of<Tall>(p.cols, p.batch);
             max_image = ib > max_image ? ib : max_image;
@@ -891,7 +953,7 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
         if (d.use_mfma) {
             d.pair_stride = has_pairs ? kNW * max_units * unit * max_batch : 0;
             d.lds_bytes = max_image + kNW * max_units * unit * max_batch * 4 * mats;
-            const int per_cu = has_pairs ? resident_wgs<Wide, true>(d.lds_bytes)
+            const int per_cu = d.extras ? resident_wgs<Wide, true>(d.lds_bytes)
                                : d.wide  ? resident_wgs<Wide>(d.lds_bytes)
                                          : resident_wgs<Tall>(d.lds_bytes);
             partition(unit, per_cu * di->cus, max_units);
@@ -947,7 +1009,7 @@ hipError_t plan_device_launch(const PlanDevice &plan, hipStream_t s) {
     sc.max_batch = plan.max_batch;
     sc.image_bytes = plan.image_bytes;
     Problem none{};
-    if (plan.pair_stride)
+    if (plan.extras)
         gemv_mfma_kernel<Wide, true><<<plan.grid, kThreads, plan.lds_bytes, s>>>(none, sc);
     else if (plan.wide)
         gemv_mfma_kernel<Wide><<<plan.grid, kThreads, plan.lds_bytes, s>>>(none, sc);

@@ -16,7 +16,7 @@ ABI_SYMBOLS = (
     "tllm_error_string", "tllm_abi_version", "tllm_ternary_gemv_f16", "tllm_ternary_gemv_i8",
     "tllm_ternary_gemv_i8_dscale", "tllm_quantize_absmax_i8", "tllm_ternary_gemm_f16",
     "tllm_linear_plan_create", "tllm_linear_plan_launch", "tllm_linear_plan_weight_bytes",
-    "tllm_linear_plan_destroy", "tllm_rmsnorm_f16", "tllm_silu_mul_f16",
+    "tllm_linear_plan_destroy", "tllm_rmsnorm_f16", "tllm_silu_mul_f16", "tllm_linear_plan_create_normed",
 )
 # include/tllm_model_file.h
 FILE_ABI_SYMBOLS = (
@@ -75,6 +75,7 @@ def lib():
     L.tllm_quantize_absmax_i8.argtypes = [vp, vp, vp, i, vp]
     L.tllm_ternary_gemm_f16.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, vp]
     L.tllm_linear_plan_create.argtypes = [C.POINTER(vp), C.POINTER(_Problem), i, i]
+    L.tllm_linear_plan_create_normed.argtypes = [C.POINTER(vp), C.POINTER(_Problem), C.POINTER(vp), f, i, i]
     L.tllm_linear_plan_launch.argtypes = [vp, vp]
     L.tllm_linear_plan_weight_bytes.argtypes = [vp]
     L.tllm_linear_plan_weight_bytes.restype = C.c_int64
@@ -167,7 +168,7 @@ SWIGLU_GATE = 1  # TLLM_PROBLEM_SWIGLU_GATE
 class LinearPlan:
     """Several independent ternary linears issued as one launch."""
 
-    def __init__(self, problems, group_size=128):
+    def __init__(self, problems, group_size=128, norm_weights=None, eps=1e-5):
         """problems: iterable of (nz, sign, scales, input, output, rows, cols, batch[, flags]);
         flags = SWIGLU_GATE marks the gate of a pair whose up projection is the next problem
         (output may be None there): the pair stores silu(gate) * up in the gate's output."""
@@ -180,7 +181,15 @@ class LinearPlan:
             arr[k] = _Problem(nz.data_ptr(), sg.data_ptr(), sc.data_ptr(), x.data_ptr(),
                               y.data_ptr() if y is not None else 0, rows, cols, batch, flags)
         self._h = C.c_void_p(0)
-        check(lib().tllm_linear_plan_create(C.byref(self._h), arr, len(problems), group_size))
+        if norm_weights is None:
+            check(lib().tllm_linear_plan_create(C.byref(self._h), arr, len(problems), group_size))
+        else:
+            # one fp16 weight tensor (or None) per problem: RMSNorm prologue on that problem's input
+            self._keep_norm = list(norm_weights)
+            ptrs = (C.c_void_p * max(len(problems), 1))(*[w.data_ptr() if w is not None else None
+                                                         for w in self._keep_norm])
+            check(lib().tllm_linear_plan_create_normed(C.byref(self._h), arr, ptrs, float(eps), len(problems),
+                                                       group_size))
 
     @property
     def weight_bytes(self):

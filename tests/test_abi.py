@@ -77,6 +77,20 @@ def test_validation_codes():
                 [P(0x1000, 0x2000, 0x3000, 0x4000, 0x9000, 64, 2048, 1, 2)]):         # unknown flag
         arr = (P * len(bad))(*bad)
         assert L.tllm_linear_plan_create(C.byref(h), arr, len(bad), 128) == -6
+    # RMSNorm prologue: batch 1, cols <= 16384, aligned weights, same weights on both halves of a pair
+    def normed(problems, norms, eps=1e-5):
+        arr = (P * len(problems))(*problems)
+        ptrs = (C.c_void_p * len(problems))(*norms)
+        return L.tllm_linear_plan_create_normed(C.byref(h), arr, ptrs, eps, len(problems), 128)
+    one = P(0x1000, 0x2000, 0x3000, 0x4000, 0x9000, 64, 2048, 1, 0)
+    assert L.tllm_linear_plan_create_normed(C.byref(h), (P * 1)(one), None, 1e-5, 1, 128) == -1
+    assert normed([P(0x1000, 0x2000, 0x3000, 0x4000, 0x9000, 64, 2048, 2, 0)], [0x7000]) == -6
+    assert normed([P(0x1000, 0x2000, 0x3000, 0x40000, 0x90000, 64, 32768, 1, 0)], [0x7000]) == -6
+    assert normed([one], [0x7002]) == -7
+    assert normed([one], [0x7000], eps=-1.0) == -6
+    up_ = P(0x1000, 0x2000, 0x3000, 0x4000, 0, 64, 2048, 1, 0)
+    assert normed([gate, up_], [0x7000, 0x8000]) == -6
+    assert normed([gate, up_], [0x7000, None]) == -6
     assert L.tllm_linear_plan_launch(None, None) == -6
     for code in range(-7, 1):
         assert L.tllm_error_string(code)

@@ -574,6 +574,74 @@ def test_swiglu_pair_vs_oracle_and_unfused(dev, oracle, rows, cols):
     plan.close()
 
 
+@pytest.mark.parametrize("cols,exact", [(4096, True), (2048, True), (8192, True), (16384, True), (11008, False)])
+def test_rmsnorm_prologue_vs_unfused_and_oracle(dev, oracle, cols, exact):
+    """q/k/v-like problems that read the residual stream through an RMSNorm prologue: equal to
+    tllm_rmsnorm_f16 followed by the plain plan (bit for bit when cols is a multiple of 2048, where
+    the sums are taken in the same order), and within tolerance of the fp64 evaluation."""
+    torch, tl = dev
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(cols)
+    x = (torch.randn((1, cols), device="cuda", generator=gen) * 3.0).to(torch.float16)
+    wn = (torch.randn(cols, device="cuda", generator=gen) * 0.2 + 1.0).to(torch.float16)
+    eps = 1e-5
+    shapes = [(4096, cols), (1024, cols), (100, cols)]
+    weights = [_rand_weight(torch, gen, r, c) for r, c in shapes]
+    outs = [torch.full((1, r), float("nan"), dtype=torch.float16, device="cuda") for r, _ in shapes]
+    fused = tl.LinearPlan([(*w, x, y, r, c, 1) for w, y, (r, c) in zip(weights, outs, shapes)],
+                          norm_weights=[wn] * 3, eps=eps)
+    fused.launch()
+    xn = torch.empty_like(x)
+    tl.rmsnorm(x, wn, xn, None, None, 1, cols, eps)
+    ref_outs = [torch.zeros((1, r), dtype=torch.float16, device="cuda") for r, _ in shapes]
+    plain = tl.LinearPlan([(*w, xn, y, r, c, 1) for w, y, (r, c) in zip(weights, ref_outs, shapes)])
+    plain.launch()
+    torch.cuda.synchronize()
+    xn_ref, _ = oracle.rmsnorm_f64(x.cpu().numpy().view(np.uint16), wn.cpu().numpy().view(np.uint16), eps)
+    xn_bits = oracle.half_bits(xn_ref[0])
+    for w, y, yr, (r, c) in zip(weights, outs, ref_outs, shapes):
+        if exact:
+            assert torch.equal(y.view(torch.int16), yr.view(torch.int16)), f"{r}x{c}"
+        pick = np.random.default_rng(r).integers(0, r, 64)
+        ref = oracle.gemv_f64(w[0][pick].cpu().numpy().view(np.uint32), w[1][pick].cpu().numpy().view(np.uint32),
+                              w[2][pick].cpu().numpy().view(np.uint16), xn_bits)
+        # the normalised vector is rounded to fp16 before the product; where the fp32 statistic lands
+        # on the other side of such a rounding, single elements of x' move by one fp16 ulp
+        assert_close(oracle, y[0][pick].cpu().numpy().astype(np.float64), ref, tol=2e-3, what=f"normed {r}x{c}")
+    fused.close()
+    plain.close()
+
+
+def test_rmsnorm_prologue_with_swiglu_pair(dev, oracle):
+    """The FFN front half of a decoder layer in ONE launch: RMSNorm, gate and up projections, SiLU*mul
+    (reference src/transformer.cpp:258-286: four launches). Equal to the four operators bit for bit."""
+    torch, tl = dev
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(31)
+    h, ffn, eps = 4096, 14336, 1e-5
+    x = (torch.randn((1, h), device="cuda", generator=gen) * 2.0).to(torch.float16)
+    wn = (torch.randn(h, device="cuda", generator=gen) * 0.2 + 1.0).to(torch.float16)
+    g_w, u_w = _rand_weight(torch, gen, ffn, h), _rand_weight(torch, gen, ffn, h)
+    out = torch.full((1, ffn), float("nan"), dtype=torch.float16, device="cuda")
+    plan = tl.LinearPlan([(*g_w, x, out, ffn, h, 1, tl.SWIGLU_GATE), (*u_w, x, None, ffn, h, 1)],
+                         norm_weights=[wn, wn], eps=eps)
+    for _ in range(2):
+        out.fill_(float("nan"))
+        plan.launch()
+        torch.cuda.synchronize()
+        xn = torch.empty_like(x)
+        tl.rmsnorm(x, wn, xn, None, None, 1, h, eps)
+        g = torch.zeros(ffn, dtype=torch.float16, device="cuda")
+        u = torch.zeros(ffn, dtype=torch.float16, device="cuda")
+        tl.ternary_gemv(*g_w, xn, g, ffn, h, 128)
+        tl.ternary_gemv(*u_w, xn, u, ffn, h, 128)
+        want = torch.empty_like(g)
+        tl.silu_mul(g, u, want, ffn)
+        torch.cuda.synchronize()
+        assert torch.equal(out[0].view(torch.int16), want.view(torch.int16))
+    plan.close()
+
+
 def test_swiglu_pairs_in_a_layer_sweep(dev, oracle):
     """Twelve 8B-shaped layers as one plan (q, k, v, o, the gate/up pair, down): large enough for the
     run-time pool, pairs in spans and in the pool alike; every output equals the separate calls."""

@@ -102,6 +102,7 @@ struct PlanDevice {
     int grid = 0;
     int max_units = 0;
     int pair_stride = 0;  // floats between the two partial-sum areas of a SwiGLU pair (0: no pairs)
+    bool fine = false;    // units of 16 rows (decode-size plans that would leave most workgroup slots empty)
     bool extras = false;  // SwiGLU pairs or RMSNorm prologues present: the kernel instance that knows them
     int image_bytes = 0;
     int lds_bytes = 0;

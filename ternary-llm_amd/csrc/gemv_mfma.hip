@@ -148,8 +148,11 @@ __device__ __forceinline__ f4 tile_product(const u4 nz, const u4 sg, const u4 (&
 
 // kExtras: the table may hold SwiGLU pairs and RMSNorm prologues (a separate instance, so that plans
 // without them keep the register allocation of the plain kernel).
-template <class G, bool kExtras = false>
-__global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Problem single, Sched sc) {
+// kFine: units of one tile per wave (16 rows for wide tiles) instead of kTilesAhead, for launches
+// that would otherwise leave most of the chip's workgroup slots empty; the tile ring then runs
+// across the walks of a wave and the B operands are reloaded for every tile.
+template <class G, bool kExtras = false, bool kFine = false>
+__global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma_kernel(Problem single, Sched sc) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     uint16_t *image = reinterpret_cast<uint16_t *>(lds);
     float *partial = reinterpret_cast<float *>(lds + sc.image_bytes);
@@ -167,7 +170,7 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
     const int li = lane & 15;  // MFMA A row / D column
     const int lq = lane >> 4;  // MFMA k quarter / D row quad
 
-    constexpr int kUnitRows = kNW * G::kRows * kTilesAhead;
+    constexpr int kUnitRows = kNW * G::kRows * (kFine ? 1 : kTilesAhead);
     int u = 0, u_end = 0, pi = 0;
     if (sc.table) {
         u = sc.wg_first[blockIdx.x];
@@ -488,6 +491,86 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
             // lanes whose result row (li & 3) is odd / is 2 or 3 (wide tiles pick one of four D rows)
             const uint64_t odd_lanes = __builtin_amdgcn_ballot_w64((li & 1) != 0);
             const uint64_t hi_lanes = __builtin_amdgcn_ballot_w64((li & 2) != 0);
+            auto process_tile = [&](const Tile<G> &t, int rb, bool live, const u4 (&B)[kMfmaPerTile], const f4 &bias,
+                                    float bias_sel) {
+                f4 d0, d1;
+                tile_product2(t.nz, t.sg, B, d0, d1);
+                const f4 d = d0 + d1;
+                const int sh = rb - min(rb, p.rows - G::kRows);  // rows a moved-back block repeats
+                if constexpr (G::kRows == 4) {
+                    // lane (row quad lq, column li): only D row 4*lq + (li & 3) pairs this column's
+                    // chunk with the row that loaded it; it is group li of row rb - sh + lq.
+                    // (bias_sel was formed the same way, so an all-zero row still gives exactly 0)
+                    const float dv = lane_select(lane_select(d[0], d[1], odd_lanes),
+                                                 lane_select(d[2], d[3], odd_lanes), hi_lanes);
+                    float x = h2f(t.sc[0]) * (dv - bias_sel);
+                    x = dpp_add<kQuadSwap1>(x);
+                    x = dpp_add<kQuadSwap2>(x);
+                    x = dpp_add<kRowHalfMirror>(x);
+                    x = dpp_add<kRowMirror>(x);
+                    if (li == 0 && lq >= sh && live) my_part[rb - sh - r_begin + lq] += x;
+                } else {
+                    float r[4];
+#pragma unroll
+                    for (int v = 0; v < 4; v++) {
+                        float x = h2f(t.sc[v]) * (d[v] - bias[v]);
+                        x = dpp_add<kQuadSwap1>(x);
+                        x = dpp_add<kQuadSwap2>(x);
+                        r[v] = x;
+                    }
+                    if ((li & 3) == 0 && bcol < p.batch && live) {
+#pragma unroll
+                        for (int v = 0; v < 4; v++)
+                            if (4 * lq + v >= sh)
+                                my_part[(size_t)(rb - sh - r_begin + 4 * lq + v) * p.batch + bcol] += r[v];
+                    }
+                }
+            };
+
+            // the B operands of a slice, and what an all-zero weight row gives with them
+            auto load_operands = [&](int slice, u4 (&B)[kMfmaPerTile], f4 &bias, float &bias_sel) {
+                // Every lane reads (no branch): the idle lanes read the zero operand with stride 0.
+                const u4 *src = b_active ? reinterpret_cast<const u4 *>(image + (size_t)bcol * img_stride +
+                                                                        slice * G::kCols) + b_chunk
+                                         : &zero_operand;
+                const int stride = b_active ? G::kChunks : 0;
+#pragma unroll
+                for (int k = 0; k < kMfmaPerTile; k++) B[k] = src[k * stride];
+                // an all-zero weight row gives the "+1" term of the code, to be subtracted
+                bias = tile_product(zero4, zero4, B);
+                // wide tiles: the one bias entry this lane uses
+                bias_sel = lane_select(lane_select(bias[0], bias[1], odd_lanes),
+                                       lane_select(bias[2], bias[3], odd_lanes), hi_lanes);
+            };
+            if constexpr (kFine) {
+                // one flat sequence of (walk, slot) pairs, three at a time through the ring
+                u4 B[kMfmaPerTile];
+                f4 bias;
+                float bias_sel = 0.0f;
+                int wi = 0, j = 0, c_begin = 0, n_rb = 0;
+                const int total = my_walks * n_slots;
+                for (int t0 = 0; t0 < total; t0 += kTilesAhead) {
+#pragma unroll
+                    for (int k = 0; k < kTilesAhead; k++) {
+                        if (t0 + k < total) {
+                            if (j == 0) {
+                                const int walk = wave + wi * kNW;
+                                const int chunk = walk / slices, slice = walk - chunk * slices;
+                                c_begin = r_begin + chunk * chunk_rows;
+                                n_rb = chunk_tiles(chunk);
+                                load_operands(slice, B, bias, bias_sel);
+                            }
+                            process_tile(ring[k], c_begin + min(j, max(n_rb, 1) - 1) * G::kRows, j < n_rb, B, bias, bias_sel);
+                            if (++j == n_slots) {
+                                j = 0;
+                                wi++;
+                            }
+                        }
+                        ring[k] = next_load();
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            } else
             for (int wi = 0; wi < my_walks; wi++) {
                 const int walk = wave + wi * kNW;
                 const int chunk = walk / slices, slice = walk - chunk * slices;
@@ -508,40 +591,7 @@ __global__ __launch_bounds__(kThreads, G::kWgPerCu) void gemv_mfma_kernel(Proble
                 const float bias_sel = lane_select(lane_select(bias[0], bias[1], odd_lanes),
                                                    lane_select(bias[2], bias[3], odd_lanes), hi_lanes);
 
-                auto process = [&](const Tile<G> &t, int rb, bool live) {
-                    f4 d0, d1;
-                    tile_product2(t.nz, t.sg, B, d0, d1);
-                    const f4 d = d0 + d1;
-                    const int sh = rb - min(rb, p.rows - G::kRows);  // rows a moved-back block repeats
-                    if constexpr (G::kRows == 4) {
-                        // lane (row quad lq, column li): only D row 4*lq + (li & 3) pairs this column's
-                        // chunk with the row that loaded it; it is group li of row rb - sh + lq.
-                        // (bias_sel was formed the same way, so an all-zero row still gives exactly 0)
-                        const float dv = lane_select(lane_select(d[0], d[1], odd_lanes),
-                                                     lane_select(d[2], d[3], odd_lanes), hi_lanes);
-                        float x = h2f(t.sc[0]) * (dv - bias_sel);
-                        x = dpp_add<kQuadSwap1>(x);
-                        x = dpp_add<kQuadSwap2>(x);
-                        x = dpp_add<kRowHalfMirror>(x);
-                        x = dpp_add<kRowMirror>(x);
-                        if (li == 0 && lq >= sh && live) my_part[rb - sh - r_begin + lq] += x;
-                    } else {
-                        float r[4];
-#pragma unroll
-                        for (int v = 0; v < 4; v++) {
-                            float x = h2f(t.sc[v]) * (d[v] - bias[v]);
-                            x = dpp_add<kQuadSwap1>(x);
-                            x = dpp_add<kQuadSwap2>(x);
-                            r[v] = x;
-                        }
-                        if ((li & 3) == 0 && bcol < p.batch && live) {
-#pragma unroll
-                            for (int v = 0; v < 4; v++)
-                                if (4 * lq + v >= sh)
-                                    my_part[(size_t)(rb - sh - r_begin + 4 * lq + v) * p.batch + bcol] += r[v];
-                        }
-                    }
-                };
+                auto process = [&](const Tile<G> &t, int rb, bool live) { process_tile(t, rb, live, B, bias, bias_sel); };
 
                 // No branch surrounds a load or an MFMA, so the wait counters stay exact and
                 // kTilesAhead - 1 tiles remain in flight while one is consumed.
@@ -611,9 +661,9 @@ DeviceInfo &device_info(int dev) {
 
 constexpr int kLdsLimit = 64 * 1024;  // per workgroup; 160 KB per CU leaves room for two or three
 
-template <class G, bool kExtras = false>
+template <class G, bool kExtras = false, bool kFine = false>
 const void *kernel_ptr() {
-    return reinterpret_cast<const void *>(&gemv_mfma_kernel<G, kExtras>);
+    return reinterpret_cast<const void *>(&gemv_mfma_kernel<G, kExtras, kFine>);
 }
 
 hipError_t prepare_device(DeviceInfo **out) {
@@ -629,6 +679,10 @@ hipError_t prepare_device(DeviceInfo **out) {
             return e;
         if (hipError_t e = hipFuncSetAttribute(kernel_ptr<Wide, true>(), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit))
             return e;
+        if (hipError_t e = hipFuncSetAttribute(kernel_ptr<Wide, false, true>(), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit))
+            return e;
+        if (hipError_t e = hipFuncSetAttribute(kernel_ptr<Wide, true, true>(), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit))
+            return e;
         di.cus = n > 0 ? n : 256;
     }
     *out = &di;
@@ -636,10 +690,10 @@ hipError_t prepare_device(DeviceInfo **out) {
 }
 
 // Resident workgroups per CU for a given dynamic LDS size (asked from the runtime, capped at 4).
-template <class G, bool kExtras = false>
+template <class G, bool kExtras = false, bool kFine = false>
 int resident_wgs(size_t lds_bytes) {
     int n = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gemv_mfma_kernel<G, kExtras>, kThreads, lds_bytes) != hipSuccess || n < 1)
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, gemv_mfma_kernel<G, kExtras, kFine>, kThreads, lds_bytes) != hipSuccess || n < 1)
         n = 1;
     return n > 4 ? 4 : n;
 }
@@ -648,6 +702,10 @@ template <class G>
 constexpr int range_unit() {  // rows: every wave walks whole groups of kTilesAhead tiles
     return kNW * G::kRows * kTilesAhead;
 }
+constexpr int kFineUnit = kNW * Wide::kRows;  // rows of a unit of the fine-grained instances: one tile per wave
+// A launch whose 48-row units would fill less than half of the workgroup slots of the chip runs in
+// units of 16 rows instead (wide tiles only): three times the workgroups, a third of the tiles each.
+bool wants_fine(int64_t coarse_units, int slots) { return coarse_units * 2 <= slots; }
 
 template <class G>
 int image_bytes_of(int cols, int batch) {
@@ -749,14 +807,17 @@ static hipError_t launch_single(const Problem &p, bool x_is_i8, float i8_scale, 
     sc.count = 1;
     const bool wide = wide_ok(p);
     sc.image_bytes = wide ? image_bytes_of<Wide>(p.cols, 1) : image_bytes_of<Tall>(p.cols, p.batch);
-    const int unit = wide ? range_unit<Wide>() : range_unit<Tall>();
+    const int wgs = (wide ? Wide::kWgPerCu : Tall::kWgPerCu) * di->cus;
+    const bool fine = wide && wants_fine((p.rows + range_unit<Wide>() - 1) / range_unit<Wide>(), wgs);
+    const int unit = fine ? kFineUnit : wide ? range_unit<Wide>() : range_unit<Tall>();
     sc.max_units = max_units_for(sc.image_bytes, p.batch, unit);
     sc.max_batch = p.batch;
-    const int wgs = (wide ? Wide::kWgPerCu : Tall::kWgPerCu) * di->cus;
     const int units = (p.rows + unit - 1) / unit;
     const int grid = units < wgs ? units : wgs;
     const size_t lds = (size_t)sc.image_bytes + (size_t)kNW * sc.max_units * unit * p.batch * 4;
-    if (wide)
+    if (fine)
+        gemv_mfma_kernel<Wide, false, true><<<grid, kThreads, lds, s>>>(p, sc);
+    else if (wide)
         gemv_mfma_kernel<Wide><<<grid, kThreads, lds, s>>>(p, sc);
     else
         gemv_mfma_kernel<Tall><<<grid, kThreads, lds, s>>>(p, sc);
@@ -946,16 +1007,25 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
             const int ib = d.wide ? image_bytes_of<Wide>(p.cols, 1) : image_bytes_of<Tall>(p.cols, p.batch);
             max_image = ib > max_image ? ib : max_image;
         }
-        const int unit = d.wide ? range_unit<Wide>() : range_unit<Tall>();
+        if (d.wide) {  // decode-size plans: fine-grained units
+            int64_t coarse = 0;
+            for (size_t i = 0; i < host.size(); i++)
+                if (!(i > 0 && (host[i - 1].flags & kProblemSwigluGate)))
+                    coarse += (host[i].rows + range_unit<Wide>() - 1) / range_unit<Wide>();
+            d.fine = wants_fine(coarse, Wide::kWgPerCu * di->cus);
+        }
+        const int unit = d.fine ? kFineUnit : d.wide ? range_unit<Wide>() : range_unit<Tall>();
         const int mats = has_pairs ? 2 : 1;
         const int max_units = max_units_for(max_image, max_batch, unit, mats);
         if (max_units < 1) d.use_mfma = false;
         if (d.use_mfma) {
             d.pair_stride = has_pairs ? kNW * max_units * unit * max_batch : 0;
             d.lds_bytes = max_image + kNW * max_units * unit * max_batch * 4 * mats;
-            const int per_cu = d.extras ? resident_wgs<Wide, true>(d.lds_bytes)
-                               : d.wide  ? resident_wgs<Wide>(d.lds_bytes)
-                                         : resident_wgs<Tall>(d.lds_bytes);
+            const int per_cu = d.extras && d.fine ? resident_wgs<Wide, true, true>(d.lds_bytes)
+                               : d.extras         ? resident_wgs<Wide, true>(d.lds_bytes)
+                               : d.fine           ? resident_wgs<Wide, false, true>(d.lds_bytes)
+                               : d.wide           ? resident_wgs<Wide>(d.lds_bytes)
+                                                  : resident_wgs<Tall>(d.lds_bytes);
             partition(unit, per_cu * di->cus, max_units);
             d.max_units = max_units;
             d.image_bytes = max_image;
@@ -1009,8 +1079,12 @@ hipError_t plan_device_launch(const PlanDevice &plan, hipStream_t s) {
     sc.max_batch = plan.max_batch;
     sc.image_bytes = plan.image_bytes;
     Problem none{};
-    if (plan.extras)
+    if (plan.extras && plan.fine)
+        gemv_mfma_kernel<Wide, true, true><<<plan.grid, kThreads, plan.lds_bytes, s>>>(none, sc);
+    else if (plan.extras)
         gemv_mfma_kernel<Wide, true><<<plan.grid, kThreads, plan.lds_bytes, s>>>(none, sc);
+    else if (plan.fine)
+        gemv_mfma_kernel<Wide, false, true><<<plan.grid, kThreads, plan.lds_bytes, s>>>(none, sc);
     else if (plan.wide)
         gemv_mfma_kernel<Wide><<<plan.grid, kThreads, plan.lds_bytes, s>>>(none, sc);
     else

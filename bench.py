@@ -188,6 +188,85 @@ def gemm_report(torch, tl, orc, seed, m_list, p_zero=0.42, calls=200, warm=20):
             "cases": cases}
 
 
+def decode_chain_report(torch, tl, problems, model, layers, reps=40):
+    """The linear-side launches of a batch-1 decode step over the sweep's own weights, issued in the
+    order a transformer needs them (every launch after the one before, as reference
+    src/transformer.cpp:193-296 does): (a) the reference's ten launches per layer, (b) q/k/v and gate/up as
+    plans, (c) RMSNorm prologue + SwiGLU pair: four launches per layer. Microseconds per token."""
+    h, qd, kvd, ffn, _ = SHAPES[model]
+    f16 = dict(dtype=torch.float16, device="cuda")
+    x = torch.randn((1, h), device="cuda").to(torch.float16)
+    xn, att = torch.empty_like(x), torch.randn((1, qd), device="cuda").to(torch.float16)
+    q, k, v = torch.zeros((1, qd), **f16), torch.zeros((1, kvd), **f16), torch.zeros((1, kvd), **f16)
+    o, g, u, d = torch.zeros((1, h), **f16), torch.zeros((1, ffn), **f16), torch.zeros((1, ffn), **f16), torch.zeros((1, h), **f16)
+    eps, L = 1e-5, []
+    for l in range(layers):
+        w = {name: problems[7 * l + i][:3] for i, name in enumerate(("q", "k", "v", "o", "g", "u", "d"))}
+        w["n1"], w["n2"] = torch.ones(h, **f16), torch.ones(h, **f16)
+        w["qkv"] = tl.LinearPlan([(*w["q"], xn, q, qd, h, 1), (*w["k"], xn, k, kvd, h, 1), (*w["v"], xn, v, kvd, h, 1)])
+        w["gu"] = tl.LinearPlan([(*w["g"], xn, g, ffn, h, 1), (*w["u"], xn, u, ffn, h, 1)])
+        w["qkv_n"] = tl.LinearPlan([(*w["q"], x, q, qd, h, 1), (*w["k"], x, k, kvd, h, 1), (*w["v"], x, v, kvd, h, 1)],
+                                   norm_weights=[w["n1"]] * 3, eps=eps)
+        w["gu_n"] = tl.LinearPlan([(*w["g"], x, g, ffn, h, 1, tl.SWIGLU_GATE), (*w["u"], x, None, ffn, h, 1)],
+                                  norm_weights=[w["n2"]] * 2, eps=eps)
+        L.append(w)
+
+    def ten():
+        for w in L:
+            tl.rmsnorm(x, w["n1"], xn, None, None, 1, h, eps)
+            tl.ternary_gemv(*w["q"], xn, q, qd, h, 128)
+            tl.ternary_gemv(*w["k"], xn, k, kvd, h, 128)
+            tl.ternary_gemv(*w["v"], xn, v, kvd, h, 128)
+            tl.ternary_gemv(*w["o"], att, o, h, qd, 128)
+            tl.rmsnorm(x, w["n2"], xn, None, None, 1, h, eps)
+            tl.ternary_gemv(*w["g"], xn, g, ffn, h, 128)
+            tl.ternary_gemv(*w["u"], xn, u, ffn, h, 128)
+            tl.silu_mul(g, u, g, ffn)
+            tl.ternary_gemv(*w["d"], g, d, h, ffn, 128)
+
+    def seven():
+        for w in L:
+            tl.rmsnorm(x, w["n1"], xn, None, None, 1, h, eps)
+            w["qkv"].launch()
+            tl.ternary_gemv(*w["o"], att, o, h, qd, 128)
+            tl.rmsnorm(x, w["n2"], xn, None, None, 1, h, eps)
+            w["gu"].launch()
+            tl.silu_mul(g, u, g, ffn)
+            tl.ternary_gemv(*w["d"], g, d, h, ffn, 128)
+
+    def four():
+        for w in L:
+            w["qkv_n"].launch()
+            tl.ternary_gemv(*w["o"], att, o, h, qd, 128)
+            w["gu_n"].launch()
+            tl.ternary_gemv(*w["d"], g, d, h, ffn, 128)
+
+    def timed(fn):
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps * 1e3
+
+    nbytes = sum(packed_bytes(p[5], p[6]) for p in problems[:7 * layers])
+    out = {"workload": f"{model}: linear-side launches of one decode step, {layers} layers, batch 1, dependent order",
+           "unit": "us per token", "packed_bytes": nbytes}
+    for name, fn, n in (("reference_10_launches_per_layer", ten, 10), ("plans_7_launches_per_layer", seven, 7),
+                        ("prologue_and_pair_4_launches_per_layer", four, 4)):
+        us = timed(fn)
+        out[name] = {"us_per_token": round(us, 1), "GBps": round(nbytes / us / 1e3, 1),
+                     "us_per_launch": round(us / (n * layers), 2)}
+    for w in L:
+        for key in ("qkv", "gu", "qkv_n", "gu_n"):
+            w[key].close()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -212,6 +291,8 @@ def main():
     ap.add_argument("--gemm-m", default="512", help='token counts M of the prefill GEMM report, e.g. "16,128,512,2048"; "" skips it')
     ap.add_argument("--gemm-calls", type=int, default=200, help="timed launches per GEMM case")
     ap.add_argument("--gemm-warm", type=int, default=20, help="untimed launches before them")
+    ap.add_argument("--decode-chain", action="store_true",
+                    help="also time the dependent launch sequence of a decode step (three variants)")
     ap.add_argument("--seed", type=int, default=20240611)
     args = ap.parse_args()
     for item in filter(None, args.matrices.split(",")):
@@ -347,6 +428,8 @@ def main():
                                      "kernel": "tllm::gemv_batch_kernel", "parity_max_rel_sampled": par_b})
         plan_b.close()
         del probs_b
+    if args.decode_chain and not CUSTOM and args.batch == 1:
+        out["decode_chain"] = decode_chain_report(torch, tl, problems, args.model, layers)
     gemm_m = [int(v) for v in args.gemm_m.split(",") if v.strip()]
     if gemm_m:
         out["gemm"] = gemm_report(torch, tl, orc, args.seed, gemm_m, args.p_zero, args.gemm_calls, args.gemm_warm)

@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <vector>
 
 #include "../../include/tllm_ternary.h"
@@ -29,6 +30,20 @@ struct Problem {
 };
 static_assert(sizeof(Problem) == sizeof(tllm_linear_problem) + 16, "tllm_linear_problem, then the prologue");
 constexpr int kProblemSwigluGate = TLLM_PROBLEM_SWIGLU_GATE;
+
+// CU count of the current device, asked once per device (256 if the runtime cannot tell). Safe to
+// call from several host threads.
+inline int current_device_cus() {
+    static std::atomic<int> cache[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    int n = cache[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) n = 256;
+        cache[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
 
 __device__ __forceinline__ float h2f(uint16_t bits) {
     return (float)__builtin_bit_cast(_Float16, bits);

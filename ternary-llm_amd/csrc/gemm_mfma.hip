@@ -485,13 +485,7 @@ struct GemmConfig {
 // Estimate: (rounds of workgroups over the CUs) x (stages per workgroup) x (time of one stage,
 // measured: 1.19 / 0.70 us for 256 / 128 activation rows) + 5 us + the traffic of a split's exchange.
 GemmConfig choose_config(const Problem &p) {
-    static int cus[64] = {};
-    int dev = 0, n_cu = 256;
-    if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64) {
-        if (!cus[dev] && hipDeviceGetAttribute(&cus[dev], hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
-            cus[dev] = 0;
-        if (cus[dev] > 0) n_cu = cus[dev];
-    }
+    const int n_cu = current_device_cus();
     const int n_tiles = (p.rows + kBN - 1) / kBN, groups = p.cols / 128;
     const float stage_us[2] = {0.70f, 1.19f};
     GemmConfig best{0, 1, 0.f};

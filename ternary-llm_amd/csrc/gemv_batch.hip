@@ -352,17 +352,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
     }
 }
 
-int device_cus() {
-    static int cus[64] = {};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-    if (!cus[dev]) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) n = 256;
-        cus[dev] = n;
-    }
-    return cus[dev];
-}
+int device_cus() { return current_device_cus(); }
 
 }  // namespace
 
@@ -376,14 +366,14 @@ constexpr size_t kLdsBytes = 4 * kImageBytes + 2 * 2 * 16 * sizeof(float);
 
 template <int T>
 static hipError_t prepare_kernel() {
-    static bool done[64] = {};
+    static std::atomic<bool> done[64];  // per device; setting the attribute twice is harmless
     int dev = 0;
     if (hipError_t e = hipGetDevice(&dev)) return e;
-    if (dev < 0 || dev >= 64 || done[dev]) return hipSuccess;
+    if (dev < 0 || dev >= 64 || done[dev].load(std::memory_order_acquire)) return hipSuccess;
     if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemv_batch_kernel<T>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes))
         return e;
-    done[dev] = true;
+    done[dev].store(true, std::memory_order_release);
     return hipSuccess;
 }
 

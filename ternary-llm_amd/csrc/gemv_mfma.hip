@@ -21,6 +21,8 @@
 //   Tall (batch 1-4): 16 rows x 512 columns. Result column j is group j % 4 of batch column j / 4.
 #include <cstdio>
 #include <cstdlib>
+#include <mutex>
+
 #include "common.h"
 #include "gemv_layout.h"
 
@@ -654,11 +656,6 @@ struct DeviceInfo {
     int cus = 0;
 };
 
-DeviceInfo &device_info(int dev) {
-    static DeviceInfo info[64];
-    return info[dev < 0 || dev >= 64 ? 0 : dev];
-}
-
 constexpr int kLdsLimit = 64 * 1024;  // per workgroup; 160 KB per CU leaves room for two or three
 
 template <class G, bool kExtras = false, bool kFine = false>
@@ -666,26 +663,23 @@ const void *kernel_ptr() {
     return reinterpret_cast<const void *>(&gemv_mfma_kernel<G, kExtras, kFine>);
 }
 
+// Per device, once: the kernels may use up to kLdsLimit of dynamic LDS. Safe from several host threads.
 hipError_t prepare_device(DeviceInfo **out) {
+    static DeviceInfo info[64];
+    static std::atomic<bool> ready[64];
     int dev = 0;
     if (hipError_t e = hipGetDevice(&dev)) return e;
-    DeviceInfo &di = device_info(dev);
-    if (di.cus == 0) {
-        int n = 0;
-        if (hipError_t e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev)) return e;
-        if (hipError_t e = hipFuncSetAttribute(kernel_ptr<Wide>(), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit))
-            return e;
-        if (hipError_t e = hipFuncSetAttribute(kernel_ptr<Tall>(), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit))
-            return e;
-        if (hipError_t e = hipFuncSetAttribute(kernel_ptr<Wide, true>(), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit))
-            return e;
-        if (hipError_t e = hipFuncSetAttribute(kernel_ptr<Wide, false, true>(), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit))
-            return e;
-        if (hipError_t e = hipFuncSetAttribute(kernel_ptr<Wide, true, true>(), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit))
-            return e;
-        di.cus = n > 0 ? n : 256;
+    if (dev < 0 || dev >= 64) return hipErrorInvalidDevice;
+    if (!ready[dev].load(std::memory_order_acquire)) {
+        static std::mutex init_mutex;
+        std::lock_guard<std::mutex> lock(init_mutex);
+        for (const void *k : {kernel_ptr<Wide>(), kernel_ptr<Tall>(), kernel_ptr<Wide, true>(),
+                              kernel_ptr<Wide, false, true>(), kernel_ptr<Wide, true, true>()})
+            if (hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit)) return e;
+        info[dev].cus = current_device_cus();
+        ready[dev].store(true, std::memory_order_release);
     }
-    *out = &di;
+    *out = &info[dev];
     return hipSuccess;
 }
 

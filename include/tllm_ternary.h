@@ -33,7 +33,7 @@ enum {
     TLLM_ERR_BAD_GROUP = -3,    /* group_size < 32, group_size % 32 != 0 or cols % group_size != 0 */
     TLLM_ERR_TOO_LARGE = -4,    /* an element count does not fit the index type, or exceeds a stated limit */
     TLLM_ERR_ALIAS = -5,        /* output overlaps the activation input */
-    TLLM_ERR_BAD_PLAN = -6,     /* plan handle is NULL, or count < 1, or batch out of range */
+    TLLM_ERR_BAD_PLAN = -6,     /* plan handle is NULL, count < 1, batch out of range, or a pair / prologue rule is broken */
     TLLM_ERR_MISALIGNED = -7    /* masks/activations not 16-byte aligned, scales/outputs not 2-byte aligned */
 };
 

@@ -62,7 +62,7 @@ const char *tllm_error_string(int code) {
         case TLLM_ERR_BAD_GROUP: return "bad group_size: must be a multiple of 32 that divides cols";
         case TLLM_ERR_TOO_LARGE: return "size exceeds the supported maximum";
         case TLLM_ERR_ALIAS: return "output overlaps the activation input";
-        case TLLM_ERR_BAD_PLAN: return "invalid plan, problem count or batch";
+        case TLLM_ERR_BAD_PLAN: return "invalid plan: handle, problem count, batch, SwiGLU pair or RMSNorm prologue";
         case TLLM_ERR_MISALIGNED: return "pointer alignment: masks/activations need 16 bytes, fp16 arrays 2";
         case -8: return "file cannot be opened, is truncated, or a write failed";   // TLLM_ERR_IO
         case -9: return "not a .tllm file of a supported version, or a header field is out of range";  // TLLM_ERR_BAD_FILE

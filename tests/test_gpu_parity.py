@@ -96,7 +96,11 @@ def test_gemv_reference_test_recipe(dev, oracle, rows, cols):
     assert rel.max() < 1e-2 or err.max() < 1e-2
 
 
-@pytest.mark.parametrize("rows,cols", [(1, 128), (3, 256), (17, 384), (100, 1152), (65, 640), (1, 4096), (15, 128)])
+@pytest.mark.parametrize("rows,cols", [(1, 128), (3, 256), (17, 384), (100, 1152), (65, 640), (1, 4096), (15, 128),
+                                       # wide tiles in units of 16 rows: row counts that end inside a tile,
+                                       # a unit or a chunk, rows that are not whole slices of 2048 columns
+                                       (16, 2048), (17, 2048), (33, 4096), (100, 2048), (70, 6144), (16, 14336),
+                                       (50, 11008), (47, 2176), (49, 8192), (18433, 2048), (20000, 2048)])
 def test_gemv_ragged_shapes(dev, oracle, rows, cols):
     nz, sg, s, x = synth.problem(rows * 7 + cols, rows, cols, dontcare_sign=True)
     ref = oracle.gemv_f64(nz, sg, s.view(np.uint16), x.view(np.uint16))
@@ -537,7 +541,8 @@ def _rand_weight(torch, gen, rows, cols):
     return nz, sg, sc
 
 
-@pytest.mark.parametrize("rows,cols", [(14336, 4096), (8192, 2048), (100, 2048), (28672, 8192)])
+@pytest.mark.parametrize("rows,cols", [(14336, 4096), (8192, 2048), (100, 2048), (28672, 8192), (11008, 4096),
+                                       (4100, 11008), (17, 2048), (20000, 2048)])
 def test_swiglu_pair_vs_oracle_and_unfused(dev, oracle, rows, cols):
     """gate/up pair in one launch with the SiLU*mul epilogue: equal, bit for bit, to the two
     projections followed by the element-wise operator, and within tolerance of the fp64 evaluation

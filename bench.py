@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the ternary linear-layer hot path on one MI355X.
 
-Default workload (BASELINE config 3): the LLaMA-3-8B decode projection sweep at batch 1 -
+Default workload (benchmark configuration 3): the LLaMA-3-8B decode projection sweep at batch 1 -
 7 ternary GEMVs per layer (q, k, v, o, gate, up, down) x 32 layers, 1.854 GB of packed
 weights + scales resident in HBM, issued as ONE launch of the multi-problem plan. A "step" is
 one sweep. The metric is the packed weight+scale stream rate in GB/s (algorithmic bytes =

@@ -64,7 +64,7 @@ def assert_close(oracle, got, ref, tol=TOL, what=""):
 
 # -------------------------------------------------------------------- GEMV
 @pytest.mark.parametrize("rows,cols,seed", [
-    (2048, 2048, 101),    # BASELINE config 1 (LLaMA-1B q_proj)
+    (2048, 2048, 101),    # benchmark configuration 1 (LLaMA-1B q_proj)
     (512, 2048, 102),     # 1B k/v_proj
     (2048, 8192, 103),    # 1B down_proj
     (1024, 4096, 104),    # 8B k/v_proj

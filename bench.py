@@ -7,7 +7,7 @@ weights + scales resident in HBM, issued as ONE launch of the multi-problem plan
 one sweep. The metric is the packed weight+scale stream rate in GB/s (algorithmic bytes =
 0.265625 * rows * cols per matrix) and its fraction of the 8 TB/s HBM peak.
 
-Prints one JSON line; see README/DESIGN for the fields. `--gpus` above 1 is refused: this build
+Prints one JSON line (value, roofline, other_batches, gemm, cpu_baseline). `--gpus` above 1 is refused: this build
 measures one GPU.
 """
 import argparse

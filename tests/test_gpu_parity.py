@@ -785,6 +785,28 @@ def test_large_plan_in_a_captured_graph(dev, oracle):
     plan.close()
 
 
+def test_random_shapes_through_every_dispatch_path(dev, oracle):
+    """Sixty seeded random (rows, cols, group, batch) problems against the oracle: whichever kernel the
+    dispatcher picks (row-wave, tall, wide in 48- or 16-row units, batched decode, passes of it, the
+    matrix-core GEMM with or without split K), the result has to be the same function of its inputs."""
+    torch, tl = dev
+    rng = np.random.default_rng(20240611)
+    batches = [1, 1, 1, 2, 3, 4, 5, 8, 16, 17, 33, 70, 130]
+    for case in range(60):
+        group = int(rng.choice([128, 128, 128, 32, 64, 256]))
+        cols = group * int(rng.integers(1, 1 + (6144 if case % 3 else 12288) // group))
+        rows = int(rng.integers(1, 700 if case % 4 else 3000))
+        batch = int(rng.choice(batches))
+        nz, sg, s, _ = synth.problem(1000 + case, rows, cols, group=group, dontcare_sign=True)
+        A = synth.acts_f16(rng, batch, cols)
+        ref = oracle.gemm_f64(A.view(np.uint16), nz, sg, s.view(np.uint16), group)
+        if batch == 1:
+            got = run_gemv(dev, nz, sg, s, A[0], group)[None, :]
+        else:
+            got = run_gemm(dev, A, nz, sg, s, group)
+        assert_close(oracle, got, ref, what=f"case {case}: rows {rows} cols {cols} group {group} batch {batch}")
+
+
 # ---------------------------------------------- full-size, size-independent
 def test_full_size_properties_8b(dev, oracle):
     """LLaMA-3-8B gate_proj (14336 x 4096) at full size: sampled rows against the oracle, plus

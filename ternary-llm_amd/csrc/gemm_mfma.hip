@@ -496,8 +496,10 @@ GemmConfig choose_config(const Problem &p) {
             if (splits > 1 && (tiles * splits > n_cu || groups / splits < 4)) break;  // only to fill idle CUs
             const long wgs = tiles * splits;
             const float stages = (float)((groups + splits - 1) / splits * 2);
-            // the exchange writes and reads every fp32 partial tile once, at about 1.5 TB/s
-            const float exchange = splits > 1 ? 2.0f * (float)wgs * (float)(bm * kBN * 4) / 1.5e6f : 0.0f;
+            // the exchange: all workgroups write their fp32 tile at once (about 5.5 us with the
+            // hand-over), then the last one of a tile reads the `splits` slots on its own, at about
+            // 29 GB/s (fitted to 14336x4096 and 4096x14336 at M = 128: 10 us with 2, 23.5 us with 8)
+            const float exchange = splits > 1 ? 5.5f + (float)splits * (float)(bm * kBN * 4) / 29.0e3f : 0.0f;
             const float us = (float)((wgs + n_cu - 1) / n_cu) * stages * stage_us[c] + 5.0f + exchange;
             if (best.us == 0.f || us < best.us) best = GemmConfig{c, splits, us};
         }

@@ -45,6 +45,9 @@ __device__ __forceinline__ __attribute__((address_space(1))) const T *as_global(
 }
 
 constexpr int kNW = 4;  // waves per workgroup
+// Most slices of a row (wide tiles: 2048 columns each) whose operand image is in LDS at one time;
+// longer rows are staged and walked in segments. 8 slices = 32 KB keep three workgroups on a CU.
+constexpr int kSegSlices = 8;
 constexpr int kThreads = kNW * kWave;
 constexpr int kMaxBatch = 4;  // activation rows the tall tiles carry
 #ifndef TLLM_TILES_AHEAD
@@ -184,9 +187,12 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
         u_end = (int)((int64_t)total * (blockIdx.x + 1) / gridDim.x);
     }
 
-    int cur = -1;  // problem whose activations are staged
+    int cur = -1;      // problem whose activations are staged
+    int cur_seg = -1;  // and which segment of its columns
+    int cur_ex = 0;    // exponent of that problem's largest activation (rows staged in segments)
     Problem p = single;
     int slices = 0, groups = 0, words = 0, img_stride = 0;
+    int seg_lo = 0, seg_n = 0;  // slices of the staged segment
 
     __shared__ int pool_task;
     for (;;) {
@@ -211,15 +217,36 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
         const int n_units = min(min(u_end - u, first_unit + p_units - u), sc.max_units);
         const int task_first_row = (u - first_unit) * kUnitRows;
         u += n_units;
-        if (pi != cur) {
-            // ------------------------------------------------ stage the activations of problem pi
-            __syncthreads();  // every wave is done with the image of the problem before
+        const bool fresh = pi != cur;
+        if (fresh) {
             if (sc.table) p = sc.table[pi];
             cur = pi;
+            cur_seg = -1;
             words = p.cols / 32;
             groups = p.cols / kChunkCols;
             slices = (p.cols + G::kCols - 1) / G::kCols;
-            img_stride = slices * G::kCols;
+        }
+        // Rows longer than kSegSlices slices are staged and walked in segments of equal length, so
+        // that the operand image never takes more than kSegSlices slices of LDS (wide tiles only).
+        const int n_seg = G::kRows == 4 && !kFine ? (slices + kSegSlices - 1) / kSegSlices : 1;  // (the host never picks a fine instance for such rows)
+        const int seg_len = (slices + n_seg - 1) / n_seg;
+
+        const int r_begin = task_first_row;
+        const int r_end = min(p.rows, r_begin + n_units * kUnitRows);
+        const bool pair = kExtras && (p.flags & kProblemSwigluGate) != 0;
+        const size_t wave_stride = (size_t)(sc.max_units * kUnitRows) * sc.max_batch;
+        for (int mat = 0; mat < (pair ? 2 : 1); mat++) {
+            float *part = partial + (size_t)mat * sc.pair_stride + (size_t)wave * wave_stride;
+            for (int k = lane; k < n_units * kUnitRows * p.batch; k += kWave) part[k] = 0.0f;
+        }
+        for (int seg = 0; seg < n_seg; seg++) {
+        if (seg != cur_seg) {
+            // ------------------------------------------------ stage the activations of problem pi
+            __syncthreads();  // every wave is done with the image that was staged before
+            cur_seg = seg;
+            seg_lo = seg * seg_len;
+            seg_n = min(seg_len, slices - seg_lo);
+            img_stride = seg_n * G::kCols;
             // eight consecutive activations as fp16 bits; int8 values convert exactly
             auto load8 = [&](int b, int c8) -> uint4 {
                 if (!sc.x_is_i8) return reinterpret_cast<const uint4 *>(p.x + (size_t)b * p.cols)[c8];
@@ -237,7 +264,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
             // pieces are numbered in image order; piece_of() loads the activations of one.
             const int pieces = img_stride / 8;
             auto piece_of = [&](int b, int c8) -> uint4 {
-                const int slice = (c8 * 8) / G::kCols;
+                const int slice = seg_lo + (c8 * 8) / G::kCols;
                 const int chunk = ((c8 * 8) % G::kCols) / kChunkCols;
                 const int g = min(slice * G::kChunks, groups - G::kChunks) + chunk;
                 if (g < slice * G::kChunks) return uint4{0u, 0u, 0u, 0u};
@@ -295,7 +322,31 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
             int stid = tid;
             asm volatile("" : "+v"(stid));
             constexpr int kKeep = 8;  // pieces per thread that stay in registers between the two steps
-            if (p.batch == 1 && pieces <= kKeep * kThreads) {
+            if (n_seg > 1) {
+                // a segment of a long row: the exponent comes from a pass over the whole row, made
+                // once per problem; the segment itself is staged like a short row
+                if (fresh && seg == 0) {
+                    uint32_t m = 0;
+                    for (int c8 = stid; c8 < p.cols / 8; c8 += kThreads) m = magnitude(m, load8(0, c8));
+#pragma unroll
+                    for (int off = 32; off > 0; off >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, off, kWave));
+                    if (lane == 0) red_amax[wave][0] = m;
+                    __syncthreads();
+                    cur_ex = exponent_of(0);
+                }
+                uint4 keep[kKeep];
+#pragma unroll
+                for (int k = 0; k < kKeep; k++) {
+                    const int c8 = stid + k * kThreads;
+                    keep[k] = c8 < pieces ? piece_of(0, c8) : uint4{0u, 0u, 0u, 0u};
+                }
+#pragma unroll
+                for (int k = 0; k < kKeep; k++) {
+                    const int c8 = stid + k * kThreads;
+                    if (c8 < pieces) write_piece(image, c8, keep[k], cur_ex);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else if (p.batch == 1 && pieces <= kKeep * kThreads) {
                 // one pass over x: all loads are issued together and kept for the image
                 uint4 keep[kKeep];
                 uint32_t m = 0;
@@ -384,8 +435,6 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
             __syncthreads();
         }
 
-        const int r_begin = task_first_row;
-        const int r_end = min(p.rows, r_begin + n_units * kUnitRows);
         // The task's rows are cut into kNW chunks; a "walk" is one chunk under one slice (the B
         // operands stay put during a walk). Walks are numbered chunk-major, slice-minor and dealt to
         // the waves round-robin, so at any time the waves of a workgroup work on neighbouring
@@ -393,12 +442,11 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
         // scales) are fetched from HBM once and shared, not once per slice.
         // chunk size: a quarter of the rows that exist, rounded up to whole groups of kTilesAhead tiles
         const int chunk_rows = ((r_end - r_begin + kNW - 1) / kNW + kUnitRows / kNW - 1) / (kUnitRows / kNW) * (kUnitRows / kNW);
-        const int n_walks = kNW * slices;
-        const int my_walks = slices;  // walks wave, wave + kNW, ...
+        const int n_walks = kNW * seg_n;
+        const int my_walks = seg_n;  // walks wave, wave + kNW, ...
         // A SwiGLU pair (flag on the gate problem; the up problem follows it in the table, same shape
         // and activations, no units of its own) runs the walks twice over the same rows, with the same
         // operand image, into two partial-sum areas; the epilogue below joins them.
-        const bool pair = kExtras && (p.flags & kProblemSwigluGate) != 0;
         for (int mat = 0; mat < (pair ? 2 : 1); mat++) {
         const uint32_t *w_nz = p.nz, *w_sg = p.sg;
         const uint16_t *w_sc = p.scales;
@@ -407,8 +455,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
             w_sg = sc.table[pi + 1].sg;
             w_sc = sc.table[pi + 1].scales;
         }
-        float *my_part = partial + (size_t)mat * sc.pair_stride + (size_t)wave * (sc.max_units * kUnitRows) * sc.max_batch;
-        for (int k = lane; k < n_units * kUnitRows * p.batch; k += kWave) my_part[k] = 0.0f;
+        float *my_part = partial + (size_t)mat * sc.pair_stride + (size_t)wave * wave_stride;
 
         // ---- which operand lanes are live, and what each lane loads
         int bcol;       // batch column of this lane's D column
@@ -450,7 +497,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
         auto load_tile = [&](int slice, int rb) -> Tile<G> {
             Tile<G> t;
             const int rbe = min(rb, p.rows - G::kRows);
-            const int c0 = min(slice * G::kChunks, groups - G::kChunks);
+            const int c0 = min((seg_lo + slice) * G::kChunks, groups - G::kChunks);
             const size_t base_a = ((size_t)rbe * words + (size_t)c0 * 4) * 4;
             const size_t base_s = ((size_t)rbe * groups + c0) * 2;
             t.nz = *reinterpret_cast<const GU4 *>(nz_g + base_a + lane_a);
@@ -476,7 +523,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
             auto next_load = [&]() -> Tile<G> {
                 // past the last walk the cursor parks on the wave's last tile
                 const int w_ = min(l_walk, n_walks - kNW + wave);
-                const int c = w_ / slices, sl = w_ - c * slices;
+                const int c = w_ / seg_n, sl = w_ - c * seg_n;
                 const int live_tiles = max(chunk_tiles(c), 1);
                 const Tile<G> t = load_tile(sl, r_begin + c * chunk_rows + min(l_slot, live_tiles - 1) * G::kRows);
                 if (++l_slot == n_slots) { l_slot = 0; l_walk += kNW; }
@@ -557,7 +604,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                         if (t0 + k < total) {
                             if (j == 0) {
                                 const int walk = wave + wi * kNW;
-                                const int chunk = walk / slices, slice = walk - chunk * slices;
+                                const int chunk = walk / seg_n, slice = walk - chunk * seg_n;
                                 c_begin = r_begin + chunk * chunk_rows;
                                 n_rb = chunk_tiles(chunk);
                                 load_operands(slice, B, bias, bias_sel);
@@ -575,7 +622,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
             } else
             for (int wi = 0; wi < my_walks; wi++) {
                 const int walk = wave + wi * kNW;
-                const int chunk = walk / slices, slice = walk - chunk * slices;
+                const int chunk = walk / seg_n, slice = walk - chunk * seg_n;
                 const int c_begin = r_begin + chunk * chunk_rows;
                 const int n_rb = chunk_tiles(chunk);  // live tiles of this walk (0: nothing to add)
                 // this slice's activations become the B operands. Every lane reads (no branch): the
@@ -610,6 +657,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
             }
         }
         }  // matrices of the task
+        }  // segments of the row
         // last task of the span, or a pool task: ask for the next pool task now (not earlier: a
         // request is a claim, and a workgroup must not claim work long before it can start it); the
         // answer arrives while the partial sums are added up
@@ -620,7 +668,6 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
         // ------------------------------------------------ add the waves' partial sums in wave order, store fp16
         {
             const int nrows = r_end - r_begin;
-            const size_t wave_stride = (size_t)(sc.max_units * kUnitRows) * sc.max_batch;
             for (int idx = tid; idx < nrows * p.batch; idx += kThreads) {
                 const int b = idx / nrows, rl = idx - b * nrows;
                 float sum = 0.0f;
@@ -703,7 +750,12 @@ bool wants_fine(int64_t coarse_units, int slots) { return coarse_units * 2 <= sl
 
 template <class G>
 int image_bytes_of(int cols, int batch) {
-    return (cols + G::kCols - 1) / G::kCols * G::kCols * 2 * batch;
+    int slices = (cols + G::kCols - 1) / G::kCols;
+    if (G::kRows == 4) {  // wide tiles: long rows are staged in equal segments of at most kSegSlices
+        const int n_seg = (slices + kSegSlices - 1) / kSegSlices;
+        slices = (slices + n_seg - 1) / n_seg;
+    }
+    return slices * G::kCols * 2 * batch;
 }
 
 // Geometry limits: a tile must fit inside the matrix (edge tiles are moved back, not clipped).
@@ -802,7 +854,8 @@ static hipError_t launch_single(const Problem &p, bool x_is_i8, float i8_scale, 
     const bool wide = wide_ok(p);
     sc.image_bytes = wide ? image_bytes_of<Wide>(p.cols, 1) : image_bytes_of<Tall>(p.cols, p.batch);
     const int wgs = (wide ? Wide::kWgPerCu : Tall::kWgPerCu) * di->cus;
-    const bool fine = wide && wants_fine((p.rows + range_unit<Wide>() - 1) / range_unit<Wide>(), wgs);
+    const bool fine = wide && p.cols <= kSegSlices * Wide::kCols &&
+                      wants_fine((p.rows + range_unit<Wide>() - 1) / range_unit<Wide>(), wgs);
     const int unit = fine ? kFineUnit : wide ? range_unit<Wide>() : range_unit<Tall>();
     sc.max_units = max_units_for(sc.image_bytes, p.batch, unit);
     sc.max_batch = p.batch;
@@ -1003,10 +1056,13 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
         }
         if (d.wide) {  // decode-size plans: fine-grained units
             int64_t coarse = 0;
-            for (size_t i = 0; i < host.size(); i++)
+            bool segmented = false;  // rows staged in segments: the coarse instances only
+            for (size_t i = 0; i < host.size(); i++) {
+                segmented = segmented || host[i].cols > kSegSlices * Wide::kCols;
                 if (!(i > 0 && (host[i - 1].flags & kProblemSwigluGate)))
                     coarse += (host[i].rows + range_unit<Wide>() - 1) / range_unit<Wide>();
-            d.fine = wants_fine(coarse, Wide::kWgPerCu * di->cus);
+            }
+            d.fine = !segmented && wants_fine(coarse, Wide::kWgPerCu * di->cus);
         }
         const int unit = d.fine ? kFineUnit : d.wide ? range_unit<Wide>() : range_unit<Tall>();
         const int mats = has_pairs ? 2 : 1;

@@ -107,6 +107,61 @@ def test_gemv_ragged_shapes(dev, oracle, rows, cols):
     assert_close(oracle, run_gemv(dev, nz, sg, s, x), ref, what=f"gemv {rows}x{cols}")
 
 
+@pytest.mark.parametrize("rows,cols", [(64, 28672), (3000, 18432), (200, 16512), (96, 57344), (50, 36992),
+                                       (2100, 28672), (16, 16384 + 2048)])
+def test_gemv_rows_staged_in_segments(dev, oracle, rows, cols):
+    """Rows longer than eight slices of 2048 columns: the operand image holds one segment of the row
+    at a time (whole and ragged last slices, one and several tasks per workgroup, up to four segments)."""
+    nz, sg, s, x = synth.problem(rows * 3 + cols, rows, cols, dontcare_sign=True)
+    ref = oracle.gemv_f64(nz, sg, s.view(np.uint16), x.view(np.uint16))
+    assert_close(oracle, run_gemv(dev, nz, sg, s, x), ref, what=f"gemv {rows}x{cols}")
+
+
+def test_plan_mixing_segmented_and_short_rows(dev, oracle):
+    """One plan with long rows (two and three segments), short rows and a SwiGLU pair over long rows;
+    several tasks per problem, so segments are restaged between tasks of one problem."""
+    torch, tl = dev
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(77)
+    shapes = [(5000, 28672), (1024, 4096), (2500, 36864), (4096, 2048), (700, 18560)]
+    problems, keep = [], []
+    for rows, cols in shapes:
+        w = _rand_weight(torch, gen, rows, cols)
+        x = torch.randn((1, cols), device="cuda", generator=gen).to(torch.float16)
+        y = torch.full((1, rows), float("nan"), dtype=torch.float16, device="cuda")
+        problems.append((*w, x, y, rows, cols, 1))
+        keep.append((w, x, y))
+    rows, cols = 3000, 20480
+    g_w, u_w = _rand_weight(torch, gen, rows, cols), _rand_weight(torch, gen, rows, cols)
+    xp = torch.randn((1, cols), device="cuda", generator=gen).to(torch.float16)
+    fused = torch.full((1, rows), float("nan"), dtype=torch.float16, device="cuda")
+    problems += [(*g_w, xp, fused, rows, cols, 1, tl.SWIGLU_GATE), (*u_w, xp, None, rows, cols, 1)]
+    plan = tl.LinearPlan(problems)
+    for _ in range(2):  # the second launch finds the counters as the first one left them
+        plan.launch()
+    torch.cuda.synchronize()
+    pick_rng = np.random.default_rng(5)
+    for (w, x, y), (r, c) in zip(keep, shapes):
+        single = torch.zeros(r, dtype=torch.float16, device="cuda")
+        tl.ternary_gemv(*w, x, single, r, c, 128)
+        torch.cuda.synchronize()
+        assert torch.isfinite(y).all()
+        pick = pick_rng.integers(0, r, 96)
+        ref = oracle.gemv_f64(w[0][pick].cpu().numpy().view(np.uint32), w[1][pick].cpu().numpy().view(np.uint32),
+                              w[2][pick].cpu().numpy().view(np.uint16), x[0].cpu().numpy().view(np.uint16))
+        assert_close(oracle, y[0][pick].cpu().numpy().astype(np.float64), ref, what=f"plan {r}x{c}")
+        assert_close(oracle, single[pick].cpu().numpy().astype(np.float64), ref, what=f"single {r}x{c}")
+    g = torch.zeros(rows, dtype=torch.float16, device="cuda")
+    u = torch.zeros(rows, dtype=torch.float16, device="cuda")
+    tl.ternary_gemv(*g_w, xp, g, rows, cols, 128)
+    tl.ternary_gemv(*u_w, xp, u, rows, cols, 128)
+    unfused = torch.empty_like(g)
+    tl.silu_mul(g, u, unfused, rows)
+    torch.cuda.synchronize()
+    assert torch.equal(fused[0].view(torch.int16), unfused.view(torch.int16))
+    plan.close()
+
+
 def test_gemv_special_matrices(dev, oracle):
     rng = np.random.default_rng(5)
     cols = 1024

@@ -228,7 +228,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
         }
         // Rows longer than kSegSlices slices are staged and walked in segments of equal length, so
         // that the operand image never takes more than kSegSlices slices of LDS (wide tiles only).
-        const int n_seg = G::kRows == 4 && !kFine ? (slices + kSegSlices - 1) / kSegSlices : 1;  // (the host never picks a fine instance for such rows)
+        const int n_seg = G::kRows == 4 && !kFine ? (slices + kSegSlices - 1) / kSegSlices : 1;  // (fine-grained instances: whole rows, the host sees to it that they fit)
         const int seg_len = (slices + n_seg - 1) / n_seg;
 
         const int r_begin = task_first_row;
@@ -749,9 +749,9 @@ constexpr int kFineUnit = kNW * Wide::kRows;  // rows of a unit of the fine-grai
 bool wants_fine(int64_t coarse_units, int slots) { return coarse_units * 2 <= slots; }
 
 template <class G>
-int image_bytes_of(int cols, int batch) {
+int image_bytes_of(int cols, int batch, bool segmented = true) {
     int slices = (cols + G::kCols - 1) / G::kCols;
-    if (G::kRows == 4) {  // wide tiles: long rows are staged in equal segments of at most kSegSlices
+    if (G::kRows == 4 && segmented) {  // wide tiles: long rows are staged in equal segments of at most kSegSlices
         const int n_seg = (slices + kSegSlices - 1) / kSegSlices;
         slices = (slices + n_seg - 1) / n_seg;
     }
@@ -852,11 +852,12 @@ static hipError_t launch_single(const Problem &p, bool x_is_i8, float i8_scale, 
     sc.table = nullptr;
     sc.count = 1;
     const bool wide = wide_ok(p);
-    sc.image_bytes = wide ? image_bytes_of<Wide>(p.cols, 1) : image_bytes_of<Tall>(p.cols, p.batch);
     const int wgs = (wide ? Wide::kWgPerCu : Tall::kWgPerCu) * di->cus;
-    const bool fine = wide && p.cols <= kSegSlices * Wide::kCols &&
+    // the fine-grained instances keep the whole row in LDS: possible while it fits
+    const bool fine = wide && image_bytes_of<Wide>(p.cols, 1, false) + kNW * kFineUnit * 4 <= kLdsLimit &&
                       wants_fine((p.rows + range_unit<Wide>() - 1) / range_unit<Wide>(), wgs);
     const int unit = fine ? kFineUnit : wide ? range_unit<Wide>() : range_unit<Tall>();
+    sc.image_bytes = wide ? image_bytes_of<Wide>(p.cols, 1, !fine) : image_bytes_of<Tall>(p.cols, p.batch);
     sc.max_units = max_units_for(sc.image_bytes, p.batch, unit);
     sc.max_batch = p.batch;
     const int units = (p.rows + unit - 1) / unit;
@@ -1050,19 +1051,20 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
     } else {
         d.wide = all_wide;
         d.use_mfma = d.extras ? all_wide : all_wide || all_tall;
-        for (const Problem &p : host) {
-            const int ib = d.wide ? image_bytes_of<Wide>(p.cols, 1) : image_bytes_of<Tall>(p.cols, p.batch);
-            max_image = ib > max_image ? ib : max_image;
-        }
         if (d.wide) {  // decode-size plans: fine-grained units
             int64_t coarse = 0;
-            bool segmented = false;  // rows staged in segments: the coarse instances only
+            int whole = 0;  // largest image of a whole row: the fine-grained instances do not stage in segments
             for (size_t i = 0; i < host.size(); i++) {
-                segmented = segmented || host[i].cols > kSegSlices * Wide::kCols;
+                whole = std::max(whole, image_bytes_of<Wide>(host[i].cols, 1, false));
                 if (!(i > 0 && (host[i - 1].flags & kProblemSwigluGate)))
                     coarse += (host[i].rows + range_unit<Wide>() - 1) / range_unit<Wide>();
             }
-            d.fine = !segmented && wants_fine(coarse, Wide::kWgPerCu * di->cus);
+            d.fine = whole + kNW * kFineUnit * 4 * (has_pairs ? 2 : 1) <= kLdsLimit &&
+                     wants_fine(coarse, Wide::kWgPerCu * di->cus);
+        }
+        for (const Problem &p : host) {
+            const int ib = d.wide ? image_bytes_of<Wide>(p.cols, 1, !d.fine) : image_bytes_of<Tall>(p.cols, p.batch);
+            max_image = ib > max_image ? ib : max_image;
         }
         const int unit = d.fine ? kFineUnit : d.wide ? range_unit<Wide>() : range_unit<Tall>();
         const int mats = has_pairs ? 2 : 1;

@@ -108,7 +108,7 @@ def test_gemv_ragged_shapes(dev, oracle, rows, cols):
 
 
 @pytest.mark.parametrize("rows,cols", [(64, 28672), (3000, 18432), (200, 16512), (96, 57344), (50, 36992),
-                                       (2100, 28672), (16, 16384 + 2048)])
+                                       (2100, 28672), (16, 16384 + 2048), (20000, 18432)])
 def test_gemv_rows_staged_in_segments(dev, oracle, rows, cols):
     """Rows longer than eight slices of 2048 columns: the operand image holds one segment of the row
     at a time (whole and ragged last slices, one and several tasks per workgroup, up to four segments)."""

@@ -89,4 +89,33 @@ inline void silu_mul_forward(const half *gate, const half *up, half *output, int
                              reinterpret_cast<uint16_t *>(output), size, stream));
 }
 
+// Reference include/kernels.cuh:50-53.
+inline void rope_forward(half *q, half *k, int batch, int seq_len, int n_heads, int n_kv_heads, int head_dim,
+                         int start_pos, float theta, hipStream_t stream = 0) {
+    report("rope_forward", tllm_rope_f16(reinterpret_cast<uint16_t *>(q), reinterpret_cast<uint16_t *>(k), batch, seq_len,
+                                         n_heads, n_kv_heads, head_dim, start_pos, theta, stream));
+}
+
+// Reference include/kernels.cuh:64-66.
+inline void add_forward(const half *a, const half *b, half *output, int size, hipStream_t stream = 0) {
+    report("add_forward", tllm_add_f16(reinterpret_cast<const uint16_t *>(a), reinterpret_cast<const uint16_t *>(b),
+                                       reinterpret_cast<uint16_t *>(output), size, stream));
+}
+
+// Reference include/kernels.cuh:68-70.
+inline void embedding_lookup(const half *table, const int *indices, half *output, int n_tokens, int dim,
+                             hipStream_t stream = 0) {
+    report("embedding_lookup", tllm_embedding_lookup_f16(reinterpret_cast<const uint16_t *>(table), indices,
+                                                         reinterpret_cast<uint16_t *>(output), n_tokens, dim, stream));
+}
+
+// Reference include/kernels.cuh:72-76.
+inline void copy_to_kv_cache(const half *k, const half *v, half *k_cache, half *v_cache, int batch, int n_kv_heads,
+                             int head_dim, int seq_len, int start_pos, int max_seq_len, hipStream_t stream = 0) {
+    report("copy_to_kv_cache",
+           tllm_copy_to_kv_cache_f16(reinterpret_cast<const uint16_t *>(k), reinterpret_cast<const uint16_t *>(v),
+                                     reinterpret_cast<uint16_t *>(k_cache), reinterpret_cast<uint16_t *>(v_cache), batch,
+                                     n_kv_heads, head_dim, seq_len, start_pos, max_seq_len, stream));
+}
+
 }  // namespace ternary

@@ -115,6 +115,45 @@ int tllm_silu_mul_f16(const uint16_t *gate, const uint16_t *up, uint16_t *output
                       tllm_stream_t stream);
 
 /*
+ * output[i] = a[i] + b[i], one correctly rounded fp16 addition per element; output may be a or b.
+ * Replaces ternary::add_forward, reference include/kernels.cuh:64-66 (kernels/elementwise.cu:18-48),
+ * the residual add of src/transformer.cpp.
+ */
+int tllm_add_f16(const uint16_t *a, const uint16_t *b, uint16_t *output, int size, tllm_stream_t stream);
+
+/*
+ * Rotary position embedding, in place: q is fp16 [batch, seq_len, n_heads, head_dim], k is
+ * [batch, seq_len, n_kv_heads, head_dim]; the pair (2i, 2i+1) of every head of token (b, s) is
+ * rotated by the angle (start_pos + s) * theta^(-2i / head_dim):
+ *   (x0, x1) -> (x0 cos - x1 sin, x0 sin + x1 cos), fp32 arithmetic, fp16 store.
+ * head_dim must be even. The angle, its sine and cosine are evaluated in fp64 and rounded to fp32
+ * (the reference evaluates them in fp32, which leaves the angle off by up to pos * 2^-23 rad).
+ * Replaces ternary::rope_forward, reference include/kernels.cuh:50-53 (kernels/rope.cu:22-104).
+ */
+int tllm_rope_f16(uint16_t *q, uint16_t *k, int batch, int seq_len, int n_heads, int n_kv_heads,
+                  int head_dim, int start_pos, float theta, tllm_stream_t stream);
+
+/*
+ * output[t, :] = table[indices[t], :] for t < n_tokens; rows of dim fp16 values, indices are int32
+ * on the device and are not range-checked (the operator does not know the table's height).
+ * Replaces ternary::embedding_lookup, reference include/kernels.cuh:68-70
+ * (kernels/elementwise.cu:54-89).
+ */
+int tllm_embedding_lookup_f16(const uint16_t *table, const int32_t *indices, uint16_t *output,
+                              int n_tokens, int dim, tllm_stream_t stream);
+
+/*
+ * Copies the new rows k, v [batch, seq_len, n_kv_heads, head_dim] into the caches
+ * [batch, n_kv_heads, max_seq_len, head_dim] at positions start_pos .. start_pos + seq_len - 1;
+ * positions at or beyond max_seq_len are dropped, as in the reference.
+ * Replaces ternary::copy_to_kv_cache, reference include/kernels.cuh:72-76
+ * (kernels/elementwise.cu:97-147).
+ */
+int tllm_copy_to_kv_cache_f16(const uint16_t *k, const uint16_t *v, uint16_t *k_cache,
+                              uint16_t *v_cache, int batch, int n_kv_heads, int head_dim,
+                              int seq_len, int start_pos, int max_seq_len, tllm_stream_t stream);
+
+/*
  * Several independent ternary linears in ONE launch (e.g. q/k/v, gate/up, or a whole
  * back-to-back projection sweep). Each problem is what one tllm_ternary_gemv_f16 /
  * small-M tllm_ternary_gemm_f16 call would take: input fp16 [batch, cols],

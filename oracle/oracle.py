@@ -63,7 +63,9 @@ def load():
     L.tllm_oracle_rmsnorm_f64.argtypes = [_u16p, _u16p, C.c_void_p, C.c_void_p, _f64p, C.c_int, C.c_int,
                                           C.c_float]
     L.tllm_oracle_silu_mul_f64.argtypes = [_u16p, _u16p, _f64p, C.c_int]
-    for f in ("rmsnorm_f64", "silu_mul_f64", "pack", "unpack", "gemv_f64", "gemv_hostloop", "gemv_hostloop_mt", "gemm_f64",
+    L.tllm_oracle_add_f64.argtypes = [_u16p, _u16p, _f64p, C.c_int]
+    L.tllm_oracle_rope_f64.argtypes = [_u16p, _f64p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_double]
+    for f in ("add_f64", "rope_f64", "rmsnorm_f64", "silu_mul_f64", "pack", "unpack", "gemv_f64", "gemv_hostloop", "gemv_hostloop_mt", "gemm_f64",
               "gemm_f32_elem", "quantize_i8", "gemv_i8_f64", "ternarize"):
         getattr(L, "tllm_oracle_" + f).restype = None
     _lib = L
@@ -173,6 +175,41 @@ def silu_mul_f64(gate, up):
     out = np.empty(gate.size, np.float64)
     load().tllm_oracle_silu_mul_f64(gate, up, out, gate.size)
     return out
+
+
+def add_f64(a, b):
+    a, b = _c(a, np.uint16).reshape(-1), _c(b, np.uint16).reshape(-1)
+    out = np.empty(a.size, np.float64)
+    load().tllm_oracle_add_f64(a, b, out, a.size)
+    return out
+
+
+def rope_f64(x, batch, seq_len, heads, head_dim, start_pos, theta):
+    """x: fp16 bits [batch, seq_len, heads, head_dim] -> rotated values, float64, same shape
+    (reference kernels/rope.cu:22-80; q and k are rotated alike, each with its own head count)."""
+    x = _c(x, np.uint16)
+    assert x.size == batch * seq_len * heads * head_dim and head_dim % 2 == 0
+    out = np.empty(x.size, np.float64)
+    load().tllm_oracle_rope_f64(x.reshape(-1), out, batch, seq_len, heads, head_dim, start_pos, float(theta))
+    return out.reshape(batch, seq_len, heads, head_dim)
+
+
+def embedding_lookup(table, indices):
+    """Rows of `table` picked by `indices` (reference kernels/elementwise.cu:54-89)."""
+    return np.asarray(table)[np.asarray(indices, dtype=np.int64)]
+
+
+def copy_to_kv_cache(k, v, k_cache, v_cache, start_pos):
+    """Returns the caches [batch, n_kv_heads, max_seq_len, head_dim] after rows k, v
+    [batch, seq_len, n_kv_heads, head_dim] went in at start_pos; positions past the cache are
+    dropped (reference kernels/elementwise.cu:97-147)."""
+    k_cache, v_cache = np.array(k_cache, copy=True), np.array(v_cache, copy=True)
+    seq_len, max_seq = k.shape[1], k_cache.shape[2]
+    n = max(0, min(seq_len, max_seq - start_pos))
+    if n:
+        k_cache[:, :, start_pos:start_pos + n, :] = np.transpose(np.asarray(k)[:, :n], (0, 2, 1, 3))
+        v_cache[:, :, start_pos:start_pos + n, :] = np.transpose(np.asarray(v)[:, :n], (0, 2, 1, 3))
+    return k_cache, v_cache
 
 
 def ternarize(w, group=128, factor=0.7):

@@ -18,6 +18,10 @@
  *   tllm_oracle_ternarize ....... ternarize/pack.py:41-101
  *   tllm_oracle_rmsnorm_f64 ..... kernels/rmsnorm.cu:20-106
  *   tllm_oracle_silu_mul_f64 .... kernels/activations.cu:18-59
+ *   tllm_oracle_add_f64 ......... kernels/elementwise.cu:18-48
+ *   tllm_oracle_rope_f64 ........ kernels/rope.cu:22-80
+ *   (embedding_lookup and copy_to_kv_cache, kernels/elementwise.cu:54-147, are pure row copies;
+ *    their restatement is numpy indexing in oracle.py)
  *
  * Pinning status (what each function is checked against in tests/test_oracle.py):
  *   pack/unpack ........ the known-answer words of tests/test_packing.py:55-81
@@ -44,6 +48,18 @@
  *                        restatement through np.linalg.norm.
  *   silu_mul_f64 ....... closed forms (silu(0)=0, silu(g)-silu(-g)=g, g>>0 -> g*u) and
  *                        scipy.special.expit.
+ *   add_f64 ............ exact by construction (the sum of two binary16 values is exact in
+ *                        binary64); checked against numpy float16 addition.
+ *   rope_f64 ........... the reference holds no test or fixture for it; pinned by closed forms
+ *                        (position 0 -> identity; theta = 1 -> every pair turns by `pos` radians,
+ *                        against math.cos/sin; the pair (1, 0) becomes (cos, sin): sign and
+ *                        interleaved pair layout; pair norms are preserved; start_pos + seq index
+ *                        composes; the angle of pair i is pos * theta^(-2i/head_dim) against a
+ *                        complex-exponential numpy restatement; q heads past n_kv_heads leave k
+ *                        untouched). The reference evaluates the angle in fp32; the oracle is the
+ *                        exact-angle rotation, from which the reference itself is off by up to
+ *                        pos * 2^-23 rad.
+ *   embedding / kv copy  index arithmetic checked by brute-force Python loops on small cases.
  */
 #include <math.h>
 #include <pthread.h>
@@ -361,6 +377,33 @@ void tllm_oracle_silu_mul_f64(const uint16_t *gate, const uint16_t *up, double *
         double g = (double)tllm_oracle_half_to_float(gate[i]);
         double u = (double)tllm_oracle_half_to_float(up[i]);
         out[i] = g / (1.0 + exp(-g)) * u;
+    }
+}
+
+/* out = a + b, exact. */
+void tllm_oracle_add_f64(const uint16_t *a, const uint16_t *b, double *out, int n) {
+    for (int i = 0; i < n; i++)
+        out[i] = (double)tllm_oracle_half_to_float(a[i]) + (double)tllm_oracle_half_to_float(b[i]);
+}
+
+/* Rotary embedding of x [tokens = batch * seq_len, heads, head_dim] (fp16 bits) into out (fp64,
+ * unrounded): pair (2i, 2i+1) of every head of token t turns by (start_pos + t % seq_len) *
+ * theta^(-2i / head_dim). */
+void tllm_oracle_rope_f64(const uint16_t *x, double *out, int batch, int seq_len, int heads, int head_dim,
+                          int start_pos, double theta) {
+    for (int64_t t = 0; t < (int64_t)batch * seq_len; t++) {
+        const double pos = (double)(start_pos + (int)(t % seq_len));
+        for (int h = 0; h < heads; h++) {
+            const int64_t base = (t * heads + h) * head_dim;
+            for (int i = 0; i < head_dim / 2; i++) {
+                const double angle = pos / pow(theta, (2.0 * i) / (double)head_dim);
+                const double c = cos(angle), s = sin(angle);
+                const double x0 = (double)tllm_oracle_half_to_float(x[base + 2 * i]);
+                const double x1 = (double)tllm_oracle_half_to_float(x[base + 2 * i + 1]);
+                out[base + 2 * i] = x0 * c - x1 * s;
+                out[base + 2 * i + 1] = x0 * s + x1 * c;
+            }
+        }
     }
 }
 

@@ -7,10 +7,14 @@ from .ops import (  # noqa: F401
     SWIGLU_GATE,
     ModelFile,
     TllmError,
+    add,
+    copy_to_kv_cache,
+    embedding_lookup,
     lib,
     lib_path,
     quantize_absmax_int8,
     rmsnorm,
+    rope,
     silu_mul,
     ternary_gemm,
     ternary_gemv,

@@ -143,6 +143,43 @@ int tllm_silu_mul_f16(const uint16_t *gate, const uint16_t *up, uint16_t *output
     return (int)tllm::launch_silu_mul(gate, up, output, size, (hipStream_t)stream);
 }
 
+int tllm_add_f16(const uint16_t *a, const uint16_t *b, uint16_t *output, int size, tllm_stream_t stream) {
+    if (!a || !b || !output) return TLLM_ERR_NULL_POINTER;
+    if (size < 1) return TLLM_ERR_BAD_SHAPE;
+    return (int)tllm::launch_add(a, b, output, size, (hipStream_t)stream);
+}
+
+int tllm_rope_f16(uint16_t *q, uint16_t *k, int batch, int seq_len, int n_heads, int n_kv_heads, int head_dim,
+                  int start_pos, float theta, tllm_stream_t stream) {
+    if (!q || !k) return TLLM_ERR_NULL_POINTER;
+    if (batch < 1 || seq_len < 1 || n_heads < 1 || n_kv_heads < 1 || head_dim < 2 || head_dim % 2 || start_pos < 0 ||
+        !(theta > 0.0f))
+        return TLLM_ERR_BAD_SHAPE;
+    const long long heads = n_heads > n_kv_heads ? n_heads : n_kv_heads;
+    if ((long long)batch * seq_len * heads * head_dim >= (1ll << 40) || (long long)start_pos + seq_len > INT32_MAX)
+        return TLLM_ERR_BAD_SHAPE;
+    if (((uintptr_t)q | (uintptr_t)k) & 3) return TLLM_ERR_MISALIGNED;
+    return (int)tllm::launch_rope(q, k, batch, seq_len, n_heads, n_kv_heads, head_dim, start_pos, theta, (hipStream_t)stream);
+}
+
+int tllm_embedding_lookup_f16(const uint16_t *table, const int32_t *indices, uint16_t *output, int n_tokens, int dim,
+                              tllm_stream_t stream) {
+    if (!table || !indices || !output) return TLLM_ERR_NULL_POINTER;
+    if (n_tokens < 1 || dim < 1) return TLLM_ERR_BAD_SHAPE;
+    return (int)tllm::launch_embedding_lookup(table, indices, output, n_tokens, dim, (hipStream_t)stream);
+}
+
+int tllm_copy_to_kv_cache_f16(const uint16_t *k, const uint16_t *v, uint16_t *k_cache, uint16_t *v_cache, int batch,
+                              int n_kv_heads, int head_dim, int seq_len, int start_pos, int max_seq_len,
+                              tllm_stream_t stream) {
+    if (!k || !v || !k_cache || !v_cache) return TLLM_ERR_NULL_POINTER;
+    if (batch < 1 || batch > 65535 || n_kv_heads < 1 || n_kv_heads > 65535 || head_dim < 1 || seq_len < 1 ||
+        start_pos < 0 || max_seq_len < 1 || (long long)start_pos + seq_len > INT32_MAX)
+        return TLLM_ERR_BAD_SHAPE;
+    return (int)tllm::launch_copy_to_kv_cache(k, v, k_cache, v_cache, batch, n_kv_heads, head_dim, seq_len, start_pos,
+                                              max_seq_len, (hipStream_t)stream);
+}
+
 static int create_plan(tllm_linear_plan **plan, const tllm_linear_problem *problems,
                        const uint16_t *const *norm_weights, float eps, int count, int group_size) {
     if (!plan || !problems) return TLLM_ERR_NULL_POINTER;

@@ -73,6 +73,14 @@ hipError_t launch_quantize_absmax_i8(const uint16_t *x, int8_t *q, float *scale,
 hipError_t launch_rmsnorm(const uint16_t *input, const uint16_t *weight, uint16_t *output, const uint16_t *residual,
                           uint16_t *residual_out, int batch, int dim, float eps, hipStream_t s);
 hipError_t launch_silu_mul(const uint16_t *gate, const uint16_t *up, uint16_t *output, int size, hipStream_t s);
+hipError_t launch_add(const uint16_t *a, const uint16_t *b, uint16_t *output, int size, hipStream_t s);
+hipError_t launch_rope(uint16_t *q, uint16_t *k, int batch, int seq_len, int n_heads, int n_kv_heads, int head_dim,
+                       int start_pos, float theta, hipStream_t s);
+hipError_t launch_embedding_lookup(const uint16_t *table, const int *indices, uint16_t *output, int n_tokens, int dim,
+                                   hipStream_t s);
+hipError_t launch_copy_to_kv_cache(const uint16_t *k, const uint16_t *v, uint16_t *k_cache, uint16_t *v_cache, int batch,
+                                   int n_kv_heads, int head_dim, int seq_len, int start_pos, int max_seq_len,
+                                   hipStream_t s);
 
 // 128-group MFMA GEMV, batch 1..4 (gemv_mfma.hip).
 bool gemv_mfma_supports(const Problem &p, int group);

@@ -1,7 +1,8 @@
-// The two decode-step element-wise operators that sit directly around the ternary linears: RMSNorm
-// (with the optional fused residual add) in front of every projection group and SiLU(gate) * up
-// between the FFN projections. Both are bandwidth-trivial (a few KB per token); fp32 arithmetic,
-// fp16 in and out, as the reference's kernels.
+// The decode-step element-wise operators around the ternary linears: RMSNorm (with the optional
+// fused residual add) in front of every projection group, SiLU(gate) * up between the FFN
+// projections, the residual add, rotary position embedding of q and k, the embedding row lookup and
+// the copy of new k/v rows into the cache. All are bandwidth-trivial (a few KB per token); fp16 in
+// and out, arithmetic as the reference's kernels unless a comment says otherwise.
 #include "common.h"
 
 namespace tllm {
@@ -142,7 +143,128 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t *gate, con
     if (i < size) output[i] = silu_mul_one(gate[i], up[i]);
 }
 
+// Reference kernels/elementwise.cu:18-48: out = a + b in fp16 (one correctly rounded fp16 addition per
+// element, what __hadd / __hadd2 give). Eight elements per lane through 16-byte loads, the tail one
+// per lane; output may be a or b.
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+__global__ __launch_bounds__(256) void add_kernel(const uint16_t *a, const uint16_t *b, uint16_t *output, int size, int vec8) {
+    const int t = blockIdx.x * 256 + threadIdx.x;
+    if (t < vec8) {
+        const half8 x = ((const half8 *)a)[t], y = ((const half8 *)b)[t];
+        ((half8 *)output)[t] = x + y;
+        return;
+    }
+    const int i = vec8 * 8 + (t - vec8);
+    if (i < size)
+        output[i] = __builtin_bit_cast(uint16_t, (_Float16)(__builtin_bit_cast(_Float16, a[i]) + __builtin_bit_cast(_Float16, b[i])));
+}
+
+// Reference kernels/rope.cu:22-80: q [batch, seq_len, n_heads, head_dim] and k [.., n_kv_heads, ..]
+// are rotated in place, pair (2i, 2i+1) of every head by the angle (start_pos + seq_idx) *
+// theta^(-2i / head_dim). One thread per (token, head slot, pair) as there; a head slot below
+// n_heads rotates q, below n_kv_heads rotates k. The reference forms the angle and its sine and
+// cosine in fp32 (the angle is then off by up to pos * 2^-23 rad); here they are computed in fp64
+// and rounded to fp32 once, the rotation itself is the reference's fp32 arithmetic.
+__global__ __launch_bounds__(256) void rope_kernel(uint16_t *q, uint16_t *k, int seq_len, int n_heads, int n_kv_heads,
+                                                   int head_dim, int start_pos, double log2_theta, long long total) {
+    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const int half_dim = head_dim / 2;
+    const int max_heads = n_heads > n_kv_heads ? n_heads : n_kv_heads;
+    const int pair = (int)(idx % half_dim);
+    long long rest = idx / half_dim;
+    const int head = (int)(rest % max_heads);
+    const long long token = rest / max_heads;  // batch_idx * seq_len + seq_idx
+    const int pos = start_pos + (int)(token % seq_len);
+    const double angle = (double)pos * exp2(-log2_theta * (2.0 * pair) / (double)head_dim);
+    double sd, cd;
+    sincos(angle, &sd, &cd);
+    const float sn = (float)sd, cs = (float)cd;
+    auto rotate = [&](uint16_t *base, int heads) {
+        uint32_t *at = (uint32_t *)(base + ((size_t)token * heads + head) * head_dim) + pair;
+        const uint32_t v = *at;
+        const float x0 = h2f((uint16_t)v), x1 = h2f((uint16_t)(v >> 16));
+        *at = (uint32_t)f2h(x0 * cs - x1 * sn) | (uint32_t)f2h(x0 * sn + x1 * cs) << 16;
+    };
+    if (head < n_heads) rotate(q, n_heads);
+    if (head < n_kv_heads) rotate(k, n_kv_heads);
+}
+
+// Reference kernels/elementwise.cu:54-89: output[t, :] = table[indices[t], :]. One workgroup per
+// token; 16-byte copies when the rows allow it.
+__global__ __launch_bounds__(256) void embedding_lookup_kernel(const uint16_t *__restrict__ table,
+                                                               const int *__restrict__ indices,
+                                                               uint16_t *__restrict__ output, int dim, int vec) {
+    const size_t src = (size_t)indices[blockIdx.x] * dim, dst = (size_t)blockIdx.x * dim;
+    if (vec) {
+        const uint4 *s4 = (const uint4 *)(table + src);
+        uint4 *d4 = (uint4 *)(output + dst);
+        for (int i = threadIdx.x; i < dim / 8; i += 256) d4[i] = s4[i];
+    } else {
+        for (int i = threadIdx.x; i < dim; i += 256) output[dst + i] = table[src + i];
+    }
+}
+
+// Reference kernels/elementwise.cu:97-147: row (batch b, position s, head h) of k and v
+// [batch, seq_len, n_kv_heads, head_dim] goes to cache row (b, h, start_pos + s) of
+// [batch, n_kv_heads, max_seq_len, head_dim]; positions at or past max_seq_len are dropped.
+__global__ __launch_bounds__(128) void copy_to_kv_cache_kernel(const uint16_t *__restrict__ k, const uint16_t *__restrict__ v,
+                                                               uint16_t *__restrict__ k_cache, uint16_t *__restrict__ v_cache,
+                                                               int n_kv_heads, int head_dim, int seq_len, int start_pos,
+                                                               int max_seq_len, int vec) {
+    const int b = blockIdx.z, h = blockIdx.y, sq = blockIdx.x;
+    const int pos = start_pos + sq;
+    if (pos >= max_seq_len) return;
+    const size_t src = (((size_t)b * seq_len + sq) * n_kv_heads + h) * head_dim;
+    const size_t dst = (((size_t)b * n_kv_heads + h) * max_seq_len + pos) * head_dim;
+    if (vec) {
+        for (int i = threadIdx.x; i < head_dim / 8; i += 128) {
+            ((uint4 *)(k_cache + dst))[i] = ((const uint4 *)(k + src))[i];
+            ((uint4 *)(v_cache + dst))[i] = ((const uint4 *)(v + src))[i];
+        }
+    } else {
+        for (int i = threadIdx.x; i < head_dim; i += 128) {
+            k_cache[dst + i] = k[src + i];
+            v_cache[dst + i] = v[src + i];
+        }
+    }
+}
+
 }  // namespace
+
+hipError_t launch_add(const uint16_t *a, const uint16_t *b, uint16_t *output, int size, hipStream_t s) {
+    const bool aligned = (((uintptr_t)a | (uintptr_t)b | (uintptr_t)output) & 15) == 0;
+    const int vec8 = aligned ? size / 8 : 0;
+    const int lanes = vec8 + (size - vec8 * 8);
+    add_kernel<<<(lanes + 255) / 256, 256, 0, s>>>(a, b, output, size, vec8);
+    return hipGetLastError();
+}
+
+hipError_t launch_rope(uint16_t *q, uint16_t *k, int batch, int seq_len, int n_heads, int n_kv_heads, int head_dim,
+                       int start_pos, float theta, hipStream_t s) {
+    const int max_heads = n_heads > n_kv_heads ? n_heads : n_kv_heads;
+    const long long total = (long long)batch * seq_len * max_heads * (head_dim / 2);
+    rope_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(q, k, seq_len, n_heads, n_kv_heads, head_dim, start_pos,
+                                                                log2((double)theta), total);
+    return hipGetLastError();
+}
+
+hipError_t launch_embedding_lookup(const uint16_t *table, const int *indices, uint16_t *output, int n_tokens, int dim,
+                                   hipStream_t s) {
+    const int vec = dim % 8 == 0 && (((uintptr_t)table | (uintptr_t)output) & 15) == 0;
+    embedding_lookup_kernel<<<n_tokens, 256, 0, s>>>(table, indices, output, dim, vec);
+    return hipGetLastError();
+}
+
+hipError_t launch_copy_to_kv_cache(const uint16_t *k, const uint16_t *v, uint16_t *k_cache, uint16_t *v_cache, int batch,
+                                   int n_kv_heads, int head_dim, int seq_len, int start_pos, int max_seq_len,
+                                   hipStream_t s) {
+    const int vec = head_dim % 8 == 0 &&
+                    (((uintptr_t)k | (uintptr_t)v | (uintptr_t)k_cache | (uintptr_t)v_cache) & 15) == 0;
+    copy_to_kv_cache_kernel<<<dim3(seq_len, n_kv_heads, batch), 128, 0, s>>>(k, v, k_cache, v_cache, n_kv_heads, head_dim,
+                                                                             seq_len, start_pos, max_seq_len, vec);
+    return hipGetLastError();
+}
 
 hipError_t launch_rmsnorm(const uint16_t *input, const uint16_t *weight, uint16_t *output, const uint16_t *residual,
                           uint16_t *residual_out, int batch, int dim, float eps, hipStream_t s) {

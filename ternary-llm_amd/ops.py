@@ -17,6 +17,7 @@ ABI_SYMBOLS = (
     "tllm_ternary_gemv_i8_dscale", "tllm_quantize_absmax_i8", "tllm_ternary_gemm_f16",
     "tllm_linear_plan_create", "tllm_linear_plan_launch", "tllm_linear_plan_weight_bytes",
     "tllm_linear_plan_destroy", "tllm_rmsnorm_f16", "tllm_silu_mul_f16", "tllm_linear_plan_create_normed",
+    "tllm_add_f16", "tllm_rope_f16", "tllm_embedding_lookup_f16", "tllm_copy_to_kv_cache_f16",
 )
 # include/tllm_model_file.h
 FILE_ABI_SYMBOLS = (
@@ -83,6 +84,10 @@ def lib():
     L.tllm_linear_plan_destroy.restype = None
     L.tllm_rmsnorm_f16.argtypes = [vp, vp, vp, vp, vp, i, i, f, vp]
     L.tllm_silu_mul_f16.argtypes = [vp, vp, vp, i, vp]
+    L.tllm_add_f16.argtypes = [vp, vp, vp, i, vp]
+    L.tllm_rope_f16.argtypes = [vp, vp, i, i, i, i, i, i, f, vp]
+    L.tllm_embedding_lookup_f16.argtypes = [vp, vp, vp, i, i, vp]
+    L.tllm_copy_to_kv_cache_f16.argtypes = [vp, vp, vp, vp, i, i, i, i, i, i, vp]
     L.tllm_ternarize_pack_f32.argtypes = [vp, i, i, i, f, vp, vp, vp]
     L.tllm_model_file_open.argtypes = [C.c_char_p, C.POINTER(vp)]
     L.tllm_model_file_close.argtypes = [vp]
@@ -160,6 +165,29 @@ def rmsnorm(input, weight, output, residual, residual_out, batch, dim, eps, stre
 def silu_mul(gate, up, output, size, stream=None):
     """SiLU(gate) * up (reference include/kernels.cuh:60-62)."""
     check(lib().tllm_silu_mul_f16(_ptr(gate), _ptr(up), _ptr(output), size, _stream(stream)))
+
+
+def add(a, b, output, size, stream=None):
+    """output = a + b in fp16 (reference include/kernels.cuh:64-66)."""
+    check(lib().tllm_add_f16(_ptr(a), _ptr(b), _ptr(output), size, _stream(stream)))
+
+
+def rope(q, k, batch, seq_len, n_heads, n_kv_heads, head_dim, start_pos, theta, stream=None):
+    """Rotary position embedding of q and k in place (reference include/kernels.cuh:50-53)."""
+    check(lib().tllm_rope_f16(_ptr(q), _ptr(k), batch, seq_len, n_heads, n_kv_heads, head_dim, start_pos, theta,
+                              _stream(stream)))
+
+
+def embedding_lookup(table, indices, output, n_tokens, dim, stream=None):
+    """output[t] = table[indices[t]] (reference include/kernels.cuh:68-70); indices: int32 on the device."""
+    check(lib().tllm_embedding_lookup_f16(_ptr(table), _ptr(indices), _ptr(output), n_tokens, dim, _stream(stream)))
+
+
+def copy_to_kv_cache(k, v, k_cache, v_cache, batch, n_kv_heads, head_dim, seq_len, start_pos, max_seq_len,
+                     stream=None):
+    """New k/v rows into the caches at start_pos (reference include/kernels.cuh:72-76)."""
+    check(lib().tllm_copy_to_kv_cache_f16(_ptr(k), _ptr(v), _ptr(k_cache), _ptr(v_cache), batch, n_kv_heads, head_dim,
+                                          seq_len, start_pos, max_seq_len, _stream(stream)))
 
 
 SWIGLU_GATE = 1  # TLLM_PROBLEM_SWIGLU_GATE

@@ -44,6 +44,16 @@ int main() {
     ternary::rmsnorm_forward(residual_buf_, attn_norm_weight, hidden_buf_, nullptr, nullptr, n_tokens, hidden,
                              rms_norm_eps);
     ternary::silu_mul_forward(gate_buf_, up_buf_, gate_buf_, n_tokens * inter);
+    // src/transformer.cpp:179-181 embedding, :225-236 RoPE and cache update, :253, 296 residual add
+    half *q_buf_ = nullptr, *k_buf_ = nullptr, *v_buf_ = nullptr, *k_cache = nullptr, *v_cache = nullptr;
+    const half *embed_tokens = nullptr;
+    const int *d_tokens = nullptr;
+    int n_heads = 32, n_kv_heads = 8, head_dim = 64, start_pos = 3, max_seq_len = 4096;
+    float rope_theta = 500000.0f;
+    ternary::embedding_lookup(embed_tokens, d_tokens, hidden_buf_, n_tokens, hidden);
+    ternary::rope_forward(q_buf_, k_buf_, 1, n_tokens, n_heads, n_kv_heads, head_dim, start_pos, rope_theta);
+    ternary::copy_to_kv_cache(k_buf_, v_buf_, k_cache, v_cache, 1, n_kv_heads, head_dim, n_tokens, start_pos, max_seq_len);
+    ternary::add_forward(residual_buf_, hidden_buf_, residual_buf_, n_tokens * hidden);
     std::printf("rejected=%d\n", rejected);
-    return rejected == 6 ? 0 : 1;
+    return rejected == 10 ? 0 : 1;
 }

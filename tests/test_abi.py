@@ -59,6 +59,17 @@ def test_validation_codes():
     assert L.tllm_rmsnorm_f16(0x10, 0x20, 0x30, None, None, 1 << 20, 1 << 12, 1e-5, None) == -4
     assert L.tllm_silu_mul_f16(0x10, None, 0x30, 4, None) == -1
     assert L.tllm_silu_mul_f16(0x10, 0x20, 0x30, 0, None) == -2
+    assert L.tllm_add_f16(0x10, None, 0x30, 4, None) == -1 and L.tllm_add_f16(0x10, 0x20, 0x30, 0, None) == -2
+    assert L.tllm_rope_f16(None, 0x20, 1, 1, 8, 2, 64, 0, 10000.0, None) == -1
+    assert L.tllm_rope_f16(0x10, 0x20, 1, 1, 8, 2, 63, 0, 10000.0, None) == -2      # odd head_dim
+    assert L.tllm_rope_f16(0x10, 0x20, 1, 1, 8, 2, 64, -1, 10000.0, None) == -2     # negative position
+    assert L.tllm_rope_f16(0x10, 0x20, 1, 1, 8, 2, 64, 0, 0.0, None) == -2          # theta must be positive
+    assert L.tllm_rope_f16(0x12, 0x20, 1, 1, 8, 2, 64, 0, 10000.0, None) == -7      # pairs are read as 4-byte words
+    assert L.tllm_embedding_lookup_f16(0x10, None, 0x30, 1, 8, None) == -1
+    assert L.tllm_embedding_lookup_f16(0x10, 0x20, 0x30, 0, 8, None) == -2
+    assert L.tllm_copy_to_kv_cache_f16(0x10, 0x20, None, 0x40, 1, 2, 64, 1, 0, 16, None) == -1
+    assert L.tllm_copy_to_kv_cache_f16(0x10, 0x20, 0x30, 0x40, 1, 2, 64, 0, 0, 16, None) == -2
+    assert L.tllm_copy_to_kv_cache_f16(0x10, 0x20, 0x30, 0x40, 1, 2, 64, 1, -1, 16, None) == -2
     h = C.c_void_p(0)
     assert L.tllm_linear_plan_create(C.byref(h), None, 1, 128) == -1
     arr = (ops._Problem * 1)(ops._Problem(0x1000, 0x2000, 0x3000, 0x4000, 0x9000, 4, 256, 17, 0))
@@ -108,4 +119,4 @@ def test_cpp_dropin_call_shapes(tmp_path):
     subprocess.run(cmd, check=True, capture_output=True, text=True)
     out = subprocess.run([str(exe)], capture_output=True, text=True)
     assert out.returncode == 0, out.stdout + out.stderr
-    assert "rejected=6" in out.stdout
+    assert "rejected=10" in out.stdout

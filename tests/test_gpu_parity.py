@@ -478,6 +478,92 @@ def test_silu_mul_tails(dev, oracle):
     assert got[0] == 0 and got[1] == 0 and got[2] == 80.0 and got[3] == 0 and got[4] == 65504.0 and got[5] == 0
     assert got[6] == np.float64(np.float16(1.0 / (1.0 + np.exp(-1.0))))
 
+@pytest.mark.parametrize("n", [1, 7, 8, 4096, 7 * 4096 + 3])
+def test_add_bit_exact(dev, oracle, n):
+    """fp16 residual add: equal, bit for bit, to the once-rounded exact sum; in place; odd start."""
+    torch, tl = dev
+    rng = np.random.default_rng(n)
+    a = oracle.half_bits(rng.normal(0, 4, n))
+    b = oracle.half_bits(rng.normal(0, 4, n) * 10.0 ** rng.integers(-6, 3, n))
+    want = oracle.half_bits(oracle.add_f64(a, b))
+    ad, bd = up(torch, a), up(torch, b)
+    out = torch.zeros(n, dtype=torch.float16, device="cuda")
+    tl.add(ad, bd, out, n)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out.cpu().numpy().view(np.uint16), want)
+    tl.add(ad, bd, ad, n)   # the reference adds into the residual buffer (src/transformer.cpp:253)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(ad.cpu().numpy().view(np.uint16), want)
+    if n > 2:
+        ad = up(torch, a)
+        out2 = torch.zeros(n, dtype=torch.float16, device="cuda")
+        tl.add(ad[1:], bd[1:], out2[1:], n - 1)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(out2.cpu().numpy().view(np.uint16)[1:], want[1:])
+
+
+@pytest.mark.parametrize("batch,seq,heads,kv_heads,hd,start,theta", [
+    (1, 1, 32, 8, 128, 0, 500000.0),      # 8B decode step, first token
+    (1, 1, 32, 8, 64, 1234, 500000.0),    # 1B decode step in mid-sequence
+    (1, 1, 64, 8, 128, 8191, 500000.0),   # 70B decode at the end of an 8K context
+    (1, 77, 32, 8, 128, 5, 10000.0),      # prefill of 77 tokens
+    (2, 3, 2, 5, 6, 9, 10000.0),          # more kv heads than q heads, tiny head
+])
+def test_rope_vs_oracle(dev, oracle, batch, seq, heads, kv_heads, hd, start, theta):
+    torch, tl = dev
+    rng = np.random.default_rng(heads * hd + start)
+    q = oracle.half_bits(rng.normal(0, 1, (batch, seq, heads, hd)))
+    k = oracle.half_bits(rng.normal(0, 1, (batch, seq, kv_heads, hd)))
+    ref_q = oracle.rope_f64(q, batch, seq, heads, hd, start, theta)
+    ref_k = oracle.rope_f64(k, batch, seq, kv_heads, hd, start, theta)
+    qd, kd = up(torch, q), up(torch, k)
+    tl.rope(qd, kd, batch, seq, heads, kv_heads, hd, start, theta)
+    torch.cuda.synchronize()
+    got_q = qd.cpu().numpy().view(np.float16).astype(np.float64)
+    got_k = kd.cpu().numpy().view(np.float16).astype(np.float64)
+    # fp32 sine/cosine of the exactly formed angle and an fp32 rotation: 1e-3 of max(|ref|, tau) as
+    # for the linears (a pair that rotates onto an axis leaves one small component)
+    assert_close(oracle, got_q.reshape(-1), ref_q.reshape(-1), what="rope q")
+    assert_close(oracle, got_k.reshape(-1), ref_k.reshape(-1), what="rope k")
+    # tighter, normwise per pair: the rotation is good to fp16 rounding of the result
+    err = np.hypot(got_q[..., 0::2] - ref_q[..., 0::2], got_q[..., 1::2] - ref_q[..., 1::2])
+    nrm = np.hypot(ref_q[..., 0::2], ref_q[..., 1::2])
+    assert (err <= 2.0 ** -10 * nrm + 1e-7).all()
+
+
+def test_embedding_lookup_bit_exact(dev, oracle):
+    torch, tl = dev
+    rng = np.random.default_rng(3)
+    for vocab, dim, n_tokens in ((1000, 2048, 1), (1000, 4096, 33), (50, 100, 7), (50, 8, 3)):
+        table = rng.integers(0, 65536, (vocab, dim)).astype(np.uint16)
+        idx = rng.integers(0, vocab, n_tokens).astype(np.int32)
+        idx[0] = vocab - 1
+        out = torch.zeros((n_tokens, dim), dtype=torch.float16, device="cuda")
+        tl.embedding_lookup(up(torch, table), torch.from_numpy(idx).cuda(), out, n_tokens, dim)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(out.cpu().numpy().view(np.uint16), oracle.embedding_lookup(table, idx))
+
+
+@pytest.mark.parametrize("batch,seq,heads,hd,start,max_seq", [
+    (1, 1, 8, 128, 0, 64), (1, 1, 8, 64, 63, 64), (1, 40, 8, 128, 10, 64), (2, 5, 3, 6, 2, 8),
+    (1, 10, 8, 128, 60, 64),   # runs past the end of the cache: the last 6 rows are dropped
+    (1, 4, 2, 64, 64, 64),     # wholly outside: nothing is written
+])
+def test_copy_to_kv_cache_bit_exact(dev, oracle, batch, seq, heads, hd, start, max_seq):
+    torch, tl = dev
+    rng = np.random.default_rng(seq * 131 + start)
+    k = rng.integers(0, 65536, (batch, seq, heads, hd)).astype(np.uint16)
+    v = rng.integers(0, 65536, (batch, seq, heads, hd)).astype(np.uint16)
+    kc = rng.integers(0, 65536, (batch, heads, max_seq, hd)).astype(np.uint16)
+    vc = rng.integers(0, 65536, (batch, heads, max_seq, hd)).astype(np.uint16)
+    want_k, want_v = oracle.copy_to_kv_cache(k, v, kc, vc, start)
+    kcd, vcd = up(torch, kc), up(torch, vc)
+    tl.copy_to_kv_cache(up(torch, k), up(torch, v), kcd, vcd, batch, heads, hd, seq, start, max_seq)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(kcd.cpu().numpy().view(np.uint16), want_k)
+    np.testing.assert_array_equal(vcd.cpu().numpy().view(np.uint16), want_v)
+
+
 # --------------------------------------------------------------- INT8 pair
 @pytest.mark.parametrize("n", [1, 63, 2048, 4096, 14336, 28672])
 def test_quantize_bit_exact(dev, oracle, n):

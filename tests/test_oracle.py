@@ -8,6 +8,7 @@ an independent unpacker (numpy unpackbits), not by the oracle's own loops.
 """
 import itertools
 import json
+import math
 import os
 
 import numpy as np
@@ -345,3 +346,70 @@ def test_silu_mul_closed_forms(oracle):
     tail = oracle.silu_mul_f64(np.array([40.0, -40.0], np.float16).view(np.uint16),
                                np.array([2.0, 2.0], np.float16).view(np.uint16))
     assert tail[0] == pytest.approx(80.0, rel=1e-15) and abs(tail[1]) < 1e-15
+
+
+def test_add_is_exact(oracle):
+    rng = np.random.default_rng(11)
+    a = rng.normal(0, 4, 2000).astype(np.float16)
+    b = (rng.normal(0, 4, 2000) * 10.0 ** rng.integers(-6, 3, 2000)).astype(np.float16)
+    out = oracle.add_f64(a.view(np.uint16), b.view(np.uint16))
+    assert (out == a.astype(np.float64) + b.astype(np.float64)).all()
+    # rounding the exact sum once is what an fp16 adder stores
+    assert (oracle.half_bits(out) == (a + b).view(np.uint16)).all()
+
+
+def test_rope_closed_forms(oracle):
+    rng = np.random.default_rng(12)
+    batch, seq, heads, hd = 2, 5, 3, 8
+    x = rng.normal(0, 1, (batch, seq, heads, hd)).astype(np.float16)
+    xv = x.astype(np.float64)
+    # position 0: identity (only the first token of each batch entry when start_pos = 0)
+    out = oracle.rope_f64(x.view(np.uint16), batch, seq, heads, hd, 0, 10000.0)
+    assert (out[:, 0] == xv[:, 0]).all()
+    # theta = 1: every pair turns by `pos` radians; (1, 0) -> (cos, sin) fixes sign and pair layout
+    unit = np.zeros((1, 4, 1, 6), np.float16)
+    unit[..., 0::2] = 1.0
+    turned = oracle.rope_f64(unit.view(np.uint16), 1, 4, 1, 6, 3, 1.0)
+    for s in range(4):
+        for i in range(3):
+            assert turned[0, s, 0, 2 * i] == pytest.approx(math.cos(3 + s), abs=1e-15)
+            assert turned[0, s, 0, 2 * i + 1] == pytest.approx(math.sin(3 + s), abs=1e-15)
+    # pair norms are preserved
+    n_in = xv[..., 0::2] ** 2 + xv[..., 1::2] ** 2
+    n_out = out[..., 0::2] ** 2 + out[..., 1::2] ** 2
+    np.testing.assert_allclose(n_out, n_in, rtol=1e-13)
+    # start_pos shifts the sequence index: token s at start 7 == token 0 at start 7 + s
+    a = oracle.rope_f64(x.view(np.uint16), batch, seq, heads, hd, 7, 500000.0)
+    for s in range(seq):
+        one = oracle.rope_f64(np.ascontiguousarray(x[:, s:s + 1]).view(np.uint16), batch, 1, heads, hd, 7 + s, 500000.0)
+        assert (a[:, s:s + 1] == one).all()
+    # complex-exponential restatement: (x0 + i x1) * exp(i * pos * theta^(-2i/hd))
+    theta, start = 500000.0, 7
+    pos = (start + np.arange(seq))[None, :, None, None]
+    freq = theta ** (-2.0 * np.arange(hd // 2) / hd)
+    z = (xv[..., 0::2] + 1j * xv[..., 1::2]) * np.exp(1j * pos * freq)
+    np.testing.assert_allclose(a[..., 0::2], z.real, rtol=1e-12, atol=1e-14)
+    np.testing.assert_allclose(a[..., 1::2], z.imag, rtol=1e-12, atol=1e-14)
+
+
+def test_embedding_and_kv_copy_index_arithmetic(oracle):
+    rng = np.random.default_rng(13)
+    table = rng.integers(0, 65536, (11, 6)).astype(np.uint16)
+    idx = np.array([3, 0, 10, 3], np.int32)
+    got = oracle.embedding_lookup(table, idx)
+    for t, i in enumerate(idx):
+        assert (got[t] == table[i]).all()
+    batch, seq, heads, hd, max_seq = 2, 3, 2, 4, 6
+    k = rng.integers(0, 65536, (batch, seq, heads, hd)).astype(np.uint16)
+    v = rng.integers(0, 65536, (batch, seq, heads, hd)).astype(np.uint16)
+    kc0 = rng.integers(0, 65536, (batch, heads, max_seq, hd)).astype(np.uint16)
+    vc0 = rng.integers(0, 65536, (batch, heads, max_seq, hd)).astype(np.uint16)
+    for start in (0, 2, 4, 5, 6):  # 4 and 5 run past the end of the cache, 6 is wholly outside
+        kc, vc = oracle.copy_to_kv_cache(k, v, kc0, vc0, start)
+        for b in range(batch):
+            for h in range(heads):
+                for p in range(max_seq):
+                    s = p - start
+                    inside = 0 <= s < seq
+                    assert (kc[b, h, p] == (k[b, s, h] if inside else kc0[b, h, p])).all()
+                    assert (vc[b, h, p] == (v[b, s, h] if inside else vc0[b, h, p])).all()

@@ -48,6 +48,7 @@ constexpr int kNW = 4;  // waves per workgroup
 // Most slices of a row (wide tiles: 2048 columns each) whose operand image is in LDS at one time;
 // longer rows are staged and walked in segments. 8 slices = 32 KB keep three workgroups on a CU.
 constexpr int kSegSlices = 8;
+constexpr int kSegElems = 16384;  // the same limit for tall tiles: elements of all batch columns together
 constexpr int kThreads = kNW * kWave;
 constexpr int kMaxBatch = 4;  // activation rows the tall tiles carry
 #ifndef TLLM_TILES_AHEAD
@@ -189,7 +190,8 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
 
     int cur = -1;      // problem whose activations are staged
     int cur_seg = -1;  // and which segment of its columns
-    int cur_ex = 0;    // exponent of that problem's largest activation (rows staged in segments)
+    constexpr int kSegBatch = G::kRows == 4 ? 1 : kMaxBatch;
+    int cur_ex[kSegBatch] = {};  // exponents of that problem's largest activations (rows staged in segments)
     Problem p = single;
     int slices = 0, groups = 0, words = 0, img_stride = 0;
     int seg_lo = 0, seg_n = 0;  // slices of the staged segment
@@ -228,7 +230,9 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
         }
         // Rows longer than kSegSlices slices are staged and walked in segments of equal length, so
         // that the operand image never takes more than kSegSlices slices of LDS (wide tiles only).
-        const int n_seg = G::kRows == 4 && !kFine ? (slices + kSegSlices - 1) / kSegSlices : 1;  // (fine-grained instances: whole rows, the host sees to it that they fit)
+        // (fine-grained instances: whole rows, the host sees to it that they fit)
+        const int seg_max = G::kRows == 4 ? kSegSlices : kSegElems / G::kCols / p.batch;
+        const int n_seg = kFine ? 1 : (slices + seg_max - 1) / seg_max;
         const int seg_len = (slices + n_seg - 1) / n_seg;
 
         const int r_begin = task_first_row;
@@ -326,25 +330,35 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                 // a segment of a long row: the exponent comes from a pass over the whole row, made
                 // once per problem; the segment itself is staged like a short row
                 if (fresh && seg == 0) {
-                    uint32_t m = 0;
-                    for (int c8 = stid; c8 < p.cols / 8; c8 += kThreads) m = magnitude(m, load8(0, c8));
 #pragma unroll
-                    for (int off = 32; off > 0; off >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, off, kWave));
-                    if (lane == 0) red_amax[wave][0] = m;
+                    for (int b = 0; b < kSegBatch; b++) {
+                        if (b >= p.batch) break;
+                        uint32_t m = 0;
+                        for (int c8 = stid; c8 < p.cols / 8; c8 += kThreads) m = magnitude(m, load8(b, c8));
+#pragma unroll
+                        for (int off = 32; off > 0; off >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, off, kWave));
+                        if (lane == 0) red_amax[wave][b] = m;
+                    }
                     __syncthreads();
-                    cur_ex = exponent_of(0);
-                }
-                uint4 keep[kKeep];
 #pragma unroll
-                for (int k = 0; k < kKeep; k++) {
-                    const int c8 = stid + k * kThreads;
-                    keep[k] = c8 < pieces ? piece_of(0, c8) : uint4{0u, 0u, 0u, 0u};
+                    for (int b = 0; b < kSegBatch; b++)
+                        if (b < p.batch) cur_ex[b] = exponent_of(b);
                 }
 #pragma unroll
-                for (int k = 0; k < kKeep; k++) {
-                    const int c8 = stid + k * kThreads;
-                    if (c8 < pieces) write_piece(image, c8, keep[k], cur_ex);
-                    __builtin_amdgcn_sched_barrier(0);
+                for (int b = 0; b < kSegBatch; b++) {
+                    if (b >= p.batch) break;
+                    uint4 keep[kKeep];
+#pragma unroll
+                    for (int k = 0; k < kKeep; k++) {
+                        const int c8 = stid + k * kThreads;
+                        keep[k] = c8 < pieces ? piece_of(b, c8) : uint4{0u, 0u, 0u, 0u};
+                    }
+#pragma unroll
+                    for (int k = 0; k < kKeep; k++) {
+                        const int c8 = stid + k * kThreads;
+                        if (c8 < pieces) write_piece(image + (size_t)b * img_stride, c8, keep[k], cur_ex[b]);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
                 }
             } else if (p.batch == 1 && pieces <= kKeep * kThreads) {
                 // one pass over x: all loads are issued together and kept for the image
@@ -751,8 +765,9 @@ bool wants_fine(int64_t coarse_units, int slots) { return coarse_units * 2 <= sl
 template <class G>
 int image_bytes_of(int cols, int batch, bool segmented = true) {
     int slices = (cols + G::kCols - 1) / G::kCols;
-    if (G::kRows == 4 && segmented) {  // wide tiles: long rows are staged in equal segments of at most kSegSlices
-        const int n_seg = (slices + kSegSlices - 1) / kSegSlices;
+    if (segmented) {  // long rows are staged in equal segments (the kernel works out the same numbers)
+        const int seg_max = G::kRows == 4 ? kSegSlices : kSegElems / G::kCols / batch;
+        const int n_seg = (slices + seg_max - 1) / seg_max;
         slices = (slices + n_seg - 1) / n_seg;
     }
     return slices * G::kCols * 2 * batch;
@@ -1045,7 +1060,13 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
         all_wide = all_wide && addressable && wide_ok(p);
         all_tall = all_tall && addressable && tall_ok(p);
     }
-    if (all_batch) {
+    // Up to this many activation rows the tall-tile MFMA kernel is the faster of the two (8B and 70B
+    // sweeps: +17 % at two rows, +6 % at three, equal at four). TLLM_TALL_MAX_BATCH overrides.
+    static const int tall_max_batch = [] {
+        const char *e = getenv("TLLM_TALL_MAX_BATCH");
+        return e ? atoi(e) : 3;
+    }();
+    if (all_batch && !(all_tall && max_batch <= tall_max_batch)) {
         d.batch_kernel = true;
         partition_blocks(gemv_batch_block_rows(), di->cus);
     } else {

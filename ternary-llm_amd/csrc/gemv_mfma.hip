@@ -48,7 +48,9 @@ constexpr int kNW = 4;  // waves per workgroup
 // Most slices of a row (wide tiles: 2048 columns each) whose operand image is in LDS at one time;
 // longer rows are staged and walked in segments. 8 slices = 32 KB keep three workgroups on a CU.
 constexpr int kSegSlices = 8;
-constexpr int kSegElems = 16384;  // the same limit for tall tiles: elements of all batch columns together
+// The same limit for tall tiles, in slices of 512 columns: 16384 elements of all batch columns
+// together, half of that at four columns (there the partial sums need the room more: measured).
+__host__ __device__ constexpr int tall_seg_slices(int batch) { return (batch >= 4 ? 8192 : 16384) / 512 / batch; }
 constexpr int kThreads = kNW * kWave;
 constexpr int kMaxBatch = 4;  // activation rows the tall tiles carry
 #ifndef TLLM_TILES_AHEAD
@@ -231,7 +233,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
         // Rows longer than kSegSlices slices are staged and walked in segments of equal length, so
         // that the operand image never takes more than kSegSlices slices of LDS (wide tiles only).
         // (fine-grained instances: whole rows, the host sees to it that they fit)
-        const int seg_max = G::kRows == 4 ? kSegSlices : kSegElems / G::kCols / p.batch;
+        const int seg_max = G::kRows == 4 ? kSegSlices : tall_seg_slices(p.batch);
         const int n_seg = kFine ? 1 : (slices + seg_max - 1) / seg_max;
         const int seg_len = (slices + n_seg - 1) / n_seg;
 
@@ -718,6 +720,9 @@ struct DeviceInfo {
 };
 
 constexpr int kLdsLimit = 64 * 1024;  // per workgroup; 160 KB per CU leaves room for two or three
+// The tall-tile instance runs two workgroups per CU (register need) and keeps one partial sum per
+// wave, row and batch column: it gets all the LDS two workgroups can have.
+constexpr int kTallLdsLimit = 78 * 1024;
 
 template <class G, bool kExtras = false, bool kFine = false>
 const void *kernel_ptr() {
@@ -736,7 +741,9 @@ hipError_t prepare_device(DeviceInfo **out) {
         std::lock_guard<std::mutex> lock(init_mutex);
         for (const void *k : {kernel_ptr<Wide>(), kernel_ptr<Tall>(), kernel_ptr<Wide, true>(),
                               kernel_ptr<Wide, false, true>(), kernel_ptr<Wide, true, true>()})
-            if (hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit)) return e;
+            if (hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                   k == kernel_ptr<Tall>() ? kTallLdsLimit : kLdsLimit))
+                return e;
         info[dev].cus = current_device_cus();
         ready[dev].store(true, std::memory_order_release);
     }
@@ -766,7 +773,7 @@ template <class G>
 int image_bytes_of(int cols, int batch, bool segmented = true) {
     int slices = (cols + G::kCols - 1) / G::kCols;
     if (segmented) {  // long rows are staged in equal segments (the kernel works out the same numbers)
-        const int seg_max = G::kRows == 4 ? kSegSlices : kSegElems / G::kCols / batch;
+        const int seg_max = G::kRows == 4 ? kSegSlices : tall_seg_slices(batch);
         const int n_seg = (slices + seg_max - 1) / seg_max;
         slices = (slices + n_seg - 1) / n_seg;
     }
@@ -780,7 +787,7 @@ bool wide_ok(const Problem &p) {
 }
 bool tall_ok(const Problem &p) {
     return p.batch >= 1 && p.batch <= kMaxBatch && p.rows >= 16 && p.cols >= Tall::kCols &&
-           image_bytes_of<Tall>(p.cols, p.batch) + kNW * range_unit<Tall>() * p.batch * 4 <= kLdsLimit;
+           image_bytes_of<Tall>(p.cols, p.batch) + kNW * range_unit<Tall>() * p.batch * 4 <= kTallLdsLimit;
 }
 
 #ifndef TLLM_MAX_TASK_UNITS
@@ -843,9 +850,9 @@ double block_pool_fraction() {
 }
 
 // units per task that the partial-sum area can hold
-int max_units_for(int image_bytes, int batch, int unit, int mats = 1) {
+int max_units_for(int image_bytes, int batch, int unit, int mats = 1, int lds_limit = kLdsLimit) {
     // one partial sum per wave, row and matrix of the task (two for a SwiGLU pair)
-    const int room_rows = (kLdsLimit - image_bytes) / (kNW * batch * 4 * mats);
+    const int room_rows = (lds_limit - image_bytes) / (kNW * batch * 4 * mats);
     const int n = room_rows / unit;
     return n > kMaxTaskUnits ? kMaxTaskUnits : n;
 }
@@ -873,7 +880,7 @@ static hipError_t launch_single(const Problem &p, bool x_is_i8, float i8_scale, 
                       wants_fine((p.rows + range_unit<Wide>() - 1) / range_unit<Wide>(), wgs);
     const int unit = fine ? kFineUnit : wide ? range_unit<Wide>() : range_unit<Tall>();
     sc.image_bytes = wide ? image_bytes_of<Wide>(p.cols, 1, !fine) : image_bytes_of<Tall>(p.cols, p.batch);
-    sc.max_units = max_units_for(sc.image_bytes, p.batch, unit);
+    sc.max_units = max_units_for(sc.image_bytes, p.batch, unit, 1, wide ? kLdsLimit : kTallLdsLimit);
     sc.max_batch = p.batch;
     const int units = (p.rows + unit - 1) / unit;
     const int grid = units < wgs ? units : wgs;
@@ -1061,10 +1068,10 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
         all_tall = all_tall && addressable && tall_ok(p);
     }
     // Up to this many activation rows the tall-tile MFMA kernel is the faster of the two (8B and 70B
-    // sweeps: +17 % at two rows, +6 % at three, equal at four). TLLM_TALL_MAX_BATCH overrides.
+    // sweeps: +17 % at two rows, +13 % at three, +5 % at four). TLLM_TALL_MAX_BATCH overrides.
     static const int tall_max_batch = [] {
         const char *e = getenv("TLLM_TALL_MAX_BATCH");
-        return e ? atoi(e) : 3;
+        return e ? atoi(e) : 4;
     }();
     if (all_batch && !(all_tall && max_batch <= tall_max_batch)) {
         d.batch_kernel = true;
@@ -1089,7 +1096,7 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
         }
         const int unit = d.fine ? kFineUnit : d.wide ? range_unit<Wide>() : range_unit<Tall>();
         const int mats = has_pairs ? 2 : 1;
-        const int max_units = max_units_for(max_image, max_batch, unit, mats);
+        const int max_units = max_units_for(max_image, max_batch, unit, mats, d.wide ? kLdsLimit : kTallLdsLimit);
         if (max_units < 1) d.use_mfma = false;
         if (d.use_mfma) {
             d.pair_stride = has_pairs ? kNW * max_units * unit * max_batch : 0;

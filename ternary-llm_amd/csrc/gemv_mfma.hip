@@ -328,41 +328,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
             int stid = tid;
             asm volatile("" : "+v"(stid));
             constexpr int kKeep = 8;  // pieces per thread that stay in registers between the two steps
-            if (n_seg > 1) {
-                // a segment of a long row: the exponent comes from a pass over the whole row, made
-                // once per problem; the segment itself is staged like a short row
-                if (fresh && seg == 0) {
-#pragma unroll
-                    for (int b = 0; b < kSegBatch; b++) {
-                        if (b >= p.batch) break;
-                        uint32_t m = 0;
-                        for (int c8 = stid; c8 < p.cols / 8; c8 += kThreads) m = magnitude(m, load8(b, c8));
-#pragma unroll
-                        for (int off = 32; off > 0; off >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, off, kWave));
-                        if (lane == 0) red_amax[wave][b] = m;
-                    }
-                    __syncthreads();
-#pragma unroll
-                    for (int b = 0; b < kSegBatch; b++)
-                        if (b < p.batch) cur_ex[b] = exponent_of(b);
-                }
-#pragma unroll
-                for (int b = 0; b < kSegBatch; b++) {
-                    if (b >= p.batch) break;
-                    uint4 keep[kKeep];
-#pragma unroll
-                    for (int k = 0; k < kKeep; k++) {
-                        const int c8 = stid + k * kThreads;
-                        keep[k] = c8 < pieces ? piece_of(b, c8) : uint4{0u, 0u, 0u, 0u};
-                    }
-#pragma unroll
-                    for (int k = 0; k < kKeep; k++) {
-                        const int c8 = stid + k * kThreads;
-                        if (c8 < pieces) write_piece(image + (size_t)b * img_stride, c8, keep[k], cur_ex[b]);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                }
-            } else if (p.batch == 1 && pieces <= kKeep * kThreads) {
+            if (n_seg == 1 && p.batch == 1 && pieces <= kKeep * kThreads) {
                 // one pass over x: all loads are issued together and kept for the image
                 uint4 keep[kKeep];
                 uint32_t m = 0;
@@ -432,20 +398,84 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                     if (c8 < pieces) write_piece(image, c8, keep[k], ex);
                     __builtin_amdgcn_sched_barrier(0);  // one piece at a time: keeps the register need low
                 }
-            } else {
-                // long rows or several batch columns: one pass for the magnitudes, one for the image
-                for (int b = 0; b < p.batch; b++) {
-                    uint32_t m = 0;
-                    for (int c8 = stid; c8 < pieces; c8 += kThreads) m = magnitude(m, piece_of(b, c8));
+            } else if constexpr (kFine) {
+                // a whole row too long for the registers (the fine-grained instances do not stage in
+                // segments): one pass for the magnitude, one for the image, piece by piece
+                uint32_t m = 0;
+                for (int c8 = stid; c8 < pieces; c8 += kThreads) m = magnitude(m, piece_of(0, c8));
 #pragma unroll
-                    for (int off = 32; off > 0; off >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, off, kWave));
-                    if (lane == 0) red_amax[wave][b] = m;
-                }
+                for (int off = 32; off > 0; off >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, off, kWave));
+                if (lane == 0) red_amax[wave][0] = m;
                 __syncthreads();
-                for (int b = 0; b < p.batch; b++) {
-                    const int ex = exponent_of(b);
-                    for (int c8 = stid; c8 < pieces; c8 += kThreads)
-                        write_piece(image + (size_t)b * img_stride, c8, piece_of(b, c8), ex);
+                const int ex = exponent_of(0);
+                for (int c8 = stid; c8 < pieces; c8 += kThreads) write_piece(image, c8, piece_of(0, c8), ex);
+            } else {
+                // Long rows or several batch columns: one pass for the magnitudes, one for the image.
+                // The (column, piece) pairs are numbered column-major and taken kFlat * kThreads at a
+                // time, so that a thread has kFlat loads in flight whatever the shape. A row staged in
+                // segments gets its exponents from one pass over the whole row, made when the problem
+                // is first seen; its segments are then written with those.
+                constexpr int kFlat = G::kRows == 4 ? kKeep / 2 : kKeep;  // loads in flight per thread (wide tiles: fewer registers to spare)
+                auto column_of = [&](int item, int per_col) -> int {  // item / per_col for at most kSegBatch columns
+                    int b = 0;
+#pragma unroll
+                    for (int c = 1; c < kSegBatch; c++) b += item >= c * per_col;
+                    return b;
+                };
+                if (n_seg == 1 || (fresh && seg == 0)) {
+                    const bool whole_row = n_seg > 1;
+                    const int per_col = whole_row ? p.cols / 8 : pieces;
+                    const int items = per_col * p.batch;
+                    uint32_t m[kSegBatch] = {};
+                    for (int base = 0; base < items; base += kFlat * kThreads) {
+                        uint4 kp[kFlat];
+                        int kb[kFlat];
+#pragma unroll
+                        for (int k = 0; k < kFlat; k++) {
+                            const int item = base + stid + k * kThreads;
+                            const int b = column_of(item, per_col);
+                            kb[k] = item < items ? b : -1;
+                            kp[k] = item >= items ? uint4{0u, 0u, 0u, 0u}
+                                    : whole_row   ? load8(b, item - b * per_col)
+                                                  : piece_of(b, item - b * per_col);
+                        }
+#pragma unroll
+                        for (int k = 0; k < kFlat; k++)
+#pragma unroll
+                            for (int c = 0; c < kSegBatch; c++)
+                                if (kb[k] == c) m[c] = magnitude(m[c], kp[k]);
+                    }
+#pragma unroll
+                    for (int c = 0; c < kSegBatch; c++) {
+#pragma unroll
+                        for (int off = 32; off > 0; off >>= 1)
+                            m[c] = max(m[c], (uint32_t)__shfl_xor((int)m[c], off, kWave));
+                        if (lane == 0) red_amax[wave][c] = m[c];
+                    }
+                    __syncthreads();
+#pragma unroll
+                    for (int c = 0; c < kSegBatch; c++)
+                        if (c < p.batch) cur_ex[c] = exponent_of(c);
+                }
+                const int items = pieces * p.batch;
+                for (int base = 0; base < items; base += kFlat * kThreads) {
+                    uint4 kp[kFlat];
+#pragma unroll
+                    for (int k = 0; k < kFlat; k++) {
+                        const int item = base + stid + k * kThreads;
+                        const int b = column_of(item, pieces);
+                        kp[k] = item < items ? piece_of(b, item - b * pieces) : uint4{0u, 0u, 0u, 0u};
+                    }
+#pragma unroll
+                    for (int k = 0; k < kFlat; k++) {
+                        const int item = base + stid + k * kThreads;
+                        const int b = column_of(item, pieces);
+                        int ex = cur_ex[0];
+#pragma unroll
+                        for (int c = 1; c < kSegBatch; c++) ex = b == c ? cur_ex[c] : ex;
+                        if (item < items) write_piece(image + (size_t)b * img_stride, item - b * pieces, kp[k], ex);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
                 }
             }
             __syncthreads();
@@ -1069,11 +1099,25 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
     }
     // Up to this many activation rows the tall-tile MFMA kernel is the faster of the two (8B and 70B
     // sweeps: +17 % at two rows, +13 % at three, +5 % at four). TLLM_TALL_MAX_BATCH overrides.
-    static const int tall_max_batch = [] {
-        const char *e = getenv("TLLM_TALL_MAX_BATCH");
-        return e ? atoi(e) : 4;
-    }();
-    if (all_batch && !(all_tall && max_batch <= tall_max_batch)) {
+    // (both variables are read at every plan creation, not once per process)
+    const char *env_batch = getenv("TLLM_TALL_MAX_BATCH");
+    const int tall_max_batch = env_batch ? atoi(env_batch) : 4;
+    // ... for plans large enough: its units (192 rows of one matrix) are what spans are cut in, and a
+    // unit of a long-row matrix must stay well below a workgroup's share of the plan (8B shapes: the
+    // tall tiles win from 24 layers on, share 3.7, and lose below 16, share 2.5; 70B: lose at 8
+    // layers, share 2.4, win at 20). TLLM_TALL_MIN_SHARE overrides the ratio.
+    bool tall_pays = all_tall && max_batch <= tall_max_batch;
+    if (tall_pays) {
+        int64_t total = 0, heaviest = 0;
+        for (const Problem &p : host) {
+            total += (int64_t)p.rows * p.cols;
+            heaviest = std::max<int64_t>(heaviest, (int64_t)range_unit<Tall>() * p.cols);
+        }
+        const char *env_share = getenv("TLLM_TALL_MIN_SHARE");
+        const double min_share = env_share ? atof(env_share) : 3.5;
+        tall_pays = (double)total / (Tall::kWgPerCu * di->cus) >= min_share * (double)heaviest;
+    }
+    if (all_batch && !tall_pays) {
         d.batch_kernel = true;
         partition_blocks(gemv_batch_block_rows(), di->cus);
     } else {

@@ -389,6 +389,36 @@ def test_batched_plan_8b_layer_batch4_and_16(dev, oracle):
 
 
 
+@pytest.mark.parametrize("batch", [2, 3, 4])
+def test_tall_tile_plan_with_batch_columns(dev, oracle, batch, monkeypatch):
+    """Plans of two to four activation rows on the tall-tile MFMA kernel (large plans take it by
+    themselves; a small one is made to here): several batch columns in one operand image, rows of
+    14336 and 36864 columns staged in segments, rows that are not whole slices, two launches."""
+    torch, tl = dev
+    monkeypatch.setenv("TLLM_TALL_MIN_SHARE", "0")
+    shapes = [(700, 4096), (128, 4096), (1800, 4096), (520, 14336), (100, 36864), (300, 1152), (64, 512)]
+    probs, host = [], []
+    for k, (rows, cols) in enumerate(shapes):
+        nz, sg, s, _ = synth.problem(9100 + k, rows, cols, dontcare_sign=True)
+        x = synth.acts_f16(np.random.default_rng(9200 + k + batch), batch, cols)
+        y = torch.full((batch, rows), float("nan"), dtype=torch.float16, device="cuda")
+        probs.append((up(torch, nz), up(torch, sg), up(torch, s), up(torch, x), y, rows, cols, batch))
+        host.append((nz, sg, s, x))
+    plan = tl.LinearPlan(probs)
+    for launch in range(2):
+        for pr in probs:
+            pr[4].fill_(float("nan"))
+        plan.launch()
+        torch.cuda.synchronize()
+        for k, (pr, (nz, sg, s, x)) in enumerate(zip(probs, host)):
+            got = pr[4].cpu().numpy().astype(np.float64)
+            rows_s = np.unique(np.random.default_rng(k).integers(0, nz.shape[0], 48))
+            ref = oracle.gemm_f64(x.view(np.uint16), nz[rows_s], sg[rows_s], s[rows_s].view(np.uint16))
+            assert np.isfinite(got).all()
+            assert_close(oracle, got[:, rows_s], ref, what=f"tall plan batch {batch} problem {k}")
+    plan.close()
+
+
 # ------------------------------------------------------------- element-wise
 def _half_out(oracle, ref):
     """fp16 rounding of an fp64 reference, as float64 (for a 1-ulp comparison)."""

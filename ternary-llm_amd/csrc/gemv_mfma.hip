@@ -48,9 +48,9 @@ constexpr int kNW = 4;  // waves per workgroup
 // Most slices of a row (wide tiles: 2048 columns each) whose operand image is in LDS at one time;
 // longer rows are staged and walked in segments. 8 slices = 32 KB keep three workgroups on a CU.
 constexpr int kSegSlices = 8;
-// The same limit for tall tiles, in slices of 512 columns: 16384 elements of all batch columns
-// together, half of that at four columns (there the partial sums need the room more: measured).
-__host__ __device__ constexpr int tall_seg_slices(int batch) { return (batch >= 4 ? 8192 : 16384) / 512 / batch; }
+// The limit for tall tiles, in slices of 512 columns: 8192 elements of all batch columns together
+// (16 KB; the partial sums need the room more).
+__host__ __device__ constexpr int tall_seg_slices(int batch) { return 8192 / 512 / batch; }
 constexpr int kThreads = kNW * kWave;
 constexpr int kMaxBatch = 4;  // activation rows the tall tiles carry
 #ifndef TLLM_TILES_AHEAD
@@ -62,7 +62,7 @@ struct Wide {
     static constexpr int kCols = 2048, kRows = 4, kChunks = 16, kScales = 1, kWgPerCu = 3;
 };
 struct Tall {
-    static constexpr int kCols = 512, kRows = 16, kChunks = 4, kScales = 4, kWgPerCu = 2;
+    static constexpr int kCols = 512, kRows = 16, kChunks = 4, kScales = 4, kWgPerCu = 3;
 };
 
 // Work is counted in units of kNW * kRows * kTilesAhead rows of one matrix. A workgroup owns a
@@ -750,9 +750,10 @@ struct DeviceInfo {
 };
 
 constexpr int kLdsLimit = 64 * 1024;  // per workgroup; 160 KB per CU leaves room for two or three
-// The tall-tile instance runs two workgroups per CU (register need) and keeps one partial sum per
-// wave, row and batch column: it gets all the LDS two workgroups can have.
-constexpr int kTallLdsLimit = 78 * 1024;
+// The tall-tile instance keeps one partial sum per wave, row and batch column: it gets all the LDS
+// that three workgroups per CU can have (three resident workgroups beat two with 78 KB each: +4.5 %
+// at four batch columns, equal at two and three).
+constexpr int kTallLdsLimit = 53 * 1024;
 
 template <class G, bool kExtras = false, bool kFine = false>
 const void *kernel_ptr() {
@@ -1103,9 +1104,9 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
     const char *env_batch = getenv("TLLM_TALL_MAX_BATCH");
     const int tall_max_batch = env_batch ? atoi(env_batch) : 4;
     // ... for plans large enough: its units (192 rows of one matrix) are what spans are cut in, and a
-    // unit of a long-row matrix must stay well below a workgroup's share of the plan (8B shapes: the
-    // tall tiles win from 24 layers on, share 3.7, and lose below 16, share 2.5; 70B: lose at 8
-    // layers, share 2.4, win at 20). TLLM_TALL_MIN_SHARE overrides the ratio.
+    // unit of a long-row matrix must not outweigh a workgroup's share of the plan by much (8B shapes:
+    // the tall tiles win from 12 layers on, share 1.2, and lose at 8; 70B: lose at 8 layers, share
+    // 1.6, win at 20, share 4). TLLM_TALL_MIN_SHARE overrides the ratio.
     bool tall_pays = all_tall && max_batch <= tall_max_batch;
     if (tall_pays) {
         int64_t total = 0, heaviest = 0;
@@ -1114,7 +1115,7 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
             heaviest = std::max<int64_t>(heaviest, (int64_t)range_unit<Tall>() * p.cols);
         }
         const char *env_share = getenv("TLLM_TALL_MIN_SHARE");
-        const double min_share = env_share ? atof(env_share) : 3.5;
+        const double min_share = env_share ? atof(env_share) : 2.0;
         tall_pays = (double)total / (Tall::kWgPerCu * di->cus) >= min_share * (double)heaviest;
     }
     if (all_batch && !tall_pays) {

@@ -312,8 +312,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
     }
 
     // ---- split K: every workgroup of a tile leaves its fp32 sums in its own slot; the one that
-    // arrives last adds all slots in split order (its own included, read back: the result does not
-    // depend on who is last) and stores. The slots are written with stores that go through to memory
+    // arrives last adds all slots in split order (its own from its registers, in its place of the
+    // order: the result does not depend on who is last) and stores. The slots are written with stores that go through to memory
     // (sc1) and are acknowledged (s_waitcnt vmcnt(0)) before the workgroup counts as arrived; the
     // reader drops what its L2 may still hold of the slots (acquire fence = invalidate, cheap) and
     // then reads them with ordinary 16-byte loads. A release fence instead of the write-through
@@ -343,13 +343,24 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
         if (!last_arrival) return;
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
         const float *slots = partial + (size_t)tile * splits * kSlot + tid * 4;
+        // the sums of this workgroup stay in registers: its own slot is not read back (same values)
+        f16v own[kNF][MF];
 #pragma unroll
         for (int i = 0; i < kNF; i++)
 #pragma unroll
-            for (int j = 0; j < MF; j++)
+            for (int j = 0; j < MF; j++) {
+                own[i][j] = acc[i][j];
 #pragma unroll
                 for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+            }
         for (int q = 0; q < splits; q++) {
+            if (q == split) {
+#pragma unroll
+                for (int i = 0; i < kNF; i++)
+#pragma unroll
+                    for (int j = 0; j < MF; j++) acc[i][j] += own[i][j];
+                continue;
+            }
             const float *slot = slots + (size_t)q * kSlot;
 #pragma unroll
             for (int i = 0; i < kNF; i++)

@@ -249,23 +249,28 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
             asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kDma + 6) : "memory");
             read_masks(w, (u + 2) % kBufs, s + 2);
             read_w(af1, u, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_row(af0[1], bf0, 1);
+            __builtin_amdgcn_sched_barrier(0);
             read_a(bf1, u, 1);
             dma_acts((u + 2) % kBufs, s + 2, 0, kQ);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int i = 1; i < kNF; i++) mfma_row(af0[i], bf0, i);
+            for (int i = 2; i < kNF; i++) mfma_row(af0[i], bf0, i);
             __builtin_amdgcn_sched_barrier(0);
             // ---- step 1 (af1/bf1): decode starts
             mfma_row(af1[0], bf1, 0);
             __builtin_amdgcn_sched_barrier(0);
             read_w(af0, u, 2);
             read_a(bf0, u, 2);
-            dma_acts((u + 2) % kBufs, s + 2, kQ, 2 * kQ);
-            d.begin(w.nz, w.sg, scale_of(w));
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 1; i < kNF; i++) {
                 mfma_row(af1[i], bf1, i);
+                if (i == 1) {
+                    dma_acts((u + 2) % kBufs, s + 2, kQ, 2 * kQ);
+                    d.begin(w.nz, w.sg, scale_of(w));
+                }
 #pragma unroll
                 for (int dw = 2 * (i - 1); dw < 2 * i; dw++) o[dw] = d.dword(dw);
                 __builtin_amdgcn_sched_barrier(0);
@@ -277,13 +282,15 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
             __builtin_amdgcn_sched_barrier(0);
             read_w(af1, u, 3);
             read_a(bf1, u, 3);
-            dma_acts((u + 2) % kBufs, s + 2, 2 * kQ, 3 * kQ);
-            *reinterpret_cast<u4 *>(Ws + (w_off ^ (0 << 4))) = u4{o[0], o[1], o[2], o[3]};
-            *reinterpret_cast<u4 *>(Ws + (w_off ^ (1 << 4))) = u4{o[4], o[5], o[6], o[7]};
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 1; i < kNF; i++) {
                 mfma_row(af0[i], bf0, i);
+                if (i == 1) {
+                    dma_acts((u + 2) % kBufs, s + 2, 2 * kQ, 3 * kQ);
+                    *reinterpret_cast<u4 *>(Ws + (w_off ^ (0 << 4))) = u4{o[0], o[1], o[2], o[3]};
+                    *reinterpret_cast<u4 *>(Ws + (w_off ^ (1 << 4))) = u4{o[4], o[5], o[6], o[7]};
+                }
 #pragma unroll
                 for (int dw = 6 + 2 * i; dw < 8 + 2 * i; dw++) o[dw] = d.dword(dw);
                 __builtin_amdgcn_sched_barrier(0);
@@ -296,6 +303,9 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
             *reinterpret_cast<u4 *>(Ws + (w_off ^ (2 << 4))) = u4{o[8], o[9], o[10], o[11]};
             *reinterpret_cast<u4 *>(Ws + (w_off ^ (3 << 4))) = u4{o[12], o[13], o[14], o[15]};
             read_w(af0, (u + 1) % kBufs, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_row(af1[1], bf1, 1);
+            __builtin_amdgcn_sched_barrier(0);
             dma_acts((u + 2) % kBufs, s + 2, 3 * kQ, kDma);
             // the activations of stage s+1 were requested during stage s-1; newer requests: the masks
             // of that stage (3) and this stage's activations (kDma)
@@ -303,7 +313,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
             read_a(bf0, (u + 1) % kBufs, 0);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int i = 1; i < kNF; i++) mfma_row(af1[i], bf1, i);
+            for (int i = 2; i < kNF; i++) mfma_row(af1[i], bf1, i);
             __builtin_amdgcn_sched_barrier(0);
             dma_masks((u + 2) % kBufs, s + 5);
             // plain barrier: a fence here would also wait for the requests in flight

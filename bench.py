@@ -46,14 +46,6 @@ def layer_matrices(model):
             ("gate_proj", ffn, h), ("up_proj", ffn, h), ("down_proj", h, ffn)]
 
 
-def plan_kernel(batch):
-    """The kernel a plan of the sweep's shapes runs at this many activation rows per matrix."""
-    if batch == 1:
-        return "tllm::gemv_mfma_kernel<Wide>"
-    return "tllm::gemv_mfma_kernel<Tall>" if batch <= int(os.environ.get("TLLM_TALL_MAX_BATCH", "4")) \
-        else "tllm::gemv_batch_kernel"
-
-
 def packed_bytes(rows, cols, group=128):
     return rows * (cols // 32) * 8 + rows * (cols // group) * 2
 
@@ -400,7 +392,7 @@ def main():
             "bound": "hbm", "achieved": round(gbps, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(gbps / HBM_PEAK_GBS, 4),
             "traffic": DEFAULT_WORKLOAD_TRAFFIC_BYTES if default_workload else None,
-            "kernel": plan_kernel(args.batch) if args.mode == "plan" else "per-matrix launches",
+            "kernel": plan.kernel if args.mode == "plan" else "per-matrix launches",
             "bytes_per_launch": sweep_bytes // launches_per_step,
         },
     }
@@ -432,7 +424,7 @@ def main():
         par_b = check_sample(orc, probs_b, [i for i in sample_idx if i < len(probs_b)])
         out["other_batches"].append({"batch": b, "ms_per_step": round(ms_b, 5), "GBps": round(gb, 2),
                                      "frac_hbm_peak": round(gb / HBM_PEAK_GBS, 4),
-                                     "kernel": plan_kernel(b), "parity_max_rel_sampled": par_b})
+                                     "kernel": plan_b.kernel, "parity_max_rel_sampled": par_b})
         plan_b.close()
         del probs_b
     if args.decode_chain and not CUSTOM and args.batch == 1:

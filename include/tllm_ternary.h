@@ -210,6 +210,10 @@ int tllm_linear_plan_create_normed(tllm_linear_plan **plan, const tllm_linear_pr
 int tllm_linear_plan_launch(const tllm_linear_plan *plan, tllm_stream_t stream);
 /* Algorithmic weight-stream bytes (masks + scales) one launch reads. */
 int64_t tllm_linear_plan_weight_bytes(const tllm_linear_plan *plan);
+/* Name of the kernel a launch of this plan runs (static string; for reports and profiles). The
+ * choice depends on the activation-row counts, the shapes and the size of the plan. No counterpart in
+ * the reference. */
+const char *tllm_linear_plan_kernel(const tllm_linear_plan *plan);
 void tllm_linear_plan_destroy(tllm_linear_plan *plan);
 
 #ifdef __cplusplus

@@ -869,7 +869,10 @@ double pool_fraction() {
     }();
     return f;
 }
-constexpr int64_t kPoolTaskWeights = 768 * 1024;
+#ifndef TLLM_POOL_TASK_WEIGHTS
+#define TLLM_POOL_TASK_WEIGHTS (768 * 1024)
+#endif
+constexpr int64_t kPoolTaskWeights = TLLM_POOL_TASK_WEIGHTS;
 // The same for the batched kernel, whose blocks are all independent (TLLM_BLOCK_POOL_FRACTION).
 double block_pool_fraction() {
     static const double f = [] {
@@ -968,7 +971,10 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
             all_units += units_in(host, i);
             min_cols = host[i].cols < min_cols ? host[i].cols : min_cols;
         }
-        if (max_task_units > 0 && all_units >= 8 * wgs) {
+        // no pool for plans that give a workgroup less than about two pool tasks of work: a quarter of
+        // the workgroups would then end with one more task than the rest (1B shapes, 16 layers: 54 us
+        // without the pool, 60.5 us with it; 8B shapes, 8 layers: 100 / 99 us)
+        if (max_task_units > 0 && all_units >= 8 * wgs && (double)all_w / wgs >= 2.3 * (double)kPoolTaskWeights) {
             const int64_t want = (int64_t)((double)all_w * pool_fraction());
             int64_t got = 0;
             int left_units = all_units;

@@ -18,6 +18,7 @@ ABI_SYMBOLS = (
     "tllm_linear_plan_create", "tllm_linear_plan_launch", "tllm_linear_plan_weight_bytes",
     "tllm_linear_plan_destroy", "tllm_rmsnorm_f16", "tllm_silu_mul_f16", "tllm_linear_plan_create_normed",
     "tllm_add_f16", "tllm_rope_f16", "tllm_embedding_lookup_f16", "tllm_copy_to_kv_cache_f16",
+    "tllm_linear_plan_kernel",
 )
 # include/tllm_model_file.h
 FILE_ABI_SYMBOLS = (
@@ -81,6 +82,8 @@ def lib():
     L.tllm_linear_plan_weight_bytes.argtypes = [vp]
     L.tllm_linear_plan_weight_bytes.restype = C.c_int64
     L.tllm_linear_plan_destroy.argtypes = [vp]
+    L.tllm_linear_plan_kernel.argtypes = [vp]
+    L.tllm_linear_plan_kernel.restype = C.c_char_p
     L.tllm_linear_plan_destroy.restype = None
     L.tllm_rmsnorm_f16.argtypes = [vp, vp, vp, vp, vp, i, i, f, vp]
     L.tllm_silu_mul_f16.argtypes = [vp, vp, vp, i, vp]
@@ -222,6 +225,11 @@ class LinearPlan:
     @property
     def weight_bytes(self):
         return int(lib().tllm_linear_plan_weight_bytes(self._h))
+
+    @property
+    def kernel(self):
+        """Name of the kernel a launch of this plan runs."""
+        return lib().tllm_linear_plan_kernel(self._h).decode()
 
     def launch(self, stream=None):
         check(lib().tllm_linear_plan_launch(self._h, _stream(stream)))

@@ -878,7 +878,7 @@ def test_swiglu_pairs_in_a_layer_sweep(dev, oracle):
 
 
 def test_linear_plan_large_sweep_shared_pool(dev, oracle):
-    """A plan big enough (16 LLaMA-1B layers, 112 matrices) that part of it is dealt out at run time
+    """A plan big enough (32 LLaMA-1B layers, 224 matrices) that part of it is dealt out at run time
     instead of belonging to a fixed span: whichever workgroup takes a piece, every output must equal
     the single-call result bit for bit, on every launch (the hand-out counters reset themselves)."""
     torch, tl = dev
@@ -886,7 +886,7 @@ def test_linear_plan_large_sweep_shared_pool(dev, oracle):
     gen = torch.Generator(device="cuda")
     gen.manual_seed(4242)
     probs = []
-    for layer in range(16):
+    for layer in range(32):
         for rows, cols in shapes:
             nz = torch.randint(-2**31, 2**31 - 1, (rows, cols // 32), dtype=torch.int32, device="cuda", generator=gen)
             sg = torch.randint(-2**31, 2**31 - 1, (rows, cols // 32), dtype=torch.int32, device="cuda", generator=gen)
@@ -927,7 +927,7 @@ def test_large_plan_in_a_captured_graph(dev, oracle):
     gen = torch.Generator(device="cuda")
     gen.manual_seed(777)
     probs = []
-    for layer in range(16):
+    for layer in range(32):   # large enough for the run-time hand-out of its tail
         for rows, cols in shapes:
             nz = torch.randint(-2**31, 2**31 - 1, (rows, cols // 32), dtype=torch.int32, device="cuda", generator=gen)
             sg = torch.randint(-2**31, 2**31 - 1, (rows, cols // 32), dtype=torch.int32, device="cuda", generator=gen)

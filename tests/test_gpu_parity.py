@@ -405,6 +405,7 @@ def test_tall_tile_plan_with_batch_columns(dev, oracle, batch, monkeypatch):
         probs.append((up(torch, nz), up(torch, sg), up(torch, s), up(torch, x), y, rows, cols, batch))
         host.append((nz, sg, s, x))
     plan = tl.LinearPlan(probs)
+    assert plan.kernel == "tllm::gemv_mfma_kernel<Tall>"
     for launch in range(2):
         for pr in probs:
             pr[4].fill_(float("nan"))
@@ -416,6 +417,31 @@ def test_tall_tile_plan_with_batch_columns(dev, oracle, batch, monkeypatch):
             ref = oracle.gemm_f64(x.view(np.uint16), nz[rows_s], sg[rows_s], s[rows_s].view(np.uint16))
             assert np.isfinite(got).all()
             assert_close(oracle, got[:, rows_s], ref, what=f"tall plan batch {batch} problem {k}")
+    plan.close()
+
+
+def test_tall_tile_plan_with_mixed_batch_sizes(dev, oracle, monkeypatch):
+    """One plan whose problems carry one to four activation rows each, on the tall-tile kernel: the
+    segment length and the operand image depend on the problem's own batch size."""
+    torch, tl = dev
+    monkeypatch.setenv("TLLM_TALL_MIN_SHARE", "0")
+    shapes = [(700, 4096, 1), (300, 14336, 3), (520, 8192, 4), (200, 36864, 2), (64, 512, 4), (900, 18432, 1)]
+    probs, host = [], []
+    for k, (rows, cols, batch) in enumerate(shapes):
+        nz, sg, s, _ = synth.problem(9300 + k, rows, cols, dontcare_sign=True)
+        x = synth.acts_f16(np.random.default_rng(9400 + k), batch, cols)
+        y = torch.full((batch, rows), float("nan"), dtype=torch.float16, device="cuda")
+        probs.append((up(torch, nz), up(torch, sg), up(torch, s), up(torch, x), y, rows, cols, batch))
+        host.append((nz, sg, s, x))
+    plan = tl.LinearPlan(probs)
+    assert plan.kernel == "tllm::gemv_mfma_kernel<Tall>"
+    for launch in range(2):
+        plan.launch()
+        torch.cuda.synchronize()
+        for k, (pr, (nz, sg, s, x)) in enumerate(zip(probs, host)):
+            got = pr[4].cpu().numpy().astype(np.float64)
+            ref = oracle.gemm_f64(x.view(np.uint16), nz, sg, s.view(np.uint16))
+            assert_close(oracle, got, ref, what=f"mixed-batch tall plan problem {k}")
     plan.close()
 
 

@@ -259,7 +259,7 @@ const char *tllm_linear_plan_kernel(const tllm_linear_plan *plan) {
     const tllm::PlanDevice &d = plan->dev;
     if (d.batch_kernel) return "tllm::gemv_batch_kernel";
     if (!d.use_mfma) return "tllm::gemv_rowwave_f16_table_kernel";
-    if (!d.wide) return "tllm::gemv_mfma_kernel<Tall>";
+    if (!d.wide) return d.fine ? "tllm::gemv_mfma_kernel<Tall, fine>" : "tllm::gemv_mfma_kernel<Tall>";
     if (d.extras) return d.fine ? "tllm::gemv_mfma_kernel<Wide, extras, fine>" : "tllm::gemv_mfma_kernel<Wide, extras>";
     return d.fine ? "tllm::gemv_mfma_kernel<Wide, fine>" : "tllm::gemv_mfma_kernel<Wide>";
 }

@@ -232,9 +232,9 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
         }
         // Rows longer than kSegSlices slices are staged and walked in segments of equal length, so
         // that the operand image never takes more than kSegSlices slices of LDS (wide tiles only).
-        // (fine-grained instances: whole rows, the host sees to it that they fit)
+        // (fine-grained wide-tile instances: whole rows, the host sees to it that they fit)
         const int seg_max = G::kRows == 4 ? kSegSlices : tall_seg_slices(p.batch);
-        const int n_seg = kFine ? 1 : (slices + seg_max - 1) / seg_max;
+        const int n_seg = kFine && G::kRows == 4 ? 1 : (slices + seg_max - 1) / seg_max;
         const int seg_len = (slices + n_seg - 1) / n_seg;
 
         const int r_begin = task_first_row;
@@ -398,7 +398,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                     if (c8 < pieces) write_piece(image, c8, keep[k], ex);
                     __builtin_amdgcn_sched_barrier(0);  // one piece at a time: keeps the register need low
                 }
-            } else if constexpr (kFine) {
+            } else if constexpr (kFine && G::kRows == 4) {
                 // a whole row too long for the registers (the fine-grained instances do not stage in
                 // segments): one pass for the magnitude, one for the image, piece by piece
                 uint32_t m = 0;
@@ -771,9 +771,11 @@ hipError_t prepare_device(DeviceInfo **out) {
         static std::mutex init_mutex;
         std::lock_guard<std::mutex> lock(init_mutex);
         for (const void *k : {kernel_ptr<Wide>(), kernel_ptr<Tall>(), kernel_ptr<Wide, true>(),
-                              kernel_ptr<Wide, false, true>(), kernel_ptr<Wide, true, true>()})
-            if (hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                   k == kernel_ptr<Tall>() ? kTallLdsLimit : kLdsLimit))
+                              kernel_ptr<Wide, false, true>(), kernel_ptr<Wide, true, true>(),
+                              kernel_ptr<Tall, false, true>()})
+            if (hipError_t e = hipFuncSetAttribute(
+                    k, hipFuncAttributeMaxDynamicSharedMemorySize,
+                    k == kernel_ptr<Tall>() || k == kernel_ptr<Tall, false, true>() ? kTallLdsLimit : kLdsLimit))
                 return e;
         info[dev].cus = current_device_cus();
         ready[dev].store(true, std::memory_order_release);
@@ -796,6 +798,7 @@ constexpr int range_unit() {  // rows: every wave walks whole groups of kTilesAh
     return kNW * G::kRows * kTilesAhead;
 }
 constexpr int kFineUnit = kNW * Wide::kRows;  // rows of a unit of the fine-grained instances: one tile per wave
+constexpr int kTallFineUnit = kNW * Tall::kRows;
 // A launch whose 48-row units would fill less than half of the workgroup slots of the chip runs in
 // units of 16 rows instead (wide tiles only): three times the workgroups, a third of the tiles each.
 bool wants_fine(int64_t coarse_units, int slots) { return coarse_units * 2 <= slots; }
@@ -1113,16 +1116,22 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
     // unit of a long-row matrix must not outweigh a workgroup's share of the plan by much (8B shapes:
     // the tall tiles win from 12 layers on, share 1.2, and lose at 8; 70B: lose at 8 layers, share
     // 1.6, win at 20, share 4). TLLM_TALL_MIN_SHARE overrides the ratio.
-    bool tall_pays = all_tall && max_batch <= tall_max_batch;
+    // Medium plans take the tall tiles in units of 64 rows (one tile per wave) when a share is at least
+    // 3.5 of those (8B shapes at 12 layers, share 3.7: +16 % at two rows, +9 % at three; 70B at 8
+    // layers, share 4.9: +18 % / +8 %; shares of 2.5 and less lose against the batched kernel).
+    bool tall_pays = all_tall && max_batch <= tall_max_batch, tall_fine = false;
     if (tall_pays) {
-        int64_t total = 0, heaviest = 0;
+        int64_t total = 0;
+        int max_cols = 0;
         for (const Problem &p : host) {
             total += (int64_t)p.rows * p.cols;
-            heaviest = std::max<int64_t>(heaviest, (int64_t)range_unit<Tall>() * p.cols);
+            max_cols = std::max(max_cols, (int)p.cols);
         }
         const char *env_share = getenv("TLLM_TALL_MIN_SHARE");
         const double min_share = env_share ? atof(env_share) : 2.0;
-        tall_pays = (double)total / (Tall::kWgPerCu * di->cus) >= min_share * (double)heaviest;
+        const double share = (double)total / (Tall::kWgPerCu * di->cus);
+        tall_pays = share >= min_share * (double)range_unit<Tall>() * max_cols;
+        if (!tall_pays) tall_pays = tall_fine = share >= 1.75 * min_share * (double)kTallFineUnit * max_cols;
     }
     if (all_batch && !tall_pays) {
         d.batch_kernel = true;
@@ -1141,11 +1150,12 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
             d.fine = whole + kNW * kFineUnit * 4 * (has_pairs ? 2 : 1) <= kLdsLimit &&
                      wants_fine(coarse, Wide::kWgPerCu * di->cus);
         }
+        if (!d.wide) d.fine = tall_fine;
         for (const Problem &p : host) {
             const int ib = d.wide ? image_bytes_of<Wide>(p.cols, 1, !d.fine) : image_bytes_of<Tall>(p.cols, p.batch);
             max_image = ib > max_image ? ib : max_image;
         }
-        const int unit = d.fine ? kFineUnit : d.wide ? range_unit<Wide>() : range_unit<Tall>();
+        const int unit = d.wide ? (d.fine ? kFineUnit : range_unit<Wide>()) : (d.fine ? kTallFineUnit : range_unit<Tall>());
         const int mats = has_pairs ? 2 : 1;
         const int max_units = max_units_for(max_image, max_batch, unit, mats, d.wide ? kLdsLimit : kTallLdsLimit);
         if (max_units < 1) d.use_mfma = false;
@@ -1154,8 +1164,9 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
             d.lds_bytes = max_image + kNW * max_units * unit * max_batch * 4 * mats;
             const int per_cu = d.extras && d.fine ? resident_wgs<Wide, true, true>(d.lds_bytes)
                                : d.extras         ? resident_wgs<Wide, true>(d.lds_bytes)
-                               : d.fine           ? resident_wgs<Wide, false, true>(d.lds_bytes)
+                               : d.wide && d.fine ? resident_wgs<Wide, false, true>(d.lds_bytes)
                                : d.wide           ? resident_wgs<Wide>(d.lds_bytes)
+                               : d.fine           ? resident_wgs<Tall, false, true>(d.lds_bytes)
                                                   : resident_wgs<Tall>(d.lds_bytes);
             partition(unit, per_cu * di->cus, max_units);
             d.max_units = max_units;
@@ -1214,8 +1225,10 @@ hipError_t plan_device_launch(const PlanDevice &plan, hipStream_t s) {
         gemv_mfma_kernel<Wide, true, true><<<plan.grid, kThreads, plan.lds_bytes, s>>>(none, sc);
     else if (plan.extras)
         gemv_mfma_kernel<Wide, true><<<plan.grid, kThreads, plan.lds_bytes, s>>>(none, sc);
-    else if (plan.fine)
+    else if (plan.fine && plan.wide)
         gemv_mfma_kernel<Wide, false, true><<<plan.grid, kThreads, plan.lds_bytes, s>>>(none, sc);
+    else if (plan.fine)
+        gemv_mfma_kernel<Tall, false, true><<<plan.grid, kThreads, plan.lds_bytes, s>>>(none, sc);
     else if (plan.wide)
         gemv_mfma_kernel<Wide><<<plan.grid, kThreads, plan.lds_bytes, s>>>(none, sc);
     else

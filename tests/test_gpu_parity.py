@@ -420,6 +420,35 @@ def test_tall_tile_plan_with_batch_columns(dev, oracle, batch, monkeypatch):
     plan.close()
 
 
+def test_tall_tile_plan_in_fine_units(dev, oracle, monkeypatch):
+    """A plan of two activation rows sized so that the tall tiles run in units of 64 rows (a share
+    per workgroup of more than 3.5 and less than 6 such units): whole output against the batched
+    kernel's single calls within tolerance, sampled rows against the oracle."""
+    torch, tl = dev
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(99)
+    batch, probs = 2, []
+    for rows, cols in [(30000, 4096)] * 12 + [(9000, 14336)] * 6 + [(30000, 4096)] * 12:
+        w = _rand_weight(torch, gen, rows, cols)
+        x = torch.randn((batch, cols), device="cuda", generator=gen).to(torch.float16)
+        y = torch.full((batch, rows), float("nan"), dtype=torch.float16, device="cuda")
+        probs.append((*w, x, y, rows, cols, batch))
+    plan = tl.LinearPlan(probs)
+    assert plan.kernel == "tllm::gemv_mfma_kernel<Tall, fine>", plan.kernel
+    for launch in range(2):
+        plan.launch()
+    torch.cuda.synchronize()
+    pick_rng = np.random.default_rng(7)
+    for k in (0, 13, 16, 29):
+        nz, sg, sc, x, y, rows, cols, b = probs[k]
+        assert torch.isfinite(y).all()
+        pick = pick_rng.integers(0, rows, 64)
+        ref = oracle.gemm_f64(x.cpu().numpy().view(np.uint16), nz[pick].cpu().numpy().view(np.uint32),
+                              sg[pick].cpu().numpy().view(np.uint32), sc[pick].cpu().numpy().view(np.uint16))
+        assert_close(oracle, y[:, pick].cpu().numpy().astype(np.float64), ref, what=f"fine tall plan problem {k}")
+    plan.close()
+
+
 def test_tall_tile_plan_with_mixed_batch_sizes(dev, oracle, monkeypatch):
     """One plan whose problems carry one to four activation rows each, on the tall-tile kernel: the
     segment length and the operand image depend on the problem's own batch size."""

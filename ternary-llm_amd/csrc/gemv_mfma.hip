@@ -799,9 +799,10 @@ constexpr int range_unit() {  // rows: every wave walks whole groups of kTilesAh
 }
 constexpr int kFineUnit = kNW * Wide::kRows;  // rows of a unit of the fine-grained instances: one tile per wave
 constexpr int kTallFineUnit = kNW * Tall::kRows;
-// A launch whose 48-row units would fill less than half of the workgroup slots of the chip runs in
-// units of 16 rows instead (wide tiles only): three times the workgroups, a third of the tiles each.
-bool wants_fine(int64_t coarse_units, int slots) { return coarse_units * 2 <= slots; }
+// A launch with fewer than six 48-row units per workgroup slot of the chip runs in units of 16 rows
+// instead: the spans end closer together (8B shapes, one launch for 1 / 2 / 4 layers: 24.9 -> 21.1,
+// 37.4 -> 33.2, 57.5 -> 49.2 us; at 8 layers, nine units per slot, the coarse units win again).
+bool wants_fine(int64_t coarse_units, int slots) { return coarse_units <= 6 * (int64_t)slots; }
 
 template <class G>
 int image_bytes_of(int cols, int batch, bool segmented = true) {

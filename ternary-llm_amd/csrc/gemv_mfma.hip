@@ -586,6 +586,9 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
             // lanes whose result row (li & 3) is odd / is 2 or 3 (wide tiles pick one of four D rows)
             const uint64_t odd_lanes = __builtin_amdgcn_ballot_w64((li & 1) != 0);
             const uint64_t hi_lanes = __builtin_amdgcn_ballot_w64((li & 2) != 0);
+            // tall tiles: the lane adds the results of rows 4 lq + v, batch column bcol, if it is the first of its quad
+            const bool adds = (li & 3) == 0 && bcol < p.batch;
+            float *part_lane = my_part + 4 * lq * p.batch + bcol;
             auto process_tile = [&](const Tile<G> &t, int rb, bool live, const u4 (&B)[kMfmaPerTile], const f4 &bias,
                                     float bias_sel) {
                 f4 d0, d1;
@@ -613,11 +616,18 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                         x = dpp_add<kQuadSwap2>(x);
                         r[v] = x;
                     }
-                    if ((li & 3) == 0 && bcol < p.batch && live) {
+                    if (adds && live) {
+                        // rows 4 lq + v of the tile, column bcol: the lane's part of the address never
+                        // changes, the tile's part is wave-uniform
+                        float *row0 = part_lane + (rb - sh - r_begin) * p.batch;
+                        if (sh == 0) {
 #pragma unroll
-                        for (int v = 0; v < 4; v++)
-                            if (4 * lq + v >= sh)
-                                my_part[(size_t)(rb - sh - r_begin + 4 * lq + v) * p.batch + bcol] += r[v];
+                            for (int v = 0; v < 4; v++) row0[v * p.batch] += r[v];
+                        } else {
+#pragma unroll
+                            for (int v = 0; v < 4; v++)
+                                if (4 * lq + v >= sh) row0[v * p.batch] += r[v];
+                        }
                     }
                 }
             };

@@ -25,7 +25,10 @@
 //     sum over the stage is complete); operands come from LDS as 16-byte chunks, XOR-swizzled by
 //     row against bank conflicts.
 // Three LDS buffers per operand, one barrier per stage; the loop body spells out the pipeline.
+#include <stdlib.h>
+
 #include <mutex>
+#include <type_traits>
 
 #include "common.h"
 
@@ -47,7 +50,10 @@ constexpr int kNF = kBN / 32;       // MFMA row fragments (32 weight rows each) 
 constexpr int kWBytes = kBN * kRowBytes;
 
 // byte offset of 16-byte chunk c (0..7) of row r inside the [128][64] fp16 LDS tile
-__device__ __forceinline__ int chunk_off(int r, int c) { return r * kRowBytes + ((c ^ (r & 7)) << 4); }
+// The swizzle keeps a 16-byte fragment read free of bank conflicts both for 8 consecutive rows on 32 banks
+// and for 16 consecutive rows on 64 banks (rows r and r + 8 lie 1 KB apart: same bank either way).
+__device__ __forceinline__ int row_swizzle(int r) { return (r & 7) ^ ((r >> 3) & 1); }
+__device__ __forceinline__ int chunk_off(int r, int c) { return r * kRowBytes + ((c ^ row_swizzle(r)) << 4); }
 
 // Decoder of 32 weights (one mask word pair) into 16 dwords; dword d holds weights (2d, 2d + 1) as
 // +-2*scale / 0. Split in steps so that the caller can spread the work between MFMAs.
@@ -117,7 +123,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
 #pragma unroll
     for (int t = 0; t < kDma; t++) {
         const int gm = min(m0 + 8 * t + (lane >> 3), M - 1);
-        a_src[t] = (GB *)A + ((size_t)gm * K + k_begin + 8 * ((lane & 7) ^ (lane >> 3))) * 2;
+        a_src[t] = (GB *)A + ((size_t)gm * K + k_begin + 8 * ((lane & 7) ^ row_swizzle(8 * t + (lane >> 3)))) * 2;
     }
     // weights: row w_row, 32-column word w_word of the stage
     const int w_row = tid >> 1, w_word = tid & 1;
@@ -415,6 +421,367 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
     }
 }
 
+
+// ------------------------------------------------------------------------------------------------
+// Eight-wave instance: two waves per SIMD, so that the loads, the decode and the LDS stores of one
+// wave run under the MFMAs of the other. Same workgroup tile (128 weight rows x 128*MF activation
+// rows) and the same LDS image of a stage; wave (wm, nh) owns activation rows 32*MF*wm .. and the
+// weight rows 64*nh .. 64*nh+63 (a 64 x 32*MF tile: 2 x MF accumulator fragments). The activation
+// tile of a wm is shared by its two waves (each requests half of its rows), the mask words and
+// scales are requested by one wave and decoded by another, so everything that lands in LDS is
+// published by the one barrier per phase.
+//
+// Phases. All LDS reads of the data of stage s happen between barrier s and barrier s+1 ("phase
+// s"): the fragments of step 0 right after barrier s (under the last MFMAs of stage s-1), those of
+// steps 1..3 one step ahead of their MFMAs. With three buffers per operand a buffer is therefore
+// free for two whole phases before it is read again:
+//   phase s: requests the activations of stage s+2 and the masks of stage s+3 (both waited for at
+//            the end of phase s+1: in-order completion, vmcnt = this phase's own requests),
+//            decodes the masks of stage s+1 (published by barrier s) into weight buffer s+1.
+constexpr int kThreads8 = 512;
+
+template <int MF>
+__global__ __launch_bounds__(kThreads8, 1) void gemm_mfma8_kernel(
+    const uint16_t *__restrict__ A, const uint32_t *__restrict__ nzB, const uint32_t *__restrict__ sgB,
+    const uint16_t *__restrict__ scB, uint16_t *__restrict__ C, int M, int N, int K, int splits,
+    float *__restrict__ partial, unsigned *__restrict__ arrivals) {
+    constexpr int kWM = MF * 32;               // activation rows per wave pair
+    constexpr int BM = 4 * kWM;
+    constexpr int kActWave = kWM * kRowBytes;  // bytes of one pair's activation tile per stage
+    constexpr int kActBytes = 4 * kActWave;
+    constexpr int kActBase = kBufs * kWBytes;
+    constexpr int kMaskBase = kActBase + kBufs * kActBytes;
+    constexpr int kMaskBytes = 4 * 1024;       // nz words 1 KB | sign words 1 KB | scale dwords 8 x 256 B
+    constexpr int kDmaPair = kWM / 8;          // 1 KB activation loads per pair and stage
+    constexpr int kDma = kDmaPair / 2;         // ... per wave
+    constexpr int kReq = kDma + 2;             // requests a wave makes per phase
+    constexpr int kNF8 = 2;                    // weight-row fragments per wave
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    typedef __attribute__((address_space(3))) unsigned char LB;
+    LB *lds_dma = (LB *)lds;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave & 3, nh = wave >> 2;
+    const int li = lane & 31, lq = lane >> 5;
+
+    const int m_tiles = (M + BM - 1) / BM;
+    const int tile = blockIdx.x / splits, split = blockIdx.x - tile * splits;
+    const int n0 = (tile / m_tiles) * kBN;
+    const int m0 = (tile % m_tiles) * BM + wm * kWM;
+    const int words = K / 32, groups = K / 128;
+    const int g_begin = (int)((long)groups * split / splits), g_end = (int)((long)groups * (split + 1) / splits);
+    const int k_begin = g_begin * 128;
+    const int last = (g_end - g_begin) * 128 / kBK - 1;
+
+    typedef __attribute__((address_space(1))) const unsigned char GB;
+    // activations: this wave requests loads nh*kDma .. of its pair's tile (rows 8t .. 8t+7 each)
+    GB *a_src[kDma];
+#pragma unroll
+    for (int t = 0; t < kDma; t++) {
+        const int gm = min(m0 + 8 * (nh * kDma + t) + (lane >> 3), M - 1);
+        a_src[t] = (GB *)A + ((size_t)gm * K + k_begin + 8 * ((lane & 7) ^ row_swizzle(8 * (nh * kDma + t) + (lane >> 3)))) * 2;
+    }
+    // masks: waves 0-3 request the non-zero words, waves 4-7 the sign words; lane l of wave w asks for
+    // word (64 (w & 3) + l) of the stage = word (idx & 1) of weight row idx >> 1
+    const int midx = 64 * (wave & 3) + lane;
+    const int mrow = min(n0 + (midx >> 1), N - 1);
+    GB *m_src = (GB *)(nh ? sgB : nzB) + ((size_t)mrow * words + k_begin / 32 + (midx & 1)) * 4;
+    // scales: lane l of wave w asks for the aligned dword that holds the scale of weight row 16 w + (l & 15)
+    const int srow = min(n0 + 16 * wave + (lane & 15), N - 1);
+    const uintptr_t s_src = reinterpret_cast<uintptr_t>(scB) + ((size_t)srow * groups + g_begin) * 2;
+    // decode: thread t turns 16 weights of row t >> 2 (columns 16 (t & 3) .. of the stage) into two chunks
+    const int w_row = tid >> 2, w_qk = tid & 3;
+    const int w_gn = min(n0 + w_row, N - 1);
+    const int w_par = (int)(((size_t)w_gn * groups + g_begin) & 1);  // scale is the high half of its dword when (w_par + group) is odd
+    const uint32_t w_sel = (w_qk & 1) ? 0x07060302u : 0x05040100u;   // which 16 weights of the word
+    const int w_off = chunk_off(w_row, 2 * w_qk);
+    const int w_mask_off = (w_row * 2 + (w_qk >> 1)) * 4;
+    const int w_scale_off = 2048 + (w_row >> 4) * 256 + (w_row & 15) * 4;
+    const int fr_off = chunk_off(li, lq);
+
+    auto dma_masks = [&](int buf, int stage) {
+        const int k0 = min(stage, last) * kBK;
+        LB *dst = lds_dma + kMaskBase + buf * kMaskBytes;
+        __builtin_amdgcn_global_load_lds((__attribute__((address_space(1))) const void *)(m_src + k0 / 8),
+                                         (__attribute__((address_space(3))) void *)(dst + nh * 1024 + (wave & 3) * 256), 4, 0, 0);
+        const uintptr_t sc_addr = s_src + (k0 / 128) * 2;
+        __builtin_amdgcn_global_load_lds((__attribute__((address_space(1))) const void *)(sc_addr & ~(uintptr_t)3),
+                                         (__attribute__((address_space(3))) void *)(dst + 2048 + wave * 256), 4, 0, 0);
+    };
+    auto dma_acts = [&](int buf, int stage, int t_begin, int t_end) {
+        const int k0 = min(stage, last) * kBK;
+#pragma unroll
+        for (int t = t_begin; t < t_end; t++)
+            __builtin_amdgcn_global_load_lds(
+                (__attribute__((address_space(1))) const void *)(a_src[t] + k0 * 2),
+                (__attribute__((address_space(3))) void *)(lds_dma + kActBase + buf * kActBytes + wm * kActWave + (nh * kDma + t) * 1024),
+                16, 0, 0);
+    };
+    // 16 weights -> 8 dwords (two chunks) of +-2*scale / 0, see Decoder above
+    struct Decoder16 {
+        uint32_t q;
+        h2 sp;
+        __device__ __forceinline__ void begin(uint32_t nz, uint32_t sg, uint32_t scale, uint32_t sel) {
+            const uint32_t neg = nz & ~sg;
+            const uint32_t t0 = __builtin_amdgcn_bitop3_b32(neg << 1, nz, 0xAAAAAAAAu, 0xE4);
+            const uint32_t t1 = __builtin_amdgcn_bitop3_b32(neg, nz >> 1, 0xAAAAAAAAu, 0xE4);
+            q = __builtin_amdgcn_perm(t1, t0, sel);
+            sp = __builtin_bit_cast(h2, scale | (scale << 16));
+        }
+        __device__ __forceinline__ uint32_t dword(int d) const {
+            us2 v = __builtin_bit_cast(us2, q);
+            v = v << (uint16_t)(14 - 2 * d);
+            const uint32_t top = __builtin_bit_cast(uint32_t, v) & 0xC000C000u;
+            return __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, top) * sp);
+        }
+    };
+
+    f16v acc[kNF8][MF];
+#pragma unroll
+    for (int i = 0; i < kNF8; i++)
+#pragma unroll
+        for (int j = 0; j < MF; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+    auto mfma_row = [&](const u4 &a, const u4 (&bf)[MF], int i) {
+#pragma unroll
+        for (int j = 0; j < MF; j++)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, a), __builtin_bit_cast(h8, bf[j]),
+                                                               acc[i][j], 0, 0, 0);
+    };
+
+    // ---- prologue: masks of stages 0..2, activations of stages 0 and 1; weights of stage 0 decoded
+    Decoder16 d;
+    u4 af0[kNF8], af1[kNF8], bf0[MF], bf1[MF];
+#pragma unroll
+    for (int i = 0; i < kNF8; i++) af1[i] = u4{0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int j = 0; j < MF; j++) bf1[j] = u4{0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int u = 0; u < kBufs; u++) dma_masks(u, u);
+    dma_acts(0, 0, 0, kDma);
+    dma_acts(1, 1, 0, kDma);
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    {
+        const unsigned char *src = lds + kMaskBase;
+        const uint32_t nz = *reinterpret_cast<const uint32_t *>(src + w_mask_off);
+        const uint32_t sg = *reinterpret_cast<const uint32_t *>(src + 1024 + w_mask_off);
+        const uint32_t sd = *reinterpret_cast<const uint32_t *>(src + w_scale_off);
+        d.begin(nz, sg, (w_par & 1) ? sd >> 16 : sd & 0xFFFFu, w_sel);
+        *reinterpret_cast<u4 *>(lds + w_off) = u4{d.dword(0), d.dword(1), d.dword(2), d.dword(3)};
+        *reinterpret_cast<u4 *>(lds + (w_off ^ 16)) = u4{d.dword(4), d.dword(5), d.dword(6), d.dword(7)};
+    }
+
+    // In the loop every LDS instruction is written out and every wait for one names how many younger
+    // ones may still be in flight (they complete in order): the fragments of a step are requested
+    // one step ahead and a wait never includes the request made just before it. (Left to itself the
+    // compiler waits for the whole queue, lgkmcnt(0), in front of each consumer.)
+    const uint32_t lds0 = (uint32_t)(uintptr_t)lds_dma;
+    uint32_t fo[4];  // this lane's fragment offset in steps 0..3
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) fo[ks] = lds0 + (uint32_t)(fr_off ^ (ks << 5));
+    const uint32_t w_rd = (uint32_t)(nh * 64 * kRowBytes);                // + buf * kWBytes
+    const uint32_t a_rd = (uint32_t)(kActBase + wm * kActWave);          // + buf * kActBytes
+    const uint32_t m_rd = lds0 + (uint32_t)(kMaskBase + w_mask_off);     // imm: buf * kMaskBytes (+ 1024)
+    const uint32_t s_rd = lds0 + (uint32_t)(kMaskBase + w_scale_off);
+    const uint32_t w_wr0 = lds0 + (uint32_t)w_off, w_wr1 = lds0 + (uint32_t)(w_off ^ 16);  // imm: buf * kWBytes
+#define TLLM_LDS_READ128(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(off))
+#define TLLM_LDS_READ32(dst, addr, off) asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(off))
+#define TLLM_LDS_WRITE128(addr, val, off) asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(addr), "v"(val), "i"(off) : "memory")
+#define TLLM_LGKM(n) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(n) : "memory")
+    auto frags = [&](u4 (&af)[kNF8], u4 (&bf)[MF], int buf, int ks) {  // kNF8 + MF reads
+        const uint32_t aw = fo[ks] + (w_rd + (uint32_t)(buf * kWBytes));
+        const uint32_t aa = fo[ks] + (a_rd + (uint32_t)(buf * kActBytes));
+        TLLM_LDS_READ128(af[0], aw, 0);
+        TLLM_LDS_READ128(af[1], aw, 32 * kRowBytes);
+        TLLM_LDS_READ128(bf[0], aa, 0);
+        if constexpr (MF == 2) TLLM_LDS_READ128(bf[1], aa, 32 * kRowBytes);
+    };
+    constexpr int kFr = kNF8 + MF;  // LDS reads of one step
+
+    // one phase; the buffer index u = s % kBufs is a compile-time constant (it sits in instruction offsets)
+    auto phase = [&](auto U, const int s) {
+        constexpr int u = decltype(U)::value;
+        constexpr int kH = kDma / 2 > 0 ? kDma / 2 : 1;
+        constexpr int kNext = (u + 1) % kBufs;
+        uint32_t o[8];
+        uint32_t m_nz, m_sg, m_sc;
+        // barrier s: publishes the weights decoded and the loads waited for in the phase before
+        TLLM_LGKM(0);
+        asm volatile("s_barrier" ::: "memory");
+        frags(af0, bf0, u, 0);                                   // in flight: kFr
+        TLLM_LDS_READ32(m_nz, m_rd, kNext * kMaskBytes);
+        TLLM_LDS_READ32(m_sg, m_rd, kNext * kMaskBytes + 1024);
+        TLLM_LDS_READ32(m_sc, s_rd, kNext * kMaskBytes);         // kFr + 3
+        __builtin_amdgcn_sched_barrier(0);
+        // last step of the stage before (all zero operands in the first phase)
+        mfma_row(af1[0], bf1, 0);
+        mfma_row(af1[1], bf1, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        dma_acts((u + 2) % kBufs, s + 2, 0, kH);
+        // ---- step 0
+        TLLM_LGKM(3);                                            // fragments of step 0 are here
+        frags(af1, bf1, u, 1);                                   // 3 + kFr
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_row(af0[0], bf0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        TLLM_LGKM(kFr);                                          // mask words and scale are here
+        __builtin_amdgcn_sched_barrier(0);
+        {
+            const int odd = (w_par + min(s + 1, last) * kBK / 128) & 1;
+            d.begin(m_nz, m_sg, odd ? m_sc >> 16 : m_sc & 0xFFFFu, w_sel);
+        }
+        o[0] = d.dword(0);
+        o[1] = d.dword(1);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_row(af0[1], bf0, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (kDma > 1) dma_acts((u + 2) % kBufs, s + 2, kH, kDma);
+        o[2] = d.dword(2);
+        o[3] = d.dword(3);
+        // ---- step 1
+        __builtin_amdgcn_sched_barrier(0);
+        TLLM_LGKM(0);                                            // fragments of step 1
+        frags(af0, bf0, u, 2);                                   // kFr
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_row(af1[0], bf1, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        o[4] = d.dword(4);
+        o[5] = d.dword(5);
+        {
+            const u4 v = {o[0], o[1], o[2], o[3]};
+            TLLM_LDS_WRITE128(w_wr0, v, kNext * kWBytes);        // kFr + 1
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_row(af1[1], bf1, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        o[6] = d.dword(6);
+        o[7] = d.dword(7);
+        dma_masks(u, s + 3);
+        {
+            const u4 v = {o[4], o[5], o[6], o[7]};
+            TLLM_LDS_WRITE128(w_wr1, v, kNext * kWBytes);        // kFr + 2
+        }
+        // ---- step 2
+        __builtin_amdgcn_sched_barrier(0);
+        TLLM_LGKM(2);                                            // fragments of step 2
+        frags(af1, bf1, u, 3);                                   // 2 + kFr
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_row(af0[0], bf0, 0);
+        mfma_row(af0[1], bf0, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        // everything requested before this phase has landed
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kReq) : "memory");
+    };
+    for (int s0 = 0; s0 <= last; s0 += kBufs) {
+        phase(std::integral_constant<int, 0>{}, s0);
+        if (s0 + 1 > last) break;
+        phase(std::integral_constant<int, 1>{}, s0 + 1);
+        if (s0 + 2 > last) break;
+        phase(std::integral_constant<int, 2>{}, s0 + 2);
+    }
+    // last step of the last stage
+    TLLM_LGKM(0);
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_row(af1[0], bf1, 0);
+    mfma_row(af1[1], bf1, 1);
+#undef TLLM_LDS_READ128
+#undef TLLM_LDS_READ32
+#undef TLLM_LDS_WRITE128
+#undef TLLM_LGKM
+    // requests past the last stage are still in flight into LDS: let them land before the workgroup ends
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    if (splits > 1) {
+        constexpr int kSlot = BM * kBN;  // floats; element (c, tid, e) of a slot at (c * kThreads8 + tid) * 4 + e
+        float *mine = partial + ((size_t)tile * splits + split) * kSlot + tid * 4;
+#pragma unroll
+        for (int i = 0; i < kNF8; i++)
+#pragma unroll
+            for (int j = 0; j < MF; j++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const f4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                    float *dst = mine + (size_t)((i * MF + j) * 4 + g) * kThreads8 * 4;
+                    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(dst), "v"(v) : "memory");
+                }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __shared__ unsigned last_arrival8;
+        __syncthreads();
+        if (tid == 0) {
+            const unsigned before = __hip_atomic_fetch_add(&arrivals[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            last_arrival8 = before == (unsigned)splits - 1;
+            if (last_arrival8) __hip_atomic_store(&arrivals[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+        if (!last_arrival8) return;
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        const float *slots = partial + (size_t)tile * splits * kSlot + tid * 4;
+        // The slots are added in split order whoever arrives last; this workgroup's own sums take
+        // their place in that order from registers. All loads of a slot are in flight together.
+        f16v own[kNF8][MF];
+#pragma unroll
+        for (int i = 0; i < kNF8; i++)
+#pragma unroll
+            for (int j = 0; j < MF; j++) {
+                own[i][j] = acc[i][j];
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+            }
+        for (int q = 0; q < splits; q++) {
+            if (q == split) {
+#pragma unroll
+                for (int i = 0; i < kNF8; i++)
+#pragma unroll
+                    for (int j = 0; j < MF; j++) acc[i][j] += own[i][j];
+                continue;
+            }
+            const float *slot = slots + (size_t)q * kSlot;
+            f4 v[kNF8 * MF * 4];
+#pragma unroll
+            for (int c = 0; c < kNF8 * MF * 4; c++) v[c] = *reinterpret_cast<const f4 *>(slot + (size_t)c * kThreads8 * 4);
+#pragma unroll
+            for (int i = 0; i < kNF8; i++)
+#pragma unroll
+                for (int j = 0; j < MF; j++)
+#pragma unroll
+                    for (int g = 0; g < 4; g++)
+#pragma unroll
+                        for (int e = 0; e < 4; e++) acc[i][j][4 * g + e] += v[(i * MF + j) * 4 + g][e];
+        }
+    }
+
+    // ---- store: lane (k half lq, column li) of fragment (i, j) holds, for activation row m, the weight
+    // rows n0 + 64 nh + 32 i + 8 g + 4 lq + v in register 4 g + v
+    const bool vec_store = (N & 3) == 0 && (reinterpret_cast<uintptr_t>(C) & 7) == 0;
+#pragma unroll
+    for (int j = 0; j < MF; j++) {
+        const int m = m0 + j * 32 + li;
+        if (m >= M) continue;
+#pragma unroll
+        for (int i = 0; i < kNF8; i++) {
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int n = n0 + nh * 64 + i * 32 + 8 * g + 4 * lq;
+                uint16_t h[4];
+#pragma unroll
+                for (int v = 0; v < 4; v++) h[v] = f2h(acc[i][j][4 * g + v] * 0.5f);
+                uint16_t *dst = C + (size_t)m * N + n;
+                if (n + 3 < N && vec_store) {
+                    *reinterpret_cast<uint2 *>(dst) = uint2{(uint32_t)h[0] | ((uint32_t)h[1] << 16),
+                                                            (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 4; v++)
+                        if (n + v < N) dst[v] = h[v];
+                }
+            }
+        }
+    }
+}
+
 // Split-K workspace: fp32 slots and arrival counters, one set per (device, stream), created on the
 // first call that needs it and grown on demand (the only allocation this file makes; never during
 // a call that does not split). Calls on one stream run in order and so may share a set.
@@ -461,18 +828,32 @@ hipError_t split_workspace(hipStream_t s, size_t floats, size_t tiles, float **p
     return hipSuccess;
 }
 
+// TLLM_GEMM_WAVES=4 selects the four-wave instance (one wave per SIMD), for comparisons.
+bool use_eight_waves() {
+    static const bool v = [] {
+        const char *e = getenv("TLLM_GEMM_WAVES");
+        return !(e && e[0] == '4');
+    }();
+    return v;
+}
+
 template <int MF>
 hipError_t launch(const Problem &p, int splits, hipStream_t s) {
     constexpr int BM = 128 * MF;
-    static bool attr_set[64] = {};
+    static std::mutex attr_mutex;
+    static bool attr_set[64][2] = {};
     int dev = 0;
     if (hipError_t e = hipGetDevice(&dev)) return e;
-    const size_t lds = kBufs * (size_t)(kWBytes + BM * kRowBytes + 3 * 1024);
-    if (dev >= 0 && dev < 64 && !attr_set[dev]) {
-        if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_mfma_kernel<MF>),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
-            return e;
-        attr_set[dev] = true;
+    const bool eight = use_eight_waves();
+    const size_t lds = kBufs * (size_t)(kWBytes + BM * kRowBytes + (eight ? 4 : 3) * 1024);
+    if (dev >= 0 && dev < 64) {
+        std::lock_guard<std::mutex> lock(attr_mutex);
+        if (!attr_set[dev][eight]) {
+            const void *k = eight ? reinterpret_cast<const void *>(&gemm_mfma8_kernel<MF>)
+                                  : reinterpret_cast<const void *>(&gemm_mfma_kernel<MF>);
+            if (hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)) return e;
+            attr_set[dev][eight] = true;
+        }
     }
     const int m_tiles = (p.batch + BM - 1) / BM, n_tiles = (p.rows + kBN - 1) / kBN;
     const int tiles = m_tiles * n_tiles;
@@ -480,8 +861,12 @@ hipError_t launch(const Problem &p, int splits, hipStream_t s) {
     unsigned *arrivals = nullptr;
     if (splits > 1)
         if (hipError_t e = split_workspace(s, (size_t)tiles * splits * BM * kBN, (size_t)tiles, &partial, &arrivals)) return e;
-    gemm_mfma_kernel<MF><<<tiles * splits, kThreads, lds, s>>>(p.x, p.nz, p.sg, p.scales, p.y, p.batch, p.rows, p.cols,
-                                                              splits, partial, arrivals);
+    if (eight)
+        gemm_mfma8_kernel<MF><<<tiles * splits, kThreads8, lds, s>>>(p.x, p.nz, p.sg, p.scales, p.y, p.batch, p.rows, p.cols,
+                                                                     splits, partial, arrivals);
+    else
+        gemm_mfma_kernel<MF><<<tiles * splits, kThreads, lds, s>>>(p.x, p.nz, p.sg, p.scales, p.y, p.batch, p.rows, p.cols,
+                                                                  splits, partial, arrivals);
     return hipGetLastError();
 }
 

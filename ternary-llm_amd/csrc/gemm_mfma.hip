@@ -545,20 +545,23 @@ __global__ __launch_bounds__(kThreads8, 1) void gemm_mfma8_kernel(
         for (int j = 0; j < MF; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
-    auto mfma_row = [&](const u4 &a, const u4 (&bf)[MF], int i) {
-#pragma unroll
-        for (int j = 0; j < MF; j++)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, a), __builtin_bit_cast(h8, bf[j]),
-                                                               acc[i][j], 0, 0, 0);
-    };
 
     // ---- prologue: masks of stages 0..2, activations of stages 0 and 1; weights of stage 0 decoded
     Decoder16 d;
-    u4 af0[kNF8], af1[kNF8], bf0[MF], bf1[MF];
+    // Three sets of fragment registers: the fragments of a step are requested two steps before its
+    // MFMAs, also across the barrier (the MFMAs of steps 2 and 3 of a stage run after the barrier that
+    // ends its phase, from registers).
+    struct Frags {
+        u4 a[kNF8], b[MF];
+    };
+    Frags R[3];
 #pragma unroll
-    for (int i = 0; i < kNF8; i++) af1[i] = u4{0u, 0u, 0u, 0u};
+    for (int q = 0; q < 3; q++) {
 #pragma unroll
-    for (int j = 0; j < MF; j++) bf1[j] = u4{0u, 0u, 0u, 0u};
+        for (int i = 0; i < kNF8; i++) R[q].a[i] = u4{0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int j = 0; j < MF; j++) R[q].b[j] = u4{0u, 0u, 0u, 0u};
+    }
 #pragma unroll
     for (int u = 0; u < kBufs; u++) dma_masks(u, u);
     dma_acts(0, 0, 0, kDma);
@@ -575,9 +578,10 @@ __global__ __launch_bounds__(kThreads8, 1) void gemm_mfma8_kernel(
     }
 
     // In the loop every LDS instruction is written out and every wait for one names how many younger
-    // ones may still be in flight (they complete in order): the fragments of a step are requested
-    // one step ahead and a wait never includes the request made just before it. (Left to itself the
-    // compiler waits for the whole queue, lgkmcnt(0), in front of each consumer.)
+    // ones may still be in flight (they complete in order), so that a wait never includes requests made
+    // just before it. (Left to itself the compiler waits for the whole queue, lgkmcnt(0), in front of
+    // each consumer.) Fragment reads are issued one at a time between MFMAs: bursts of them from all
+    // eight waves at once fill the LDS queue and hold the MFMAs behind them.
     const uint32_t lds0 = (uint32_t)(uintptr_t)lds_dma;
     uint32_t fo[4];  // this lane's fragment offset in steps 0..3
 #pragma unroll
@@ -591,89 +595,117 @@ __global__ __launch_bounds__(kThreads8, 1) void gemm_mfma8_kernel(
 #define TLLM_LDS_READ32(dst, addr, off) asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(off))
 #define TLLM_LDS_WRITE128(addr, val, off) asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(addr), "v"(val), "i"(off) : "memory")
 #define TLLM_LGKM(n) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(n) : "memory")
-    auto frags = [&](u4 (&af)[kNF8], u4 (&bf)[MF], int buf, int ks) {  // kNF8 + MF reads
+#define TLLM_FENCE() __builtin_amdgcn_sched_barrier(0)
+    constexpr int kFr = kNF8 + MF;  // LDS reads of one step
+    // read number r (0 .. kFr-1) of the fragments of step ks: weight rows first, then activation rows
+    auto frag_read = [&](Frags &f, int buf, int ks, int r) {
         const uint32_t aw = fo[ks] + (w_rd + (uint32_t)(buf * kWBytes));
         const uint32_t aa = fo[ks] + (a_rd + (uint32_t)(buf * kActBytes));
-        TLLM_LDS_READ128(af[0], aw, 0);
-        TLLM_LDS_READ128(af[1], aw, 32 * kRowBytes);
-        TLLM_LDS_READ128(bf[0], aa, 0);
-        if constexpr (MF == 2) TLLM_LDS_READ128(bf[1], aa, 32 * kRowBytes);
+        if (r == 0) TLLM_LDS_READ128(f.a[0], aw, 0);
+        if (r == 1) TLLM_LDS_READ128(f.a[1], aw, 32 * kRowBytes);
+        if (r == 2) TLLM_LDS_READ128(f.b[0], aa, 0);
+        if constexpr (MF == 2)
+            if (r == 3) TLLM_LDS_READ128(f.b[1], aa, 32 * kRowBytes);
     };
-    constexpr int kFr = kNF8 + MF;  // LDS reads of one step
+    // MFMA number m (0 .. 2 MF - 1) of a step
+    auto mfma_one = [&](const Frags &f, int m) {
+        const int i = m / MF, j = m % MF;
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, f.a[i]), __builtin_bit_cast(h8, f.b[j]),
+                                                           acc[i][j], 0, 0, 0);
+    };
+    constexpr int kMf = kNF8 * MF;  // MFMAs of one step
+    // a slot: the MFMAs of one step (from set `use`) with the fragment reads of the step two ahead
+    // (into set `get`) between them, one read behind each of the first MFMAs
+    auto slot_spread = [&](const Frags &use, Frags &get, int buf, int ks) {
+#pragma unroll
+        for (int m = 0; m < (kMf > kFr ? kMf : kFr); m++) {
+            if (m < kMf) mfma_one(use, m);
+            TLLM_FENCE();
+            if (m < kFr) frag_read(get, buf, ks, m);
+            TLLM_FENCE();
+        }
+    };
 
     // one phase; the buffer index u = s % kBufs is a compile-time constant (it sits in instruction offsets)
     auto phase = [&](auto U, const int s) {
         constexpr int u = decltype(U)::value;
         constexpr int kH = kDma / 2 > 0 ? kDma / 2 : 1;
         constexpr int kNext = (u + 1) % kBufs;
+        // slot j of this phase reads into set (4 u + j) % 3 and multiplies from set (4 u + j + 1) % 3
+        constexpr int g0 = (4 * u + 0) % 3, g1 = (4 * u + 1) % 3, g2 = (4 * u + 2) % 3, g3 = (4 * u + 3) % 3;
         uint32_t o[8];
         uint32_t m_nz, m_sg, m_sc;
         // barrier s: publishes the weights decoded and the loads waited for in the phase before
         TLLM_LGKM(0);
         asm volatile("s_barrier" ::: "memory");
-        frags(af0, bf0, u, 0);                                   // in flight: kFr
+        TLLM_FENCE();
+        // ---- slot 0: step 2 of the stage before (zero operands in the first phase); fragments of step 0
+        slot_spread(R[g1], R[g0], u, 0);
         TLLM_LDS_READ32(m_nz, m_rd, kNext * kMaskBytes);
         TLLM_LDS_READ32(m_sg, m_rd, kNext * kMaskBytes + 1024);
-        TLLM_LDS_READ32(m_sc, s_rd, kNext * kMaskBytes);         // kFr + 3
-        __builtin_amdgcn_sched_barrier(0);
-        // last step of the stage before (all zero operands in the first phase)
-        mfma_row(af1[0], bf1, 0);
-        mfma_row(af1[1], bf1, 1);
-        __builtin_amdgcn_sched_barrier(0);
+        TLLM_LDS_READ32(m_sc, s_rd, kNext * kMaskBytes);
         dma_acts((u + 2) % kBufs, s + 2, 0, kH);
-        // ---- step 0
-        TLLM_LGKM(3);                                            // fragments of step 0 are here
-        frags(af1, bf1, u, 1);                                   // 3 + kFr
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_row(af0[0], bf0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        TLLM_LGKM(kFr);                                          // mask words and scale are here
-        __builtin_amdgcn_sched_barrier(0);
+        TLLM_FENCE();
+        // ---- slot 1: step 3 of the stage before; fragments of step 1
+        slot_spread(R[g2], R[g1], u, 1);
+        if (kDma > 1) dma_acts((u + 2) % kBufs, s + 2, kH, kDma);
+        TLLM_FENCE();
+        // ---- slot 2: step 0; fragments of step 2. In flight behind what it needs: the reads of slot 1.
+        TLLM_LGKM(kFr);
+        TLLM_FENCE();
         {
             const int odd = (w_par + min(s + 1, last) * kBK / 128) & 1;
             d.begin(m_nz, m_sg, odd ? m_sc >> 16 : m_sc & 0xFFFFu, w_sel);
         }
-        o[0] = d.dword(0);
-        o[1] = d.dword(1);
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_row(af0[1], bf0, 1);
-        __builtin_amdgcn_sched_barrier(0);
-        if (kDma > 1) dma_acts((u + 2) % kBufs, s + 2, kH, kDma);
-        o[2] = d.dword(2);
-        o[3] = d.dword(3);
-        // ---- step 1
-        __builtin_amdgcn_sched_barrier(0);
-        TLLM_LGKM(0);                                            // fragments of step 1
-        frags(af0, bf0, u, 2);                                   // kFr
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_row(af1[0], bf1, 0);
-        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int m = 0; m < (kMf > kFr ? kMf : kFr); m++) {
+            if (m < kMf) mfma_one(R[g0], m);
+            TLLM_FENCE();
+            if (m < kFr) frag_read(R[g2], u, 2, m);
+            if (m < 4) o[m] = d.dword(m);
+            TLLM_FENCE();
+        }
+#pragma unroll
+        for (int m = (kMf > kFr ? kMf : kFr); m < 4; m++) o[m] = d.dword(m);
+        // ---- slot 3: step 1; fragments of step 3, requested early in the slot so that the wait in
+        // front of the barrier finds them done. In flight behind what it needs: the reads of slot 2.
+        TLLM_LGKM(kFr);
+        TLLM_FENCE();
+#pragma unroll
+        for (int r = 0; r < kFr; r++) frag_read(R[g3], u, 3, r);
+        TLLM_FENCE();
+        mfma_one(R[g1], 0);
+        TLLM_FENCE();
         o[4] = d.dword(4);
         o[5] = d.dword(5);
         {
             const u4 v = {o[0], o[1], o[2], o[3]};
-            TLLM_LDS_WRITE128(w_wr0, v, kNext * kWBytes);        // kFr + 1
+            TLLM_LDS_WRITE128(w_wr0, v, kNext * kWBytes);
         }
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_row(af1[1], bf1, 1);
-        __builtin_amdgcn_sched_barrier(0);
+        TLLM_FENCE();
+        mfma_one(R[g1], 1);
+        TLLM_FENCE();
         o[6] = d.dword(6);
         o[7] = d.dword(7);
         dma_masks(u, s + 3);
         {
             const u4 v = {o[4], o[5], o[6], o[7]};
-            TLLM_LDS_WRITE128(w_wr1, v, kNext * kWBytes);        // kFr + 2
+            TLLM_LDS_WRITE128(w_wr1, v, kNext * kWBytes);
         }
-        // ---- step 2
-        __builtin_amdgcn_sched_barrier(0);
-        TLLM_LGKM(2);                                            // fragments of step 2
-        frags(af1, bf1, u, 3);                                   // 2 + kFr
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_row(af0[0], bf0, 0);
-        mfma_row(af0[1], bf0, 1);
-        __builtin_amdgcn_sched_barrier(0);
+        TLLM_FENCE();
+#pragma unroll
+        for (int m = 2; m < kMf; m++) mfma_one(R[g1], m);
+        TLLM_FENCE();
         // everything requested before this phase has landed
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kReq) : "memory");
+        if (s == last) {  // steps 2 and 3 of the last stage
+            TLLM_LGKM(0);
+            TLLM_FENCE();
+#pragma unroll
+            for (int m = 0; m < kMf; m++) mfma_one(R[g2], m);
+#pragma unroll
+            for (int m = 0; m < kMf; m++) mfma_one(R[g3], m);
+        }
     };
     for (int s0 = 0; s0 <= last; s0 += kBufs) {
         phase(std::integral_constant<int, 0>{}, s0);
@@ -682,15 +714,11 @@ __global__ __launch_bounds__(kThreads8, 1) void gemm_mfma8_kernel(
         if (s0 + 2 > last) break;
         phase(std::integral_constant<int, 2>{}, s0 + 2);
     }
-    // last step of the last stage
-    TLLM_LGKM(0);
-    __builtin_amdgcn_sched_barrier(0);
-    mfma_row(af1[0], bf1, 0);
-    mfma_row(af1[1], bf1, 1);
 #undef TLLM_LDS_READ128
 #undef TLLM_LDS_READ32
 #undef TLLM_LDS_WRITE128
 #undef TLLM_LGKM
+#undef TLLM_FENCE
     // requests past the last stage are still in flight into LDS: let them land before the workgroup ends
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 

@@ -810,6 +810,402 @@ __global__ __launch_bounds__(kThreads8, 1) void gemm_mfma8_kernel(
     }
 }
 
+
+// ------------------------------------------------------------------------------------------------
+// Four-wave instance with hand-placed instructions: one wave per SIMD, wave tile 128 weight rows x
+// 32*MF activation rows (4 x MF accumulator fragments), the same LDS image of a stage as above.
+// What a wave issues besides its MFMAs (fragment reads, the decode, direct-to-LDS loads) is dealt out
+// one or two instructions at a time into the gaps between the MFMAs, every LDS instruction is written
+// out, and every wait names how many younger requests may stay in flight. Activation tiles and mask
+// words are private to a wave / thread (requested and read by the same one); only the decoded
+// weights are shared, published by the one barrier per phase.
+//   phase s: fragment reads of stage s (two steps ahead of their MFMAs, also across the barrier);
+//            requests the activations of stage s+2 and the masks of stage s+3 (waited for at the end
+//            of phase s+1: in-order completion, vmcnt = this phase's own requests);
+//            decodes the masks of stage s+1 into weight buffer s+1.
+template <int MF>
+__global__ __launch_bounds__(kThreads, 1) void gemm_mfma4_kernel(
+    const uint16_t *__restrict__ A, const uint32_t *__restrict__ nzB, const uint32_t *__restrict__ sgB,
+    const uint16_t *__restrict__ scB, uint16_t *__restrict__ C, int M, int N, int K, int splits,
+    float *__restrict__ partial, unsigned *__restrict__ arrivals) {
+    constexpr int kWM = MF * 32;
+    constexpr int BM = 4 * kWM;
+    constexpr int kActWave = kWM * kRowBytes;
+    constexpr int kActBytes = 4 * kActWave;
+    constexpr int kActBase = kBufs * kWBytes;
+    constexpr int kMaskBase = kActBase + kBufs * kActBytes;
+    constexpr int kMaskBytes = 3 * 1024;  // per wave 768 bytes: nz words | sign words | scale dwords, 256 bytes each
+    constexpr int kDma = kWM / 8;         // 1 KB activation loads per wave and stage
+    constexpr int kReq = kDma + 3;        // requests a wave makes per phase
+    constexpr int kFr = kNF + MF;         // LDS reads of one step
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    typedef __attribute__((address_space(3))) unsigned char LB;
+    LB *lds_dma = (LB *)lds;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 31, lq = lane >> 5;
+
+    const int m_tiles = (M + BM - 1) / BM;
+    const int tile = blockIdx.x / splits, split = blockIdx.x - tile * splits;
+    const int n0 = (tile / m_tiles) * kBN;
+    const int m0 = (tile % m_tiles) * BM + wave * kWM;
+    const int words = K / 32, groups = K / 128;
+    const int g_begin = (int)((long)groups * split / splits), g_end = (int)((long)groups * (split + 1) / splits);
+    const int k_begin = g_begin * 128;
+    const int last = (g_end - g_begin) * 128 / kBK - 1;
+
+    typedef __attribute__((address_space(1))) const unsigned char GB;
+    // Global addresses: a uniform base (which moves with the stage) plus a 32-bit lane offset that never changes.
+    GB *a_base = (GB *)A + (size_t)k_begin * 2;
+    uint32_t a_off[kDma];  // load t: rows 8t .. 8t+7 of the wave's tile, 128 bytes each, chunk order = LDS order
+#pragma unroll
+    for (int t = 0; t < kDma; t++) {
+        const int gm = min(m0 + 8 * t + (lane >> 3), M - 1);
+        a_off[t] = (uint32_t)(((size_t)gm * K + 8 * ((lane & 7) ^ row_swizzle(8 * t + (lane >> 3)))) * 2);
+    }
+    const int w_row = tid >> 1, w_word = tid & 1;  // this thread decodes 32 weights: one mask word pair per stage
+    const int gn = min(n0 + w_row, N - 1);
+    GB *nz_base = (GB *)nzB + (size_t)(k_begin / 32) * 4;
+    GB *sg_base = (GB *)sgB + (size_t)(k_begin / 32) * 4;
+    const uint32_t m_off = (uint32_t)(((size_t)gn * words + w_word) * 4);
+    // the scale of a group travels as the aligned dword that holds it
+    const size_t sc_elem = (size_t)gn * groups + g_begin;
+    GB *sc_base = (GB *)scB;
+    const uint32_t sc_off = (uint32_t)((sc_elem * 2) & ~(size_t)3);   // + 4 * ((sc_elem & 1) + group) / 2 ...
+    const int w_par = (int)(sc_elem & 1);
+
+    f16v acc[kNF][MF];
+#pragma unroll
+    for (int i = 0; i < kNF; i++)
+#pragma unroll
+        for (int j = 0; j < MF; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+    struct Frags {
+        u4 a[kNF], b[MF];
+    };
+    Frags R[3];
+#pragma unroll
+    for (int q = 0; q < 3; q++) {
+#pragma unroll
+        for (int i = 0; i < kNF; i++) R[q].a[i] = u4{0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int j = 0; j < MF; j++) R[q].b[j] = u4{0u, 0u, 0u, 0u};
+    }
+
+    // LDS addresses (bytes from the start of LDS); buffer and fragment offsets sit in the instructions
+    const uint32_t lds0 = (uint32_t)(uintptr_t)lds_dma;
+    const int fr_off = chunk_off(li, lq);
+    uint32_t fw[4], fa[4];  // fragment reads of steps 0..3: weights, activations (buffers 0 and 1)
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+        fw[ks] = lds0 + (uint32_t)(fr_off ^ (ks << 5));
+        fa[ks] = fw[ks] + (uint32_t)(kActBase + wave * kActWave);
+    }
+    const int w_off = chunk_off(w_row, w_word * 4);
+    uint32_t w_wr[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) w_wr[c] = lds0 + (uint32_t)(w_off ^ (c << 4));
+    const uint32_t m_rd = lds0 + (uint32_t)(kMaskBase + wave * 768 + lane * 4);
+    const uint32_t m_rdb[3] = {m_rd, m_rd + (uint32_t)kMaskBytes, m_rd + 2u * (uint32_t)kMaskBytes};  // ds_read2 offsets are 8 bits
+    // the scale is the low or the high half of its dword: the half flips from group to group
+    const uint32_t s_rd_a = m_rd + 512u + 2u * (uint32_t)w_par, s_rd_b = m_rd + 512u + 2u * (uint32_t)(w_par ^ 1);
+
+#define TLLM_GPTR(p) ((__attribute__((address_space(1))) const void *)(p))
+#define TLLM_LPTR(p) ((__attribute__((address_space(3))) void *)(p))
+    // stage index -> first column of the stage relative to k_begin (requests past the end repeat the last stage)
+    auto stage_k0 = [&](int stage) -> int { return min(stage, last) * kBK; };
+    auto dma_masks = [&](int buf, int stage) {
+        const int k0 = stage_k0(stage);
+        LB *dst = lds_dma + kMaskBase + buf * kMaskBytes + wave * 768;
+        __builtin_amdgcn_global_load_lds(TLLM_GPTR(nz_base + (k0 / 8) + m_off), TLLM_LPTR(dst), 4, 0, 0);
+        __builtin_amdgcn_global_load_lds(TLLM_GPTR(sg_base + (k0 / 8) + m_off), TLLM_LPTR(dst + 256), 4, 0, 0);
+        // group k0 / 128 of this row: element sc_elem + k0 / 128, in dword (sc_elem + k0 / 128) / 2
+        const uint32_t g2 = (uint32_t)(((w_par + k0 / 128) >> 1) * 4);
+        __builtin_amdgcn_global_load_lds(TLLM_GPTR(sc_base + (sc_off + g2)), TLLM_LPTR(dst + 512), 4, 0, 0);
+    };
+    auto dma_act = [&](int buf, int stage, int t) {
+        const int k0 = stage_k0(stage);
+        __builtin_amdgcn_global_load_lds(TLLM_GPTR(a_base + (size_t)(k0 * 2) + a_off[t]),
+                                         TLLM_LPTR(lds_dma + kActBase + buf * kActBytes + wave * kActWave + t * 1024), 16, 0, 0);
+    };
+
+    // ---- prologue: masks of stages 0..2, activations of stages 0 and 1; weights of stage 0 decoded
+#pragma unroll
+    for (int u = 0; u < kBufs; u++) dma_masks(u, u);
+#pragma unroll
+    for (int t = 0; t < kDma; t++) dma_act(0, 0, t);
+#pragma unroll
+    for (int t = 0; t < kDma; t++) dma_act(1, 1, t);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    Decoder d;
+    {
+        const unsigned char *src = lds + kMaskBase + wave * 768 + lane * 4;
+        const uint32_t nz = *reinterpret_cast<const uint32_t *>(src);
+        const uint32_t sg = *reinterpret_cast<const uint32_t *>(src + 256);
+        const uint32_t sd = *reinterpret_cast<const uint32_t *>(src + 512);
+        d.begin(nz, sg, (w_par & 1) ? sd >> 16 : sd & 0xFFFFu);
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+            *reinterpret_cast<u4 *>(lds + (w_off ^ (c << 4))) = u4{d.dword(4 * c), d.dword(4 * c + 1), d.dword(4 * c + 2), d.dword(4 * c + 3)};
+    }
+
+#define TLLM_LDS_READ128(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(off))
+#define TLLM_LDS_READ2(dst, addr, o0, o1) asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(dst) : "v"(addr), "i"(o0), "i"(o1))
+#define TLLM_LDS_READ16(dst, addr, off) asm volatile("ds_read_u16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(off))
+#define TLLM_LDS_WRITE128(addr, val, off) asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(addr), "v"(val), "i"(off) : "memory")
+#define TLLM_LGKM(n) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(n) : "memory")
+#define TLLM_FENCE() __builtin_amdgcn_sched_barrier(0)
+    // fragment reads of step ks of the stage in buffer u into set g
+#define TLLM_RW(g, i, ks) TLLM_LDS_READ128(R[g].a[i], fw[ks], u * kWBytes + (i) * 32 * kRowBytes)
+#define TLLM_RA(g, j, ks)                                                                              \
+    do {                                                                                               \
+        if constexpr ((j) < MF) {                                                                      \
+            if constexpr (u * kActBytes + (j) * 32 * kRowBytes < 65536)                                \
+                TLLM_LDS_READ128(R[g].b[(j) < MF ? (j) : 0], fa[ks], u * kActBytes + (j) * 32 * kRowBytes);            \
+            else                                                                                       \
+                TLLM_LDS_READ128(R[g].b[(j) < MF ? (j) : 0], fa_hi, u * kActBytes + (j) * 32 * kRowBytes - 65536);     \
+        }                                                                                              \
+    } while (0)
+    // MFMA (i, j) of a step from set g
+#define TLLM_MM(g, i, j)                                                                               \
+    do {                                                                                               \
+        if constexpr ((j) < MF)                                                                        \
+            acc[i][(j) < MF ? (j) : 0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(                       \
+                __builtin_bit_cast(h8, R[g].a[i]), __builtin_bit_cast(h8, R[g].b[(j) < MF ? (j) : 0]), \
+                acc[i][(j) < MF ? (j) : 0], 0, 0, 0);                                                  \
+        TLLM_FENCE();                                                                                  \
+    } while (0)
+#define TLLM_DMA(t)                                                    \
+    do {                                                               \
+        if constexpr ((t) < kDma) dma_act((u + 2) % kBufs, s + 2, (t) < kDma ? (t) : 0); \
+        TLLM_FENCE();                                                  \
+    } while (0)
+
+    auto phase = [&](auto U, const int s) {
+        constexpr int u = decltype(U)::value;
+        constexpr int kNext = (u + 1) % kBufs;
+        // slot j of this phase reads into set (4 u + j) % 3 and multiplies from set (4 u + j + 1) % 3
+        constexpr int g0 = (4 * u + 0) % 3, g1 = (4 * u + 1) % 3, g2 = (4 * u + 2) % 3, g3 = (4 * u + 3) % 3;
+        uint32_t o[16];
+        uint32_t m_w[2], m_sc;
+        const uint32_t fa_hi_base = 65536u;
+        // barrier s: publishes the weights decoded in the phase before
+        TLLM_LGKM(0);
+        asm volatile("s_barrier" ::: "memory");
+        TLLM_FENCE();
+        // address of the scale half for stage s + 1 (group (s + 1) / 2 of this split)
+        const uint32_t s_rd = ((stage_k0(s + 1) / 128) & 1) ? s_rd_b : s_rd_a;
+        uint32_t fa_hi[4];  // only formed where a buffer offset does not fit the instruction (third buffer at MF = 2)
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) fa_hi[ks] = fa[ks] + fa_hi_base;
+#define fa_hi fa_hi[ks_]
+        // ---- slot 0: MFMAs of step 2 of the stage before (zero operands in the first phase); fragments of step 0
+        {
+            constexpr int ks_ = 0;
+            TLLM_MM(g1, 0, 0); TLLM_RW(g0, 0, 0); TLLM_FENCE();
+            TLLM_MM(g1, 0, 1); TLLM_RW(g0, 1, 0); TLLM_FENCE();
+            TLLM_MM(g1, 1, 0); TLLM_RW(g0, 2, 0); TLLM_FENCE();
+            TLLM_MM(g1, 1, 1); TLLM_RW(g0, 3, 0); TLLM_FENCE();
+            TLLM_MM(g1, 2, 0); TLLM_RA(g0, 0, 0); TLLM_FENCE();
+            TLLM_MM(g1, 2, 1); TLLM_RA(g0, 1, 0); TLLM_FENCE();
+            TLLM_MM(g1, 3, 0);
+            TLLM_LDS_READ2(m_w, m_rdb[kNext], 0, 64);
+            TLLM_LDS_READ16(m_sc, s_rd, kNext * kMaskBytes);
+            TLLM_FENCE();
+            TLLM_MM(g1, 3, 1); TLLM_DMA(0); TLLM_DMA(1);
+        }
+        // ---- slot 1: MFMAs of step 3 of the stage before; fragments of step 1
+        {
+            constexpr int ks_ = 1;
+            TLLM_MM(g2, 0, 0); TLLM_RW(g1, 0, 1); TLLM_FENCE();
+            TLLM_MM(g2, 0, 1); TLLM_RW(g1, 1, 1); TLLM_FENCE();
+            TLLM_MM(g2, 1, 0); TLLM_RW(g1, 2, 1); TLLM_FENCE();
+            TLLM_MM(g2, 1, 1); TLLM_RW(g1, 3, 1); TLLM_FENCE();
+            TLLM_MM(g2, 2, 0); TLLM_RA(g1, 0, 1); TLLM_FENCE();
+            TLLM_MM(g2, 2, 1); TLLM_RA(g1, 1, 1); TLLM_FENCE();
+            TLLM_MM(g2, 3, 0); TLLM_DMA(2); TLLM_DMA(3);
+            TLLM_MM(g2, 3, 1); TLLM_DMA(4); TLLM_DMA(5);
+        }
+        // ---- slot 2: MFMAs of step 0; fragments of step 2; first half of the decode.
+        // In flight behind what is needed (fragments of step 0, mask words, scale): the reads of slot 1.
+        TLLM_LGKM(kFr);
+        TLLM_FENCE();
+        {
+            constexpr int ks_ = 2;
+            d.begin(m_w[0], m_w[1], m_sc);
+            TLLM_FENCE();
+            TLLM_MM(g0, 0, 0); TLLM_RW(g2, 0, 2); o[0] = d.dword(0); o[1] = d.dword(1); TLLM_FENCE();
+            TLLM_MM(g0, 0, 1); TLLM_RW(g2, 1, 2); o[2] = d.dword(2); o[3] = d.dword(3); TLLM_FENCE();
+            TLLM_MM(g0, 1, 0); TLLM_RW(g2, 2, 2); o[4] = d.dword(4); o[5] = d.dword(5); TLLM_FENCE();
+            TLLM_MM(g0, 1, 1); TLLM_RW(g2, 3, 2); o[6] = d.dword(6); o[7] = d.dword(7); TLLM_FENCE();
+            TLLM_MM(g0, 2, 0); TLLM_RA(g2, 0, 2); o[8] = d.dword(8); o[9] = d.dword(9); TLLM_FENCE();
+            TLLM_MM(g0, 2, 1); TLLM_RA(g2, 1, 2); o[10] = d.dword(10); TLLM_FENCE();
+            TLLM_MM(g0, 3, 0); TLLM_DMA(6); TLLM_DMA(7);
+            o[11] = d.dword(11);
+            TLLM_FENCE();
+            TLLM_MM(g0, 3, 1);
+            {
+                const u4 v0 = {o[0], o[1], o[2], o[3]}, v1 = {o[4], o[5], o[6], o[7]};
+                TLLM_LDS_WRITE128(w_wr[0], v0, kNext * kWBytes);
+                TLLM_LDS_WRITE128(w_wr[1], v1, kNext * kWBytes);
+            }
+            TLLM_FENCE();
+        }
+        // ---- slot 3: MFMAs of step 1; fragments of step 3, requested early in the slot so that the wait
+        // in front of the barrier finds them done. In flight behind what is needed: the reads and the two
+        // stores of slot 2.
+        TLLM_LGKM(kFr + 2);
+        TLLM_FENCE();
+        {
+            constexpr int ks_ = 3;
+            TLLM_MM(g1, 0, 0); TLLM_RW(g3, 0, 3); TLLM_RW(g3, 1, 3); TLLM_FENCE();
+            TLLM_MM(g1, 0, 1); TLLM_RW(g3, 2, 3); TLLM_RW(g3, 3, 3); TLLM_FENCE();
+            TLLM_MM(g1, 1, 0); TLLM_RA(g3, 0, 3); TLLM_RA(g3, 1, 3); TLLM_FENCE();
+            TLLM_MM(g1, 1, 1); o[12] = d.dword(12); o[13] = d.dword(13); TLLM_FENCE();
+            TLLM_MM(g1, 2, 0); o[14] = d.dword(14); o[15] = d.dword(15); TLLM_FENCE();
+            TLLM_MM(g1, 2, 1);
+            {
+                const u4 v2 = {o[8], o[9], o[10], o[11]};
+                TLLM_LDS_WRITE128(w_wr[2], v2, kNext * kWBytes);
+            }
+            TLLM_FENCE();
+            TLLM_MM(g1, 3, 0);
+            {
+                const u4 v3 = {o[12], o[13], o[14], o[15]};
+                TLLM_LDS_WRITE128(w_wr[3], v3, kNext * kWBytes);
+            }
+            TLLM_FENCE();
+            TLLM_MM(g1, 3, 1);
+            dma_masks(u, s + 3);
+            TLLM_FENCE();
+        }
+#undef fa_hi
+        // everything requested before this phase has landed
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kReq) : "memory");
+        if (s == last) {  // steps 2 and 3 of the last stage
+            TLLM_LGKM(0);
+            TLLM_FENCE();
+            TLLM_MM(g2, 0, 0); TLLM_MM(g2, 0, 1); TLLM_MM(g2, 1, 0); TLLM_MM(g2, 1, 1);
+            TLLM_MM(g2, 2, 0); TLLM_MM(g2, 2, 1); TLLM_MM(g2, 3, 0); TLLM_MM(g2, 3, 1);
+            TLLM_MM(g3, 0, 0); TLLM_MM(g3, 0, 1); TLLM_MM(g3, 1, 0); TLLM_MM(g3, 1, 1);
+            TLLM_MM(g3, 2, 0); TLLM_MM(g3, 2, 1); TLLM_MM(g3, 3, 0); TLLM_MM(g3, 3, 1);
+        }
+    };
+    for (int s0 = 0; s0 <= last; s0 += kBufs) {
+        phase(std::integral_constant<int, 0>{}, s0);
+        if (s0 + 1 > last) break;
+        phase(std::integral_constant<int, 1>{}, s0 + 1);
+        if (s0 + 2 > last) break;
+        phase(std::integral_constant<int, 2>{}, s0 + 2);
+    }
+#undef TLLM_LDS_READ128
+#undef TLLM_LDS_READ2
+#undef TLLM_LDS_READ16
+#undef TLLM_LDS_WRITE128
+#undef TLLM_LGKM
+#undef TLLM_FENCE
+#undef TLLM_RW
+#undef TLLM_RA
+#undef TLLM_MM
+#undef TLLM_DMA
+#undef TLLM_GPTR
+#undef TLLM_LPTR
+    // requests past the last stage are still in flight into LDS: let them land before the workgroup ends
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    if (splits > 1) {
+        constexpr int kSlot = BM * kBN;  // floats; element (c, tid, e) of a slot at (c * kThreads + tid) * 4 + e
+        float *mine = partial + ((size_t)tile * splits + split) * kSlot + tid * 4;
+#pragma unroll
+        for (int i = 0; i < kNF; i++)
+#pragma unroll
+            for (int j = 0; j < MF; j++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const f4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                    float *dst = mine + (size_t)((i * MF + j) * 4 + g) * kThreads * 4;
+                    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(dst), "v"(v) : "memory");
+                }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __shared__ unsigned last_arrival4;
+        __syncthreads();
+        if (tid == 0) {
+            const unsigned before = __hip_atomic_fetch_add(&arrivals[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            last_arrival4 = before == (unsigned)splits - 1;
+            if (last_arrival4) __hip_atomic_store(&arrivals[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+        if (!last_arrival4) return;
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        const float *slots = partial + (size_t)tile * splits * kSlot + tid * 4;
+        // The slots are added in split order whoever arrives last; this workgroup's own sums take their
+        // place in that order from registers. The loads of one fragment row are in flight together.
+        f16v own[kNF][MF];
+#pragma unroll
+        for (int i = 0; i < kNF; i++)
+#pragma unroll
+            for (int j = 0; j < MF; j++) {
+                own[i][j] = acc[i][j];
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+            }
+        for (int q = 0; q < splits; q++) {
+            if (q == split) {
+#pragma unroll
+                for (int i = 0; i < kNF; i++)
+#pragma unroll
+                    for (int j = 0; j < MF; j++) acc[i][j] += own[i][j];
+                continue;
+            }
+            const float *slot = slots + (size_t)q * kSlot;
+#pragma unroll
+            for (int i = 0; i < kNF; i++) {
+                f4 v[MF * 4];
+#pragma unroll
+                for (int c = 0; c < MF * 4; c++) v[c] = *reinterpret_cast<const f4 *>(slot + (size_t)(i * MF * 4 + c) * kThreads * 4);
+#pragma unroll
+                for (int j = 0; j < MF; j++)
+#pragma unroll
+                    for (int g = 0; g < 4; g++)
+#pragma unroll
+                        for (int e = 0; e < 4; e++) acc[i][j][4 * g + e] += v[j * 4 + g][e];
+            }
+        }
+    }
+
+    // ---- store: lane (k half lq, column li) of fragment (i, j) holds, for activation row m, the weight
+    // rows n0 + 32 i + 8 g + 4 lq + v in register 4 g + v
+    const bool vec_store = (N & 3) == 0 && (reinterpret_cast<uintptr_t>(C) & 7) == 0;
+#pragma unroll
+    for (int j = 0; j < MF; j++) {
+        const int m = m0 + j * 32 + li;
+        if (m >= M) continue;
+#pragma unroll
+        for (int i = 0; i < kNF; i++) {
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int n = n0 + i * 32 + 8 * g + 4 * lq;
+                uint16_t h[4];
+#pragma unroll
+                for (int v = 0; v < 4; v++) h[v] = f2h(acc[i][j][4 * g + v] * 0.5f);
+                uint16_t *dst = C + (size_t)m * N + n;
+                if (n + 3 < N && vec_store) {
+                    *reinterpret_cast<uint2 *>(dst) = uint2{(uint32_t)h[0] | ((uint32_t)h[1] << 16),
+                                                            (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 4; v++)
+                        if (n + v < N) dst[v] = h[v];
+                }
+            }
+        }
+    }
+}
+
 // Split-K workspace: fp32 slots and arrival counters, one set per (device, stream), created on the
 // first call that needs it and grown on demand (the only allocation this file makes; never during
 // a call that does not split). Calls on one stream run in order and so may share a set.
@@ -856,11 +1252,12 @@ hipError_t split_workspace(hipStream_t s, size_t floats, size_t tiles, float **p
     return hipSuccess;
 }
 
-// TLLM_GEMM_WAVES=4 selects the four-wave instance (one wave per SIMD), for comparisons.
-bool use_eight_waves() {
-    static const bool v = [] {
+// TLLM_GEMM_WAVES picks the instance, for comparisons: 4 = four waves with hand-placed instructions (default),
+// 8 = eight waves, 1 = the first four-wave kernel (instruction order left to the compiler).
+int gemm_instance() {
+    static const int v = [] {
         const char *e = getenv("TLLM_GEMM_WAVES");
-        return !(e && e[0] == '4');
+        return e && e[0] == '8' ? 8 : e && e[0] == '1' ? 1 : 4;
     }();
     return v;
 }
@@ -869,18 +1266,19 @@ template <int MF>
 hipError_t launch(const Problem &p, int splits, hipStream_t s) {
     constexpr int BM = 128 * MF;
     static std::mutex attr_mutex;
-    static bool attr_set[64][2] = {};
+    static bool attr_set[64][3] = {};
     int dev = 0;
     if (hipError_t e = hipGetDevice(&dev)) return e;
-    const bool eight = use_eight_waves();
-    const size_t lds = kBufs * (size_t)(kWBytes + BM * kRowBytes + (eight ? 4 : 3) * 1024);
+    const int inst = gemm_instance(), slot = inst == 8 ? 2 : inst == 4 ? 1 : 0;
+    const size_t lds = kBufs * (size_t)(kWBytes + BM * kRowBytes + (inst == 8 ? 4 : 3) * 1024);
     if (dev >= 0 && dev < 64) {
         std::lock_guard<std::mutex> lock(attr_mutex);
-        if (!attr_set[dev][eight]) {
-            const void *k = eight ? reinterpret_cast<const void *>(&gemm_mfma8_kernel<MF>)
-                                  : reinterpret_cast<const void *>(&gemm_mfma_kernel<MF>);
+        if (!attr_set[dev][slot]) {
+            const void *k = inst == 8   ? reinterpret_cast<const void *>(&gemm_mfma8_kernel<MF>)
+                            : inst == 4 ? reinterpret_cast<const void *>(&gemm_mfma4_kernel<MF>)
+                                        : reinterpret_cast<const void *>(&gemm_mfma_kernel<MF>);
             if (hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)) return e;
-            attr_set[dev][eight] = true;
+            attr_set[dev][slot] = true;
         }
     }
     const int m_tiles = (p.batch + BM - 1) / BM, n_tiles = (p.rows + kBN - 1) / kBN;
@@ -889,9 +1287,12 @@ hipError_t launch(const Problem &p, int splits, hipStream_t s) {
     unsigned *arrivals = nullptr;
     if (splits > 1)
         if (hipError_t e = split_workspace(s, (size_t)tiles * splits * BM * kBN, (size_t)tiles, &partial, &arrivals)) return e;
-    if (eight)
+    if (inst == 8)
         gemm_mfma8_kernel<MF><<<tiles * splits, kThreads8, lds, s>>>(p.x, p.nz, p.sg, p.scales, p.y, p.batch, p.rows, p.cols,
                                                                      splits, partial, arrivals);
+    else if (inst == 4)
+        gemm_mfma4_kernel<MF><<<tiles * splits, kThreads, lds, s>>>(p.x, p.nz, p.sg, p.scales, p.y, p.batch, p.rows, p.cols,
+                                                                   splits, partial, arrivals);
     else
         gemm_mfma_kernel<MF><<<tiles * splits, kThreads, lds, s>>>(p.x, p.nz, p.sg, p.scales, p.y, p.batch, p.rows, p.cols,
                                                                   splits, partial, arrivals);

@@ -88,12 +88,28 @@ int tllm_quantize_absmax_i8(const uint16_t *input, int8_t *output, float *scale,
  * A fp16 [M,K] row-major, packed weight [N,K], C fp16 [M,N] row-major.
  * Replaces ternary::ternary_gemm, reference include/kernels.cuh:37-40
  * (kernels/ternary_gemm.cu:33-195). Any M >= 1 is accepted.
- * Allocation: none per call, except that the first call on a stream whose shape leaves CUs idle
- * (few weight tiles) creates a per-stream fp32 workspace for splitting K, grown on demand.
+ * Allocation: none per call, with one exception. Shapes with few weight tiles (M > 16 and N * M small
+ * against the chip) split K over several workgroups per tile, which exchange fp32 partial sums through a
+ * workspace that belongs to (device, stream): the first such call on a stream creates it (and a call with
+ * a larger need grows it: stream synchronisation, free, allocation). tllm_gemm_workspace_reserve does
+ * that ahead of time. While `stream` is being captured into a graph nothing is allocated: a call whose
+ * workspace is missing or too small then runs without the split (same result up to the order of the
+ * fp32 additions, slower). Calls that use one stream's workspace must not overlap in time: replays of a
+ * captured graph on another stream count as calls on the stream the graph was captured on.
  */
 int tllm_ternary_gemm_f16(const uint16_t *A, const uint32_t *nz_B, const uint32_t *sign_B,
                           const uint16_t *scales_B, uint16_t *C, int M, int N, int K,
                           int group_size, tllm_stream_t stream);
+
+/*
+ * Creates, or grows, the split-K workspace of `stream` for the GEMM shape (M, N, K) so that later
+ * tllm_ternary_gemm_f16 calls of that shape (or a smaller need) on that stream allocate nothing, e.g.
+ * before capturing them into a graph. May synchronise the stream. No counterpart in the reference (its
+ * GEMM needs no workspace). tllm_gemm_workspace_release frees every workspace of the process; no GEMM
+ * call may be in flight.
+ */
+int tllm_gemm_workspace_reserve(int M, int N, int K, int group_size, tllm_stream_t stream);
+void tllm_gemm_workspace_release(void);
 
 /*
  * output[b, i] = fp16( t[b, i] / sqrt(mean_i t[b, i]^2 + eps) * weight[i] ),  t = input (+ residual), fp32.

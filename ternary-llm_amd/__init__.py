@@ -10,6 +10,8 @@ from .ops import (  # noqa: F401
     add,
     copy_to_kv_cache,
     embedding_lookup,
+    gemm_workspace_release,
+    gemm_workspace_reserve,
     lib,
     lib_path,
     quantize_absmax_int8,

@@ -87,6 +87,18 @@ int tllm_ternary_gemm_f16(const uint16_t *A, const uint32_t *nz_B, const uint32_
     return tllm::run_linear(p, group_size, (hipStream_t)stream);
 }
 
+int tllm_gemm_workspace_reserve(int M, int N, int K, int group_size, tllm_stream_t stream) {
+    if (M < 1 || N < 1 || K < 1 || K % 32 != 0) return TLLM_ERR_BAD_SHAPE;
+    if (group_size < 32 || group_size % 32 != 0 || K % group_size != 0) return TLLM_ERR_BAD_GROUP;
+    if ((int64_t)M * K > INT32_MAX || (int64_t)M * N > INT32_MAX) return TLLM_ERR_TOO_LARGE;
+    // only the shape matters here: the pointers are never dereferenced
+    Problem p{nullptr, nullptr, nullptr, nullptr, nullptr, N, K, M, 0};
+    if (group_size != 128 || M <= 16) return TLLM_OK;  // paths that never split K
+    return (int)tllm::gemm_mfma_reserve(p, (hipStream_t)stream);
+}
+
+void tllm_gemm_workspace_release(void) { tllm::gemm_mfma_release_all(); }
+
 static int gemv_i8_common(const uint32_t *nz, const uint32_t *sg, const uint16_t *scales,
                           const int8_t *xq, float scale_value, const float *scale_dev,
                           uint16_t *y, int rows, int cols, int group, tllm_stream_t stream) {

@@ -101,6 +101,9 @@ hipError_t launch_gemv_batch_table(const Problem *table, const int *unit_prefix,
 bool gemm_mfma_supports(const Problem &p, int group);
 hipError_t launch_gemm_mfma(const Problem &p, hipStream_t s);
 float gemm_mfma_cost_us(const Problem &p);  // rough time of launch_gemm_mfma, to choose between kernels
+// Creates (or grows) the split-K workspace of stream s for this shape, if the shape splits K at all.
+hipError_t gemm_mfma_reserve(const Problem &p, hipStream_t s);
+void gemm_mfma_release_all();  // frees every split-K workspace (nothing may still be running on them)
 
 // Picks the kernel for one linear (fast 128-group paths when they apply, else the row-wave kernel).
 hipError_t dispatch_linear(const Problem &p, int group, hipStream_t s);

@@ -5,8 +5,8 @@
 // Here the product scale * w is formed exactly in fp16 (w in {-1,0,+1}), so the only difference to
 // the reference is the order of the fp32 additions.
 //
-// Tiling. A workgroup (4 waves) computes 128 weight rows x BM activation rows; every wave owns all
-// 128 weight rows and BM/4 activation rows of its own. Per stage of 64 columns of K:
+// Tiling. A workgroup (4 waves, one per SIMD) computes 128 weight rows x BM activation rows; every wave
+// owns all 128 weight rows and BM/4 activation rows of its own. Per stage of 64 columns of K:
 //   * weights: each thread decodes one 32-bit mask word pair of one weight row into LDS. One
 //     v_bitop3 puts the 2-bit field (negative, non-zero) of every even/odd weight in place, two
 //     v_perm gather the fields of weights (2f, 2f+1) into the two halves of one dword; shifted to
@@ -20,11 +20,10 @@
 //     16-byte chunk that belongs at byte 16 p of the destination block under the row swizzle, so
 //     every load reads eight full 128-byte lines. (Loading the MFMA operand straight into
 //     registers instead needs 16 different rows per 16 lanes and was 2.5 times slower.)
-//   * each wave multiplies with v_mfma_f32_16x16x32_f16; inside a stage the MFMA with index ks
-//     sums columns 16q + 8ks .. + 7 for lane quad q (both operands use the same assignment, so the
-//     sum over the stage is complete); operands come from LDS as 16-byte chunks, XOR-swizzled by
-//     row against bank conflicts.
-// Three LDS buffers per operand, one barrier per stage; the loop body spells out the pipeline.
+//   * each wave multiplies with v_mfma_f32_32x32x16_f16 in four steps of 16 columns; lane half q of
+//     step ks sums columns 16 ks + 8 q .. + 7 (both operands use the same assignment); operands come
+//     from LDS as 16-byte chunks, XOR-swizzled by row against bank conflicts.
+// Three LDS buffers per operand, one barrier per stage; the kernel spells out the pipeline.
 #include <stdlib.h>
 
 #include <mutex>
@@ -43,7 +42,7 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 
 constexpr int kBN = 128;     // weight rows per workgroup
-constexpr int kBK = 64;      // K columns per stage (two MFMA steps of 32)
+constexpr int kBK = 64;      // K columns per stage (four MFMA steps of 16)
 constexpr int kThreads = 256;
 constexpr int kRowBytes = kBK * 2;  // one LDS row: 64 fp16 = 8 chunks of 16 bytes
 constexpr int kNF = kBN / 32;       // MFMA row fragments (32 weight rows each) per wave
@@ -80,740 +79,8 @@ struct Decoder {
 
 constexpr int kBufs = 3;  // LDS buffers per operand (stages in flight)
 
-template <int MF>  // MFMA column fragments (32 activation rows each) per wave
-__global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
-    const uint16_t *__restrict__ A, const uint32_t *__restrict__ nzB, const uint32_t *__restrict__ sgB,
-    const uint16_t *__restrict__ scB, uint16_t *__restrict__ C, int M, int N, int K, int splits,
-    float *__restrict__ partial, unsigned *__restrict__ arrivals) {
-    constexpr int kWM = MF * 32;             // activation rows per wave
-    constexpr int BM = 4 * kWM;
-    constexpr int kActWave = kWM * kRowBytes;  // bytes of one wave's activation tile per stage
-    constexpr int kActBytes = 4 * kActWave;
-    constexpr int kActBase = kBufs * kWBytes;  // weights buffers first, activation buffers behind them
-    constexpr int kMaskBase = kActBase + kBufs * kActBytes;  // raw mask words and scales: 3 planes of 1 KB per buffer
-    constexpr int kMaskBytes = 3 * 1024;
-    constexpr int kDma = kWM / 8;              // direct-to-LDS loads per wave and stage (8 rows of 128 bytes each)
-    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    typedef __attribute__((address_space(3))) unsigned char LB;
-    LB *lds_dma = (LB *)lds;  // the same memory as a local-address-space pointer, for the direct loads
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int li = lane & 31, lq = lane >> 5;  // MFMA 32x32x16: operand row / column, k half
-
-    // tile coordinates: consecutive workgroups share the weight tile (same n0), so it stays in L2
-    // With splits > 1, `splits` consecutive workgroups share a tile and take consecutive ranges of
-    // whole scale groups of K; the last of them to finish adds the partial sums (below).
-    const int m_tiles = (M + BM - 1) / BM;
-    const int tile = blockIdx.x / splits, split = blockIdx.x - tile * splits;
-    const int n0 = (tile / m_tiles) * kBN;
-    const int m0 = (tile % m_tiles) * BM + wave * kWM;
-    const int words = K / 32, groups = K / 128;
-    const int g_begin = (int)((long)groups * split / splits), g_end = (int)((long)groups * (split + 1) / splits);
-    const int k_begin = g_begin * 128;
-    const int last = (g_end - g_begin) * 128 / kBK - 1;  // index of this workgroup's last stage
-
-    // activations: load t of a stage brings rows 8t .. 8t+7 of the wave's tile, 128 bytes each, straight
-    // into LDS. The hardware puts lane p's 16 bytes at byte 16 p of the 1 KB block, so lane p asks for
-    // the chunk that belongs there under the row swizzle: row p / 8, chunk (p % 8) ^ (p / 8).
-    // Rows past M re-read row M-1; their results are not stored.
-    typedef __attribute__((address_space(1))) const unsigned char GB;
-    GB *a_src[kDma];
-#pragma unroll
-    for (int t = 0; t < kDma; t++) {
-        const int gm = min(m0 + 8 * t + (lane >> 3), M - 1);
-        a_src[t] = (GB *)A + ((size_t)gm * K + k_begin + 8 * ((lane & 7) ^ row_swizzle(8 * t + (lane >> 3)))) * 2;
-    }
-    // weights: row w_row, 32-column word w_word of the stage
-    const int w_row = tid >> 1, w_word = tid & 1;
-    const int gn = min(n0 + w_row, N - 1);
-    GB *nz_src = (GB *)nzB + ((size_t)gn * words + k_begin / 32 + w_word) * 4;
-    GB *sg_src = (GB *)sgB + ((size_t)gn * words + k_begin / 32 + w_word) * 4;
-    // the scale of group g travels as the aligned dword that contains it; sc_half picks the half
-    GB *sc_src = (GB *)scB + ((size_t)gn * groups + g_begin) * 2;
-    const int w_off = chunk_off(w_row, w_word * 4);      // chunk c of the word: w_off ^ (c << 4)
-    const int fr_off = chunk_off(li, lq);                // fragment i, step ks: (fr_off ^ (ks << 5)) + i * 32 rows
-
-    struct Masks {
-        uint32_t nz, sg, sc;
-        bool hi;  // the scale is the high half of sc
-    };
-    // Mask words and scales also come through LDS: thread t asks for its own three dwords, which the
-    // hardware puts at byte 4 t of each 1 KB plane, and reads them back itself (no barrier involved).
-    auto dma_masks = [&](int buf, int stage) {
-        const int k0 = min(stage, last) * kBK;
-        LB *dst = lds_dma + kMaskBase + buf * kMaskBytes + wave * 256;
-        __builtin_amdgcn_global_load_lds((__attribute__((address_space(1))) const void *)(nz_src + k0 / 8),
-                                         (__attribute__((address_space(3))) void *)dst, 4, 0, 0);
-        __builtin_amdgcn_global_load_lds((__attribute__((address_space(1))) const void *)(sg_src + k0 / 8),
-                                         (__attribute__((address_space(3))) void *)(dst + 1024), 4, 0, 0);
-        const uintptr_t sc_addr = reinterpret_cast<uintptr_t>(sc_src) + (k0 / 128) * 2;
-        __builtin_amdgcn_global_load_lds((__attribute__((address_space(1))) const void *)(sc_addr & ~(uintptr_t)3),
-                                         (__attribute__((address_space(3))) void *)(dst + 2048), 4, 0, 0);
-    };
-    auto read_masks = [&](Masks &w, int buf, int stage) {
-        const unsigned char *src = lds + kMaskBase + buf * kMaskBytes + tid * 4;
-        w.nz = *reinterpret_cast<const uint32_t *>(src);
-        w.sg = *reinterpret_cast<const uint32_t *>(src + 1024);
-        w.sc = *reinterpret_cast<const uint32_t *>(src + 2048);  // the dword that holds the scale
-        const uintptr_t sc_addr = reinterpret_cast<uintptr_t>(sc_src) + (min(stage, last) * kBK / 128) * 2;
-        w.hi = (sc_addr & 2) != 0;
-    };
-    auto scale_of = [](const Masks &w) -> uint32_t { return w.hi ? w.sc >> 16 : w.sc & 0xFFFFu; };
-    auto dma_acts = [&](int buf, int stage, int t_begin, int t_end) {
-        const int k0 = min(stage, last) * kBK;
-#pragma unroll
-        for (int t = t_begin; t < t_end; t++)
-            __builtin_amdgcn_global_load_lds(
-                (__attribute__((address_space(1))) const void *)(a_src[t] + k0 * 2),
-                (__attribute__((address_space(3))) void *)(lds_dma + kActBase + buf * kActBytes + wave * kActWave + t * 1024),
-                16, 0, 0);
-    };
-    auto read_w = [&](u4 (&af)[kNF], int buf, int ks) {
-        const unsigned char *Ws = lds + buf * kWBytes + (fr_off ^ (ks << 5));
-#pragma unroll
-        for (int i = 0; i < kNF; i++) af[i] = *reinterpret_cast<const u4 *>(Ws + i * 32 * kRowBytes);
-    };
-    auto read_a = [&](u4 (&bf)[MF], int buf, int ks) {
-        const unsigned char *As = lds + kActBase + buf * kActBytes + wave * kActWave + (fr_off ^ (ks << 5));
-#pragma unroll
-        for (int j = 0; j < MF; j++) bf[j] = *reinterpret_cast<const u4 *>(As + j * 32 * kRowBytes);
-    };
-
-    f16v acc[kNF][MF];
-#pragma unroll
-    for (int i = 0; i < kNF; i++)
-#pragma unroll
-        for (int j = 0; j < MF; j++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
-    auto mfma_row = [&](const u4 &a, const u4 (&bf)[MF], int i) {
-#pragma unroll
-        for (int j = 0; j < MF; j++)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, a), __builtin_bit_cast(h8, bf[j]),
-                                                               acc[i][j], 0, 0, 0);
-    };
-    auto decode_all = [&](const Masks &w, int buf) {
-        Decoder d;
-        d.begin(w.nz, w.sg, scale_of(w));
-        unsigned char *Ws = lds + buf * kWBytes;
-#pragma unroll
-        for (int c = 0; c < 4; c++)
-            *reinterpret_cast<u4 *>(Ws + (w_off ^ (c << 4))) =
-                u4{d.dword(4 * c), d.dword(4 * c + 1), d.dword(4 * c + 2), d.dword(4 * c + 3)};
-    };
-
-    // Software pipeline, per stage s (buffer indices modulo 3). Everything that comes from global
-    // memory is written into LDS by the load itself; such loads complete in order, so "at most n
-    // still in flight" is the test for the older ones. A stage is four MFMA steps of 16 columns;
-    // the fragments of a step are read from LDS during the step before, after its first MFMAs.
-    //   top:    activations of stage s+2 are requested;
-    //   step 0: the masks of stage s+2 (requested in stage s-3) are read from LDS;
-    //   steps 1-3: between the MFMAs the masks are decoded into weight buffer s+2;
-    //   step 3: fragments of step 0 of stage s+1 are read; at the end the masks of stage s+5 are
-    //           requested into the mask buffer just read; barrier.
-    // The barrier at the end of stage s publishes weight buffer s+2 before its first read (step 3 of
-    // stage s+1); that buffer was last read in step 2 of stage s-1. Activation and mask buffers are
-    // private to a wave, ordered by the wave's own waits.
-    Masks w;
-    u4 af0[kNF], af1[kNF], bf0[MF], bf1[MF];
-    dma_acts(0, 0, 0, kDma);
-    dma_acts(1, 1, 0, kDma);
-#pragma unroll
-    for (int u = 0; u < kBufs; u++) dma_masks(u, u);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    read_masks(w, 0, 0);
-    decode_all(w, 0);
-    read_masks(w, 1, 1);
-    decode_all(w, 1);
-    dma_masks(0, 3);
-    dma_masks(1, 4);
-    // everything requested so far has landed: the in-loop waits count only requests made in the loop
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    read_w(af0, 0, 0);
-    read_a(bf0, 0, 0);
-    for (int s0 = 0; s0 <= last; s0 += kBufs) {
-#pragma unroll
-        for (int u = 0; u < kBufs; u++) {
-            const int s = s0 + u;
-            if (s > last) break;
-            // Every LDS read is issued right AFTER the first MFMAs of a step, one step before its
-            // data is used: the wait in front of a step's first MFMA then finds nothing younger in
-            // the LDS queue and costs nothing.
-            Decoder d;
-            unsigned char *Ws = lds + ((u + 2) % kBufs) * kWBytes;
-            uint32_t o[16];
-            // the activation requests of stage s+2 are spread over the four steps (a quarter each, behind
-            // the step's first MFMAs): issued back to back they hold the wave up
-            constexpr int kQ = kDma / 4;
-            // ---- step 0 (af0/bf0)
-            mfma_row(af0[0], bf0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            // masks of stage s+2: requested in stage s-3; newer requests: 2 stages of (kDma + 3)
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kDma + 6) : "memory");
-            read_masks(w, (u + 2) % kBufs, s + 2);
-            read_w(af1, u, 1);
-            __builtin_amdgcn_sched_barrier(0);
-            mfma_row(af0[1], bf0, 1);
-            __builtin_amdgcn_sched_barrier(0);
-            read_a(bf1, u, 1);
-            dma_acts((u + 2) % kBufs, s + 2, 0, kQ);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int i = 2; i < kNF; i++) mfma_row(af0[i], bf0, i);
-            __builtin_amdgcn_sched_barrier(0);
-            // ---- step 1 (af1/bf1): decode starts
-            mfma_row(af1[0], bf1, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            read_w(af0, u, 2);
-            read_a(bf0, u, 2);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int i = 1; i < kNF; i++) {
-                mfma_row(af1[i], bf1, i);
-                if (i == 1) {
-                    dma_acts((u + 2) % kBufs, s + 2, kQ, 2 * kQ);
-                    d.begin(w.nz, w.sg, scale_of(w));
-                }
-#pragma unroll
-                for (int dw = 2 * (i - 1); dw < 2 * i; dw++) o[dw] = d.dword(dw);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            // ---- step 2 (af0/bf0)
-            mfma_row(af0[0], bf0, 0);
-            o[6] = d.dword(6);
-            o[7] = d.dword(7);
-            __builtin_amdgcn_sched_barrier(0);
-            read_w(af1, u, 3);
-            read_a(bf1, u, 3);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int i = 1; i < kNF; i++) {
-                mfma_row(af0[i], bf0, i);
-                if (i == 1) {
-                    dma_acts((u + 2) % kBufs, s + 2, 2 * kQ, 3 * kQ);
-                    *reinterpret_cast<u4 *>(Ws + (w_off ^ (0 << 4))) = u4{o[0], o[1], o[2], o[3]};
-                    *reinterpret_cast<u4 *>(Ws + (w_off ^ (1 << 4))) = u4{o[4], o[5], o[6], o[7]};
-                }
-#pragma unroll
-                for (int dw = 6 + 2 * i; dw < 8 + 2 * i; dw++) o[dw] = d.dword(dw);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            // ---- step 3 (af1/bf1): fragments of step 0 of the next stage
-            mfma_row(af1[0], bf1, 0);
-            o[14] = d.dword(14);
-            o[15] = d.dword(15);
-            __builtin_amdgcn_sched_barrier(0);
-            *reinterpret_cast<u4 *>(Ws + (w_off ^ (2 << 4))) = u4{o[8], o[9], o[10], o[11]};
-            *reinterpret_cast<u4 *>(Ws + (w_off ^ (3 << 4))) = u4{o[12], o[13], o[14], o[15]};
-            read_w(af0, (u + 1) % kBufs, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            mfma_row(af1[1], bf1, 1);
-            __builtin_amdgcn_sched_barrier(0);
-            dma_acts((u + 2) % kBufs, s + 2, 3 * kQ, kDma);
-            // the activations of stage s+1 were requested during stage s-1; newer requests: the masks
-            // of that stage (3) and this stage's activations (kDma)
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kDma + 3) : "memory");
-            read_a(bf0, (u + 1) % kBufs, 0);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int i = 2; i < kNF; i++) mfma_row(af1[i], bf1, i);
-            __builtin_amdgcn_sched_barrier(0);
-            dma_masks((u + 2) % kBufs, s + 5);
-            // plain barrier: a fence here would also wait for the requests in flight
-            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        }
-    }
-
-    // ---- split K: every workgroup of a tile leaves its fp32 sums in its own slot; the one that
-    // arrives last adds all slots in split order (its own from its registers, in its place of the
-    // order: the result does not depend on who is last) and stores. The slots are written with stores that go through to memory
-    // (sc1) and are acknowledged (s_waitcnt vmcnt(0)) before the workgroup counts as arrived; the
-    // reader drops what its L2 may still hold of the slots (acquire fence = invalidate, cheap) and
-    // then reads them with ordinary 16-byte loads. A release fence instead of the write-through
-    // stores would write back the whole L2 of the XCD and cost more than the GEMM.
-    if (splits > 1) {
-        constexpr int kSlot = BM * kBN;  // floats; element (c, tid, e) of a slot at (c * kThreads + tid) * 4 + e
-        float *mine = partial + ((size_t)tile * splits + split) * kSlot + tid * 4;
-#pragma unroll
-        for (int i = 0; i < kNF; i++)
-#pragma unroll
-            for (int j = 0; j < MF; j++)
-#pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const f4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-                    float *dst = mine + (size_t)((i * MF + j) * 4 + g) * kThreads * 4;
-                    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(dst), "v"(v) : "memory");
-                }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __shared__ unsigned last_arrival;
-        __syncthreads();
-        if (tid == 0) {
-            const unsigned before = __hip_atomic_fetch_add(&arrivals[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            last_arrival = before == (unsigned)splits - 1;
-            if (last_arrival) __hip_atomic_store(&arrivals[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
-        }
-        __syncthreads();
-        if (!last_arrival) return;
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-        const float *slots = partial + (size_t)tile * splits * kSlot + tid * 4;
-        // the sums of this workgroup stay in registers: its own slot is not read back (same values)
-        f16v own[kNF][MF];
-#pragma unroll
-        for (int i = 0; i < kNF; i++)
-#pragma unroll
-            for (int j = 0; j < MF; j++) {
-                own[i][j] = acc[i][j];
-#pragma unroll
-                for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
-            }
-        for (int q = 0; q < splits; q++) {
-            if (q == split) {
-#pragma unroll
-                for (int i = 0; i < kNF; i++)
-#pragma unroll
-                    for (int j = 0; j < MF; j++) acc[i][j] += own[i][j];
-                continue;
-            }
-            const float *slot = slots + (size_t)q * kSlot;
-#pragma unroll
-            for (int i = 0; i < kNF; i++)
-#pragma unroll
-                for (int j = 0; j < MF; j++)
-#pragma unroll
-                    for (int g = 0; g < 4; g++) {
-                        const f4 v = *reinterpret_cast<const f4 *>(slot + (size_t)((i * MF + j) * 4 + g) * kThreads * 4);
-#pragma unroll
-                        for (int e = 0; e < 4; e++) acc[i][j][4 * g + e] += v[e];
-                    }
-        }
-    }
-
-    // ---- store: lane (k half lq, column li) of fragment (i, j) holds, for activation row m, the weight
-    // rows n0 + 32 i + 8 g + 4 lq + v in register 4 g + v (g, v = 0..3)
-    uint16_t *Cg = C;
-    const bool vec_store = (N & 3) == 0 && (reinterpret_cast<uintptr_t>(C) & 7) == 0;
-#pragma unroll
-    for (int j = 0; j < MF; j++) {
-        const int m = m0 + j * 32 + li;
-        if (m >= M) continue;
-#pragma unroll
-        for (int i = 0; i < kNF; i++) {
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const int n = n0 + i * 32 + 8 * g + 4 * lq;
-                uint16_t h[4];
-#pragma unroll
-                for (int v = 0; v < 4; v++) h[v] = f2h(acc[i][j][4 * g + v] * 0.5f);
-                uint16_t *dst = Cg + (size_t)m * N + n;
-                if (n + 3 < N && vec_store) {
-                    *reinterpret_cast<uint2 *>(dst) = uint2{(uint32_t)h[0] | ((uint32_t)h[1] << 16),
-                                                            (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
-                } else {
-#pragma unroll
-                    for (int v = 0; v < 4; v++)
-                        if (n + v < N) dst[v] = h[v];
-                }
-            }
-        }
-    }
-}
-
-
-// ------------------------------------------------------------------------------------------------
-// Eight-wave instance: two waves per SIMD, so that the loads, the decode and the LDS stores of one
-// wave run under the MFMAs of the other. Same workgroup tile (128 weight rows x 128*MF activation
-// rows) and the same LDS image of a stage; wave (wm, nh) owns activation rows 32*MF*wm .. and the
-// weight rows 64*nh .. 64*nh+63 (a 64 x 32*MF tile: 2 x MF accumulator fragments). The activation
-// tile of a wm is shared by its two waves (each requests half of its rows), the mask words and
-// scales are requested by one wave and decoded by another, so everything that lands in LDS is
-// published by the one barrier per phase.
-//
-// Phases. All LDS reads of the data of stage s happen between barrier s and barrier s+1 ("phase
-// s"): the fragments of step 0 right after barrier s (under the last MFMAs of stage s-1), those of
-// steps 1..3 one step ahead of their MFMAs. With three buffers per operand a buffer is therefore
-// free for two whole phases before it is read again:
-//   phase s: requests the activations of stage s+2 and the masks of stage s+3 (both waited for at
-//            the end of phase s+1: in-order completion, vmcnt = this phase's own requests),
-//            decodes the masks of stage s+1 (published by barrier s) into weight buffer s+1.
-constexpr int kThreads8 = 512;
-
-template <int MF>
-__global__ __launch_bounds__(kThreads8, 1) void gemm_mfma8_kernel(
-    const uint16_t *__restrict__ A, const uint32_t *__restrict__ nzB, const uint32_t *__restrict__ sgB,
-    const uint16_t *__restrict__ scB, uint16_t *__restrict__ C, int M, int N, int K, int splits,
-    float *__restrict__ partial, unsigned *__restrict__ arrivals) {
-    constexpr int kWM = MF * 32;               // activation rows per wave pair
-    constexpr int BM = 4 * kWM;
-    constexpr int kActWave = kWM * kRowBytes;  // bytes of one pair's activation tile per stage
-    constexpr int kActBytes = 4 * kActWave;
-    constexpr int kActBase = kBufs * kWBytes;
-    constexpr int kMaskBase = kActBase + kBufs * kActBytes;
-    constexpr int kMaskBytes = 4 * 1024;       // nz words 1 KB | sign words 1 KB | scale dwords 8 x 256 B
-    constexpr int kDmaPair = kWM / 8;          // 1 KB activation loads per pair and stage
-    constexpr int kDma = kDmaPair / 2;         // ... per wave
-    constexpr int kReq = kDma + 2;             // requests a wave makes per phase
-    constexpr int kNF8 = 2;                    // weight-row fragments per wave
-    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    typedef __attribute__((address_space(3))) unsigned char LB;
-    LB *lds_dma = (LB *)lds;
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave & 3, nh = wave >> 2;
-    const int li = lane & 31, lq = lane >> 5;
-
-    const int m_tiles = (M + BM - 1) / BM;
-    const int tile = blockIdx.x / splits, split = blockIdx.x - tile * splits;
-    const int n0 = (tile / m_tiles) * kBN;
-    const int m0 = (tile % m_tiles) * BM + wm * kWM;
-    const int words = K / 32, groups = K / 128;
-    const int g_begin = (int)((long)groups * split / splits), g_end = (int)((long)groups * (split + 1) / splits);
-    const int k_begin = g_begin * 128;
-    const int last = (g_end - g_begin) * 128 / kBK - 1;
-
-    typedef __attribute__((address_space(1))) const unsigned char GB;
-    // activations: this wave requests loads nh*kDma .. of its pair's tile (rows 8t .. 8t+7 each)
-    GB *a_src[kDma];
-#pragma unroll
-    for (int t = 0; t < kDma; t++) {
-        const int gm = min(m0 + 8 * (nh * kDma + t) + (lane >> 3), M - 1);
-        a_src[t] = (GB *)A + ((size_t)gm * K + k_begin + 8 * ((lane & 7) ^ row_swizzle(8 * (nh * kDma + t) + (lane >> 3)))) * 2;
-    }
-    // masks: waves 0-3 request the non-zero words, waves 4-7 the sign words; lane l of wave w asks for
-    // word (64 (w & 3) + l) of the stage = word (idx & 1) of weight row idx >> 1
-    const int midx = 64 * (wave & 3) + lane;
-    const int mrow = min(n0 + (midx >> 1), N - 1);
-    GB *m_src = (GB *)(nh ? sgB : nzB) + ((size_t)mrow * words + k_begin / 32 + (midx & 1)) * 4;
-    // scales: lane l of wave w asks for the aligned dword that holds the scale of weight row 16 w + (l & 15)
-    const int srow = min(n0 + 16 * wave + (lane & 15), N - 1);
-    const uintptr_t s_src = reinterpret_cast<uintptr_t>(scB) + ((size_t)srow * groups + g_begin) * 2;
-    // decode: thread t turns 16 weights of row t >> 2 (columns 16 (t & 3) .. of the stage) into two chunks
-    const int w_row = tid >> 2, w_qk = tid & 3;
-    const int w_gn = min(n0 + w_row, N - 1);
-    const int w_par = (int)(((size_t)w_gn * groups + g_begin) & 1);  // scale is the high half of its dword when (w_par + group) is odd
-    const uint32_t w_sel = (w_qk & 1) ? 0x07060302u : 0x05040100u;   // which 16 weights of the word
-    const int w_off = chunk_off(w_row, 2 * w_qk);
-    const int w_mask_off = (w_row * 2 + (w_qk >> 1)) * 4;
-    const int w_scale_off = 2048 + (w_row >> 4) * 256 + (w_row & 15) * 4;
-    const int fr_off = chunk_off(li, lq);
-
-    auto dma_masks = [&](int buf, int stage) {
-        const int k0 = min(stage, last) * kBK;
-        LB *dst = lds_dma + kMaskBase + buf * kMaskBytes;
-        __builtin_amdgcn_global_load_lds((__attribute__((address_space(1))) const void *)(m_src + k0 / 8),
-                                         (__attribute__((address_space(3))) void *)(dst + nh * 1024 + (wave & 3) * 256), 4, 0, 0);
-        const uintptr_t sc_addr = s_src + (k0 / 128) * 2;
-        __builtin_amdgcn_global_load_lds((__attribute__((address_space(1))) const void *)(sc_addr & ~(uintptr_t)3),
-                                         (__attribute__((address_space(3))) void *)(dst + 2048 + wave * 256), 4, 0, 0);
-    };
-    auto dma_acts = [&](int buf, int stage, int t_begin, int t_end) {
-        const int k0 = min(stage, last) * kBK;
-#pragma unroll
-        for (int t = t_begin; t < t_end; t++)
-            __builtin_amdgcn_global_load_lds(
-                (__attribute__((address_space(1))) const void *)(a_src[t] + k0 * 2),
-                (__attribute__((address_space(3))) void *)(lds_dma + kActBase + buf * kActBytes + wm * kActWave + (nh * kDma + t) * 1024),
-                16, 0, 0);
-    };
-    // 16 weights -> 8 dwords (two chunks) of +-2*scale / 0, see Decoder above
-    struct Decoder16 {
-        uint32_t q;
-        h2 sp;
-        __device__ __forceinline__ void begin(uint32_t nz, uint32_t sg, uint32_t scale, uint32_t sel) {
-            const uint32_t neg = nz & ~sg;
-            const uint32_t t0 = __builtin_amdgcn_bitop3_b32(neg << 1, nz, 0xAAAAAAAAu, 0xE4);
-            const uint32_t t1 = __builtin_amdgcn_bitop3_b32(neg, nz >> 1, 0xAAAAAAAAu, 0xE4);
-            q = __builtin_amdgcn_perm(t1, t0, sel);
-            sp = __builtin_bit_cast(h2, scale | (scale << 16));
-        }
-        __device__ __forceinline__ uint32_t dword(int d) const {
-            us2 v = __builtin_bit_cast(us2, q);
-            v = v << (uint16_t)(14 - 2 * d);
-            const uint32_t top = __builtin_bit_cast(uint32_t, v) & 0xC000C000u;
-            return __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, top) * sp);
-        }
-    };
-
-    f16v acc[kNF8][MF];
-#pragma unroll
-    for (int i = 0; i < kNF8; i++)
-#pragma unroll
-        for (int j = 0; j < MF; j++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
-
-    // ---- prologue: masks of stages 0..2, activations of stages 0 and 1; weights of stage 0 decoded
-    Decoder16 d;
-    // Three sets of fragment registers: the fragments of a step are requested two steps before its
-    // MFMAs, also across the barrier (the MFMAs of steps 2 and 3 of a stage run after the barrier that
-    // ends its phase, from registers).
-    struct Frags {
-        u4 a[kNF8], b[MF];
-    };
-    Frags R[3];
-#pragma unroll
-    for (int q = 0; q < 3; q++) {
-#pragma unroll
-        for (int i = 0; i < kNF8; i++) R[q].a[i] = u4{0u, 0u, 0u, 0u};
-#pragma unroll
-        for (int j = 0; j < MF; j++) R[q].b[j] = u4{0u, 0u, 0u, 0u};
-    }
-#pragma unroll
-    for (int u = 0; u < kBufs; u++) dma_masks(u, u);
-    dma_acts(0, 0, 0, kDma);
-    dma_acts(1, 1, 0, kDma);
-    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-    {
-        const unsigned char *src = lds + kMaskBase;
-        const uint32_t nz = *reinterpret_cast<const uint32_t *>(src + w_mask_off);
-        const uint32_t sg = *reinterpret_cast<const uint32_t *>(src + 1024 + w_mask_off);
-        const uint32_t sd = *reinterpret_cast<const uint32_t *>(src + w_scale_off);
-        d.begin(nz, sg, (w_par & 1) ? sd >> 16 : sd & 0xFFFFu, w_sel);
-        *reinterpret_cast<u4 *>(lds + w_off) = u4{d.dword(0), d.dword(1), d.dword(2), d.dword(3)};
-        *reinterpret_cast<u4 *>(lds + (w_off ^ 16)) = u4{d.dword(4), d.dword(5), d.dword(6), d.dword(7)};
-    }
-
-    // In the loop every LDS instruction is written out and every wait for one names how many younger
-    // ones may still be in flight (they complete in order), so that a wait never includes requests made
-    // just before it. (Left to itself the compiler waits for the whole queue, lgkmcnt(0), in front of
-    // each consumer.) Fragment reads are issued one at a time between MFMAs: bursts of them from all
-    // eight waves at once fill the LDS queue and hold the MFMAs behind them.
-    const uint32_t lds0 = (uint32_t)(uintptr_t)lds_dma;
-    uint32_t fo[4];  // this lane's fragment offset in steps 0..3
-#pragma unroll
-    for (int ks = 0; ks < 4; ks++) fo[ks] = lds0 + (uint32_t)(fr_off ^ (ks << 5));
-    const uint32_t w_rd = (uint32_t)(nh * 64 * kRowBytes);                // + buf * kWBytes
-    const uint32_t a_rd = (uint32_t)(kActBase + wm * kActWave);          // + buf * kActBytes
-    const uint32_t m_rd = lds0 + (uint32_t)(kMaskBase + w_mask_off);     // imm: buf * kMaskBytes (+ 1024)
-    const uint32_t s_rd = lds0 + (uint32_t)(kMaskBase + w_scale_off);
-    const uint32_t w_wr0 = lds0 + (uint32_t)w_off, w_wr1 = lds0 + (uint32_t)(w_off ^ 16);  // imm: buf * kWBytes
-#define TLLM_LDS_READ128(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(off))
-#define TLLM_LDS_READ32(dst, addr, off) asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(off))
-#define TLLM_LDS_WRITE128(addr, val, off) asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(addr), "v"(val), "i"(off) : "memory")
-#define TLLM_LGKM(n) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(n) : "memory")
-#define TLLM_FENCE() __builtin_amdgcn_sched_barrier(0)
-    constexpr int kFr = kNF8 + MF;  // LDS reads of one step
-    // read number r (0 .. kFr-1) of the fragments of step ks: weight rows first, then activation rows
-    auto frag_read = [&](Frags &f, int buf, int ks, int r) {
-        const uint32_t aw = fo[ks] + (w_rd + (uint32_t)(buf * kWBytes));
-        const uint32_t aa = fo[ks] + (a_rd + (uint32_t)(buf * kActBytes));
-        if (r == 0) TLLM_LDS_READ128(f.a[0], aw, 0);
-        if (r == 1) TLLM_LDS_READ128(f.a[1], aw, 32 * kRowBytes);
-        if (r == 2) TLLM_LDS_READ128(f.b[0], aa, 0);
-        if constexpr (MF == 2)
-            if (r == 3) TLLM_LDS_READ128(f.b[1], aa, 32 * kRowBytes);
-    };
-    // MFMA number m (0 .. 2 MF - 1) of a step
-    auto mfma_one = [&](const Frags &f, int m) {
-        const int i = m / MF, j = m % MF;
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, f.a[i]), __builtin_bit_cast(h8, f.b[j]),
-                                                           acc[i][j], 0, 0, 0);
-    };
-    constexpr int kMf = kNF8 * MF;  // MFMAs of one step
-    // a slot: the MFMAs of one step (from set `use`) with the fragment reads of the step two ahead
-    // (into set `get`) between them, one read behind each of the first MFMAs
-    auto slot_spread = [&](const Frags &use, Frags &get, int buf, int ks) {
-#pragma unroll
-        for (int m = 0; m < (kMf > kFr ? kMf : kFr); m++) {
-            if (m < kMf) mfma_one(use, m);
-            TLLM_FENCE();
-            if (m < kFr) frag_read(get, buf, ks, m);
-            TLLM_FENCE();
-        }
-    };
-
-    // one phase; the buffer index u = s % kBufs is a compile-time constant (it sits in instruction offsets)
-    auto phase = [&](auto U, const int s) {
-        constexpr int u = decltype(U)::value;
-        constexpr int kH = kDma / 2 > 0 ? kDma / 2 : 1;
-        constexpr int kNext = (u + 1) % kBufs;
-        // slot j of this phase reads into set (4 u + j) % 3 and multiplies from set (4 u + j + 1) % 3
-        constexpr int g0 = (4 * u + 0) % 3, g1 = (4 * u + 1) % 3, g2 = (4 * u + 2) % 3, g3 = (4 * u + 3) % 3;
-        uint32_t o[8];
-        uint32_t m_nz, m_sg, m_sc;
-        // barrier s: publishes the weights decoded and the loads waited for in the phase before
-        TLLM_LGKM(0);
-        asm volatile("s_barrier" ::: "memory");
-        TLLM_FENCE();
-        // ---- slot 0: step 2 of the stage before (zero operands in the first phase); fragments of step 0
-        slot_spread(R[g1], R[g0], u, 0);
-        TLLM_LDS_READ32(m_nz, m_rd, kNext * kMaskBytes);
-        TLLM_LDS_READ32(m_sg, m_rd, kNext * kMaskBytes + 1024);
-        TLLM_LDS_READ32(m_sc, s_rd, kNext * kMaskBytes);
-        dma_acts((u + 2) % kBufs, s + 2, 0, kH);
-        TLLM_FENCE();
-        // ---- slot 1: step 3 of the stage before; fragments of step 1
-        slot_spread(R[g2], R[g1], u, 1);
-        if (kDma > 1) dma_acts((u + 2) % kBufs, s + 2, kH, kDma);
-        TLLM_FENCE();
-        // ---- slot 2: step 0; fragments of step 2. In flight behind what it needs: the reads of slot 1.
-        TLLM_LGKM(kFr);
-        TLLM_FENCE();
-        {
-            const int odd = (w_par + min(s + 1, last) * kBK / 128) & 1;
-            d.begin(m_nz, m_sg, odd ? m_sc >> 16 : m_sc & 0xFFFFu, w_sel);
-        }
-#pragma unroll
-        for (int m = 0; m < (kMf > kFr ? kMf : kFr); m++) {
-            if (m < kMf) mfma_one(R[g0], m);
-            TLLM_FENCE();
-            if (m < kFr) frag_read(R[g2], u, 2, m);
-            if (m < 4) o[m] = d.dword(m);
-            TLLM_FENCE();
-        }
-#pragma unroll
-        for (int m = (kMf > kFr ? kMf : kFr); m < 4; m++) o[m] = d.dword(m);
-        // ---- slot 3: step 1; fragments of step 3, requested early in the slot so that the wait in
-        // front of the barrier finds them done. In flight behind what it needs: the reads of slot 2.
-        TLLM_LGKM(kFr);
-        TLLM_FENCE();
-#pragma unroll
-        for (int r = 0; r < kFr; r++) frag_read(R[g3], u, 3, r);
-        TLLM_FENCE();
-        mfma_one(R[g1], 0);
-        TLLM_FENCE();
-        o[4] = d.dword(4);
-        o[5] = d.dword(5);
-        {
-            const u4 v = {o[0], o[1], o[2], o[3]};
-            TLLM_LDS_WRITE128(w_wr0, v, kNext * kWBytes);
-        }
-        TLLM_FENCE();
-        mfma_one(R[g1], 1);
-        TLLM_FENCE();
-        o[6] = d.dword(6);
-        o[7] = d.dword(7);
-        dma_masks(u, s + 3);
-        {
-            const u4 v = {o[4], o[5], o[6], o[7]};
-            TLLM_LDS_WRITE128(w_wr1, v, kNext * kWBytes);
-        }
-        TLLM_FENCE();
-#pragma unroll
-        for (int m = 2; m < kMf; m++) mfma_one(R[g1], m);
-        TLLM_FENCE();
-        // everything requested before this phase has landed
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kReq) : "memory");
-        if (s == last) {  // steps 2 and 3 of the last stage
-            TLLM_LGKM(0);
-            TLLM_FENCE();
-#pragma unroll
-            for (int m = 0; m < kMf; m++) mfma_one(R[g2], m);
-#pragma unroll
-            for (int m = 0; m < kMf; m++) mfma_one(R[g3], m);
-        }
-    };
-    for (int s0 = 0; s0 <= last; s0 += kBufs) {
-        phase(std::integral_constant<int, 0>{}, s0);
-        if (s0 + 1 > last) break;
-        phase(std::integral_constant<int, 1>{}, s0 + 1);
-        if (s0 + 2 > last) break;
-        phase(std::integral_constant<int, 2>{}, s0 + 2);
-    }
-#undef TLLM_LDS_READ128
-#undef TLLM_LDS_READ32
-#undef TLLM_LDS_WRITE128
-#undef TLLM_LGKM
-#undef TLLM_FENCE
-    // requests past the last stage are still in flight into LDS: let them land before the workgroup ends
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-
-    if (splits > 1) {
-        constexpr int kSlot = BM * kBN;  // floats; element (c, tid, e) of a slot at (c * kThreads8 + tid) * 4 + e
-        float *mine = partial + ((size_t)tile * splits + split) * kSlot + tid * 4;
-#pragma unroll
-        for (int i = 0; i < kNF8; i++)
-#pragma unroll
-            for (int j = 0; j < MF; j++)
-#pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const f4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-                    float *dst = mine + (size_t)((i * MF + j) * 4 + g) * kThreads8 * 4;
-                    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(dst), "v"(v) : "memory");
-                }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __shared__ unsigned last_arrival8;
-        __syncthreads();
-        if (tid == 0) {
-            const unsigned before = __hip_atomic_fetch_add(&arrivals[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            last_arrival8 = before == (unsigned)splits - 1;
-            if (last_arrival8) __hip_atomic_store(&arrivals[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-        __syncthreads();
-        if (!last_arrival8) return;
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-        const float *slots = partial + (size_t)tile * splits * kSlot + tid * 4;
-        // The slots are added in split order whoever arrives last; this workgroup's own sums take
-        // their place in that order from registers. All loads of a slot are in flight together.
-        f16v own[kNF8][MF];
-#pragma unroll
-        for (int i = 0; i < kNF8; i++)
-#pragma unroll
-            for (int j = 0; j < MF; j++) {
-                own[i][j] = acc[i][j];
-#pragma unroll
-                for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
-            }
-        for (int q = 0; q < splits; q++) {
-            if (q == split) {
-#pragma unroll
-                for (int i = 0; i < kNF8; i++)
-#pragma unroll
-                    for (int j = 0; j < MF; j++) acc[i][j] += own[i][j];
-                continue;
-            }
-            const float *slot = slots + (size_t)q * kSlot;
-            f4 v[kNF8 * MF * 4];
-#pragma unroll
-            for (int c = 0; c < kNF8 * MF * 4; c++) v[c] = *reinterpret_cast<const f4 *>(slot + (size_t)c * kThreads8 * 4);
-#pragma unroll
-            for (int i = 0; i < kNF8; i++)
-#pragma unroll
-                for (int j = 0; j < MF; j++)
-#pragma unroll
-                    for (int g = 0; g < 4; g++)
-#pragma unroll
-                        for (int e = 0; e < 4; e++) acc[i][j][4 * g + e] += v[(i * MF + j) * 4 + g][e];
-        }
-    }
-
-    // ---- store: lane (k half lq, column li) of fragment (i, j) holds, for activation row m, the weight
-    // rows n0 + 64 nh + 32 i + 8 g + 4 lq + v in register 4 g + v
-    const bool vec_store = (N & 3) == 0 && (reinterpret_cast<uintptr_t>(C) & 7) == 0;
-#pragma unroll
-    for (int j = 0; j < MF; j++) {
-        const int m = m0 + j * 32 + li;
-        if (m >= M) continue;
-#pragma unroll
-        for (int i = 0; i < kNF8; i++) {
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const int n = n0 + nh * 64 + i * 32 + 8 * g + 4 * lq;
-                uint16_t h[4];
-#pragma unroll
-                for (int v = 0; v < 4; v++) h[v] = f2h(acc[i][j][4 * g + v] * 0.5f);
-                uint16_t *dst = C + (size_t)m * N + n;
-                if (n + 3 < N && vec_store) {
-                    *reinterpret_cast<uint2 *>(dst) = uint2{(uint32_t)h[0] | ((uint32_t)h[1] << 16),
-                                                            (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
-                } else {
-#pragma unroll
-                    for (int v = 0; v < 4; v++)
-                        if (n + v < N) dst[v] = h[v];
-                }
-            }
-        }
-    }
-}
-
-
-// ------------------------------------------------------------------------------------------------
-// Four-wave instance with hand-placed instructions: one wave per SIMD, wave tile 128 weight rows x
-// 32*MF activation rows (4 x MF accumulator fragments), the same LDS image of a stage as above.
+// The kernel: one wave per SIMD, wave tile 128 weight rows x 32*MF activation rows (4 x MF accumulator
+// fragments of 32 x 32).
 // What a wave issues besides its MFMAs (fragment reads, the decode, direct-to-LDS loads) is dealt out
 // one or two instructions at a time into the gaps between the MFMAs, every LDS instruction is written
 // out, and every wait names how many younger requests may stay in flight. Activation tiles and mask
@@ -824,7 +91,7 @@ __global__ __launch_bounds__(kThreads8, 1) void gemm_mfma8_kernel(
 //            of phase s+1: in-order completion, vmcnt = this phase's own requests);
 //            decodes the masks of stage s+1 into weight buffer s+1.
 template <int MF>
-__global__ __launch_bounds__(kThreads, 1) void gemm_mfma4_kernel(
+__global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
     const uint16_t *__restrict__ A, const uint32_t *__restrict__ nzB, const uint32_t *__restrict__ sgB,
     const uint16_t *__restrict__ scB, uint16_t *__restrict__ C, int M, int N, int K, int splits,
     float *__restrict__ partial, unsigned *__restrict__ arrivals) {
@@ -1206,96 +473,95 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma4_kernel(
     }
 }
 
-// Split-K workspace: fp32 slots and arrival counters, one set per (device, stream), created on the
-// first call that needs it and grown on demand (the only allocation this file makes; never during
-// a call that does not split). Calls on one stream run in order and so may share a set.
+// ---- split-K exchange memory: fp32 slots and one arrival counter per tile.
+//
+// Ordinary calls use a workspace per (device, stream), created by tllm_gemm_workspace_reserve or by the
+// first call that needs it and grown on demand; calls on one stream run in order and so may share it.
+// Nothing is allocated, freed or synchronised while the stream is being captured into a graph: a call
+// that would have to falls back to one workgroup per tile (no exchange).
 struct SplitWorkspace {
     int device = -1;
     hipStream_t stream = nullptr;
     float *partial = nullptr;
     size_t floats = 0;
     unsigned *arrivals = nullptr;
-    size_t tiles = 0;
 };
+constexpr size_t kArrivalSlots = 1024;  // tiles of a split launch (at most one per CU pair)
 std::mutex g_ws_mutex;
 std::vector<SplitWorkspace> g_ws;
 
-hipError_t split_workspace(hipStream_t s, size_t floats, size_t tiles, float **partial, unsigned **arrivals) {
+__global__ void clear_arrivals_kernel(unsigned *arrivals, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) arrivals[i] = 0u;
+}
+
+// may_allocate = false: only hands out what exists. *partial stays null when the workspace is too small.
+hipError_t split_workspace(hipStream_t s, size_t floats, bool may_allocate, float **partial, unsigned **arrivals) {
     int dev = 0;
     if (hipError_t e = hipGetDevice(&dev)) return e;
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     SplitWorkspace *w = nullptr;
     for (SplitWorkspace &c : g_ws)
         if (c.device == dev && c.stream == s) w = &c;
+    if ((!w || w->floats < floats) && !may_allocate) return hipSuccess;
     if (!w) {
         g_ws.push_back(SplitWorkspace{});
         w = &g_ws.back();
         w->device = dev;
         w->stream = s;
     }
-    if (w->floats < floats || w->tiles < tiles) {
+    if (w->floats < floats) {
         if (hipError_t e = hipStreamSynchronize(s)) return e;  // earlier launches may still use the old buffers
         if (w->partial) (void)hipFree(w->partial);
-        if (w->arrivals) (void)hipFree(w->arrivals);
         w->partial = nullptr;
-        w->arrivals = nullptr;
-        w->floats = w->tiles = 0;
-        const size_t nf = floats > w->floats ? floats : w->floats, nt = tiles > 1024 ? tiles : 1024;
-        if (hipError_t e = hipMalloc(reinterpret_cast<void **>(&w->partial), nf * sizeof(float))) return e;
-        if (hipError_t e = hipMalloc(reinterpret_cast<void **>(&w->arrivals), nt * sizeof(unsigned))) return e;
-        if (hipError_t e = hipMemset(w->arrivals, 0, nt * sizeof(unsigned))) return e;
-        w->floats = nf;
-        w->tiles = nt;
+        w->floats = 0;
+        if (hipError_t e = hipMalloc(reinterpret_cast<void **>(&w->partial), floats * sizeof(float))) return e;
+        w->floats = floats;
+        if (!w->arrivals) {
+            if (hipError_t e = hipMalloc(reinterpret_cast<void **>(&w->arrivals), kArrivalSlots * sizeof(unsigned))) return e;
+            // cleared once, in stream order; every launch leaves the counters at zero again
+            clear_arrivals_kernel<<<(int)(kArrivalSlots / 256), 256, 0, s>>>(w->arrivals, (int)kArrivalSlots);
+            if (hipError_t e = hipGetLastError()) return e;
+        }
     }
     *partial = w->partial;
     *arrivals = w->arrivals;
     return hipSuccess;
 }
 
-// TLLM_GEMM_WAVES picks the instance, for comparisons: 4 = four waves with hand-placed instructions (default),
-// 8 = eight waves, 1 = the first four-wave kernel (instruction order left to the compiler).
-int gemm_instance() {
-    static const int v = [] {
-        const char *e = getenv("TLLM_GEMM_WAVES");
-        return e && e[0] == '8' ? 8 : e && e[0] == '1' ? 1 : 4;
-    }();
-    return v;
+struct GemmConfig {
+    int height;  // 0: 128 activation rows per workgroup, 1: 256
+    int splits;  // workgroups per tile along K
+    float us;    // estimated time
+};
+GemmConfig choose_config(const Problem &p);
+
+size_t split_floats(const Problem &p, const GemmConfig &c) {
+    const int bm = 128 << c.height;
+    const size_t tiles = (size_t)((p.batch + bm - 1) / bm) * ((p.rows + kBN - 1) / kBN);
+    return c.splits > 1 ? tiles * c.splits * bm * kBN : 0;
 }
 
 template <int MF>
-hipError_t launch(const Problem &p, int splits, hipStream_t s) {
+hipError_t launch(const Problem &p, int splits, float *partial, unsigned *arrivals, hipStream_t s) {
     constexpr int BM = 128 * MF;
     static std::mutex attr_mutex;
-    static bool attr_set[64][3] = {};
+    static bool attr_set[64] = {};
     int dev = 0;
     if (hipError_t e = hipGetDevice(&dev)) return e;
-    const int inst = gemm_instance(), slot = inst == 8 ? 2 : inst == 4 ? 1 : 0;
-    const size_t lds = kBufs * (size_t)(kWBytes + BM * kRowBytes + (inst == 8 ? 4 : 3) * 1024);
+    const size_t lds = kBufs * (size_t)(kWBytes + BM * kRowBytes + 3 * 1024);
     if (dev >= 0 && dev < 64) {
         std::lock_guard<std::mutex> lock(attr_mutex);
-        if (!attr_set[dev][slot]) {
-            const void *k = inst == 8   ? reinterpret_cast<const void *>(&gemm_mfma8_kernel<MF>)
-                            : inst == 4 ? reinterpret_cast<const void *>(&gemm_mfma4_kernel<MF>)
-                                        : reinterpret_cast<const void *>(&gemm_mfma_kernel<MF>);
-            if (hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)) return e;
-            attr_set[dev][slot] = true;
+        if (!attr_set[dev]) {
+            if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_mfma_kernel<MF>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
+                return e;
+            attr_set[dev] = true;
         }
     }
     const int m_tiles = (p.batch + BM - 1) / BM, n_tiles = (p.rows + kBN - 1) / kBN;
-    const int tiles = m_tiles * n_tiles;
-    float *partial = nullptr;
-    unsigned *arrivals = nullptr;
-    if (splits > 1)
-        if (hipError_t e = split_workspace(s, (size_t)tiles * splits * BM * kBN, (size_t)tiles, &partial, &arrivals)) return e;
-    if (inst == 8)
-        gemm_mfma8_kernel<MF><<<tiles * splits, kThreads8, lds, s>>>(p.x, p.nz, p.sg, p.scales, p.y, p.batch, p.rows, p.cols,
-                                                                     splits, partial, arrivals);
-    else if (inst == 4)
-        gemm_mfma4_kernel<MF><<<tiles * splits, kThreads, lds, s>>>(p.x, p.nz, p.sg, p.scales, p.y, p.batch, p.rows, p.cols,
-                                                                   splits, partial, arrivals);
-    else
-        gemm_mfma_kernel<MF><<<tiles * splits, kThreads, lds, s>>>(p.x, p.nz, p.sg, p.scales, p.y, p.batch, p.rows, p.cols,
-                                                                  splits, partial, arrivals);
+    gemm_mfma_kernel<MF><<<m_tiles * n_tiles * splits, kThreads, lds, s>>>(p.x, p.nz, p.sg, p.scales, p.y, p.batch, p.rows,
+                                                                          p.cols, splits, partial, arrivals);
     return hipGetLastError();
 }
 
@@ -1309,12 +575,6 @@ bool gemm_mfma_supports(const Problem &p, int group) {
 }
 
 namespace {
-struct GemmConfig {
-    int height;  // 0: 128 activation rows per workgroup, 1: 256
-    int splits;  // workgroups per tile along K
-    float us;    // estimated time
-};
-
 // One workgroup occupies a CU (LDS). Taller tiles do more per stage, shorter tiles fill the chip
 // when there are few of them, and when even those leave CUs idle K is split across workgroups.
 // Estimate: (rounds of workgroups over the CUs) x (stages per workgroup) x (time of one stage,
@@ -1346,9 +606,36 @@ GemmConfig choose_config(const Problem &p) {
 float gemm_mfma_cost_us(const Problem &p) { return choose_config(p).us; }
 
 hipError_t launch_gemm_mfma(const Problem &p, hipStream_t s) {
+    GemmConfig c = choose_config(p);
+    float *partial = nullptr;
+    unsigned *arrivals = nullptr;
+    if (c.splits > 1) {
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipError_t e = hipStreamIsCapturing(s, &cap)) return e;
+        if (hipError_t e = split_workspace(s, split_floats(p, c), cap == hipStreamCaptureStatusNone, &partial, &arrivals)) return e;
+        if (!partial) c.splits = 1;  // under capture without a reserved workspace: one workgroup per tile
+    }
+    return c.height == 1 ? launch<2>(p, c.splits, partial, arrivals, s) : launch<1>(p, c.splits, partial, arrivals, s);
+}
+
+hipError_t gemm_mfma_reserve(const Problem &p, hipStream_t s) {
     const GemmConfig c = choose_config(p);
-    if (c.height == 1) return launch<2>(p, c.splits, s);
-    return launch<1>(p, c.splits, s);
+    float *partial = nullptr;
+    unsigned *arrivals = nullptr;
+    return c.splits > 1 ? split_workspace(s, split_floats(p, c), true, &partial, &arrivals) : hipSuccess;
+}
+
+void gemm_mfma_release_all() {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    for (SplitWorkspace &w : g_ws) {
+        (void)hipSetDevice(w.device);
+        if (w.partial) (void)hipFree(w.partial);
+        if (w.arrivals) (void)hipFree(w.arrivals);
+    }
+    g_ws.clear();
+    (void)hipSetDevice(dev);
 }
 
 }  // namespace tllm

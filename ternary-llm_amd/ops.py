@@ -18,7 +18,7 @@ ABI_SYMBOLS = (
     "tllm_linear_plan_create", "tllm_linear_plan_launch", "tllm_linear_plan_weight_bytes",
     "tllm_linear_plan_destroy", "tllm_rmsnorm_f16", "tllm_silu_mul_f16", "tllm_linear_plan_create_normed",
     "tllm_add_f16", "tllm_rope_f16", "tllm_embedding_lookup_f16", "tllm_copy_to_kv_cache_f16",
-    "tllm_linear_plan_kernel",
+    "tllm_linear_plan_kernel", "tllm_gemm_workspace_reserve", "tllm_gemm_workspace_release",
 )
 # include/tllm_model_file.h
 FILE_ABI_SYMBOLS = (
@@ -76,6 +76,9 @@ def lib():
     L.tllm_ternary_gemv_i8_dscale.argtypes = [vp, vp, vp, vp, vp, vp, i, i, i, vp]
     L.tllm_quantize_absmax_i8.argtypes = [vp, vp, vp, i, vp]
     L.tllm_ternary_gemm_f16.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, vp]
+    L.tllm_gemm_workspace_reserve.argtypes = [i, i, i, i, vp]
+    L.tllm_gemm_workspace_release.argtypes = []
+    L.tllm_gemm_workspace_release.restype = None
     L.tllm_linear_plan_create.argtypes = [C.POINTER(vp), C.POINTER(_Problem), i, i]
     L.tllm_linear_plan_create_normed.argtypes = [C.POINTER(vp), C.POINTER(_Problem), C.POINTER(vp), f, i, i]
     L.tllm_linear_plan_launch.argtypes = [vp, vp]
@@ -157,6 +160,16 @@ def ternary_gemm(A, nz_B, sign_B, scales_B, Cout, M, N, K, group_size=128, strea
     """C[M,N] = A[M,K] @ W[N,K]^T (reference include/kernels.cuh:37-40)."""
     check(lib().tllm_ternary_gemm_f16(_ptr(A), _ptr(nz_B), _ptr(sign_B), _ptr(scales_B), _ptr(Cout),
                                       M, N, K, group_size, _stream(stream)))
+
+
+def gemm_workspace_reserve(M, N, K, group_size=128, stream=None):
+    """Creates the split-K workspace of the stream for this GEMM shape ahead of time (e.g. before graph capture)."""
+    check(lib().tllm_gemm_workspace_reserve(M, N, K, group_size, _stream(stream)))
+
+
+def gemm_workspace_release():
+    """Frees every split-K workspace of the process (no GEMM may be in flight)."""
+    lib().tllm_gemm_workspace_release()
 
 
 def rmsnorm(input, weight, output, residual, residual_out, batch, dim, eps, stream=None):

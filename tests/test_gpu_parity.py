@@ -1057,3 +1057,134 @@ def test_full_size_properties_8b(dev, oracle):
     x4 = (x.astype(np.float32) * 4).astype(np.float16)
     np.testing.assert_array_equal(run_gemv(dev, nz, sg, s, x4), 4 * y)
     np.testing.assert_array_equal(run_gemv(dev, nz[1000:1777], sg[1000:1777], s[1000:1777], x), y[1000:1777])
+
+
+# ---------------------------------------------------------- benchmark configurations 4 and 5 at full size
+def _device_problem(torch, rows, cols, p_zero, lo, hi, gen):
+    """Seeded packed weights made on the device (the 70B matrices are too large to pack with numpy in
+    test time): i.i.d. P(0) = p_zero, random sign bits also under zero weights, fp16 scales U[lo, hi]."""
+    words = cols // 32
+    pw = (torch.ones(32, dtype=torch.int64, device="cuda") << torch.arange(32, device="cuda"))
+    nz = torch.empty((rows, words), dtype=torch.int32, device="cuda")
+    step = max(1, (1 << 24) // cols)
+    for r0 in range(0, rows, step):
+        r1 = min(rows, r0 + step)
+        v = ((torch.rand((r1 - r0, words, 32), device="cuda", generator=gen) >= p_zero).to(torch.int64) * pw).sum(dim=2)
+        nz[r0:r1] = torch.where(v >= 2 ** 31, v - 2 ** 32, v).to(torch.int32)
+    sg = torch.randint(-2 ** 31, 2 ** 31 - 1, (rows, words), dtype=torch.int32, device="cuda", generator=gen)
+    sc = (torch.rand((rows, cols // 128), device="cuda", generator=gen) * (hi - lo) + lo).to(torch.float16)
+    return nz, sg, sc
+
+
+def _check_sampled(oracle, torch, A, nz, sg, sc, out, n_rows, n_cols, seed, what):
+    """out[M, N] against the fp64 oracle on sampled activation rows x weight rows; everything finite."""
+    assert bool(torch.isfinite(out).all()), f"{what}: non-finite output"
+    M, N = out.shape
+    rng = np.random.default_rng(seed)
+    ms_ = np.unique(rng.integers(0, M, n_rows))
+    ns_ = np.unique(np.concatenate([rng.integers(0, N, n_cols), [0, N - 1]]))
+    ref = oracle.gemm_f64(A[ms_].cpu().numpy().view(np.uint16), nz[ns_].cpu().numpy().view(np.uint32),
+                          sg[ns_].cpu().numpy().view(np.uint32), sc[ns_].cpu().numpy().view(np.uint16))
+    full = out.float()
+    tau = float(torch.sqrt(torch.mean(full * full)).item()) / 64.0
+    got = out[ms_][:, ns_].cpu().numpy().astype(np.float64)
+    rel = float((np.abs(got - ref) / np.maximum(np.abs(ref), tau)).max())
+    assert rel <= TOL, f"{what}: max_rel {rel:.3e} (tau {tau:.3e})"
+
+
+@pytest.mark.parametrize("N,K", [(14336, 4096), (4096, 14336)])
+@pytest.mark.parametrize("M", [16, 128, 512, 2048])
+def test_cfg4_prefill_gemm_every_m(dev, oracle, M, N, K):
+    """Benchmark configuration 4: X [M, K] N(0,1) against the LLaMA-3-8B gate/up (14336 x 4096) and down
+    (4096 x 14336) matrices, every token count of the configuration. M = 2048 is the only case with eight
+    256-row tiles; M = 128 runs the split-K path on both shapes."""
+    torch, tl = dev
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(400 + M + N)
+    nz, sg, sc = _device_problem(torch, N, K, 0.42, 0.01, 0.03, gen)
+    A = torch.randn((M, K), device="cuda", generator=gen).to(torch.float16)
+    Cm = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    tl.ternary_gemm(A, nz, sg, sc, Cm, M, N, K, 128)
+    torch.cuda.synchronize()
+    _check_sampled(oracle, torch, A, nz, sg, sc, Cm, 6, 80, M + N, f"cfg4 M={M} {N}x{K}")
+
+
+LLAMA70B_LAYER = [(8192, 8192), (1024, 8192), (1024, 8192), (8192, 8192), (28672, 8192), (28672, 8192), (8192, 28672)]
+
+
+@pytest.mark.parametrize("p_zero", [0.2, 0.42, 0.7])
+@pytest.mark.parametrize("batch", [1, 16])
+def test_cfg5_llama70b_layer_plan(dev, oracle, batch, p_zero):
+    """Benchmark configuration 5: one full LLaMA-70B decoder layer (q, k, v, o, gate, up, down at hidden 8192,
+    ffn 28672: 855.6 M weights) as one plan launch at batch 1 and batch 16, fp16 scales U[0.005, 0.02], zero
+    fractions 0.2 / 0.42 / 0.7; sampled rows of every matrix against the oracle. The batch-16 matrices
+    also go through the reference's own entry point for that case (ternary_gemm with M = 16)."""
+    torch, tl = dev
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(int(500 + 100 * p_zero + batch))
+    probs = []
+    for rows, cols in LLAMA70B_LAYER:
+        nz, sg, sc = _device_problem(torch, rows, cols, p_zero, 0.005, 0.02, gen)
+        x = torch.randn((batch, cols), device="cuda", generator=gen).to(torch.float16)
+        y = torch.full((batch, rows), float("nan"), dtype=torch.float16, device="cuda")
+        probs.append((nz, sg, sc, x, y, rows, cols, batch))
+    plan = tl.LinearPlan(probs)
+    plan.launch()
+    torch.cuda.synchronize()
+    for k, (nz, sg, sc, x, y, rows, cols, _) in enumerate(probs):
+        _check_sampled(oracle, torch, x, nz, sg, sc, y, 4, 48, 31 * k + batch, f"cfg5 {rows}x{cols} batch {batch} P0={p_zero}")
+    plan.close()
+    if batch == 16 and p_zero == 0.42:
+        for k in (1, 4, 6):
+            nz, sg, sc, x, y, rows, cols, _ = probs[k]
+            Cm = torch.full((batch, rows), float("nan"), dtype=torch.float16, device="cuda")
+            tl.ternary_gemm(x, nz, sg, sc, Cm, batch, rows, cols, 128)
+            torch.cuda.synchronize()
+            _check_sampled(oracle, torch, x, nz, sg, sc, Cm, 4, 48, k, f"cfg5 gemm entry {rows}x{cols} M=16")
+
+
+def test_gemm_split_k_under_graph_capture(dev, oracle):
+    """A GEMM whose shape splits K, captured into a HIP graph: with the workspace reserved beforehand the
+    captured launch is the split one (bit-identical to the eager call); captured on a stream that has no
+    workspace the call allocates nothing and runs without the split (same values within the bar). Every
+    replay, with eager work between replays, gives the same bits."""
+    torch, tl = dev
+    M, N, K = 256, 1024, 4096
+    nz, sg, s, _ = synth.problem(4300, N, K)
+    A = synth.acts_f16(np.random.default_rng(4301), M, K)
+    rows = np.unique(np.random.default_rng(1).integers(0, M, 6))
+    ref = oracle.gemm_f64(A[rows].view(np.uint16), nz, sg, s.view(np.uint16))
+    dA, dnz, dsg, ds = up(torch, A), up(torch, nz), up(torch, sg), up(torch, s)
+    eager = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    tl.ternary_gemm(dA, dnz, dsg, ds, eager, M, N, K, 128)
+    torch.cuda.synchronize()
+    assert_close(oracle, eager.cpu().numpy().astype(np.float64)[rows], ref, what="eager split-K")
+    for reserve in (True, False):
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        out = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            if reserve:
+                tl.gemm_workspace_reserve(M, N, K, 128, stream=side)
+            side.synchronize()
+            with torch.cuda.graph(graph, stream=side):
+                tl.ternary_gemm(dA, dnz, dsg, ds, out, M, N, K, 128, stream=side)
+        torch.cuda.synchronize()
+        first = None
+        for replay in range(3):
+            out.fill_(float("nan"))
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            got = out.cpu().numpy()
+            assert_close(oracle, got.astype(np.float64)[rows], ref, what=f"captured GEMM reserve={reserve} replay {replay}")
+            if reserve:
+                assert torch.equal(out.view(torch.int16), eager.view(torch.int16)), f"replay {replay}: differs from the eager split call"
+            if first is None:
+                first = got.view(np.uint16).copy()
+            assert np.array_equal(got.view(np.uint16), first), f"reserve={reserve} replay {replay}: bits changed"
+            if replay == 1:   # eager work between replays
+                tl.ternary_gemm(dA, dnz, dsg, ds, eager, M, N, K, 128)
+                torch.cuda.synchronize()
+        del graph

@@ -34,7 +34,9 @@ enum {
     TLLM_ERR_TOO_LARGE = -4,    /* an element count does not fit the index type, or exceeds a stated limit */
     TLLM_ERR_ALIAS = -5,        /* output overlaps the activation input */
     TLLM_ERR_BAD_PLAN = -6,     /* plan handle is NULL, count < 1, batch out of range, or a pair / prologue rule is broken */
-    TLLM_ERR_MISALIGNED = -7    /* masks/activations not 16-byte aligned, scales/outputs not 2-byte aligned */
+    TLLM_ERR_MISALIGNED = -7,   /* masks/activations not 16-byte aligned, scales/outputs not 2-byte aligned */
+    /* -8 and -9 belong to tllm_model_file.h */
+    TLLM_ERR_SCRATCH_TOO_SMALL = -10 /* tllm_ternary_gemm_f16_static: the shape needs more exchange memory than the fixed scratch */
 };
 
 /* Human-readable text for a negative TLLM_ERR_* code (host pointer, static storage). */
@@ -100,6 +102,23 @@ int tllm_quantize_absmax_i8(const uint16_t *input, int8_t *output, float *scale,
 int tllm_ternary_gemm_f16(const uint16_t *A, const uint32_t *nz_B, const uint32_t *sign_B,
                           const uint16_t *scales_B, uint16_t *C, int M, int N, int K,
                           int group_size, tllm_stream_t stream);
+
+/*
+ * tllm_ternary_gemm_f16 for callers that cannot allocate device memory (code under HIP graph capture,
+ * serving loops and harnesses that forbid hipMalloc): same arguments, same kernels, same results bit for
+ * bit, but the split-K exchange goes through a fixed array of TLLM_GEMM_STATIC_SCRATCH_BYTES in device
+ * memory that the library holds on every GPU it runs on until the process ends. The call never
+ * allocates, frees or synchronises. A shape whose exchange would not fit is rejected with
+ * TLLM_ERR_SCRATCH_TOO_SMALL before anything is launched (with the tile shapes of this library the need
+ * is at most CUs * 128 KiB: every shape fits on a 256-CU MI355X). All calls on one GPU share the one
+ * array: calls that overlap in time on one GPU (two streams, two threads, two graph branches) race on it;
+ * issue them on one stream, or use tllm_ternary_gemm_f16 with its per-stream workspaces.
+ * No counterpart in the reference, whose GEMM needs no exchange memory.
+ */
+#define TLLM_GEMM_STATIC_SCRATCH_BYTES (32 * 1024 * 1024 + 4096)
+int tllm_ternary_gemm_f16_static(const uint16_t *A, const uint32_t *nz_B, const uint32_t *sign_B,
+                                 const uint16_t *scales_B, uint16_t *C, int M, int N, int K,
+                                 int group_size, tllm_stream_t stream);
 
 /*
  * Creates, or grows, the split-K workspace of `stream` for the GEMM shape (M, N, K) so that later

@@ -19,6 +19,7 @@ from .ops import (  # noqa: F401
     rope,
     silu_mul,
     ternary_gemm,
+    ternary_gemm_static,
     ternary_gemv,
     ternary_gemv_int8,
     ternarize_pack,

@@ -66,6 +66,9 @@ const char *tllm_error_string(int code) {
         case TLLM_ERR_MISALIGNED: return "pointer alignment: masks/activations need 16 bytes, fp16 arrays 2";
         case -8: return "file cannot be opened, is truncated, or a write failed";   // TLLM_ERR_IO
         case -9: return "not a .tllm file of a supported version, or a header field is out of range";  // TLLM_ERR_BAD_FILE
+        case TLLM_ERR_SCRATCH_TOO_SMALL:
+            return "the split-K exchange of this GEMM shape needs more than the fixed device scratch of "
+                   "tllm_ternary_gemm_f16_static (TLLM_GEMM_STATIC_SCRATCH_BYTES): use tllm_ternary_gemm_f16";
         default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error code";
     }
 }
@@ -85,6 +88,16 @@ int tllm_ternary_gemm_f16(const uint16_t *A, const uint32_t *nz_B, const uint32_
     if (M < 1) return TLLM_ERR_BAD_SHAPE;
     Problem p{nz_B, sign_B, scales_B, A, C, N, K, M, 0};
     return tllm::run_linear(p, group_size, (hipStream_t)stream);
+}
+
+int tllm_ternary_gemm_f16_static(const uint16_t *A, const uint32_t *nz_B, const uint32_t *sign_B,
+                                 const uint16_t *scales_B, uint16_t *C, int M, int N, int K,
+                                 int group_size, tllm_stream_t stream) {
+    if (M < 1) return TLLM_ERR_BAD_SHAPE;
+    Problem p{nz_B, sign_B, scales_B, A, C, N, K, M, 0};
+    if (int e = tllm::check_linear(p, group_size)) return e;
+    if (tllm::dispatch_takes_gemm(p, group_size) && !tllm::gemm_mfma_static_fits(p)) return TLLM_ERR_SCRATCH_TOO_SMALL;
+    return (int)tllm::dispatch_linear(p, group_size, (hipStream_t)stream, true);
 }
 
 int tllm_gemm_workspace_reserve(int M, int N, int K, int group_size, tllm_stream_t stream) {

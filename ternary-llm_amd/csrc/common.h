@@ -104,9 +104,15 @@ float gemm_mfma_cost_us(const Problem &p);  // rough time of launch_gemm_mfma, t
 // Creates (or grows) the split-K workspace of stream s for this shape, if the shape splits K at all.
 hipError_t gemm_mfma_reserve(const Problem &p, hipStream_t s);
 void gemm_mfma_release_all();  // frees every split-K workspace (nothing may still be running on them)
+// The same launch with the split-K exchange in the library's fixed device array (no allocation, ever).
+bool gemm_mfma_static_fits(const Problem &p);
+hipError_t launch_gemm_mfma_static(const Problem &p, hipStream_t s);
 
 // Picks the kernel for one linear (fast 128-group paths when they apply, else the row-wave kernel).
-hipError_t dispatch_linear(const Problem &p, int group, hipStream_t s);
+// static_scratch: a GEMM that splits K exchanges its partial sums through the fixed device array.
+hipError_t dispatch_linear(const Problem &p, int group, hipStream_t s, bool static_scratch = false);
+// True if dispatch_linear would run the prefill GEMM kernel (the only path that may need exchange memory).
+bool dispatch_takes_gemm(const Problem &p, int group);
 
 // Device-resident schedule of a multi-problem launch.
 struct PlanDevice {

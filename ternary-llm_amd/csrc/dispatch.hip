@@ -21,29 +21,42 @@ int forced_path() {
 }
 }  // namespace
 
-hipError_t dispatch_linear(const Problem &p, int group, hipStream_t s) {
-    if (group != 128) return launch_gemv_rowwave_f16(p, group, s);
-    if (p.batch == 1 && gemv_mfma_supports(p, group)) return launch_gemv_mfma(p, s);
+namespace {
+// The activation rows go through the batched decode kernel in passes of 16 (true), or not (false).
+bool streams_in_passes(const Problem &p, int group) {
     Problem probe = p;
     probe.batch = p.batch < kBatchRows ? p.batch : kBatchRows;
-    if (p.batch > 1 && gemv_batch_supports(probe, group)) {
-        const int passes = (p.batch + kBatchRows - 1) / kBatchRows;
-        const bool gemm_ok = gemm_mfma_supports(p, group);
-        bool stream = passes == 1 || !gemm_ok || (float)passes * gemv_batch_cost_us(probe) < gemm_mfma_cost_us(p);
-        if (passes > 1 && gemm_ok && forced_path()) stream = forced_path() == 2;
-        if (stream) {
-            for (int b0 = 0; b0 < p.batch; b0 += kBatchRows) {
-                Problem q = p;
-                q.batch = p.batch - b0 < kBatchRows ? p.batch - b0 : kBatchRows;
-                q.x = p.x + (size_t)b0 * p.cols;
-                q.y = p.y + (size_t)b0 * p.rows;
-                if (hipError_t e = launch_gemv_batch(q, s)) return e;
-            }
-            return hipSuccess;
+    if (p.batch <= 1 || !gemv_batch_supports(probe, group)) return false;
+    const int passes = (p.batch + kBatchRows - 1) / kBatchRows;
+    const bool gemm_ok = gemm_mfma_supports(p, group);
+    bool stream = passes == 1 || !gemm_ok || (float)passes * gemv_batch_cost_us(probe) < gemm_mfma_cost_us(p);
+    if (passes > 1 && gemm_ok && forced_path()) stream = forced_path() == 2;
+    return stream;
+}
+}  // namespace
+
+bool dispatch_takes_gemm(const Problem &p, int group) {
+    if (group != 128) return false;
+    if (p.batch == 1 && gemv_mfma_supports(p, group)) return false;
+    if (streams_in_passes(p, group)) return false;
+    return !gemv_mfma_supports(p, group) && gemm_mfma_supports(p, group);
+}
+
+hipError_t dispatch_linear(const Problem &p, int group, hipStream_t s, bool static_scratch) {
+    if (group != 128) return launch_gemv_rowwave_f16(p, group, s);
+    if (p.batch == 1 && gemv_mfma_supports(p, group)) return launch_gemv_mfma(p, s);
+    if (streams_in_passes(p, group)) {
+        for (int b0 = 0; b0 < p.batch; b0 += kBatchRows) {
+            Problem q = p;
+            q.batch = p.batch - b0 < kBatchRows ? p.batch - b0 : kBatchRows;
+            q.x = p.x + (size_t)b0 * p.cols;
+            q.y = p.y + (size_t)b0 * p.rows;
+            if (hipError_t e = launch_gemv_batch(q, s)) return e;
         }
+        return hipSuccess;
     }
     if (gemv_mfma_supports(p, group)) return launch_gemv_mfma(p, s);
-    if (gemm_mfma_supports(p, group)) return launch_gemm_mfma(p, s);
+    if (gemm_mfma_supports(p, group)) return static_scratch ? launch_gemm_mfma_static(p, s) : launch_gemm_mfma(p, s);
     // wider batches: four activation rows at a time through the tall-tile kernel
     for (int b0 = 0; b0 < p.batch; b0 += kTallBatch) {
         Problem q = p;

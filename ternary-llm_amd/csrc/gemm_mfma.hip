@@ -529,6 +529,29 @@ hipError_t split_workspace(hipStream_t s, size_t floats, bool may_allocate, floa
     return hipSuccess;
 }
 
+// The exchange memory of tllm_ternary_gemm_f16_static: a fixed array in device memory, one copy per GPU,
+// held until the process ends. Arrival counters first (zero when the module is loaded, left at zero by
+// every launch), then the fp32 slots.
+constexpr size_t kStaticSlotFloats = (size_t)TLLM_GEMM_STATIC_SCRATCH_BYTES / 4 - kArrivalSlots;
+static __device__ __align__(256) unsigned char scratch[TLLM_GEMM_STATIC_SCRATCH_BYTES];
+
+// Device address of `scratch` on the current device, asked once per device.
+hipError_t static_scratch(unsigned char **out) {
+    static std::mutex m;
+    static unsigned char *ptr[64] = {};
+    int dev = 0;
+    if (hipError_t e = hipGetDevice(&dev)) return e;
+    if (dev < 0 || dev >= 64) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(m);
+    if (!ptr[dev]) {
+        unsigned char *p = nullptr;
+        if (hipError_t e = hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(scratch))) return e;
+        ptr[dev] = p;
+    }
+    *out = ptr[dev];
+    return hipSuccess;
+}
+
 struct GemmConfig {
     int height;  // 0: 128 activation rows per workgroup, 1: 256
     int splits;  // workgroups per tile along K
@@ -636,6 +659,21 @@ void gemm_mfma_release_all() {
     }
     g_ws.clear();
     (void)hipSetDevice(dev);
+}
+
+bool gemm_mfma_static_fits(const Problem &p) { return split_floats(p, choose_config(p)) <= kStaticSlotFloats; }
+
+hipError_t launch_gemm_mfma_static(const Problem &p, hipStream_t s) {
+    const GemmConfig c = choose_config(p);
+    float *partial = nullptr;
+    unsigned *arrivals = nullptr;
+    if (c.splits > 1) {
+        unsigned char *base = nullptr;
+        if (hipError_t e = static_scratch(&base)) return e;
+        arrivals = reinterpret_cast<unsigned *>(base);
+        partial = reinterpret_cast<float *>(base) + kArrivalSlots;
+    }
+    return c.height == 1 ? launch<2>(p, c.splits, partial, arrivals, s) : launch<1>(p, c.splits, partial, arrivals, s);
 }
 
 }  // namespace tllm

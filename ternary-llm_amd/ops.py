@@ -19,6 +19,7 @@ ABI_SYMBOLS = (
     "tllm_linear_plan_destroy", "tllm_rmsnorm_f16", "tllm_silu_mul_f16", "tllm_linear_plan_create_normed",
     "tllm_add_f16", "tllm_rope_f16", "tllm_embedding_lookup_f16", "tllm_copy_to_kv_cache_f16",
     "tllm_linear_plan_kernel", "tllm_gemm_workspace_reserve", "tllm_gemm_workspace_release",
+    "tllm_ternary_gemm_f16_static",
 )
 # include/tllm_model_file.h
 FILE_ABI_SYMBOLS = (
@@ -76,6 +77,7 @@ def lib():
     L.tllm_ternary_gemv_i8_dscale.argtypes = [vp, vp, vp, vp, vp, vp, i, i, i, vp]
     L.tllm_quantize_absmax_i8.argtypes = [vp, vp, vp, i, vp]
     L.tllm_ternary_gemm_f16.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, vp]
+    L.tllm_ternary_gemm_f16_static.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, vp]
     L.tllm_gemm_workspace_reserve.argtypes = [i, i, i, i, vp]
     L.tllm_gemm_workspace_release.argtypes = []
     L.tllm_gemm_workspace_release.restype = None
@@ -160,6 +162,12 @@ def ternary_gemm(A, nz_B, sign_B, scales_B, Cout, M, N, K, group_size=128, strea
     """C[M,N] = A[M,K] @ W[N,K]^T (reference include/kernels.cuh:37-40)."""
     check(lib().tllm_ternary_gemm_f16(_ptr(A), _ptr(nz_B), _ptr(sign_B), _ptr(scales_B), _ptr(Cout),
                                       M, N, K, group_size, _stream(stream)))
+
+
+def ternary_gemm_static(A, nz_B, sign_B, scales_B, Cout, M, N, K, group_size=128, stream=None):
+    """ternary_gemm that never allocates: the split-K exchange uses the library's fixed device array."""
+    check(lib().tllm_ternary_gemm_f16_static(_ptr(A), _ptr(nz_B), _ptr(sign_B), _ptr(scales_B), _ptr(Cout),
+                                             M, N, K, group_size, _stream(stream)))
 
 
 def gemm_workspace_reserve(M, N, K, group_size=128, stream=None):

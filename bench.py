@@ -1,14 +1,29 @@
 #!/usr/bin/env python3
 """Benchmark of the ternary linear-layer hot path on one MI355X.
 
-Default workload (benchmark configuration 3): the LLaMA-3-8B decode projection sweep at batch 1 -
-7 ternary GEMVs per layer (q, k, v, o, gate, up, down) x 32 layers, 1.854 GB of packed
-weights + scales resident in HBM, issued as ONE launch of the multi-problem plan. A "step" is
-one sweep. The metric is the packed weight+scale stream rate in GB/s (algorithmic bytes =
-0.265625 * rows * cols per matrix) and its fraction of the 8 TB/s HBM peak.
+Headline workload (benchmark configuration 3): the LLaMA-3-8B decode projection sweep at batch 1 -
+7 ternary GEMVs per layer (q, k, v, o, gate, up, down) x 32 layers, 1.854 GB of packed weights + scales
+resident in HBM, issued as ONE launch of the multi-problem plan. A "step" is one sweep. The metric is the
+packed weight+scale stream rate in GB/s (algorithmic bytes = 0.265625 * rows * cols per matrix) and its
+fraction of the 8 TB/s HBM peak.
 
-Prints one JSON line (value, roofline, other_batches, gemm, cpu_baseline). `--gpus` above 1 is refused: this build
-measures one GPU.
+The same run measures every other benchmark configuration and reports them in `configs`:
+  cfg1  one 2048 x 2048 GEMV (cache-resident, and rotated over > 512 MB of distinct matrices)
+  cfg2  the LLaMA-1B layer set x 16 layers as one plan (cache-resident 258 MB, and rotated over 775 MB)
+  cfg3  the 8B sweep at batch 1 (the headline), 4 and 16
+  cfg4  the prefill GEMM, M in {16, 128, 512, 2048} x {gate/up 14336 x 4096, down 4096 x 14336}
+  cfg5  LLaMA-70B, all 80 layers resident (18.2 GB packed), batch 1 and 16 (--sparsity-sweep adds
+        P(0) = 0.2 and 0.7)
+plus `single_calls` (the reference's own call pattern, one operator call per matrix, replayed from a
+captured HIP graph so that no host time is in the figure: fp16 and int8 activations, and the dependent
+chain of a decode step), `copy_ceiling` (what this GPU streams with a plain read / copy kernel) and
+`cpu_baseline` (the reference's host loop, restated in C, on this machine's cores).
+
+Every time is taken with HIP events on the launch stream around back-to-back launches, after an untimed
+settle phase (the GPU idles near 100 MHz and needs tens of milliseconds of load to reach its working
+clocks); `mean`, `median` and `min` are per step, the last two over groups of consecutive steps.
+
+Prints one JSON line. `--gpus` above 1 is refused: this build measures one GPU.
 """
 import argparse
 import json
@@ -22,10 +37,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes one launch of the default workload moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by
-# a copy kernel of known size (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); valid for the default workload only.
-DEFAULT_WORKLOAD_TRAFFIC_BYTES = 1980595008
-MFMA_F16_PEAK_TFLOPS = 2500.0
+MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense FP16 matrix peak
+# HBM bytes one launch of the headline workload moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
+# copy kernel of known size (profiles/gemv_mfma_wide__llama8b_sweep_b1.md); valid for that workload only.
+HEADLINE_TRAFFIC_BYTES = 1980595008
+HEADLINE_TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this workload (profiles/gemv_mfma_wide__llama8b_sweep_b1.md), not read in this run"
 
 SHAPES = {
     # name: (hidden, q_dim, kv_dim, ffn, layers)
@@ -33,7 +49,6 @@ SHAPES = {
     "llama8b": (4096, 4096, 1024, 14336, 32),
     "llama70b": (8192, 8192, 1024, 28672, 80),
 }
-
 
 CUSTOM = []  # filled by --matrices "ROWSxCOLS,..." (replaces the model's per-layer matrix list)
 
@@ -66,7 +81,7 @@ def gen_masks(torch, rows, cols, p_zero, gen):
     return nz, sg
 
 
-def build_sweep(torch, model, layers, batch, p_zero, scale_lo, scale_hi, seed):
+def build_sweep(torch, model, layers, batch, p_zero, scale_lo, scale_hi, seed, unit_rms=False):
     gen = torch.Generator(device="cuda")
     gen.manual_seed(seed)
     problems, meta = [], []
@@ -75,11 +90,26 @@ def build_sweep(torch, model, layers, batch, p_zero, scale_lo, scale_hi, seed):
             nz, sg = gen_masks(torch, rows, cols, p_zero, gen)
             sc = (torch.rand((rows, cols // 128), device="cuda", generator=gen) * (scale_hi - scale_lo)
                   + scale_lo).to(torch.float16)
-            x = torch.randn((batch, cols), device="cuda", generator=gen).to(torch.float16)
+            x = torch.randn((batch, cols), device="cuda", generator=gen)
+            if unit_rms:
+                x = x / torch.sqrt(torch.mean(x * x, dim=1, keepdim=True))
+            x = x.to(torch.float16)
             y = torch.zeros((batch, rows), dtype=torch.float16, device="cuda")
             problems.append((nz, sg, sc, x, y, rows, cols, batch))
             meta.append((layer, name))
     return problems, meta
+
+
+def with_batch(torch, problems, batch, seed):
+    """The same weights with `batch` activation rows per matrix."""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(seed)
+    out = []
+    for (nz, sg, sc, _, _, rows, cols, _) in problems:
+        x = torch.randn((batch, cols), device="cuda", generator=gen).to(torch.float16)
+        y = torch.zeros((batch, rows), dtype=torch.float16, device="cuda")
+        out.append((nz, sg, sc, x, y, rows, cols, batch))
+    return out
 
 
 def check_sample(oracle, problems, idxs, rows_per=64, seed=0):
@@ -96,79 +126,180 @@ def check_sample(oracle, problems, idxs, rows_per=64, seed=0):
         got = y[:, pick].cpu().numpy().astype(np.float64)
         ref = oracle.gemm_f64(xs, nzs, sgs, scs)
         # the error floor uses the rms of the whole output vector, not of the sample
-        full = y.cpu().numpy().astype(np.float64)
-        tau = float(np.sqrt(np.mean(full * full))) / 64.0
+        full = y.float()
+        tau = float((full * full).mean().sqrt().item()) / 64.0
         rel = np.abs(got - ref) / np.maximum(np.abs(ref), tau)
         worst = max(worst, float(rel.max()))
     return worst
 
 
-def cpu_baseline(oracle, problems, n_layer_mats, threads, mt_layers=8):
-    """The reference's fp32 host loop (oracle restatement), batch 1: single-threaded over ONE layer's
-    matrices (the reference's own form) and split by rows over `threads` host threads over the
-    first `mt_layers` layers. About 20 core-seconds of CPU work in total."""
-    def host(pr):
-        nz, sg, sc, x, y, rows, cols, batch = pr
-        return (nz.cpu().numpy().view(np.uint32), sg.cpu().numpy().view(np.uint32),
-                sc.cpu().numpy().astype(np.float32), x[0].cpu().numpy().astype(np.float32), rows, cols)
+class Timer:
+    """HIP-event timing of back-to-back launches on torch's current stream (the stream every launch of
+    this file uses). Untimed: launches for `settle_ms`, then `warmup` more. Timed: `steps` launches, with an
+    event between groups of consecutive launches so that a median and a minimum exist beside the mean."""
 
-    st_bytes, t_st = 0, 0.0
-    for pr in problems[:n_layer_mats]:
-        nzh, sgh, sch, xh, rows, cols = host(pr)
+    def __init__(self, torch, settle_ms):
+        self.torch = torch
+        self.settle_ms = settle_ms
+
+    def run(self, fn, steps, warmup):
+        torch = self.torch
+        untimed = 0
         t0 = time.perf_counter()
-        oracle.gemv_hostloop(nzh, sgh, sch, xh, threads=1)
-        t_st += time.perf_counter() - t0
-        st_bytes += packed_bytes(rows, cols)
-    mt_bytes, t_mt = 0, 0.0
-    mt_probs = problems[:n_layer_mats * mt_layers]
-    for pr in mt_probs:
-        nzh, sgh, sch, xh, rows, cols = host(pr)
-        t0 = time.perf_counter()
-        oracle.gemv_hostloop(nzh, sgh, sch, xh, threads=threads)
-        t_mt += time.perf_counter() - t0
-        mt_bytes += packed_bytes(rows, cols)
-    return {
-        "value": round(mt_bytes / t_mt / 1e9, 4), "unit": "GB/s", "cores": threads, "kind": "port",
-        "sample": f"{len(mt_probs)} GEMVs = {len(mt_probs) // n_layer_mats} decoder layers ({mt_bytes} packed bytes) "
-                  f"in {t_mt:.2f} s with rows split over {threads} threads; single thread: one layer "
-                  f"({st_bytes} packed bytes) in {t_st:.2f} s; loop = tests/test_ternary_gemv.cu:40-75 restated in C",
-        "single_thread_GBps": round(st_bytes / t_st / 1e9, 4),
-    }
+        while (time.perf_counter() - t0) * 1e3 < self.settle_ms:
+            for _ in range(10):
+                fn()
+            untimed += 10
+            torch.cuda.synchronize()
+        for _ in range(warmup):
+            fn()
+        untimed += warmup
+        torch.cuda.synchronize()
+        group = max(1, steps // 20)
+        n_groups = (steps + group - 1) // group
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(n_groups + 1)]
+        done = 0
+        ev[0].record()
+        for g in range(n_groups):
+            n = min(group, steps - done)
+            for _ in range(n):
+                fn()
+            done += n
+            ev[g + 1].record()
+        torch.cuda.synchronize()
+        per = []
+        done = 0
+        for g in range(n_groups):
+            n = min(group, steps - done)
+            done += n
+            per.append(ev[g].elapsed_time(ev[g + 1]) / n)
+        total = ev[0].elapsed_time(ev[n_groups])
+        return {"mean_ms": total / steps, "median_ms": float(np.median(per)), "min_ms": float(np.min(per)),
+                "steps": steps, "untimed_launches": untimed, "steps_per_timing_group": group}
 
 
-MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense FP16 matrix peak
+def stats_us(t):
+    return {"us": round(t["mean_ms"] * 1e3, 2), "us_median": round(t["median_ms"] * 1e3, 2),
+            "us_min": round(t["min_ms"] * 1e3, 2), "steps": t["steps"], "untimed_launches": t["untimed_launches"]}
 
 
-def gemm_report(torch, tl, orc, seed, m_list, p_zero=0.42, calls=200, warm=20, settle_ms=200.0):
-    """Prefill GEMM (cfg4): LLaMA-3-8B gate/up 14336x4096 and down 4096x14336, M tokens each.
-    Times `calls` back-to-back launches with events on the launch stream, checks sampled outputs
-    against the FP64 oracle, and reports dense-equivalent 2*M*N*K flops. Every case first runs
-    untimed for `settle_ms`: the host-side oracle check of the case before leaves the GPU idle long
-    enough for its clocks to drop (133 MHz), and they need tens of milliseconds of work to come back."""
+def hbm_row(name, t, nbytes, kernel, parity=None, note=None):
+    gbps = nbytes / (t["mean_ms"] * 1e-3) / 1e9
+    row = {"config": name, **stats_us(t), "packed_bytes": nbytes, "GBps": round(gbps, 1),
+           "GBps_best": round(nbytes / (t["min_ms"] * 1e-3) / 1e9, 1), "bound": "hbm",
+           "frac_hbm_peak": round(gbps / HBM_PEAK_GBS, 4), "kernel": kernel}
+    if parity is not None:
+        row["parity_max_rel_sampled"] = parity
+    if note:
+        row["note"] = note
+    return row
+
+
+def capture(torch, fn):
+    """Records fn's launches into a HIP graph on a side stream; returns the graph (replay() = one step)."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        fn()                      # warm-up on the capture stream (per-stream state is created here, not under capture)
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            fn()
+    torch.cuda.synchronize()
+    return graph
+
+
+def cfg1_rows(torch, tl, orc, timer, seed):
+    """One 2048 x 2048 GEMV per call (the reference's own test shape, 1.1 MB packed). A call is far below
+    the launch floor, so the row is latency, not bandwidth. Calls are replayed from a captured graph (no
+    host time): 256 calls on ONE matrix (cache-resident) and 512 calls over 512 distinct matrices
+    (582 MB, beyond L2 and the 256 MB Infinity Cache)."""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(seed + 11)
+    rows = cols = 2048
+    n_distinct = 512
+    nz, sg = gen_masks(torch, rows * 8, cols, 0.42, gen)    # 8 matrices of random bits, reused with offsets below
+    nz_all = nz.repeat(n_distinct // 8, 1).contiguous()
+    sg_all = sg.repeat(n_distinct // 8, 1).contiguous()
+    sc_all = (torch.rand((rows * n_distinct, cols // 128), device="cuda", generator=gen) * 0.02 + 0.01).to(torch.float16)
+    x = torch.randn((1, cols), device="cuda", generator=gen).to(torch.float16)
+    y = torch.zeros((n_distinct, rows), dtype=torch.float16, device="cuda")
+    mats = [(nz_all[i * rows:(i + 1) * rows], sg_all[i * rows:(i + 1) * rows], sc_all[i * rows:(i + 1) * rows]) for i in range(n_distinct)]
+
+    def same():
+        for _ in range(256):
+            tl.ternary_gemv(*mats[0], x, y[0], rows, cols, 128)
+
+    def rotated():
+        for i in range(n_distinct):
+            tl.ternary_gemv(*mats[i], x, y[i], rows, cols, 128)
+
+    out = []
+    nbytes = packed_bytes(rows, cols)
+    for name, fn, calls, note in (("cfg1: 2048x2048 GEMV, same matrix (cache-resident)", same, 256,
+                                   "1.1 MB of weights stay in L2: latency of one launch, not HBM bandwidth"),
+                                  ("cfg1: 2048x2048 GEMV, rotated over 512 distinct matrices (582 MB)", rotated, n_distinct,
+                                   "every call reads weights that left the caches")):
+        graph = capture(torch, fn)
+        t = timer.run(graph.replay, 20, 3)
+        per_call = {k: v / calls for k, v in t.items() if k.endswith("_ms")}
+        row = hbm_row(name, {**t, **per_call}, nbytes, "tllm::gemv_mfma_kernel<Wide, fine>", note=note)
+        row["calls_per_graph_replay"] = calls
+        out.append(row)
+        del graph
+    probs = [(mats[3][0], mats[3][1], mats[3][2], x, y[3:4], rows, cols, 1)]
+    out[1]["parity_max_rel_sampled"] = check_sample(orc, probs, [0])
+    return out
+
+
+def plan_rows(torch, tl, orc, timer, label, model, layers, batches, p_zero, lo, hi, seed, steps, warmup, copies=1,
+              unit_rms=False, problems=None):
+    """A model's projection sweep as one plan launch per step, for each batch size. copies > 1: that many
+    distinct weight sets, launched in turn (a step = one set), so that no set is still in a cache when its
+    turn comes again."""
+    sets = [problems] if problems is not None else []
+    while len(sets) < copies:
+        sets.append(build_sweep(torch, model, layers, 1, p_zero, lo, hi, seed + 1000 * len(sets), unit_rms)[0])
+    nbytes = sum(packed_bytes(p[5], p[6]) for p in sets[0])
+    rows = []
+    for b in batches:
+        psets = [s if b == 1 else with_batch(torch, s, b, seed + 100 + b) for s in sets]
+        plans = [tl.LinearPlan(ps) for ps in psets]
+        turn = [0]
+
+        def step():
+            plans[turn[0] % len(plans)].launch()
+            turn[0] += 1
+
+        t = timer.run(step, steps, warmup)
+        n = len(psets[0])
+        parity = check_sample(orc, psets[-1], sorted(set([0, 1, 4, 6, n - 1, n // 2])))
+        note = None
+        if copies > 1:
+            note = f"rotated over {copies} distinct weight sets ({copies * nbytes} bytes)"
+        elif nbytes < 512 * 1024 * 1024:
+            note = "cache-resident: the set fits the 256 MB Infinity Cache, so the figure is not an HBM rate"
+        rows.append(hbm_row(f"{label}, batch {b}", t, nbytes, plans[0].kernel, parity, note))
+        rows[-1]["matrices_per_launch"] = n
+        for pl in plans:
+            pl.close()
+        del psets, plans
+    return rows, sets[0]
+
+
+def gemm_rows(torch, tl, orc, timer, seed, m_list, p_zero, calls, warm):
+    """Prefill GEMM (cfg4): LLaMA-3-8B gate/up 14336x4096 and down 4096x14336, M tokens each; dense-equivalent
+    2*M*N*K flops against the FP16 matrix peak (M = 16 is HBM-bound and also gets its weight-stream rate)."""
     gen = torch.Generator(device="cuda")
     gen.manual_seed(seed + 4)
-    cases = []
+    rows = []
     for (n, k) in ((14336, 4096), (4096, 14336)):
         nz, sg = gen_masks(torch, n, k, p_zero, gen)
         sc = (torch.rand((n, k // 128), device="cuda", generator=gen) * 0.02 + 0.01).to(torch.float16)
         for m in m_list:
             a = torch.randn((m, k), device="cuda", generator=gen).to(torch.float16)
             c = torch.zeros((m, n), dtype=torch.float16, device="cuda")
-            t_settle = time.perf_counter()
-            while (time.perf_counter() - t_settle) * 1e3 < settle_ms:
-                for _ in range(20):
-                    tl.ternary_gemm(a, nz, sg, sc, c, m, n, k, 128)
-                torch.cuda.synchronize()
-            for _ in range(warm):
-                tl.ternary_gemm(a, nz, sg, sc, c, m, n, k, 128)
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            for _ in range(calls):
-                tl.ternary_gemm(a, nz, sg, sc, c, m, n, k, 128)
-            e1.record()
-            torch.cuda.synchronize()
-            us = e0.elapsed_time(e1) / calls * 1e3
+            t = timer.run(lambda: tl.ternary_gemm(a, nz, sg, sc, c, m, n, k, 128), calls, warm)
             rng = np.random.default_rng(m + n)
             ms_ = np.unique(rng.integers(0, m, 4))
             ns_ = np.unique(rng.integers(0, n, 96))
@@ -178,28 +309,70 @@ def gemm_report(torch, tl, orc, seed, m_list, p_zero=0.42, calls=200, warm=20, s
             tau = float(torch.sqrt(torch.mean(full * full)).item()) / 64.0
             got = full.cpu().numpy().astype(np.float64)[np.ix_(ms_, ns_)]
             rel = float((np.abs(got - ref) / np.maximum(np.abs(ref), tau)).max())
-            tflops = 2.0 * m * n * k / us / 1e6
-            cases.append({"M": m, "N": n, "K": k, "us": round(us, 2), "tflops": round(tflops, 1),
-                          "frac_mfma_peak": round(tflops / MFMA_F16_PEAK_TFLOPS, 4), "max_rel_sampled": rel})
+            tflops = 2.0 * m * n * k / (t["mean_ms"] * 1e-3) / 1e12
+            row = {"config": f"cfg4: prefill GEMM M={m}, W {n}x{k}", "M": m, "N": n, "K": k, **stats_us(t),
+                   "tflops": round(tflops, 1), "tflops_best": round(2.0 * m * n * k / (t["min_ms"] * 1e-3) / 1e12, 1),
+                   "bound": "mfma" if m > 16 else "hbm", "frac_mfma_peak": round(tflops / MFMA_F16_PEAK_TFLOPS, 4),
+                   "kernel": "tllm::gemm_mfma_kernel" if m > 16 else "tllm::gemv_batch_kernel", "max_rel_sampled": rel}
+            if m <= 16:
+                gb = packed_bytes(n, k) / (t["mean_ms"] * 1e-3) / 1e9
+                row["GBps"] = round(gb, 1)
+                row["frac_hbm_peak"] = round(gb / HBM_PEAK_GBS, 4)
+            rows.append(row)
             del a, c, full
         del nz, sg, sc
-    m512 = [c for c in cases if c["M"] == 512]
-    agg = None
-    if m512:
-        agg = sum(2.0 * c["M"] * c["N"] * c["K"] for c in m512) / sum(c["us"] for c in m512) / 1e6
-    return {"workload": "cfg4: prefill GEMM, LLaMA-3-8B gate/up 14336x4096 and down 4096x14336",
-            "unit": "TFLOP/s (2*M*N*K)", "bound": "mfma", "peak": MFMA_F16_PEAK_TFLOPS,
-            "kernel": "tllm::gemm_mfma_kernel", "calls_timed": calls,
-            "m512_tflops": round(agg, 1) if agg else None,
-            "m512_frac": round(agg / MFMA_F16_PEAK_TFLOPS, 4) if agg else None,
-            "cases": cases}
+    return rows
 
 
-def decode_chain_report(torch, tl, problems, model, layers, reps=40):
-    """The linear-side launches of a batch-1 decode step over the sweep's own weights, issued in the
-    order a transformer needs them (every launch after the one before, as reference
-    src/transformer.cpp:193-296 does): (a) the reference's ten launches per layer, (b) q/k/v and gate/up as
-    plans, (c) RMSNorm prologue + SwiGLU pair: four launches per layer. Microseconds per token."""
+def single_call_rows(torch, tl, timer, problems, model, layers):
+    """The reference's call pattern on the headline weights: one operator call per matrix
+    (src/transformer.cpp:102-118), all calls of a sweep captured once into a HIP graph and replayed, so the
+    time holds launch and kernel costs but no host time. fp16 activations (ternary_gemv), int8 activations
+    (quantize_absmax_int8 once per layer input + ternary_gemv_int8 with the device-resident scale), and the
+    dependent chain of a decode step's linear side in its three forms."""
+    n = len(problems)
+    nbytes = sum(packed_bytes(p[5], p[6]) for p in problems)
+    out = []
+
+    def f16_calls():
+        for nz, sg, sc, x, y, rows, cols, _ in problems:
+            tl.ternary_gemv(nz, sg, sc, x, y, rows, cols, 128)
+
+    q8 = {c: torch.zeros(c, dtype=torch.int8, device="cuda") for c in {p[6] for p in problems}}
+    qs = {c: torch.zeros(1, dtype=torch.float32, device="cuda") for c in q8}
+
+    def i8_calls():   # the reference's ternary_linear_int8 (src/transformer.cpp:132-142), without its device-to-host copy of the scale
+        for nz, sg, sc, x, y, rows, cols, _ in problems:
+            tl.quantize_absmax_int8(x, q8[cols], qs[cols], cols)
+            tl.ternary_gemv_int8(nz, sg, sc, q8[cols], qs[cols], y, rows, cols, 128)
+
+    for name, fn, kernel in ((f"single calls, fp16 activations: {n} x ternary_gemv from one graph", f16_calls, "tllm::gemv_mfma_kernel<Wide, fine>"),
+                             (f"single calls, int8 activations: {n} x (quantize_absmax_int8 + ternary_gemv_int8) from one graph", i8_calls,
+                              "tllm::gemv_mfma_kernel<Wide, fine> on int8 activations")):
+        graph = capture(torch, fn)
+        t = timer.run(graph.replay, 30, 5)
+        row = hbm_row(name, t, nbytes, kernel)
+        row["us_per_call"] = round(t["mean_ms"] * 1e3 / n, 2)
+        out.append(row)
+        del graph
+    chain = decode_chain(torch, tl, problems, model, layers)
+    for name, fn, launches in chain["variants"]:
+        graph = capture(torch, fn)
+        t = timer.run(graph.replay, 30, 5)
+        row = hbm_row(f"decode chain ({name}), {layers} layers, dependent order, from one graph", t, nbytes, "several")
+        row["launches_per_token"] = launches * layers
+        row["us_per_launch"] = round(t["mean_ms"] * 1e3 / (launches * layers), 2)
+        out.append(row)
+        del graph
+    chain["close"]()
+    return out
+
+
+def decode_chain(torch, tl, problems, model, layers):
+    """The linear-side launches of a batch-1 decode step over the sweep's own weights, issued in the order a
+    transformer needs them (every launch after the one before, as reference src/transformer.cpp:193-296
+    does): (a) the reference's ten launches per layer, (b) q/k/v and gate/up as plans, (c) RMSNorm prologue +
+    SwiGLU pair: four launches per layer."""
     h, qd, kvd, ffn, _ = SHAPES[model]
     f16 = dict(dtype=torch.float16, device="cuda")
     x = torch.randn((1, h), device="cuda").to(torch.float16)
@@ -248,41 +421,89 @@ def decode_chain_report(torch, tl, problems, model, layers, reps=40):
             w["gu_n"].launch()
             tl.ternary_gemv(*w["d"], g, d, h, ffn, 128)
 
-    def timed(fn):
-        for _ in range(10):
-            fn()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(reps):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / reps * 1e3
+    def close():
+        for w in L:
+            for key in ("qkv", "gu", "qkv_n", "gu_n"):
+                w[key].close()
 
-    nbytes = sum(packed_bytes(p[5], p[6]) for p in problems[:7 * layers])
-    out = {"workload": f"{model}: linear-side launches of one decode step, {layers} layers, batch 1, dependent order",
-           "unit": "us per token", "packed_bytes": nbytes}
-    for name, fn, n in (("reference_10_launches_per_layer", ten, 10), ("plans_7_launches_per_layer", seven, 7),
-                        ("prologue_and_pair_4_launches_per_layer", four, 4)):
-        us = timed(fn)
-        out[name] = {"us_per_token": round(us, 1), "GBps": round(nbytes / us / 1e3, 1),
-                     "us_per_launch": round(us / (n * layers), 2)}
-    for w in L:
-        for key in ("qkv", "gu", "qkv_n", "gu_n"):
-            w[key].close()
-    return out
+    return {"variants": (("the reference's 10 launches per layer", ten, 10), ("q/k/v and gate/up as plans: 7 per layer", seven, 7),
+                         ("RMSNorm prologue + SwiGLU pair: 4 per layer", four, 4)), "close": close}
+
+
+def copy_ceiling(torch, tl, timer):
+    """What this GPU moves with nothing to compute: a read-only pass over 4 GiB (the library's streaming kernel:
+    16-byte non-temporal loads; a few launch shapes are tried and the best is kept) and a device-to-device copy of
+    2 GiB (bytes read + bytes written)."""
+    src = torch.ones(1 << 30, dtype=torch.int32, device="cuda")
+    best = None
+    for shape in ("3,16", "8,8", "24,4", "32,8"):   # workgroups per CU, loads in flight per thread
+        os.environ["TLLM_READ_SHAPE"] = shape
+        t = timer.run(lambda: tl.read_stream(src), 20, 3)
+        rate = src.numel() * 4 / (t["mean_ms"] * 1e-3) / 1e9
+        if best is None or rate > best[0]:
+            best = (rate, src.numel() * 4 / (t["min_ms"] * 1e-3) / 1e9, shape)
+    os.environ.pop("TLLM_READ_SHAPE", None)
+    half = src[: 1 << 29]
+    dst = torch.empty_like(half)
+    t2 = timer.run(lambda: dst.copy_(half), 20, 3)
+    copy = 2 * half.numel() * 4 / (t2["mean_ms"] * 1e-3) / 1e9
+    del src, dst
+    return {"read_only_GBps": round(best[0], 1), "read_only_GBps_best": round(best[1], 1), "read_only_frac_hbm_peak": round(best[0] / HBM_PEAK_GBS, 4),
+            "read_only_launch_shape": best[2], "copy_read_plus_write_GBps": round(copy, 1),
+            "what": "tllm_read_stream over 4 GiB (best of four launch shapes); torch copy_ of 2 GiB (hipMemcpy device to device)"}
+
+
+def cpu_baseline(oracle, torch, shape_sets, threads):
+    """The reference's fp32 host loop (tests/test_ternary_gemv.cu:40-75, restated in C in oracle/), batch 1,
+    on this machine's host cores: every matrix shape of configurations 1-3 and one full 70B layer, single
+    threaded (the reference's own form) and split by rows over `threads` threads. A bounded sample: about
+    10-20 s of CPU time."""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(99)
+    rows_out = []
+    tot = {"st_bytes": 0, "st_s": 0.0, "mt_bytes": 0, "mt_s": 0.0}
+    for label, shapes in shape_sets:
+        st_b = st_t = mt_t = 0.0
+        for (rows, cols) in shapes:
+            nz, sg = gen_masks(torch, rows, cols, 0.42, gen)
+            sc = (torch.rand((rows, cols // 128), device="cuda", generator=gen) * 0.02 + 0.01).float()
+            x = torch.randn(cols, device="cuda", generator=gen).to(torch.float16).float()
+            nzh, sgh = nz.cpu().numpy().view(np.uint32), sg.cpu().numpy().view(np.uint32)
+            sch, xh = sc.cpu().numpy(), x.cpu().numpy()
+            t0 = time.perf_counter()
+            oracle.gemv_hostloop(nzh, sgh, sch, xh, threads=1)
+            st_t += time.perf_counter() - t0
+            t0 = time.perf_counter()
+            oracle.gemv_hostloop(nzh, sgh, sch, xh, threads=threads)
+            mt_t += time.perf_counter() - t0
+            st_b += packed_bytes(rows, cols)
+            del nz, sg, sc, x
+        rows_out.append({"shapes": label, "packed_bytes": int(st_b), "single_thread_ms": round(st_t * 1e3, 2),
+                         "single_thread_GBps": round(st_b / st_t / 1e9, 4), f"threads_{threads}_ms": round(mt_t * 1e3, 2),
+                         f"threads_{threads}_GBps": round(st_b / mt_t / 1e9, 4)})
+        tot["st_bytes"] += st_b
+        tot["st_s"] += st_t
+        tot["mt_bytes"] += st_b
+        tot["mt_s"] += mt_t
+    return {
+        "value": round(tot["mt_bytes"] / tot["mt_s"] / 1e9, 4), "unit": "GB/s", "cores": threads, "kind": "port",
+        "sample": f"one GEMV per matrix shape of configurations 1-3 and of one LLaMA-70B layer ({int(tot['st_bytes'])} packed bytes in all), "
+                  f"rows split over {threads} threads: {tot['mt_s']:.2f} s; single thread: {tot['st_s']:.2f} s; "
+                  "loop = tests/test_ternary_gemv.cu:40-75 restated in C; the 80-layer 70B figure would be 80 x the layer's time",
+        "single_thread_GBps": round(tot["st_bytes"] / tot["st_s"] / 1e9, 4),
+        "per_shape_set": rows_out,
+    }
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    # A step is 0.35 ms. The GPU idles at ~100 MHz and takes tens of milliseconds of load to settle at
-    # its working clocks: 5 warm-up steps give 0.367 ms per step over the next 20, 500 give 0.345.
+    # A step is 0.33 ms. The GPU idles at ~100 MHz and takes tens of milliseconds of load to settle at its working
+    # clocks, so every timed region is preceded by --settle-ms of the same launches, whatever --warmup says.
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--settle-ms", type=float, default=200.0,
-                    help="untimed steps for this long before the warm-up steps (lets the clocks settle)")
+                    help="untimed launches for this long before the warm-up launches of every timed region")
     ap.add_argument("--model", default="llama8b", choices=sorted(SHAPES))
     ap.add_argument("--layers", type=int, default=0, help="0 = the model's own layer count")
     ap.add_argument("--batch", type=int, default=1)
@@ -291,15 +512,14 @@ def main():
                     help="plan: the whole sweep as one launch; calls: one operator call per matrix")
     ap.add_argument("--matrices", default="", help='per-layer matrix list "ROWSxCOLS,..." instead of the model\'s')
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--copy-calibration", action="store_true",
-                    help="also run a 1 GiB -> 1 GiB elementwise copy kernel (reference for HBM byte counters)")
-    ap.add_argument("--also-batch", default="4", help='extra activation-row counts measured on the same weights '
-                    '(cfg3 asks for batch 1 and 4), e.g. "4,16"; "" skips')
-    ap.add_argument("--gemm-m", default="512", help='token counts M of the prefill GEMM report, e.g. "16,128,512,2048"; "" skips it')
+    ap.add_argument("--only-headline", action="store_true", help="skip configs, single_calls and copy_ceiling (profiling runs)")
+    ap.add_argument("--configs", default="1,2,3,4,5", help="benchmark configurations to add to `configs`")
+    ap.add_argument("--also-batch", default="4,16", help="extra activation-row counts of configuration 3")
+    ap.add_argument("--gemm-m", default="16,128,512,2048", help="token counts M of configuration 4")
     ap.add_argument("--gemm-calls", type=int, default=200, help="timed launches per GEMM case")
-    ap.add_argument("--gemm-warm", type=int, default=20, help="untimed launches before them")
-    ap.add_argument("--decode-chain", action="store_true",
-                    help="also time the dependent launch sequence of a decode step (three variants)")
+    ap.add_argument("--gemm-warm", type=int, default=20, help="untimed launches before them (after the settle phase)")
+    ap.add_argument("--sparsity-sweep", action="store_true", help="configuration 5 also at P(0) = 0.2 and 0.7")
+    ap.add_argument("--no-single-calls", action="store_true")
     ap.add_argument("--seed", type=int, default=20240611)
     args = ap.parse_args()
     for item in filter(None, args.matrices.split(",")):
@@ -315,6 +535,11 @@ def main():
         print("bench.py needs the MI355X (no CPU fallback exists).", file=sys.stderr)
         sys.exit(2)
     tl.lib()
+    from oracle import oracle as orc
+    if not os.path.exists(orc.LIB):
+        orc.build()
+    orc.load()
+    timer = Timer(torch, args.settle_ms)
     layers = args.layers or SHAPES[args.model][4]
     lo, hi = (0.005, 0.02) if args.model == "llama70b" else (0.01, 0.03)
     problems, meta = build_sweep(torch, args.model, layers, args.batch, args.p_zero, lo, hi, args.seed)
@@ -325,9 +550,7 @@ def main():
     if args.mode == "plan":
         plan = tl.LinearPlan(problems)
         assert plan.weight_bytes == sweep_bytes
-
-        def step():
-            plan.launch()
+        step = plan.launch
         launches_per_step = 1
     else:
         def step():
@@ -338,53 +561,22 @@ def main():
                     tl.ternary_gemm(x, nz, sg, sc, y, batch, rows, cols, 128)
         launches_per_step = len(problems)
 
-    default_workload = (args.model == "llama8b" and not CUSTOM and args.batch == 1 and args.mode == "plan"
-                        and layers == SHAPES["llama8b"][4] and args.p_zero == 0.42)
-    # Clock settle: the GPU idles near 100 MHz and needs tens of milliseconds under load to reach its
-    # working clocks, however many warm-up steps are asked for. Untimed, before the warm-up steps.
-    def settle(fn):
-        t_settle = time.perf_counter()
-        while (time.perf_counter() - t_settle) * 1e3 < args.settle_ms:
-            for _ in range(20):
-                fn()
-            torch.cuda.synchronize()
-
-    settle(step)
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    headline = (args.model == "llama8b" and not CUSTOM and args.batch == 1 and args.mode == "plan"
+                and layers == SHAPES["llama8b"][4] and args.p_zero == 0.42)
     t0 = time.perf_counter()
-    ev0.record()          # recorded on torch's current stream: the stream every launch above uses
-    for _ in range(args.steps):
-        step()
-    ev1.record()
-    torch.cuda.synchronize()
+    t = timer.run(step, args.steps, args.warmup)
     wall_ms = (time.perf_counter() - t0) * 1e3
-    dev_ms = ev0.elapsed_time(ev1)
-    ms_per_step = dev_ms / args.steps
+    ms_per_step = t["mean_ms"]
     gbps = sweep_bytes / (ms_per_step * 1e-3) / 1e9
-
-    if args.copy_calibration:
-        src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            torch.mul(src, 1.0, out=dst)  # vectorized elementwise kernel: reads 2^30 B, writes 2^30 B
-        torch.cuda.synchronize()
-        del src, dst
-
-    from oracle import oracle as orc
-    if not os.path.exists(orc.LIB):
-        orc.build()
-    orc.load()
     sample_idx = sorted(set([0, 1, 4, 6, len(problems) - 1, len(problems) // 2]))
     parity = check_sample(orc, problems, [i for i in sample_idx if i < len(problems)])
 
     out = {
         "metric": "ternary GEMV packed-weight GB/s (% HBM peak) at B=1; GEMM TOPS at M=512",
-        "value": round(gbps, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "settle_ms": args.settle_ms,
-        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f16",
+        "value": round(gbps, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "settle_ms": args.settle_ms, "untimed_launches": t["untimed_launches"],
+        "ms_per_step": round(ms_per_step, 5), "ms_per_step_median": round(t["median_ms"], 5), "ms_per_step_min": round(t["min_ms"], 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
         "dtype_detail": "fp16 activations x 2-bit ternary weights (fp16 group scales), fp32 accumulation, fp16 outputs",
         "data": "synthetic (seeded; P(0)=%.2f, fp16 scales U[%.3f,%.3f], x ~ N(0,1))" % (args.p_zero, lo, hi),
         "config": {
@@ -393,56 +585,69 @@ def main():
             "mode": args.mode, "launches_per_step": launches_per_step, "group_size": 128,
         },
         "pct_hbm_peak": round(100.0 * gbps / HBM_PEAK_GBS, 2),
-        "wall_ms_per_step": round(wall_ms / args.steps, 5),
+        "timing": "HIP events on the launch stream around back-to-back launches; mean over all timed steps, median and min over "
+                  f"groups of {t['steps_per_timing_group']} consecutive steps; {t['untimed_launches']} untimed launches first "
+                  f"({args.settle_ms:.0f} ms settle + {args.warmup} warm-up)",
+        "wall_ms_per_step_with_untimed": round(wall_ms / args.steps, 5),
         "parity_max_rel_sampled": parity,
         "roofline": {
             "bound": "hbm", "achieved": round(gbps, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(gbps / HBM_PEAK_GBS, 4),
-            "traffic": DEFAULT_WORKLOAD_TRAFFIC_BYTES if default_workload else None,
+            "frac_best_group": round(sweep_bytes / (t["min_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "traffic": HEADLINE_TRAFFIC_BYTES if headline else None,
+            "traffic_source": HEADLINE_TRAFFIC_SOURCE if headline else None,
             "kernel": plan.kernel if args.mode == "plan" else "per-matrix launches",
             "bytes_per_launch": sweep_bytes // launches_per_step,
         },
     }
-    extra = [int(v) for v in args.also_batch.split(",") if v.strip()] if args.mode == "plan" else []
-    if extra:
-        out["other_batches"] = []
-    for b in extra:
-        # the same weights with b activation rows per matrix: one plan launch streams them once for all rows
-        g2 = torch.Generator(device="cuda")
-        g2.manual_seed(args.seed + 100 + b)
-        probs_b = []
-        for (nz, sg, sc, _, _, rows, cols, _) in problems:
-            xb = torch.randn((b, cols), device="cuda", generator=g2).to(torch.float16)
-            yb = torch.zeros((b, rows), dtype=torch.float16, device="cuda")
-            probs_b.append((nz, sg, sc, xb, yb, rows, cols, b))
-        plan_b = tl.LinearPlan(probs_b)
-        settle(plan_b.launch)
-        for _ in range(args.warmup):
-            plan_b.launch()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(args.steps):
-            plan_b.launch()
-        e1.record()
-        torch.cuda.synchronize()
-        ms_b = e0.elapsed_time(e1) / args.steps
-        gb = sweep_bytes / (ms_b * 1e-3) / 1e9
-        par_b = check_sample(orc, probs_b, [i for i in sample_idx if i < len(probs_b)])
-        out["other_batches"].append({"batch": b, "ms_per_step": round(ms_b, 5), "GBps": round(gb, 2),
-                                     "frac_hbm_peak": round(gb / HBM_PEAK_GBS, 4),
-                                     "kernel": plan_b.kernel, "parity_max_rel_sampled": par_b})
-        plan_b.close()
-        del probs_b
-    if args.decode_chain and not CUSTOM and args.batch == 1:
-        out["decode_chain"] = decode_chain_report(torch, tl, problems, args.model, layers)
-    gemm_m = [int(v) for v in args.gemm_m.split(",") if v.strip()]
-    if gemm_m:
-        out["gemm"] = gemm_report(torch, tl, orc, args.seed, gemm_m, args.p_zero, args.gemm_calls, args.gemm_warm,
-                                  args.settle_ms)
+    if not args.only_headline:
+        want = {int(v) for v in args.configs.split(",") if v.strip()}
+        cfgs = []
+        cfg_steps = max(50, min(args.steps, 400))
+        if 1 in want:
+            cfgs += cfg1_rows(torch, tl, orc, timer, args.seed)
+        if 2 in want:
+            r, _ = plan_rows(torch, tl, orc, timer, "cfg2: llama1b 16-layer sweep (unit-RMS activations)", "llama1b", 16, [1], 0.42, 0.01, 0.03,
+                             args.seed + 2, cfg_steps, 20, unit_rms=True)
+            cfgs += r
+            r, _ = plan_rows(torch, tl, orc, timer, "cfg2: llama1b 16-layer sweep, rotated", "llama1b", 16, [1], 0.42, 0.01, 0.03,
+                             args.seed + 2, cfg_steps, 20, copies=3, unit_rms=True)
+            cfgs += r
+        if 3 in want and headline:
+            cfgs.append(hbm_row("cfg3: llama8b 32-layer sweep, batch 1 (the headline value)", t, sweep_bytes, plan.kernel, parity))
+            extra = [int(v) for v in args.also_batch.split(",") if v.strip()]
+            r, _ = plan_rows(torch, tl, orc, timer, "cfg3: llama8b 32-layer sweep", "llama8b", 32, extra, 0.42, 0.01, 0.03,
+                             args.seed, cfg_steps, 20, problems=problems)
+            cfgs += r
+        if 4 in want:
+            gemm_m = [int(v) for v in args.gemm_m.split(",") if v.strip()]
+            g = gemm_rows(torch, tl, orc, timer, args.seed, gemm_m, 0.42, args.gemm_calls, args.gemm_warm)
+            cfgs += g
+            m512 = [c for c in g if c["M"] == 512]
+            if m512:
+                agg = sum(2.0 * c["M"] * c["N"] * c["K"] for c in m512) / sum(c["us"] for c in m512) / 1e6
+                out["gemm_m512"] = {"tflops_both_shapes": round(agg, 1), "frac_mfma_peak": round(agg / MFMA_F16_PEAK_TFLOPS, 4),
+                                    "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s (2*M*N*K)",
+                                    "per_shape": [{k: c[k] for k in ("N", "K", "us", "tflops", "frac_mfma_peak")} for c in m512]}
+        if not args.no_single_calls and headline:
+            out["single_calls"] = single_call_rows(torch, tl, timer, problems, "llama8b", 32)
+        if 5 in want:
+            zs = [0.42] + ([0.2, 0.7] if args.sparsity_sweep else [])
+            for pz in zs:
+                r, _ = plan_rows(torch, tl, orc, timer, f"cfg5: llama70b 80-layer sweep resident, P(0)={pz}", "llama70b", 80, [1, 16],
+                                 pz, 0.005, 0.02, args.seed + 5, 40, 5)
+                cfgs += r
+        out["configs"] = cfgs
+        out["copy_ceiling"] = copy_ceiling(torch, tl, timer)
     if not args.no_cpu_baseline:
         threads = min(os.cpu_count() or 1, 16)
-        out["cpu_baseline"] = cpu_baseline(orc, problems, n_mats, threads)
+        sets = [("cfg1: 2048x2048", [(2048, 2048)]),
+                ("cfg2: one llama1b layer", [(r, c) for _, r, c in layer_matrices("llama1b")] if not CUSTOM else [(2048, 2048)]),
+                ("cfg3: one llama8b layer", [(4096, 4096), (1024, 4096), (1024, 4096), (4096, 4096), (14336, 4096), (14336, 4096), (4096, 14336)]),
+                ("cfg5: one llama70b layer", [(8192, 8192), (1024, 8192), (1024, 8192), (8192, 8192), (28672, 8192), (28672, 8192), (8192, 28672)])]
+        if CUSTOM:
+            sets = sets[:1]
+        out["cpu_baseline"] = cpu_baseline(orc, torch, sets, threads)
     print(json.dumps(out))
 
 

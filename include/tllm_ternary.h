@@ -251,6 +251,14 @@ int64_t tllm_linear_plan_weight_bytes(const tllm_linear_plan *plan);
 const char *tllm_linear_plan_kernel(const tllm_linear_plan *plan);
 void tllm_linear_plan_destroy(tllm_linear_plan *plan);
 
+/*
+ * Measurement aid: one pass of 16-byte loads over `bytes` of device memory (16-byte aligned), nothing
+ * written (`sink` may be NULL). Timed, it gives the read-only streaming ceiling of the GPU at hand, the
+ * figure a weight stream can be compared with besides the published HBM peak. No counterpart in the
+ * reference operators; its benchmark prints a copy bandwidth for the same purpose (tests/benchmark.cu:87-95).
+ */
+int tllm_read_stream(const void *src, size_t bytes, uint32_t *sink, tllm_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -15,6 +15,7 @@ from .ops import (  # noqa: F401
     lib,
     lib_path,
     quantize_absmax_int8,
+    read_stream,
     rmsnorm,
     rope,
     silu_mul,

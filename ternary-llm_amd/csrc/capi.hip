@@ -205,6 +205,13 @@ int tllm_copy_to_kv_cache_f16(const uint16_t *k, const uint16_t *v, uint16_t *k_
                                               max_seq_len, (hipStream_t)stream);
 }
 
+int tllm_read_stream(const void *src, size_t bytes, uint32_t *sink, tllm_stream_t stream) {
+    if (!src) return TLLM_ERR_NULL_POINTER;
+    if (bytes < 16) return TLLM_ERR_BAD_SHAPE;
+    if (tllm::misaligned(src, 16)) return TLLM_ERR_MISALIGNED;
+    return (int)tllm::launch_read_stream(src, bytes, sink, (hipStream_t)stream);
+}
+
 static int create_plan(tllm_linear_plan **plan, const tllm_linear_problem *problems,
                        const uint16_t *const *norm_weights, float eps, int count, int group_size) {
     if (!plan || !problems) return TLLM_ERR_NULL_POINTER;

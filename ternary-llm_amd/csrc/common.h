@@ -12,6 +12,14 @@ namespace tllm {
 
 constexpr int kWave = 64;
 
+// Load of weight-stream data that is read once per launch: marked non-temporal, so that it does not
+// displace what is reused (activations, scales) from the caches. -DTLLM_STREAM_PLAIN keeps ordinary loads.
+#ifdef TLLM_STREAM_PLAIN
+#define TLLM_STREAM_LOAD(ptr) (*(ptr))
+#else
+#define TLLM_STREAM_LOAD(ptr) __builtin_nontemporal_load(ptr)
+#endif
+
 // One ternary linear: y[batch, rows] = x[batch, cols] * W^T with W packed as two bit planes.
 struct Problem {
     const uint32_t *nz;
@@ -81,6 +89,9 @@ hipError_t launch_embedding_lookup(const uint16_t *table, const int *indices, ui
 hipError_t launch_copy_to_kv_cache(const uint16_t *k, const uint16_t *v, uint16_t *k_cache, uint16_t *v_cache, int batch,
                                    int n_kv_heads, int head_dim, int seq_len, int start_pos, int max_seq_len,
                                    hipStream_t s);
+
+// Measurement aid (elementwise.hip): reads `bytes` of device memory once.
+hipError_t launch_read_stream(const void *src, size_t bytes, uint32_t *sink, hipStream_t s);
 
 // 128-group MFMA GEMV, batch 1..4 (gemv_mfma.hip).
 bool gemv_mfma_supports(const Problem &p, int group);

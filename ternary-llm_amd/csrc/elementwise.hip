@@ -3,6 +3,9 @@
 // projections, the residual add, rotary position embedding of q and k, the embedding row lookup and
 // the copy of new k/v rows into the cache. All are bandwidth-trivial (a few KB per token); fp16 in
 // and out, arithmetic as the reference's kernels unless a comment says otherwise.
+#include <cstdio>
+#include <cstdlib>
+
 #include "common.h"
 
 namespace tllm {
@@ -291,6 +294,41 @@ hipError_t launch_silu_mul(const uint16_t *gate, const uint16_t *up, uint16_t *o
     const int vec8 = aligned ? size / 8 : 0;
     const int lanes = vec8 + (size - vec8 * 8);
     silu_mul_kernel<<<(lanes + 255) / 256, 256, 0, s>>>(gate, up, output, size, vec8);
+    return hipGetLastError();
+}
+
+// ---- measurement aid: how fast can this GPU stream memory into registers at all?
+// Every thread reads 16 bytes at a time, grid-stride, keeps eight loads in flight and folds the values
+// into one word; the word is stored only if it equals a value it cannot have (keeps the loads alive).
+typedef uint32_t u4v __attribute__((ext_vector_type(4)));
+template <int kFlight>
+__global__ __launch_bounds__(256) void read_stream_kernel(const u4v *__restrict__ src, size_t n16, uint32_t *sink) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    uint32_t acc = 0;
+    for (; i + (kFlight - 1) * stride < n16; i += kFlight * stride) {
+        u4v v[kFlight];
+#pragma unroll
+        for (int k = 0; k < kFlight; k++) v[k] = __builtin_nontemporal_load(src + i + k * stride);
+#pragma unroll
+        for (int k = 0; k < kFlight; k++) acc ^= v[k].x ^ v[k].y ^ v[k].z ^ v[k].w;
+    }
+    for (; i < n16; i += stride) {
+        const u4v v = src[i];
+        acc ^= v.x ^ v.y ^ v.z ^ v.w;
+    }
+    if (acc == 0x9E3779B9u && sink) *sink = acc;
+}
+
+hipError_t launch_read_stream(const void *src, size_t bytes, uint32_t *sink, hipStream_t s) {
+    // TLLM_READ_SHAPE="wgs_per_cu,loads_in_flight" (tuning aid); default 8 workgroups per CU, 8 loads per thread
+    int per_cu = 8, flight = 8;
+    if (const char *e = getenv("TLLM_READ_SHAPE")) sscanf(e, "%d,%d", &per_cu, &flight);
+    const int grid = current_device_cus() * (per_cu < 1 ? 1 : per_cu > 64 ? 64 : per_cu);
+    const u4v *p = reinterpret_cast<const u4v *>(src);
+    if (flight >= 16) read_stream_kernel<16><<<grid, 256, 0, s>>>(p, bytes / 16, sink);
+    else if (flight >= 8) read_stream_kernel<8><<<grid, 256, 0, s>>>(p, bytes / 16, sink);
+    else read_stream_kernel<4><<<grid, 256, 0, s>>>(p, bytes / 16, sink);
     return hipGetLastError();
 }
 

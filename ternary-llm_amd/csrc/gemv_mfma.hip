@@ -546,8 +546,16 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
             const int c0 = min((seg_lo + slice) * G::kChunks, groups - G::kChunks);
             const size_t base_a = ((size_t)rbe * words + (size_t)c0 * 4) * 4;
             const size_t base_s = ((size_t)rbe * groups + c0) * 2;
-            t.nz = *reinterpret_cast<const GU4 *>(nz_g + base_a + lane_a);
-            t.sg = *reinterpret_cast<const GU4 *>(sg_g + base_a + lane_a);
+            if constexpr (G::kRows == 4) {
+                // wide tiles read every mask line once, whole (a quad of lanes = 64 bytes, the next quad the
+                // rest of the line): streamed past the caches. Tall tiles come back to a line for the next
+                // slice and keep ordinary loads (non-temporal ones cost them 12 %).
+                t.nz = TLLM_STREAM_LOAD(reinterpret_cast<const GU4 *>(nz_g + base_a + lane_a));
+                t.sg = TLLM_STREAM_LOAD(reinterpret_cast<const GU4 *>(sg_g + base_a + lane_a));
+            } else {
+                t.nz = *reinterpret_cast<const GU4 *>(nz_g + base_a + lane_a);
+                t.sg = *reinterpret_cast<const GU4 *>(sg_g + base_a + lane_a);
+            }
 #pragma unroll
             for (int v = 0; v < G::kScales; v++)
                 t.sc[v] = *reinterpret_cast<const GU16 *>(sc_g + base_s + lane_s[v]);

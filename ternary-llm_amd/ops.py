@@ -19,7 +19,7 @@ ABI_SYMBOLS = (
     "tllm_linear_plan_destroy", "tllm_rmsnorm_f16", "tllm_silu_mul_f16", "tllm_linear_plan_create_normed",
     "tllm_add_f16", "tllm_rope_f16", "tllm_embedding_lookup_f16", "tllm_copy_to_kv_cache_f16",
     "tllm_linear_plan_kernel", "tllm_gemm_workspace_reserve", "tllm_gemm_workspace_release",
-    "tllm_ternary_gemm_f16_static",
+    "tllm_ternary_gemm_f16_static", "tllm_read_stream",
 )
 # include/tllm_model_file.h
 FILE_ABI_SYMBOLS = (
@@ -79,6 +79,7 @@ def lib():
     L.tllm_ternary_gemm_f16.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, vp]
     L.tllm_ternary_gemm_f16_static.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, vp]
     L.tllm_gemm_workspace_reserve.argtypes = [i, i, i, i, vp]
+    L.tllm_read_stream.argtypes = [vp, C.c_size_t, vp, vp]
     L.tllm_gemm_workspace_release.argtypes = []
     L.tllm_gemm_workspace_release.restype = None
     L.tllm_linear_plan_create.argtypes = [C.POINTER(vp), C.POINTER(_Problem), i, i]
@@ -168,6 +169,11 @@ def ternary_gemm_static(A, nz_B, sign_B, scales_B, Cout, M, N, K, group_size=128
     """ternary_gemm that never allocates: the split-K exchange uses the library's fixed device array."""
     check(lib().tllm_ternary_gemm_f16_static(_ptr(A), _ptr(nz_B), _ptr(sign_B), _ptr(scales_B), _ptr(Cout),
                                              M, N, K, group_size, _stream(stream)))
+
+
+def read_stream(buf, stream=None):
+    """Measurement aid: one read-only pass over a device tensor (the streaming ceiling of the GPU)."""
+    check(lib().tllm_read_stream(_ptr(buf), buf.numel() * buf.element_size(), None, _stream(stream)))
 
 
 def gemm_workspace_reserve(M, N, K, group_size=128, stream=None):

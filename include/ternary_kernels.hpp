@@ -5,14 +5,19 @@
 // (include/kernels.cuh:45-48, 60-62) with the same names, argument order and default stream,
 // so the call expressions in src/transformer.cpp:107-116, 132-142, 193-196, 201-217, 258-261,
 // 266-278, 285-286 compile unchanged against this header. `half` is HIP's __half (hip/hip_fp16.h) and the
-// stream is a hipStream_t. Like the reference these return void; a rejected call is
-// reported through the optional handler below instead of being silently dropped.
+// stream is a hipStream_t. Like the reference these return void. The C ABI underneath checks what the
+// reference never checked (null pointers, cols % group_size, 16-byte alignment of masks and activations,
+// output overlapping the input) and REJECTS such a call without writing the output: the rejection goes
+// to the handler below (default: a line on stderr) and stays readable in ternary::last_error() until the
+// caller clears it, so a caller ported from the reference cannot consume a stale buffer unnoticed.
+// Compile with -DTERNARY_ABORT_ON_ERROR to abort on the first rejected call instead.
 #pragma once
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime_api.h>
 
 #include <cstdint>
 #include <cstdio>
+#include <cstdlib>
 
 #include "tllm_ternary.h"
 
@@ -29,8 +34,19 @@ inline error_handler_t &error_handler() {
     return h;
 }
 
+// First non-zero code since the caller last set it to 0 (negative: TLLM_ERR_*, positive: hipError_t).
+inline int &last_error() {
+    static int e = 0;
+    return e;
+}
+
 inline void report(const char *op, int code) {
-    if (code != 0 && error_handler()) error_handler()(op, code);
+    if (code == 0) return;
+    if (!last_error()) last_error() = code;
+    if (error_handler()) error_handler()(op, code);
+#ifdef TERNARY_ABORT_ON_ERROR
+    std::abort();
+#endif
 }
 
 // Reference include/kernels.cuh:11-14.

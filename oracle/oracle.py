@@ -65,6 +65,7 @@ def load():
     L.tllm_oracle_silu_mul_f64.argtypes = [_u16p, _u16p, _f64p, C.c_int]
     L.tllm_oracle_add_f64.argtypes = [_u16p, _u16p, _f64p, C.c_int]
     L.tllm_oracle_rope_f64.argtypes = [_u16p, _f64p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_double]
+    L.tllm_oracle_rope_f32angle.argtypes = [_u16p, _u16p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float]
     for f in ("add_f64", "rope_f64", "rmsnorm_f64", "silu_mul_f64", "pack", "unpack", "gemv_f64", "gemv_hostloop", "gemv_hostloop_mt", "gemm_f64",
               "gemm_f32_elem", "quantize_i8", "gemv_i8_f64", "ternarize"):
         getattr(L, "tllm_oracle_" + f).restype = None
@@ -191,6 +192,15 @@ def rope_f64(x, batch, seq_len, heads, head_dim, start_pos, theta):
     assert x.size == batch * seq_len * heads * head_dim and head_dim % 2 == 0
     out = np.empty(x.size, np.float64)
     load().tllm_oracle_rope_f64(x.reshape(-1), out, batch, seq_len, heads, head_dim, start_pos, float(theta))
+    return out.reshape(batch, seq_len, heads, head_dim)
+
+
+def rope_f32angle(x, batch, seq_len, heads, head_dim, start_pos, theta):
+    """The rotation in the reference's fp32 arithmetic (kernels/rope.cu:49-64): fp16 bits in, fp16 bits out."""
+    x = _c(x, np.uint16)
+    assert x.size == batch * seq_len * heads * head_dim and head_dim % 2 == 0
+    out = np.empty(x.size, np.uint16)
+    load().tllm_oracle_rope_f32angle(x.reshape(-1), out, batch, seq_len, heads, head_dim, start_pos, float(theta))
     return out.reshape(batch, seq_len, heads, head_dim)
 
 

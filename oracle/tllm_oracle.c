@@ -20,6 +20,7 @@
  *   tllm_oracle_silu_mul_f64 .... kernels/activations.cu:18-59
  *   tllm_oracle_add_f64 ......... kernels/elementwise.cu:18-48
  *   tllm_oracle_rope_f64 ........ kernels/rope.cu:22-80
+ *   tllm_oracle_rope_f32angle ... kernels/rope.cu:49-64 (the reference's fp32 angle arithmetic)
  *   (embedding_lookup and copy_to_kv_cache, kernels/elementwise.cu:54-147, are pure row copies;
  *    their restatement is numpy indexing in oracle.py)
  *
@@ -402,6 +403,31 @@ void tllm_oracle_rope_f64(const uint16_t *x, double *out, int batch, int seq_len
                 const double x1 = (double)tllm_oracle_half_to_float(x[base + 2 * i + 1]);
                 out[base + 2 * i] = x0 * c - x1 * s;
                 out[base + 2 * i + 1] = x0 * s + x1 * c;
+            }
+        }
+    }
+}
+
+/* The same rotation in the reference's own arithmetic (kernels/rope.cu:49-64): frequency, angle, sine and
+ * cosine formed in fp32 (`1.0f / powf(theta, 2i / head_dim)`, `(float)pos * freq`, `cosf`, `sinf`), the
+ * rotation in fp32, the result rounded to fp16 (returned as fp16 bits). The host's powf/sinf/cosf stand in
+ * for the device's: all are within an ulp or two of the exact functions of the fp32 angle, which itself
+ * is off from the exact angle by up to about pos * 2^-23 rad. Used to bound the distance between the
+ * exact-angle rotation the library computes and what the reference stores. */
+void tllm_oracle_rope_f32angle(const uint16_t *x, uint16_t *out, int batch, int seq_len, int heads, int head_dim,
+                               int start_pos, float theta) {
+    for (int64_t t = 0; t < (int64_t)batch * seq_len; t++) {
+        const int pos = start_pos + (int)(t % seq_len);
+        for (int h = 0; h < heads; h++) {
+            const int64_t base = (t * heads + h) * head_dim;
+            for (int i = 0; i < head_dim / 2; i++) {
+                const float freq = 1.0f / powf(theta, (2.0f * (float)i) / (float)head_dim);
+                const float angle = (float)pos * freq;
+                const float c = cosf(angle), sn = sinf(angle);
+                const float x0 = tllm_oracle_half_to_float(x[base + 2 * i]);
+                const float x1 = tllm_oracle_half_to_float(x[base + 2 * i + 1]);
+                out[base + 2 * i] = tllm_oracle_float_to_half(x0 * c - x1 * sn);
+                out[base + 2 * i + 1] = tllm_oracle_float_to_half(x0 * sn + x1 * c);
             }
         }
     }

@@ -4,6 +4,7 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <algorithm>
 #include <new>
 #include <string>
 #include <vector>
@@ -106,14 +107,27 @@ int tllm_model_file_open(const char *path, tllm_model_file **file) {
     fclose(f);
     if (!ok) return TLLM_ERR_IO;
     if (h.magic != kMagic || h.version != kVersion) return TLLM_ERR_BAD_FILE;
+    // Every size is bounded BEFORE any arithmetic on it: the fields come from an untrusted file, and an
+    // overflowed product would pass the truncation check below and send uploads to wild pool offsets.
+    constexpr uint32_t kMaxDim = 1u << 24;       // rows or columns of one matrix
+    constexpr uint64_t kMaxElems = 1ull << 40;   // weights of one matrix, vocabulary table elements
     if (!h.vocab_size || !h.hidden_dim || !h.intermediate_dim || !h.n_heads || !h.n_kv_heads || !h.head_dim ||
-        h.group_size < 32 || h.group_size % 32 != 0 || h.n_layers > 4096)
+        h.group_size < 32 || h.group_size % 32 != 0 || h.group_size > kMaxDim || h.n_layers > 4096 ||
+        h.vocab_size > kMaxDim || h.hidden_dim > kMaxDim || h.intermediate_dim > kMaxDim || h.n_heads > kMaxDim ||
+        h.n_kv_heads > kMaxDim || h.head_dim > kMaxDim)
         return TLLM_ERR_BAD_FILE;
+    const uint64_t q64 = (uint64_t)h.n_heads * h.head_dim, kv64 = (uint64_t)h.n_kv_heads * h.head_dim;
+    if (q64 > kMaxDim || kv64 > kMaxDim) return TLLM_ERR_BAD_FILE;
     const int gs = (int)h.group_size;
     const int hidden_pad = pad32((int)h.hidden_dim);
-    const int q_dim = (int)(h.n_heads * h.head_dim), kv_dim = (int)(h.n_kv_heads * h.head_dim);
+    const int q_dim = (int)q64, kv_dim = (int)kv64;
     const int q_pad = pad32(q_dim), inter_pad = pad32((int)h.intermediate_dim);
     if (hidden_pad % gs || q_pad % gs || inter_pad % gs) return TLLM_ERR_BAD_FILE;
+    {
+        const uint64_t widest = (uint64_t)std::max(std::max(hidden_pad, q_pad), inter_pad);
+        const uint64_t tallest = std::max<uint64_t>(std::max<uint64_t>(h.intermediate_dim, h.vocab_size), std::max<uint64_t>(q64, h.hidden_dim));
+        if (widest * tallest > kMaxElems) return TLLM_ERR_BAD_FILE;   // with <= 4096 layers x 7 matrices the sums stay below 2^63
+    }
 
     tllm_model_file *m = new (std::nothrow) tllm_model_file;
     if (!m) return TLLM_ERR_TOO_LARGE;

@@ -413,3 +413,22 @@ def test_embedding_and_kv_copy_index_arithmetic(oracle):
                     inside = 0 <= s < seq
                     assert (kc[b, h, p] == (k[b, s, h] if inside else kc0[b, h, p])).all()
                     assert (vc[b, h, p] == (v[b, s, h] if inside else vc0[b, h, p])).all()
+
+
+def test_rope_fp32_angle_restatement(oracle):
+    """tllm_oracle_rope_f32angle restates the reference's fp32 arithmetic (kernels/rope.cu:49-64). Pinned by:
+    position 0 is the identity (cos 0 = 1, sin 0 = 0: the fp16 inputs come back bit for bit); theta = 1 makes
+    every frequency exactly 1, so the fp32 angle is exact for integer positions below 2^24 and the result must
+    equal the exact-angle rotation up to fp32 sine/cosine and fp16 rounding; and in general it stays within
+    pos * 2^-22 rad of the exact-angle rotation (the fp32 product pos * freq and powf are each good to an ulp)."""
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((2, 3, 4, 64)).astype(np.float16)
+    xb = x.view(np.uint16)
+    same = oracle.rope_f32angle(xb, 2, 3, 4, 64, 0, 10000.0)
+    assert np.array_equal(same[:, 0], xb[:, 0])                      # tokens at position 0
+    norm = np.sqrt((x.astype(np.float64).reshape(2, 3, 4, 32, 2) ** 2).sum(-1)).repeat(2, -1).reshape(x.shape)
+    for pos, theta in ((1234, 1.0), (8191, 1.0), (1234, 10000.0), (8191, 500000.0), (100000, 500000.0)):
+        exact = oracle.rope_f64(xb, 2, 3, 4, 64, pos, theta)
+        ref32 = oracle.rope_f32angle(xb, 2, 3, 4, 64, pos, theta).view(np.float16).astype(np.float64)
+        slack = (0.0 if theta == 1.0 else (pos + 2) * 2.0 ** -22) + 2.0 ** -10
+        assert (np.abs(ref32 - exact) <= slack * norm + 1e-7).all(), (pos, theta, float(np.abs(ref32 - exact).max()))

@@ -158,6 +158,45 @@ def test_model_file_rejects_bad_files(tmp_path):
         tl.write_synthetic_model(path, seed=1, **dict(DIMS, hidden_dim=200))   # not a multiple of the group
 
 
+def test_model_file_rejects_hostile_headers(tmp_path):
+    """Header fields of an untrusted file whose products overflow 32 or 64 bits (heads x head_dim,
+    rows x columns, the vocabulary table) must be refused as a bad file, not wrapped into offsets that pass
+    the truncation check."""
+    import struct
+    path = str(tmp_path / "t.tllm")
+    tl.write_synthetic_model(path, seed=1, **DIMS)
+    good = bytearray(open(path, "rb").read()[:256])
+    names = ("magic", "version", "arch", "vocab_size", "hidden_dim", "intermediate_dim", "n_layers", "n_heads",
+             "n_kv_heads", "max_seq_len", "head_dim", "rope_theta_bits", "group_size", "rms_norm_eps_bits", "flags")
+
+    def with_fields(**kw):
+        h = bytearray(good)
+        for k, v in kw.items():
+            struct.pack_into("<I", h, 4 * names.index(k), v)
+        return bytes(h)
+
+    hostile = [
+        dict(n_heads=0x10000, head_dim=0x10000),               # product wraps to 0 in 32 bits
+        dict(n_heads=0x8000, head_dim=0x20001),                # product wraps to a small number
+        dict(hidden_dim=0xFFFFFFE0),                           # negative as int, pad32 overflows
+        dict(vocab_size=0xFFFFFFFF),
+        dict(intermediate_dim=0x80000000),
+        dict(hidden_dim=1 << 23, intermediate_dim=1 << 23, n_layers=4096),   # each size allowed, a matrix of 2^46 weights
+        dict(group_size=0x80000000),
+        dict(n_layers=0xFFFFFFFF),
+        dict(n_kv_heads=0xFFFFFFFF, head_dim=2),
+    ]
+    for k, fields in enumerate(hostile):
+        f = tmp_path / f"hostile{k}.tllm"
+        f.write_bytes(with_fields(**fields) + b"\0" * 4096)
+        with pytest.raises(tl.TllmError) as e:
+            tl.ModelFile(str(f))
+        assert e.value.code == -9, (fields, e.value.code)
+    ok = tmp_path / "still_good.tllm"
+    ok.write_bytes(open(path, "rb").read())
+    tl.ModelFile(str(ok)).close()
+
+
 @pytest.mark.gpu
 def test_model_file_upload_and_sweep(tmp_path, oracle):
     """File -> one device pool -> one plan over every linear of the file -> oracle on the bytes

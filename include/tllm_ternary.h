@@ -246,10 +246,13 @@ int tllm_linear_plan_create(tllm_linear_plan **plan, const tllm_linear_problem *
 int tllm_linear_plan_create_normed(tllm_linear_plan **plan, const tllm_linear_problem *problems,
                                    const uint16_t *const *norm_weights, float eps, int count,
                                    int group_size);
-/* One launch over every problem of the plan. Allocation-free. Launches of ONE plan must not overlap in
- * time (two streams, or two graph branches): besides the outputs they share two device counters that
- * deal the tail of a large plan out to the workgroups; the kernel resets them when it ends, so
- * launches that follow each other on a stream, or replays of a captured graph, need no clearing. */
+/* One launch over every problem of the plan. Allocation-free. Besides the outputs a launch uses two device
+ * counters that deal the tail of a large plan out to the workgroups (the kernel resets them when it ends, so
+ * replays of a captured graph need no clearing). The plan holds 16 such pairs and launches take them in turn:
+ * launches of one plan may overlap in time (several streams, graph branches) as long as no two of them that
+ * are in flight together are 16 launches apart or were captured as the same launch (a captured launch keeps the
+ * pair it was captured with: do not replay one graph concurrently with itself). They still write the same
+ * outputs, like two calls of any operator on the same buffers. */
 int tllm_linear_plan_launch(const tllm_linear_plan *plan, tllm_stream_t stream);
 /* Algorithmic weight-stream bytes (masks + scales) one launch reads. */
 int64_t tllm_linear_plan_weight_bytes(const tllm_linear_plan *plan);

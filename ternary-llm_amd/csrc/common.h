@@ -125,6 +125,10 @@ hipError_t dispatch_linear(const Problem &p, int group, hipStream_t s, bool stat
 // True if dispatch_linear would run the prefill GEMM kernel (the only path that may need exchange memory).
 bool dispatch_takes_gemm(const Problem &p, int group);
 
+// Launches of one plan that are in flight at the same time need hand-out counters of their own: a launch
+// takes pair (launch number % kPlanSlots), so any kPlanSlots consecutive launches never share one.
+constexpr int kPlanSlots = 16;
+
 // Device-resident schedule of a multi-problem launch.
 struct PlanDevice {
     Problem *problems = nullptr;  // device copy of the table
@@ -141,7 +145,8 @@ struct PlanDevice {
     int *pool_first = nullptr;  // shared pool of small tasks (MFMA kernel, large plans)
     int pool_count = 0;
     int pool_begin = 0, pool_end = 0;  // batched kernel: blocks handed out at run time, their problems in pool_first
-    int *counters = nullptr;
+    int *counters = nullptr;  // kPlanSlots pairs of hand-out counters; a launch takes the next pair in turn
+    std::atomic<unsigned> *next_slot = nullptr;
     int grid = 0;
     int max_units = 0;
     int pair_stride = 0;  // floats between the two partial-sum areas of a SwiGLU pair (0: no pairs)

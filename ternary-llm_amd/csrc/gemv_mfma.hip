@@ -22,6 +22,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <mutex>
+#include <new>
 
 #include "common.h"
 #include "gemv_layout.h"
@@ -851,7 +852,8 @@ constexpr int kMaxTaskUnits = TLLM_MAX_TASK_UNITS;  // longer tasks amortise the
 // The workgroups of one launch all start together, three per CU, and the CU serves its oldest
 // waves first: measured on the 8B sweep with equal spans, the first 256 workgroups (one per CU)
 // finished after 233 us, the second 256 after 280 us and the last after 333 us; the odd XCDs
-// (workgroup index % 8) ran 8 % slower than the even ones, and what is left after these two effects
+// (workgroups go to the eight XCDs in turn, so XCD = index % 8 and its parity = index & 1) ran 8 % slower
+// than the even ones, and what is left after these two effects
 // is +-2 %. Spans are therefore cut in proportion to the speed of the place a workgroup will run in,
 // so that they end together. TLLM_SPAN_SHARES="s0,s1,s2,odd" overrides the four factors.
 struct SpanShares {
@@ -1200,7 +1202,7 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
     const size_t bytes_wg = round16(sizeof(int) * wg_first.size());
     const size_t bytes_pool = round16(sizeof(int) * pool_first.size());
     char *base = nullptr;
-    if (hipError_t e = hipMalloc(&base, bytes_table + bytes_prefix + bytes_wg + bytes_pool + 16)) return e;
+    if (hipError_t e = hipMalloc(&base, bytes_table + bytes_prefix + bytes_wg + bytes_pool + 8 * kPlanSlots)) return e;
     d.problems = reinterpret_cast<Problem *>(base);
     d.unit_prefix = reinterpret_cast<int *>(base + bytes_table);
     d.wg_first = reinterpret_cast<int *>(base + bytes_table + bytes_prefix);
@@ -1212,9 +1214,12 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
         e = hipMemcpy(d.wg_first, wg_first.data(), sizeof(int) * wg_first.size(), hipMemcpyHostToDevice);
     if (!e && !pool_first.empty())
         e = hipMemcpy(d.pool_first, pool_first.data(), sizeof(int) * pool_first.size(), hipMemcpyHostToDevice);
-    if (!e) e = hipMemset(d.counters, 0, 16);
+    if (!e) e = hipMemset(d.counters, 0, 8 * kPlanSlots);
+    d.next_slot = new (std::nothrow) std::atomic<unsigned>(0);
+    if (!e && !d.next_slot) e = hipErrorOutOfMemory;
     if (e) {
         (void)hipFree(base);
+        delete d.next_slot;
         return e;
     }
     *out = d;
@@ -1222,9 +1227,10 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
 }
 
 hipError_t plan_device_launch(const PlanDevice &plan, hipStream_t s) {
+    int *counters = plan.counters + 2 * (plan.next_slot->fetch_add(1, std::memory_order_relaxed) % kPlanSlots);
     if (plan.batch_kernel)
         return launch_gemv_batch_table(plan.problems, plan.unit_prefix, plan.wg_first, plan.grid, plan.pool_begin,
-                                       plan.pool_end, plan.pool_first, plan.counters, s);
+                                       plan.pool_end, plan.pool_first, counters, s);
     if (!plan.use_mfma)
         return launch_gemv_rowwave_f16_table(plan.problems, plan.count, plan.max_rows, plan.max_batch, 128, s);
     Sched sc{};
@@ -1233,7 +1239,7 @@ hipError_t plan_device_launch(const PlanDevice &plan, hipStream_t s) {
     sc.wg_first = plan.wg_first;
     sc.pool_first = plan.pool_first;
     sc.pool_count = plan.pool_count;
-    sc.counters = plan.counters;
+    sc.counters = counters;
     sc.count = plan.count;
     sc.pair_stride = plan.pair_stride;
     sc.max_units = plan.max_units;
@@ -1258,6 +1264,8 @@ hipError_t plan_device_launch(const PlanDevice &plan, hipStream_t s) {
 void plan_device_destroy(PlanDevice *plan) {
     if (plan->problems) (void)hipFree(plan->problems);
     plan->problems = nullptr;
+    delete plan->next_slot;
+    plan->next_slot = nullptr;
 }
 
 }  // namespace tllm

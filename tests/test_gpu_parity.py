@@ -1017,6 +1017,41 @@ def test_large_plan_in_a_captured_graph(dev, oracle):
     plan.close()
 
 
+def test_plan_launches_overlapping_on_two_streams(dev, oracle):
+    """Launches of one large plan (its tail is handed out through device counters) issued on two streams so that
+    they overlap in time: each launch has counters of its own, every launch must produce the bits of a launch
+    that ran alone (all launches write the same values into the same outputs)."""
+    torch, tl = dev
+    shapes = [(2048, 2048), (512, 2048), (512, 2048), (2048, 2048), (8192, 2048), (8192, 2048), (2048, 8192)]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(778)
+    probs = []
+    for layer in range(32):
+        for rows, cols in shapes:
+            nz = torch.randint(-2**31, 2**31 - 1, (rows, cols // 32), dtype=torch.int32, device="cuda", generator=gen)
+            sg = torch.randint(-2**31, 2**31 - 1, (rows, cols // 32), dtype=torch.int32, device="cuda", generator=gen)
+            sc = (torch.rand((rows, cols // 128), device="cuda", generator=gen) * 0.02 + 0.01).to(torch.float16)
+            x = torch.randn((1, cols), device="cuda", generator=gen).to(torch.float16)
+            y = torch.zeros((1, rows), dtype=torch.float16, device="cuda")
+            probs.append((nz, sg, sc, x, y, rows, cols, 1))
+    plan = tl.LinearPlan(probs)
+    plan.launch()
+    torch.cuda.synchronize()
+    alone = [p[4].clone() for p in probs]
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    for rep in range(3):
+        for p in probs:
+            p[4].fill_(float("nan"))
+        torch.cuda.synchronize()
+        for _ in range(5):
+            plan.launch(stream=s1)
+            plan.launch(stream=s2)
+        torch.cuda.synchronize()
+        for k, (p, a) in enumerate(zip(probs, alone)):
+            assert torch.equal(p[4].view(torch.int16), a.view(torch.int16)), f"round {rep} problem {k}"
+    plan.close()
+
+
 def test_random_shapes_through_every_dispatch_path(dev, oracle):
     """Sixty seeded random (rows, cols, group, batch) problems against the oracle: whichever kernel the
     dispatcher picks (row-wave, tall, wide in 48- or 16-row units, batched decode, passes of it, the

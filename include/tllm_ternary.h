@@ -98,14 +98,18 @@ int tllm_quantize_absmax_i8(const uint16_t *input, int8_t *output, float *scale,
  * A fp16 [M,K] row-major, packed weight [N,K], C fp16 [M,N] row-major.
  * Replaces ternary::ternary_gemm, reference include/kernels.cuh:37-40
  * (kernels/ternary_gemm.cu:33-195). Any M >= 1 is accepted.
- * Allocation: none per call, with one exception. Shapes with few weight tiles (M > 16 and N * M small
- * against the chip) split K over several workgroups per tile, which exchange fp32 partial sums through a
- * workspace that belongs to (device, stream): the first such call on a stream creates it (and a call with
- * a larger need grows it: stream synchronisation, free, allocation). tllm_gemm_workspace_reserve does
- * that ahead of time. While `stream` is being captured into a graph nothing is allocated: a call whose
- * workspace is missing or too small then runs without the split (same result up to the order of the
- * fp32 additions, slower). Calls that use one stream's workspace must not overlap in time: replays of a
- * captured graph on another stream count as calls on the stream the graph was captured on.
+ * Allocation: none per call, with one exception: a workspace that belongs to (device, stream). Two kinds
+ * of shapes use it. Shapes with few weight tiles (M > 16 and N * M small against the chip) split K over
+ * several workgroups per tile, which exchange fp32 partial sums through it; tall shapes (M of about 512 and
+ * more on wide matrices) run a kernel that reads the activations from a copy in matrix-core fragment order,
+ * which a small kernel writes there first (M rounded up to 32, times K, times 2 bytes; such a shape is only
+ * chosen while that stays within TLLM_GEMM_STATIC_SCRATCH_BYTES). The first such call on a stream creates
+ * the workspace (and a call with a larger need grows it: stream synchronisation, free, allocation).
+ * tllm_gemm_workspace_reserve does that ahead of time. While `stream` is being captured into a graph
+ * nothing is allocated: a call whose workspace is missing or too small then runs the kernel that needs
+ * none (same result up to the order of the fp32 additions, slower). Calls that use one stream's workspace
+ * must not overlap in time: replays of a captured graph on another stream count as calls on the stream
+ * the graph was captured on.
  */
 int tllm_ternary_gemm_f16(const uint16_t *A, const uint32_t *nz_B, const uint32_t *sign_B,
                           const uint16_t *scales_B, uint16_t *C, int M, int N, int K,
@@ -114,11 +118,12 @@ int tllm_ternary_gemm_f16(const uint16_t *A, const uint32_t *nz_B, const uint32_
 /*
  * tllm_ternary_gemm_f16 for callers that cannot allocate device memory (code under HIP graph capture,
  * serving loops and harnesses that forbid hipMalloc): same arguments, same kernels, same results bit for
- * bit, but the split-K exchange goes through a fixed array of TLLM_GEMM_STATIC_SCRATCH_BYTES in device
- * memory that the library holds on every GPU it runs on until the process ends. The call never
- * allocates, frees or synchronises. A shape whose exchange would not fit is rejected with
- * TLLM_ERR_SCRATCH_TOO_SMALL before anything is launched (with the tile shapes of this library the need
- * is at most CUs * 128 KiB: every shape fits on a 256-CU MI355X). All calls on one GPU share the one
+ * bit, but the workspace (split-K exchange or fragment-ordered activations) is a fixed array of
+ * TLLM_GEMM_STATIC_SCRATCH_BYTES in device memory that the library holds on every GPU it runs on until
+ * the process ends. The call never allocates, frees or synchronises. Both entry points choose their kernel among those whose workspace
+ * fits the array (a split needs at most CUs * 128 KiB; the copy of the activations is used up to 32 MiB),
+ * so on a 256-CU MI355X every shape runs; a configuration that would not fit is rejected with
+ * TLLM_ERR_SCRATCH_TOO_SMALL before anything is launched. All calls on one GPU share the one
  * array: calls that overlap in time on one GPU (two streams, two threads, two graph branches) race on it;
  * issue them on one stream, or use tllm_ternary_gemm_f16 with its per-stream workspaces.
  * No counterpart in the reference, whose GEMM needs no exchange memory.

@@ -1019,10 +1019,8 @@ GemmConfig choose_config(const Problem &p, size_t limit_floats) {
     // The eight-wave kernel: 0.85 us per stage (0.69 - 0.92 measured, the clock falls with the load), 9 us of
     // start, first loads, pair exchange and stores, and the copy of the activations into fragment order
     // (read + write at about 4 TB/s behind 2.5 us of its own start).
-    static const int forced = [] {
-        const char *e = getenv("TLLM_GEMM_PINGPONG");  // 0: never, 1: whenever the shape allows
-        return e ? atoi(e) : -1;
-    }();
+    const char *env = getenv("TLLM_GEMM_PINGPONG");  // 0: never, 1: whenever the shape allows (read at every call: tests switch it)
+    const int forced = env ? atoi(env) : -1;
     const GemmConfig pp{1, 1, true, 0.f};
     if (forced != 0 && workspace_floats(p, pp) <= limit_floats) {
         const long tiles = (long)n_tiles * ((p.batch + 255) / 256);

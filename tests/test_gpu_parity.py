@@ -239,6 +239,32 @@ def test_gemm_vs_oracle(dev, oracle, M, N, K):
     assert_close(oracle, run_gemm(dev, A, nz, sg, s), ref, what=f"gemm {M}x{N}x{K}")
 
 
+@pytest.mark.parametrize("M,N,K", [(600, 300, 640), (33, 128, 128), (257, 1000, 1152), (100, 129, 256), (512, 136, 384),
+                                   (16, 64, 128), (1023, 260, 640)])  # K not a multiple of 512: these go to the GEMM kernels
+def test_gemm_eight_wave_kernel_edges(dev, oracle, M, N, K):
+    """The eight-wave kernel (chosen by itself only for tall problems) forced onto shapes with ragged edges:
+    M not a multiple of 256 or of 32, N not a multiple of 128 or of 8 (the narrow store path), a single
+    scale group, more tiles than CUs. Against the fp64 oracle, and against the four-wave kernel (the two
+    differ only in the order of the fp32 additions)."""
+    nz, sg, s, _ = synth.problem(M * 7 + N, N, K, dontcare_sign=True)
+    A = synth.acts_f16(np.random.default_rng(M + K + 5), M, K)
+    ref = oracle.gemm_f64(A.view(np.uint16), nz, sg, s.view(np.uint16))
+    old = os.environ.get("TLLM_GEMM_PINGPONG")
+    try:
+        os.environ["TLLM_GEMM_PINGPONG"] = "1"
+        got = run_gemm(dev, A, nz, sg, s)
+        os.environ["TLLM_GEMM_PINGPONG"] = "0"
+        other = run_gemm(dev, A, nz, sg, s)
+    finally:
+        if old is None:
+            os.environ.pop("TLLM_GEMM_PINGPONG", None)
+        else:
+            os.environ["TLLM_GEMM_PINGPONG"] = old
+    assert_close(oracle, got, ref, what=f"eight-wave gemm {M}x{N}x{K}")
+    assert_close(oracle, other, ref, what=f"four-wave gemm {M}x{N}x{K}")
+    assert_close(oracle, got, other, tol=2e-3, what=f"eight-wave against four-wave {M}x{N}x{K}")
+
+
 @pytest.mark.parametrize("group,M", [(32, 3), (64, 20), (256, 5)])
 def test_gemm_other_group_sizes(dev, oracle, group, M):
     """Group sizes the .tllm files do not use still give the reference's result (general kernel)."""

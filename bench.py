@@ -313,7 +313,7 @@ def gemm_rows(torch, tl, orc, timer, seed, m_list, p_zero, calls, warm):
             row = {"config": f"cfg4: prefill GEMM M={m}, W {n}x{k}", "M": m, "N": n, "K": k, **stats_us(t),
                    "tflops": round(tflops, 1), "tflops_best": round(2.0 * m * n * k / (t["min_ms"] * 1e-3) / 1e12, 1),
                    "bound": "mfma" if m > 16 else "hbm", "frac_mfma_peak": round(tflops / MFMA_F16_PEAK_TFLOPS, 4),
-                   "kernel": "tllm::gemm_mfma_kernel" if m > 16 else "tllm::gemv_batch_kernel", "max_rel_sampled": rel}
+                   "kernel": tl.gemm_kernel(m, n, k), "max_rel_sampled": rel}
             if m <= 16:
                 gb = packed_bytes(n, k) / (t["mean_ms"] * 1e-3) / 1e9
                 row["GBps"] = round(gb, 1)

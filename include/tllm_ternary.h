@@ -134,6 +134,13 @@ int tllm_ternary_gemm_f16_static(const uint16_t *A, const uint32_t *nz_B, const 
                                  int group_size, tllm_stream_t stream);
 
 /*
+ * Name of the kernel tllm_ternary_gemm_f16 runs for a shape on the current device (static string, "" for a
+ * shape the entry point would reject; for reports and profiles: the choice depends on M, N, K and the
+ * number of CUs). No counterpart in the reference.
+ */
+const char *tllm_ternary_gemm_kernel(int M, int N, int K, int group_size);
+
+/*
  * Creates, or grows, the split-K workspace of `stream` for the GEMM shape (M, N, K) so that later
  * tllm_ternary_gemm_f16 calls of that shape (or a smaller need) on that stream allocate nothing, e.g.
  * before capturing them into a graph. May synchronise the stream. No counterpart in the reference (its

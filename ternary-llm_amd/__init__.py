@@ -10,6 +10,7 @@ from .ops import (  # noqa: F401
     add,
     copy_to_kv_cache,
     embedding_lookup,
+    gemm_kernel,
     gemm_workspace_release,
     gemm_workspace_reserve,
     lib,

@@ -112,6 +112,12 @@ int tllm_gemm_workspace_reserve(int M, int N, int K, int group_size, tllm_stream
 
 void tllm_gemm_workspace_release(void) { tllm::gemm_mfma_release_all(); }
 
+const char *tllm_ternary_gemm_kernel(int M, int N, int K, int group_size) {
+    if (M < 1 || N < 1 || K < 1 || K % 32 != 0 || group_size < 32 || group_size % 32 != 0 || K % group_size != 0) return "";
+    Problem p{nullptr, nullptr, nullptr, nullptr, nullptr, N, K, M, 0};
+    return tllm::dispatch_kernel_name(p, group_size);
+}
+
 static int gemv_i8_common(const uint32_t *nz, const uint32_t *sg, const uint16_t *scales,
                           const int8_t *xq, float scale_value, const float *scale_dev,
                           uint16_t *y, int rows, int cols, int group, tllm_stream_t stream) {

@@ -111,7 +111,8 @@ hipError_t launch_gemv_batch_table(const Problem *table, const int *unit_prefix,
 // 128-group MFMA GEMM for M >= 16 (gemm_mfma.hip); Problem.batch is M, rows is N, cols is K.
 bool gemm_mfma_supports(const Problem &p, int group);
 hipError_t launch_gemm_mfma(const Problem &p, hipStream_t s);
-float gemm_mfma_cost_us(const Problem &p);  // rough time of launch_gemm_mfma, to choose between kernels
+float gemm_mfma_cost_us(const Problem &p);
+const char *gemm_mfma_kernel_name(const Problem &p);  // the kernel launch_gemm_mfma would run (static string)  // rough time of launch_gemm_mfma, to choose between kernels
 // Creates (or grows) the split-K workspace of stream s for this shape, if the shape splits K at all.
 hipError_t gemm_mfma_reserve(const Problem &p, hipStream_t s);
 void gemm_mfma_release_all();  // frees every split-K workspace (nothing may still be running on them)
@@ -124,6 +125,8 @@ hipError_t launch_gemm_mfma_static(const Problem &p, hipStream_t s);
 hipError_t dispatch_linear(const Problem &p, int group, hipStream_t s, bool static_scratch = false);
 // True if dispatch_linear would run the prefill GEMM kernel (the only path that may need exchange memory).
 bool dispatch_takes_gemm(const Problem &p, int group);
+// Name of the kernel dispatch_linear would launch for this shape (static string; pointers may be null).
+const char *dispatch_kernel_name(const Problem &p, int group);
 
 // Launches of one plan that are in flight at the same time need hand-out counters of their own: a launch
 // takes pair (launch number % kPlanSlots), so any kPlanSlots consecutive launches never share one.

@@ -71,4 +71,14 @@ hipError_t dispatch_linear(const Problem &p, int group, hipStream_t s, bool stat
     return hipSuccess;
 }
 
+
+const char *dispatch_kernel_name(const Problem &p, int group) {
+    if (group != 128) return "tllm::gemv_rowwave_f16_kernel";
+    if (p.batch == 1 && gemv_mfma_supports(p, group)) return "tllm::gemv_mfma_kernel";
+    if (streams_in_passes(p, group)) return "tllm::gemv_batch_kernel";
+    if (gemv_mfma_supports(p, group)) return "tllm::gemv_mfma_kernel<Tall>";
+    if (gemm_mfma_supports(p, group)) return gemm_mfma_kernel_name(p);
+    return "tllm::gemv_mfma_kernel<Tall>, passes";
+}
+
 }  // namespace tllm

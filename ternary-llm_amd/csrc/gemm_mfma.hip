@@ -499,18 +499,26 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
 constexpr int kPpThreads = 512;
 constexpr int kPpMaskBuf = 8 * 768;  // per wave: nz words | sign words | scale dwords, 256 bytes each
 
-// A [M, K] row-major -> fragment order, rows past M as zeros. One thread per 16 bytes; a workgroup copies 32
-// rows x 64 columns (four 16-column steps): every wave reads eight whole 128-byte lines (8 rows) and writes
-// eight 128-byte runs (8 consecutive lanes of a fragment each).
+// A [M, K] row-major -> fragment order, rows past M as zeros. A workgroup copies 32 rows x 256 columns in four
+// passes of 64 columns (four 16-column steps): every wave reads eight whole 128-byte lines (8 rows) per
+// pass and writes eight 128-byte runs (8 consecutive lanes of a fragment each); the four loads of a thread
+// are in flight together.
 __global__ __launch_bounds__(256) void tile_acts_kernel(const uint16_t *__restrict__ A, u4 *__restrict__ At, int M, int K) {
-    const int ksteps = K / 16, kq_count = ksteps / 4;
-    const int mb = (int)blockIdx.x / kq_count, kq = (int)blockIdx.x % kq_count;
+    const int ksteps = K / 16, kq_count = ksteps / 4, wg_per_row = (kq_count + 3) / 4;
+    const int mb = (int)blockIdx.x / wg_per_row, kq0 = ((int)blockIdx.x % wg_per_row) * 4;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = 8 * wave + (lane >> 3), c = lane & 7;  // row inside the block, 16-byte chunk inside the 128 bytes
     const int row = 32 * mb + r;
-    u4 v = {0u, 0u, 0u, 0u};
-    if (row < M) v = __builtin_nontemporal_load(reinterpret_cast<const u4 *>(A + (size_t)row * K + 64 * kq + 8 * c));
-    At[((size_t)mb * ksteps + 4 * kq + (c >> 1)) * 64 + (c & 1) * 32 + r] = v;
+    u4 v[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        v[q] = u4{0u, 0u, 0u, 0u};
+        if (row < M && kq0 + q < kq_count)
+            v[q] = __builtin_nontemporal_load(reinterpret_cast<const u4 *>(A + (size_t)row * K + 64 * (kq0 + q) + 8 * c));
+    }
+#pragma unroll
+    for (int q = 0; q < 4; q++)
+        if (kq0 + q < kq_count) At[((size_t)mb * ksteps + 4 * (kq0 + q) + (c >> 1)) * 64 + (c & 1) * 32 + r] = v[q];
 }
 
 template <int MF>
@@ -972,7 +980,7 @@ hipError_t launch_pingpong(const Problem &p, float *workspace, hipStream_t s) {
         }
     }
     u4 *At = reinterpret_cast<u4 *>(workspace);
-    tile_acts_kernel<<<(unsigned)(((p.batch + 31) / 32) * (p.cols / 64)), 256, 0, s>>>(p.x, At, p.batch, p.cols);
+    tile_acts_kernel<<<(unsigned)(((p.batch + 31) / 32) * ((p.cols / 64 + 3) / 4)), 256, 0, s>>>(p.x, At, p.batch, p.cols);
     if (hipError_t e = hipGetLastError()) return e;
     const int m_tiles = (p.batch + BM - 1) / BM, n_tiles = (p.rows + kBN - 1) / kBN;
     gemm_pp_kernel<MF><<<m_tiles * n_tiles, kPpThreads, lds, s>>>(reinterpret_cast<const uint16_t *>(At), p.nz, p.sg, p.scales, p.y,
@@ -1035,6 +1043,13 @@ GemmConfig choose_config(const Problem &p, size_t limit_floats) {
 // Configurations are chosen among those whose workspace fits the fixed array of the entry point that
 // allocates nothing, so that both entry points run the same kernels on every shape.
 float gemm_mfma_cost_us(const Problem &p) { return choose_config(p, kStaticSlotFloats).us; }
+
+const char *gemm_mfma_kernel_name(const Problem &p) {
+    const GemmConfig c = choose_config(p, kStaticSlotFloats);
+    if (c.pingpong) return "tllm::gemm_pp_kernel<2> after tllm::tile_acts_kernel";
+    if (c.height == 1) return c.splits > 1 ? "tllm::gemm_mfma_kernel<2>, K split" : "tllm::gemm_mfma_kernel<2>";
+    return c.splits > 1 ? "tllm::gemm_mfma_kernel<1>, K split" : "tllm::gemm_mfma_kernel<1>";
+}
 
 namespace {
 hipError_t launch_config(const Problem &p, const GemmConfig &c, float *workspace, unsigned *arrivals, hipStream_t s) {

@@ -19,7 +19,7 @@ ABI_SYMBOLS = (
     "tllm_linear_plan_destroy", "tllm_rmsnorm_f16", "tllm_silu_mul_f16", "tllm_linear_plan_create_normed",
     "tllm_add_f16", "tllm_rope_f16", "tllm_embedding_lookup_f16", "tllm_copy_to_kv_cache_f16",
     "tllm_linear_plan_kernel", "tllm_gemm_workspace_reserve", "tllm_gemm_workspace_release",
-    "tllm_ternary_gemm_f16_static", "tllm_read_stream",
+    "tllm_ternary_gemm_f16_static", "tllm_read_stream", "tllm_ternary_gemm_kernel",
 )
 # include/tllm_model_file.h
 FILE_ABI_SYMBOLS = (
@@ -90,6 +90,8 @@ def lib():
     L.tllm_linear_plan_destroy.argtypes = [vp]
     L.tllm_linear_plan_kernel.argtypes = [vp]
     L.tllm_linear_plan_kernel.restype = C.c_char_p
+    L.tllm_ternary_gemm_kernel.argtypes = [i, i, i, i]
+    L.tllm_ternary_gemm_kernel.restype = C.c_char_p
     L.tllm_linear_plan_destroy.restype = None
     L.tllm_rmsnorm_f16.argtypes = [vp, vp, vp, vp, vp, i, i, f, vp]
     L.tllm_silu_mul_f16.argtypes = [vp, vp, vp, i, vp]
@@ -174,6 +176,11 @@ def ternary_gemm_static(A, nz_B, sign_B, scales_B, Cout, M, N, K, group_size=128
 def read_stream(buf, stream=None):
     """Measurement aid: one read-only pass over a device tensor (the streaming ceiling of the GPU)."""
     check(lib().tllm_read_stream(_ptr(buf), buf.numel() * buf.element_size(), None, _stream(stream)))
+
+
+def gemm_kernel(M, N, K, group_size=128):
+    """Name of the kernel ternary_gemm runs for this shape on the current device."""
+    return lib().tllm_ternary_gemm_kernel(M, N, K, group_size).decode()
 
 
 def gemm_workspace_reserve(M, N, K, group_size=128, stream=None):

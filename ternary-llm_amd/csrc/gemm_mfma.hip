@@ -395,7 +395,11 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
                 for (int g = 0; g < 4; g++) {
                     const f4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
                     float *dst = mine + (size_t)((i * MF + j) * 4 + g) * kThreads * 4;
-                    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(dst), "v"(v) : "memory");
+                    // A store of more than 8 bytes still reads its data registers for two issue slots after it
+                    // has issued; the compiler keeps other writers away from its own stores but cannot see into
+                    // this one, so the slots are filled here (without them the next address computation landed
+                    // in the data registers of the store before it and a quarter of the lanes stored garbage).
+                    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(dst), "v"(v) : "memory");
                 }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __shared__ unsigned last_arrival4;
@@ -744,6 +748,9 @@ __global__ __launch_bounds__(kPpThreads, 1) void gemm_pp_kernel(
     // ---- the two waves of a pair add their sums: fragment t = i * MF + j stays with wave kh = t & 1, the other
     // half crosses through LDS (free now); a + b = b + a, so both get the same bits whoever adds
     {
+        // the compiler cannot see that the LDS writes below read matrix results: the slots a 16-pass
+        // product needs before its result may be read by a memory instruction
+        asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 3" ::: "memory");
         constexpr int kKeep = kTiles / 2;
         const uint32_t xw = lds0 + (uint32_t)(wave * kKeep * 4096 + lane * 16);
         const uint32_t xr = lds0 + (uint32_t)((wave ^ 4) * kKeep * 4096 + lane * 16);

@@ -1170,6 +1170,69 @@ def test_cfg4_prefill_gemm_every_m(dev, oracle, M, N, K):
     _check_sampled(oracle, torch, A, nz, sg, sc, Cm, 6, 80, M + N, f"cfg4 M={M} {N}x{K}")
 
 
+def _dense_weights(torch, nz, sg, sc):
+    """fp32 [N, K] matrix of the packed weights (bit set in the sign plane: +scale, clear: -scale)."""
+    rows, words = nz.shape
+    sh = torch.arange(32, device="cuda", dtype=torch.int64)
+    out = torch.empty((rows, words * 32), dtype=torch.float32, device="cuda")
+    step = max(1, (1 << 23) // (words * 32))
+    for r0 in range(0, rows, step):
+        r1 = min(rows, r0 + step)
+        a = ((nz[r0:r1].to(torch.int64).unsqueeze(-1) >> sh) & 1).reshape(r1 - r0, -1)
+        b = ((sg[r0:r1].to(torch.int64).unsqueeze(-1) >> sh) & 1).reshape(r1 - r0, -1)
+        out[r0:r1] = (a * (2 * b - 1)).float() * sc[r0:r1].float().repeat_interleave(128, dim=1)
+    return out
+
+
+@pytest.mark.parametrize("M,N,K", [
+    (1024, 4096, 14336),   # 256-row tiles, K split in two (128 tiles on 256 CUs)
+    (640, 4096, 14336),    # the same with a ragged last tile of activation rows
+    (512, 4096, 14336),    # 128-row tiles, K split
+    (2048, 4096, 14336),   # 256-row tiles, no split
+    (512, 1024, 4096),     # few tiles: K split eight ways
+    (256, 256, 8192),
+    (130, 512, 2048),
+    (1024, 14336, 4096),   # the eight-wave kernel
+    (300, 2048, 2176),
+])
+def test_gemm_every_output_against_dense_product(dev, oracle, M, N, K):
+    """Every element of C, not a sample: the packed weights are expanded to an fp32 matrix on the GPU and
+    multiplied by the activations in fp32 (torch), which is itself checked against the fp64 oracle on sampled
+    rows and columns. A fault confined to a few lanes and registers of one exchange step (1 output in 256)
+    passes a sampled check more often than not; this test is the one that sees it. Each shape runs as the
+    library chooses and with the eight-wave kernel forced."""
+    torch, tl = dev
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(7000 + M + N + K)
+    nz, sg, sc = _device_problem(torch, N, K, 0.42, 0.01, 0.03, gen)
+    A = torch.randn((M, K), device="cuda", generator=gen).to(torch.float16)
+    W = _dense_weights(torch, nz, sg, sc)
+    ref = A.float() @ W.t()
+    del W
+    _check_sampled(oracle, torch, A, nz, sg, sc, ref, 4, 40, M + K, f"dense fp32 product {M}x{N}x{K}")
+    tau = float(torch.sqrt(torch.mean(ref * ref)).item()) / 64.0
+    old = os.environ.get("TLLM_GEMM_PINGPONG")
+    try:
+        for force in (None, "1"):
+            if force is None:
+                os.environ.pop("TLLM_GEMM_PINGPONG", None)
+            else:
+                os.environ["TLLM_GEMM_PINGPONG"] = force
+            for rep in range(2):
+                Cm = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+                tl.ternary_gemm(A, nz, sg, sc, Cm, M, N, K, 128)
+                torch.cuda.synchronize()
+                rel = (Cm.float() - ref).abs() / torch.clamp(ref.abs(), min=tau)
+                bad = int((~(rel <= TOL)).sum().item())
+                assert bad == 0, (f"gemm {M}x{N}x{K} ({tl.gemm_kernel(M, N, K)}, forced={force}, repetition {rep}): "
+                                  f"{bad} of {M * N} outputs beyond {TOL}, max_rel {float(rel.max()):.3e}")
+    finally:
+        if old is None:
+            os.environ.pop("TLLM_GEMM_PINGPONG", None)
+        else:
+            os.environ["TLLM_GEMM_PINGPONG"] = old
+
+
 LLAMA70B_LAYER = [(8192, 8192), (1024, 8192), (1024, 8192), (8192, 8192), (28672, 8192), (28672, 8192), (8192, 28672)]
 
 

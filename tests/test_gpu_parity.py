@@ -1233,6 +1233,46 @@ def test_gemm_every_output_against_dense_product(dev, oracle, M, N, K):
             os.environ["TLLM_GEMM_PINGPONG"] = old
 
 
+@pytest.mark.parametrize("batch", [1, 2, 4, 16])
+def test_decode_plan_every_output_against_dense_product(dev, oracle, batch):
+    """The decode kernels (one plan launch over the LLaMA-3-8B projections and a 70B-sized matrix pair) with
+    every output row compared, not a sample, against the fp32 product of the expanded weights; the single-call
+    entry points on the same operands must agree with the plan."""
+    torch, tl = dev
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(7100 + batch)
+    shapes = [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336), (28672, 8192), (8192, 28672), (1000, 1536)]
+    probs, refs = [], []
+    for rows, cols in shapes:
+        nz, sg, sc = _device_problem(torch, rows, cols, 0.42, 0.01, 0.03, gen)
+        x = torch.randn((batch, cols), device="cuda", generator=gen).to(torch.float16)
+        y = torch.full((batch, rows), float("nan"), dtype=torch.float16, device="cuda")
+        W = _dense_weights(torch, nz, sg, sc)
+        refs.append(x.float() @ W.t())
+        del W
+        probs.append((nz, sg, sc, x, y, rows, cols, batch))
+    _check_sampled(oracle, torch, probs[2][3], probs[2][0], probs[2][1], probs[2][2], refs[2], 2, 40, batch,
+                   "dense fp32 product 14336x4096")
+    plan = tl.LinearPlan(probs)
+    plan.launch()
+    torch.cuda.synchronize()
+    plan.close()
+    for (nz, sg, sc, x, y, rows, cols, _), ref in zip(probs, refs):
+        tau = float(torch.sqrt(torch.mean(ref * ref)).item()) / 64.0
+        rel = (y.float() - ref).abs() / torch.clamp(ref.abs(), min=tau)
+        bad = int((~(rel <= TOL)).sum().item())
+        assert bad == 0, f"plan {rows}x{cols} batch {batch}: {bad} of {batch * rows} outputs beyond {TOL}, max_rel {float(rel.max()):.3e}"
+        single = torch.full((batch, rows), float("nan"), dtype=torch.float16, device="cuda")
+        if batch == 1:
+            tl.ternary_gemv(nz, sg, sc, x[0], single[0], rows, cols, 128)
+        else:
+            tl.ternary_gemm(x, nz, sg, sc, single, batch, rows, cols, 128)
+        torch.cuda.synchronize()
+        rel = (single.float() - ref).abs() / torch.clamp(ref.abs(), min=tau)
+        bad = int((~(rel <= TOL)).sum().item())
+        assert bad == 0, f"single call {rows}x{cols} batch {batch}: {bad} outputs beyond {TOL}, max_rel {float(rel.max()):.3e}"
+
+
 LLAMA70B_LAYER = [(8192, 8192), (1024, 8192), (1024, 8192), (8192, 8192), (28672, 8192), (28672, 8192), (8192, 28672)]
 
 

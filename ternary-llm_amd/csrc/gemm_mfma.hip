@@ -848,6 +848,353 @@ __global__ __launch_bounds__(kPpThreads, 1) void gemm_pp_kernel(
     }
 }
 
+// ---- The row-split kernel: eight waves that split the weight rows, weights decoded straight into MFMA operand
+// registers.
+//
+// A workgroup computes 256 weight rows x 32 MF activation rows; wave w owns weight rows 32 w .. 32 w + 31 (one A-operand
+// fragment) and all the activation rows (MF accumulator fragments). What this changes against the kernels above:
+//   * decoded weights never pass through LDS (its write port was the slowest unit of those kernels): lane (li, lq) of wave
+//     w loads the mask words of its own row, and the byte of a word IS the eight weights of one MFMA operand: one
+//     v_perm puts byte t of the even-weight and odd-weight codes into the two halves of a dword, then a packed shift,
+//     an AND and a packed multiply per weight pair: 13 vector instructions per MFMA step, used by MF MFMAs.
+//     K is walked in an order that makes this possible: a block of 256 columns is four chunks of 64; in step t of chunk u
+//     lane half lq multiplies the 8 columns 256 b + 64 u + 32 lq + 8 t .. + 7, i.e. byte t of mask word 2 u + lq. Both
+//     operands use the same assignment, and a sum does not care in which order the columns are taken.
+//     A lane loads mask words 4 lq .. 4 lq + 3 of a block (16 bytes per plane) and the two half-waves then trade words
+//     with v_permlane32_swap; the two scales of a block come as one dword.
+//   * the activations of the tile come straight from A[M][K] (no reordered copy): the load instruction writes them into
+//     LDS (global_load_lds, 16 bytes per lane) in 1 KB pieces of 16 rows x 64 bytes, lane 16 t + r fetching step t of
+//     row r, so that the B operand of (step t, fragment j) is one conflict-free ds_read_b128 per lane. A chunk is
+//     MF x 4 KB; four chunks are in flight (ring of four slots, one barrier per chunk, taken one step before the
+//     chunk's end so that the first fragment reads of the next chunk are already on their way).
+//   * the vector work of step s + 1 is dealt out between the MFMAs of step s.
+// Tiles that do not fill the last round of workgroups over the CUs are split along K between several workgroups
+// (`splits`), which exchange fp32 sums through memory like the kernels above; the tiles before them (`full_tiles`)
+// run whole. The workgroups of one XCD take consecutive work items of both kinds.
+constexpr int kNsBN = 256;
+constexpr int kNsThreads = 512;
+constexpr int kNsPitch = 2 * kNsBN + 16;  // bytes per activation row of the output tile in LDS
+
+template <int MF>
+__global__ __launch_bounds__(kNsThreads, 1) void gemm_ns_kernel(
+    const uint16_t *__restrict__ A, const uint32_t *__restrict__ nzB, const uint32_t *__restrict__ sgB,
+    const uint16_t *__restrict__ scB, uint16_t *__restrict__ C, int M, int N, int K, int full_tiles, int splits,
+    float *__restrict__ partial, unsigned *__restrict__ arrivals) {
+    constexpr int BM = 32 * MF;
+    constexpr int kChunk = 4 * MF * 1024;  // bytes of one chunk: four steps of MF fragments
+    constexpr int kDma = MF / 2;           // 1 KB pieces per wave and chunk
+    static_assert(MF == 4, "the ring of four chunks is addressed with 16-bit offsets: 4 x 16 KB");
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    typedef __attribute__((address_space(3))) unsigned char LB;
+    typedef __attribute__((address_space(1))) const unsigned char GB;
+    LB *lds_l = (LB *)lds;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 31, lq = lane >> 5;
+
+    // ---- which tile, which part of K. Workgroup ids go round the XCDs: XCD x takes the x-th eighth of the whole tiles
+    // first and the x-th eighth of the parts of split tiles afterwards.
+    const int m_tiles = (M + BM - 1) / BM, n_tiles = (N + kNsBN - 1) / kNsBN;
+    const int tiles = m_tiles * n_tiles, parts = (tiles - full_tiles) * splits;
+    const int full_per = (full_tiles + 7) / 8, part_per = (parts + 7) / 8;
+    const int xcd = (int)blockIdx.x & 7, slot_in_xcd = (int)blockIdx.x >> 3;
+    int tile, split = 0;
+    if (slot_in_xcd < full_per) {
+        tile = xcd * full_per + slot_in_xcd;
+        if (tile >= full_tiles) return;
+    } else {
+        const int part = xcd * part_per + (slot_in_xcd - full_per);
+        if (part >= parts) return;
+        tile = full_tiles + part / splits;
+        split = part - (part / splits) * splits;
+    }
+    const bool is_split = tile >= full_tiles && splits > 1;
+    const int n0 = (tile / m_tiles) * kNsBN;
+    const int m0 = (tile % m_tiles) * BM;
+    const int words = K / 32, groups = K / 128, blocks = K / 256;
+    const int chunks = blocks * 4;
+    const int b_begin = is_split ? (int)((long)blocks * split / splits) : 0;
+    const int b_end = is_split ? (int)((long)blocks * (split + 1) / splits) : blocks;
+
+    const int row = min(n0 + 32 * wave + li, N - 1);
+    GB *nz_g = (GB *)nzB + ((size_t)row * words + 4 * lq) * 4;
+    GB *sg_g = (GB *)sgB + ((size_t)row * words + 4 * lq) * 4;
+    GB *sc_g = (GB *)scB + (size_t)row * groups * 2;  // two scales per block: one aligned dword (groups is even)
+
+    // activation pieces this wave copies per chunk: piece p = wave * kDma + i covers fragment j = p / 4, rows
+    // 16 h .. 16 h + 15 of it (h = (p / 2) % 2), column half q = p % 2; lane L of the copy fetches step L / 16 of row
+    // L % 16. Rows past M repeat the last row (their outputs are not stored).
+    GB *a_src[kDma];
+    int a_dst[kDma];
+#pragma unroll
+    for (int i = 0; i < kDma; i++) {
+        const int p = wave * kDma + i, j = p >> 2, h = (p >> 1) & 1, q = p & 1;
+        const int m = min(m0 + 32 * j + 16 * h + (lane & 15), M - 1);
+        a_src[i] = (GB *)A + ((size_t)m * K + 32 * q + 8 * (lane >> 4)) * 2;
+        a_dst[i] = p * 1024;
+    }
+    const uint32_t lds0 = (uint32_t)(uintptr_t)lds_l;
+    const uint32_t b_rd = lds0 + (uint32_t)((((li >> 4) * 2 + lq) * 1024) + (li & 15) * 16);
+#define TLLM_GPTR(p) ((__attribute__((address_space(1))) const void *)(p))
+#define TLLM_LPTR(p) ((__attribute__((address_space(3))) void *)(p))
+    // The destination of an asm load is "+v": the register that is being filled is then the one the variable had
+    // before, and no copy of a register still in flight can appear on a loop edge.
+#define TLLM_LDS_READ128(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "+v"(dst) : "v"(addr), "i"(off))
+#define TLLM_FENCE() __builtin_amdgcn_sched_barrier(0)
+    auto dma_chunk = [&](int c, int slot) {
+        const int off = min(c, chunks - 1) * 128;
+#pragma unroll
+        for (int i = 0; i < kDma; i++)
+            __builtin_amdgcn_global_load_lds(TLLM_GPTR(a_src[i] + off), TLLM_LPTR(lds_l + slot * kChunk + a_dst[i]), 16, 0, 0);
+    };
+    u4 nx_nz = {0u, 0u, 0u, 0u}, nx_sg = {0u, 0u, 0u, 0u};
+    uint32_t nx_sc = 0;
+    auto load_masks = [&](int b) {
+        const int bb = min(b, blocks - 1);
+        GB *p0 = nz_g + (size_t)bb * 32;
+        GB *p1 = sg_g + (size_t)bb * 32;
+        GB *p2 = sc_g + (size_t)bb * 4;
+        asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(nx_nz) : "v"(p0) : "memory");
+        asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(nx_sg) : "v"(p1) : "memory");
+        asm volatile("global_load_dword %0, %1, off" : "+v"(nx_sc) : "v"(p2) : "memory");
+    };
+
+    f16v acc[MF];
+#pragma unroll
+    for (int j = 0; j < MF; j++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[j][r] = 0.f;
+
+    uint32_t cu_nz[4], cu_sg[4];  // mask word 2 u + lq of the current block
+    h2 sp2[2];                    // its two scales, each in both halves
+    u4 Bv[2][MF];
+#pragma unroll
+    for (int q = 0; q < 2; q++)
+#pragma unroll
+        for (int j = 0; j < MF; j++) Bv[q][j] = u4{0u, 0u, 0u, 0u};
+    u4 av[2];
+    uint32_t t0 = 0, t1 = 0, qn = 0;
+    h2 sp = {};
+    auto codes = [&](int u) {  // the two-bit codes (negative, non-zero) of mask word u: even weights in t0, odd weights in t1
+        const uint32_t m_nz = cu_nz[u], m_sg = cu_sg[u];
+        sp = sp2[u >> 1];
+        const uint32_t neg = m_nz & ~m_sg;
+        t0 = __builtin_amdgcn_bitop3_b32(neg << 1, m_nz, 0xAAAAAAAAu, 0xE4);
+        t1 = __builtin_amdgcn_bitop3_b32(neg, m_nz >> 1, 0xAAAAAAAAu, 0xE4);
+    };
+    auto pick = [&](int t) {  // byte t of the even codes into the low half, of the odd codes into the high half
+        qn = __builtin_amdgcn_perm(t1, t0, 0x0C000C00u | (uint32_t)t | ((uint32_t)(4 + t) << 16));
+    };
+    auto pair = [&](int e) -> uint32_t {  // weights 2 e, 2 e + 1 of the byte as +-2 scale / 0
+        us2 v = __builtin_bit_cast(us2, qn);
+        v = v << (uint16_t)(14 - 2 * e);
+        uint32_t top = __builtin_bit_cast(uint32_t, v);
+        if (e > 0) top &= 0xC000C000u;  // (for e = 0 the shift leaves nothing below the field)
+        return __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, top) * sp);
+    };
+    auto take_masks = [&]() {  // the loads into nx_* are complete where this is called
+        asm volatile("" : "+v"(nx_nz), "+v"(nx_sg), "+v"(nx_sc));
+        // v_permlane32_swap(a, b): a keeps its lower half-wave and takes b's lower half-wave as its upper one; b takes
+        // a's upper half-wave as its lower one and keeps its upper one
+        const auto s01 = __builtin_amdgcn_permlane32_swap(nx_nz[0], nx_nz[1], false, false);
+        const auto s23 = __builtin_amdgcn_permlane32_swap(nx_nz[2], nx_nz[3], false, false);
+        const auto g01 = __builtin_amdgcn_permlane32_swap(nx_sg[0], nx_sg[1], false, false);
+        const auto g23 = __builtin_amdgcn_permlane32_swap(nx_sg[2], nx_sg[3], false, false);
+        cu_nz[0] = s01[0]; cu_nz[2] = s01[1]; cu_nz[1] = s23[0]; cu_nz[3] = s23[1];
+        cu_sg[0] = g01[0]; cu_sg[2] = g01[1]; cu_sg[1] = g23[0]; cu_sg[3] = g23[1];
+        sp2[0] = __builtin_bit_cast(h2, __builtin_amdgcn_perm(nx_sc, nx_sc, 0x01000100u));
+        sp2[1] = __builtin_bit_cast(h2, __builtin_amdgcn_perm(nx_sc, nx_sc, 0x03020302u));
+#pragma unroll
+        for (int u = 0; u < 4; u++) asm volatile("" : "+v"(cu_nz[u]), "+v"(cu_sg[u]));
+        asm volatile("" : "+v"(sp2[0]), "+v"(sp2[1]));
+    };
+
+    // ---- prologue: masks of the first two blocks, the first four chunks; operands of the first step.
+    // Requests complete in order; every wait below names how many younger ones may still be in flight.
+    const int c_begin = 4 * b_begin;
+    load_masks(b_begin);
+    dma_chunk(c_begin, 0);
+    dma_chunk(c_begin + 1, 1);
+    dma_chunk(c_begin + 2, 2);
+    TLLM_FENCE();
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kDma) : "memory");
+    __builtin_amdgcn_s_barrier();
+    TLLM_FENCE();
+    take_masks();
+    load_masks(b_begin + 1);
+    dma_chunk(c_begin + 3, 3);
+    TLLM_FENCE();
+#pragma unroll
+    for (int j = 0; j < MF; j++) TLLM_LDS_READ128(Bv[0][j], b_rd, j * 4096);
+    codes(0);
+    pick(0);
+    av[0] = u4{pair(0), pair(1), pair(2), pair(3)};
+    TLLM_FENCE();
+
+    // One step: the MFMAs of step s = (chunk c in ring slot u, t) with the decode of step s + 1 between them; the
+    // activation fragments of step s + 1 are requested first. The last step of a chunk begins by taking the workgroup
+    // across the barrier that frees the chunk's slot (every wave has its last fragments of it) and proves that the next
+    // chunk has landed (every wave has waited for its own pieces); the slot is refilled with chunk c + 4. Request order
+    // is: masks of block b + 2 (asked for in the last step of block b), then the chunks; a chunk's wait therefore
+    // leaves the two younger chunks in flight and, in the two steps that follow a mask request, those three loads too.
+    auto kstep = [&](auto U, auto T, int c) {
+        constexpr int u = decltype(U)::value, t = decltype(T)::value;
+        constexpr int cur = t & 1, nxt = cur ^ 1;
+        constexpr int ru = t == 3 ? ((u + 1) & 3) : u, rt = (t + 1) & 3;
+        if (t == 3) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            if (u < 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kDma + 3) : "memory");
+            else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kDma) : "memory");
+            __builtin_amdgcn_s_barrier();
+            TLLM_FENCE();
+            if (u == 3) {
+                take_masks();
+                load_masks((c + 1) / 4 + 1);
+            }
+            dma_chunk(c + 4, u);
+            TLLM_FENCE();
+        }
+#pragma unroll
+        for (int j = 0; j < MF; j++) TLLM_LDS_READ128(Bv[nxt][j], b_rd, ru * kChunk + j * 4096 + rt * 256);
+        if (t != 3) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(MF) : "memory");
+        TLLM_FENCE();
+        u4(&R)[MF] = Bv[cur];
+        u4 &a_cur = av[cur];
+        uint32_t an[4];
+#pragma unroll
+        for (int j = 0; j < MF; j++) {
+            asm volatile("" : "+v"(R[j]));
+            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, a_cur), __builtin_bit_cast(h8, R[j]), acc[j], 0, 0, 0);
+            TLLM_FENCE();
+            if (j == 0) {
+                if (t == 3) codes(ru);
+                pick(rt);
+            }
+            an[j] = pair(j);
+            asm volatile("" : "+v"(an[j]));  // computed here, between the MFMAs, not where it is used
+            TLLM_FENCE();
+        }
+        av[nxt] = u4{an[0], an[1], an[2], an[3]};
+    };
+    std::integral_constant<int, 0> i0;
+    std::integral_constant<int, 1> i1;
+    std::integral_constant<int, 2> i2;
+    std::integral_constant<int, 3> i3;
+    for (int b = b_begin; b < b_end; b++) {
+        kstep(i0, i0, 4 * b); kstep(i0, i1, 4 * b); kstep(i0, i2, 4 * b); kstep(i0, i3, 4 * b);
+        kstep(i1, i0, 4 * b + 1); kstep(i1, i1, 4 * b + 1); kstep(i1, i2, 4 * b + 1); kstep(i1, i3, 4 * b + 1);
+        kstep(i2, i0, 4 * b + 2); kstep(i2, i1, 4 * b + 2); kstep(i2, i2, 4 * b + 2); kstep(i2, i3, 4 * b + 2);
+        kstep(i3, i0, 4 * b + 3); kstep(i3, i1, 4 * b + 3); kstep(i3, i2, 4 * b + 3); kstep(i3, i3, 4 * b + 3);
+    }
+    TLLM_FENCE();
+    // copies and fragment reads past the last step are still in flight into LDS and registers
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    // the compiler cannot see that the asm stores below read matrix results: the slots a 16-pass product needs before
+    // its result may be read by a memory instruction
+    asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 3" ::: "memory");
+#undef TLLM_LDS_READ128
+#undef TLLM_FENCE
+#undef TLLM_GPTR
+#undef TLLM_LPTR
+
+    if (is_split) {
+        // fp32 sums of this part into its slot (element (j, g, tid, e) at ((j * 4 + g) * 512 + tid) * 4 + e), written
+        // through to memory; the last part of a tile to arrive adds all slots in part order, its own sums from its
+        // registers in their place of that order
+        constexpr int kSlot = BM * kNsBN;
+        const int st = tile - full_tiles;
+        float *mine = partial + ((size_t)st * splits + split) * kSlot + tid * 4;
+#pragma unroll
+        for (int j = 0; j < MF; j++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const f4 v = {acc[j][4 * g], acc[j][4 * g + 1], acc[j][4 * g + 2], acc[j][4 * g + 3]};
+                float *dst = mine + (size_t)(j * 4 + g) * kNsThreads * 4;
+                // (two idle issue slots: a store of more than 8 bytes still reads its data registers after it has issued)
+                asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(dst), "v"(v) : "memory");
+            }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __shared__ unsigned last_arrival_ns;
+        __syncthreads();
+        if (tid == 0) {
+            const unsigned before = __hip_atomic_fetch_add(&arrivals[st], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            last_arrival_ns = before == (unsigned)splits - 1;
+            if (last_arrival_ns) __hip_atomic_store(&arrivals[st], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+        if (!last_arrival_ns) return;
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        const float *slots = partial + (size_t)st * splits * kSlot + tid * 4;
+        f16v own[MF];
+#pragma unroll
+        for (int j = 0; j < MF; j++) {
+            own[j] = acc[j];
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[j][r] = 0.f;
+        }
+        for (int q = 0; q < splits; q++) {
+            if (q == split) {
+#pragma unroll
+                for (int j = 0; j < MF; j++) acc[j] += own[j];
+                continue;
+            }
+            const float *slot = slots + (size_t)q * kSlot;
+#pragma unroll
+            for (int j = 0; j < MF; j++) {
+                f4 v[4];
+#pragma unroll
+                for (int g = 0; g < 4; g++) v[g] = *reinterpret_cast<const f4 *>(slot + (size_t)(j * 4 + g) * kNsThreads * 4);
+#pragma unroll
+                for (int g = 0; g < 4; g++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) acc[j][4 * g + e] += v[g][e];
+            }
+        }
+    }
+
+    // ---- store. Register 4 g + v of fragment j is weight row n0 + 32 wave + 8 g + 4 lq + v for activation row
+    // m0 + 32 j + li: stored as they are these are 8-byte pieces in 32 different lines per instruction. The tile goes
+    // through LDS instead (the ring is free now) and leaves as whole 512-byte rows, two rows per instruction.
+    const bool wide_store = (N & 7) == 0 && (reinterpret_cast<uintptr_t>(C) & 15) == 0;
+    if (wide_store) {
+        __syncthreads();  // every wave is done with the ring
+#pragma unroll
+        for (int j = 0; j < MF; j++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                uint16_t hv[4];
+#pragma unroll
+                for (int v = 0; v < 4; v++) hv[v] = f2h(acc[j][4 * g + v] * 0.5f);
+                *reinterpret_cast<uint2 *>(lds + (32 * j + li) * kNsPitch + (32 * wave + 8 * g + 4 * lq) * 2) =
+                    uint2{(uint32_t)hv[0] | ((uint32_t)hv[1] << 16), (uint32_t)hv[2] | ((uint32_t)hv[3] << 16)};
+            }
+        __syncthreads();
+        const int piece = lane & 31;
+        const int n = n0 + piece * 8;
+#pragma unroll
+        for (int r = 0; r < BM / 16; r++) {
+            const int ml = wave * (BM / 8) + 2 * r + lq;
+            const int m = m0 + ml;
+            if (m < M && n < N) *reinterpret_cast<u4 *>(C + (size_t)m * N + n) = *reinterpret_cast<const u4 *>(lds + ml * kNsPitch + piece * 16);
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < MF; j++) {
+            const int m = m0 + j * 32 + li;
+            if (m >= M) continue;
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int n = n0 + 32 * wave + 8 * g + 4 * lq;
+#pragma unroll
+                for (int v = 0; v < 4; v++)
+                    if (n + v < N) C[(size_t)m * N + n + v] = f2h(acc[j][4 * g + v] * 0.5f);
+            }
+        }
+    }
+}
+
 // ---- split-K exchange memory: fp32 slots and one arrival counter per tile.
 //
 // Ordinary calls use a workspace per (device, stream), created by tllm_gemm_workspace_reserve or by the
@@ -928,16 +1275,22 @@ hipError_t static_scratch(unsigned char **out) {
 }
 
 struct GemmConfig {
-    int height;   // 0: 128 activation rows per workgroup, 1: 256
-    int splits;   // workgroups per tile along K (four-wave kernel)
+    int height;   // 0: 128 activation rows per workgroup, 1: 256 (four-wave and eight-wave ping-pong kernels)
+    int splits;   // workgroups per tile along K (four-wave kernel: every tile; row-split kernel: the tiles after full_tiles)
     bool pingpong;  // the eight-wave kernel (256 activation rows, one workgroup per tile, fragment-ordered activations)
     float us;     // estimated time
+    bool rowsplit = false;  // the row-split kernel (256 weight rows x 128 activation rows per workgroup)
+    int full_tiles = 0;     // row-split kernel: tiles computed by one workgroup each
 };
 GemmConfig choose_config(const Problem &p, size_t workspace_floats);
 
 // Workspace a configuration needs, in floats: the fp32 slots of a split, or the fragment-ordered copy of the
 // activations (rows rounded up to 32) of the eight-wave kernel. The two never occur together.
 size_t workspace_floats(const Problem &p, const GemmConfig &c) {
+    if (c.rowsplit) {
+        const size_t tiles = (size_t)((p.batch + 127) / 128) * ((p.rows + kNsBN - 1) / kNsBN);
+        return c.splits > 1 ? (tiles - c.full_tiles) * c.splits * 128 * kNsBN : 0;
+    }
     if (c.pingpong) return (size_t)((p.batch + 31) / 32) * 32 * p.cols / 2;
     const int bm = 128 << c.height;
     const size_t tiles = (size_t)((p.batch + bm - 1) / bm) * ((p.rows + kBN - 1) / kBN);
@@ -995,6 +1348,32 @@ hipError_t launch_pingpong(const Problem &p, float *workspace, hipStream_t s) {
     return hipGetLastError();
 }
 
+hipError_t launch_rowsplit(const Problem &p, const GemmConfig &c, float *partial, unsigned *arrivals, hipStream_t s) {
+    constexpr int MF = 4, BM = 32 * MF;
+    static std::mutex attr_mutex;
+    static bool attr_set[64] = {};
+    int dev = 0;
+    if (hipError_t e = hipGetDevice(&dev)) return e;
+    // loop: a ring of four activation chunks; afterwards the output tile, one padded row per activation row
+    const size_t ring = 4 * (size_t)(4 * MF * 1024), out_tile = (size_t)BM * kNsPitch;
+    const size_t lds = ring > out_tile ? ring : out_tile;
+    if (dev >= 0 && dev < 64) {
+        std::lock_guard<std::mutex> lock(attr_mutex);
+        if (!attr_set[dev]) {
+            if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_ns_kernel<MF>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
+                return e;
+            attr_set[dev] = true;
+        }
+    }
+    const int tiles = ((p.batch + BM - 1) / BM) * ((p.rows + kNsBN - 1) / kNsBN);
+    const int parts = (tiles - c.full_tiles) * c.splits;
+    const int wgs = 8 * ((c.full_tiles + 7) / 8 + (parts + 7) / 8);
+    gemm_ns_kernel<MF><<<wgs, kNsThreads, lds, s>>>(p.x, p.nz, p.sg, p.scales, p.y, p.batch, p.rows, p.cols, c.full_tiles,
+                                                    c.splits, partial, arrivals);
+    return hipGetLastError();
+}
+
 }  // namespace
 
 bool gemm_mfma_supports(const Problem &p, int group) {
@@ -1043,6 +1422,42 @@ GemmConfig choose_config(const Problem &p, size_t limit_floats) {
                          (float)p.batch * (float)p.cols * 4.0f / 4.0e6f;
         if (forced == 1 || us < best.us) best = GemmConfig{1, 1, true, us};
     }
+    // The row-split kernel: 3.3 us per block of 256 columns (1490 - 1530 cycles per chunk of 64 at the 1.8 GHz the chip
+    // holds under this load), 9 us of launch, first loads and stores. The tiles that do not fill the last round over the
+    // CUs are split along K (at most as far as the CUs reach, two blocks per part at least, and while the slots fit the
+    // workspace) when that is cheaper than a last round of whole tiles; an exchange costs about 6 us + 1.5 us per part
+    // (fitted to 4096 x 14336 at M = 128 ... 512). Tiles are 128 activation rows high: not for fewer than 96.
+    const char *env_rs = getenv("TLLM_GEMM_ROWSPLIT");  // 0: never, 1: whenever the shape allows (read at every call)
+    const int forced_rs = env_rs ? atoi(env_rs) : -1;
+    const bool rs_ok = p.cols % 256 == 0 && !((reinterpret_cast<uintptr_t>(p.x) | reinterpret_cast<uintptr_t>(p.nz) |
+                                                reinterpret_cast<uintptr_t>(p.sg)) & 15);
+    if (forced_rs != 0 && rs_ok && forced != 1 && (forced_rs == 1 || p.batch >= 96)) {
+        const int blocks = p.cols / 256;
+        const int tiles = ((p.batch + 127) / 128) * ((p.rows + kNsBN - 1) / kNsBN);
+        const float block_us = 3.3f, fixed_us = 9.0f;
+        GemmConfig rs{0, 1, false, 0.f};
+        rs.rowsplit = true;
+        rs.full_tiles = tiles;
+        rs.us = (float)((tiles + n_cu - 1) / n_cu) * (float)blocks * block_us + fixed_us;
+        const int rem = tiles % n_cu;
+        if (rem) {
+            int splits = n_cu / rem;
+            if (splits > 8) splits = 8;
+            if (splits > blocks / 2) splits = blocks / 2;
+            while (splits > 1 && (size_t)rem * splits * 128 * kNsBN > limit_floats) splits--;
+            if (splits > 1) {
+                const float exchange = 6.0f + 1.5f * (float)splits;
+                const float us = (float)(tiles / n_cu) * (float)blocks * block_us + (float)((blocks + splits - 1) / splits) * block_us +
+                                 exchange + fixed_us;
+                if (us < rs.us) {
+                    rs.splits = splits;
+                    rs.full_tiles = tiles - rem;
+                    rs.us = us;
+                }
+            }
+        }
+        if (forced_rs == 1 || rs.us < best.us) best = rs;
+    }
     return best;
 }
 }  // namespace
@@ -1053,6 +1468,7 @@ float gemm_mfma_cost_us(const Problem &p) { return choose_config(p, kStaticSlotF
 
 const char *gemm_mfma_kernel_name(const Problem &p) {
     const GemmConfig c = choose_config(p, kStaticSlotFloats);
+    if (c.rowsplit) return c.splits > 1 ? "tllm::gemm_ns_kernel<4>, last tiles K split" : "tllm::gemm_ns_kernel<4>";
     if (c.pingpong) return "tllm::gemm_pp_kernel<2> after tllm::tile_acts_kernel";
     if (c.height == 1) return c.splits > 1 ? "tllm::gemm_mfma_kernel<2>, K split" : "tllm::gemm_mfma_kernel<2>";
     return c.splits > 1 ? "tllm::gemm_mfma_kernel<1>, K split" : "tllm::gemm_mfma_kernel<1>";
@@ -1060,6 +1476,7 @@ const char *gemm_mfma_kernel_name(const Problem &p) {
 
 namespace {
 hipError_t launch_config(const Problem &p, const GemmConfig &c, float *workspace, unsigned *arrivals, hipStream_t s) {
+    if (c.rowsplit) return launch_rowsplit(p, c, workspace, arrivals, s);
     if (c.pingpong) return launch_pingpong(p, workspace, s);
     return c.height == 1 ? launch<2>(p, c.splits, workspace, arrivals, s) : launch<1>(p, c.splits, workspace, arrivals, s);
 }

@@ -62,6 +62,31 @@ def assert_close(oracle, got, ref, tol=TOL, what=""):
     assert rep["max_rel"] <= tol, f"{what}: {rep}"
 
 
+class gemm_forced:
+    """Forces the GEMM kernel choice through the environment switches the library reads at every call:
+    gemm_forced(pingpong=1), gemm_forced(rowsplit=1), gemm_forced(pingpong=0, rowsplit=0), gemm_forced() for the
+    library's own choice."""
+    NAMES = {"pingpong": "TLLM_GEMM_PINGPONG", "rowsplit": "TLLM_GEMM_ROWSPLIT"}
+
+    def __init__(self, **kw):
+        self.want = {self.NAMES[k]: str(v) for k, v in kw.items()}
+
+    def __enter__(self):
+        self.old = {n: os.environ.get(n) for n in self.NAMES.values()}
+        for n in self.NAMES.values():
+            os.environ.pop(n, None)
+        os.environ.update(self.want)
+        return self
+
+    def __exit__(self, *exc):
+        for n, v in self.old.items():
+            if v is None:
+                os.environ.pop(n, None)
+            else:
+                os.environ[n] = v
+        return False
+
+
 # -------------------------------------------------------------------- GEMV
 @pytest.mark.parametrize("rows,cols,seed", [
     (2048, 2048, 101),    # benchmark configuration 1 (LLaMA-1B q_proj)
@@ -249,20 +274,36 @@ def test_gemm_eight_wave_kernel_edges(dev, oracle, M, N, K):
     nz, sg, s, _ = synth.problem(M * 7 + N, N, K, dontcare_sign=True)
     A = synth.acts_f16(np.random.default_rng(M + K + 5), M, K)
     ref = oracle.gemm_f64(A.view(np.uint16), nz, sg, s.view(np.uint16))
-    old = os.environ.get("TLLM_GEMM_PINGPONG")
-    try:
-        os.environ["TLLM_GEMM_PINGPONG"] = "1"
+    with gemm_forced(pingpong=1, rowsplit=0):
         got = run_gemm(dev, A, nz, sg, s)
-        os.environ["TLLM_GEMM_PINGPONG"] = "0"
+    with gemm_forced(pingpong=0, rowsplit=0):
         other = run_gemm(dev, A, nz, sg, s)
-    finally:
-        if old is None:
-            os.environ.pop("TLLM_GEMM_PINGPONG", None)
-        else:
-            os.environ["TLLM_GEMM_PINGPONG"] = old
     assert_close(oracle, got, ref, what=f"eight-wave gemm {M}x{N}x{K}")
     assert_close(oracle, other, ref, what=f"four-wave gemm {M}x{N}x{K}")
     assert_close(oracle, got, other, tol=2e-3, what=f"eight-wave against four-wave {M}x{N}x{K}")
+
+
+@pytest.mark.parametrize("M,N,K", [(600, 300, 768), (33, 130, 256), (257, 1000, 1280), (100, 129, 512), (1023, 260, 512),
+                                   (128, 256, 256), (129, 257, 512), (16, 64, 256), (260, 300, 6144)])
+def test_gemm_row_split_kernel_edges(dev, oracle, M, N, K):
+    """The row-split kernel (chosen by itself for tall problems) forced onto shapes with ragged edges: M not a
+    multiple of 128 or of 16, N not a multiple of 256 or of 8 (the narrow store path), a single block of 256 columns,
+    tiles that are split along K (260 x 300 x 6144: six tiles in eight parts each). Against the fp64 oracle and against the
+    four-wave kernel."""
+    torch, tl = dev
+    nz, sg, s, _ = synth.problem(M * 5 + N + K, N, K, dontcare_sign=True)
+    A = synth.acts_f16(np.random.default_rng(M + K + 9), M, K)
+    ref = oracle.gemm_f64(A.view(np.uint16), nz, sg, s.view(np.uint16))
+    with gemm_forced(rowsplit=1):
+        assert "gemm_ns_kernel" in tl.gemm_kernel(M, N, K)
+        assert ("K split" in tl.gemm_kernel(M, N, K)) == (K == 6144)
+        got = run_gemm(dev, A, nz, sg, s)
+        again = run_gemm(dev, A, nz, sg, s)
+    with gemm_forced(pingpong=0, rowsplit=0):
+        other = run_gemm(dev, A, nz, sg, s)
+    assert_close(oracle, got, ref, what=f"row-split gemm {M}x{N}x{K}")
+    assert np.array_equal(got, again), "the row-split kernel must give the same bits on every call"
+    assert_close(oracle, got, other, tol=2e-3, what=f"row-split against four-wave {M}x{N}x{K}")
 
 
 @pytest.mark.parametrize("group,M", [(32, 3), (64, 20), (256, 5)])
@@ -1200,7 +1241,8 @@ def test_gemm_every_output_against_dense_product(dev, oracle, M, N, K):
     multiplied by the activations in fp32 (torch), which is itself checked against the fp64 oracle on sampled
     rows and columns. A fault confined to a few lanes and registers of one exchange step (1 output in 256)
     passes a sampled check more often than not; this test is the one that sees it. Each shape runs as the
-    library chooses and with the eight-wave kernel forced."""
+    library chooses, with the eight-wave kernel forced, with the row-split kernel forced and with the four-wave
+    kernels only."""
     torch, tl = dev
     gen = torch.Generator(device="cuda")
     gen.manual_seed(7000 + M + N + K)
@@ -1211,13 +1253,8 @@ def test_gemm_every_output_against_dense_product(dev, oracle, M, N, K):
     del W
     _check_sampled(oracle, torch, A, nz, sg, sc, ref, 4, 40, M + K, f"dense fp32 product {M}x{N}x{K}")
     tau = float(torch.sqrt(torch.mean(ref * ref)).item()) / 64.0
-    old = os.environ.get("TLLM_GEMM_PINGPONG")
-    try:
-        for force in (None, "1"):
-            if force is None:
-                os.environ.pop("TLLM_GEMM_PINGPONG", None)
-            else:
-                os.environ["TLLM_GEMM_PINGPONG"] = force
+    for force in ({}, {"pingpong": 1, "rowsplit": 0}, {"rowsplit": 1}, {"pingpong": 0, "rowsplit": 0}):
+        with gemm_forced(**force):
             for rep in range(2):
                 Cm = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
                 tl.ternary_gemm(A, nz, sg, sc, Cm, M, N, K, 128)
@@ -1226,11 +1263,6 @@ def test_gemm_every_output_against_dense_product(dev, oracle, M, N, K):
                 bad = int((~(rel <= TOL)).sum().item())
                 assert bad == 0, (f"gemm {M}x{N}x{K} ({tl.gemm_kernel(M, N, K)}, forced={force}, repetition {rep}): "
                                   f"{bad} of {M * N} outputs beyond {TOL}, max_rel {float(rel.max()):.3e}")
-    finally:
-        if old is None:
-            os.environ.pop("TLLM_GEMM_PINGPONG", None)
-        else:
-            os.environ["TLLM_GEMM_PINGPONG"] = old
 
 
 @pytest.mark.parametrize("batch", [1, 2, 4, 16])

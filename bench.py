@@ -289,17 +289,36 @@ def plan_rows(torch, tl, orc, timer, label, model, layers, batches, p_zero, lo, 
 
 def gemm_rows(torch, tl, orc, timer, seed, m_list, p_zero, calls, warm):
     """Prefill GEMM (cfg4): LLaMA-3-8B gate/up 14336x4096 and down 4096x14336, M tokens each; dense-equivalent
-    2*M*N*K flops against the FP16 matrix peak (M = 16 is HBM-bound and also gets its weight-stream rate)."""
+    2*M*N*K flops against the FP16 matrix peak (M = 16 is HBM-bound and also gets its weight-stream rate).
+    For M > 16 the same shape is also timed as a dense fp16 product of the vendor library (torch.matmul on a
+    dense fp16 matrix with the same value distribution: 42 % zeros, +-scale): what the matrix cores of this
+    box deliver on these operands when the weights need no decoding (`dense_fp16_us`, `vs_dense_fp16` =
+    that time / ours)."""
     gen = torch.Generator(device="cuda")
     gen.manual_seed(seed + 4)
     rows = []
     for (n, k) in ((14336, 4096), (4096, 14336)):
         nz, sg = gen_masks(torch, n, k, p_zero, gen)
         sc = (torch.rand((n, k // 128), device="cuda", generator=gen) * 0.02 + 0.01).to(torch.float16)
+        dense = None
+        if any(m > 16 for m in m_list):
+            dense = torch.empty((n, k), dtype=torch.float16, device="cuda")
+            step = max(1, (1 << 24) // k)
+            for r0 in range(0, n, step):
+                r1 = min(n, r0 + step)
+                u = torch.rand((r1 - r0, k), device="cuda", generator=gen)
+                w = torch.where(u < p_zero, 0.0, torch.where(u < (1.0 + p_zero) / 2, 1.0, -1.0))
+                dense[r0:r1] = (w * sc[r0:r1].float().repeat_interleave(128, dim=1)).to(torch.float16)
+                del u, w
         for m in m_list:
             a = torch.randn((m, k), device="cuda", generator=gen).to(torch.float16)
             c = torch.zeros((m, n), dtype=torch.float16, device="cuda")
             t = timer.run(lambda: tl.ternary_gemm(a, nz, sg, sc, c, m, n, k, 128), calls, warm)
+            t_dense = None
+            if dense is not None and m > 16:
+                cd = torch.empty((m, n), dtype=torch.float16, device="cuda")
+                t_dense = timer.run(lambda: torch.matmul(a, dense.t(), out=cd), calls, warm)
+                del cd
             rng = np.random.default_rng(m + n)
             ms_ = np.unique(rng.integers(0, m, 4))
             ns_ = np.unique(rng.integers(0, n, 96))
@@ -314,12 +333,17 @@ def gemm_rows(torch, tl, orc, timer, seed, m_list, p_zero, calls, warm):
                    "tflops": round(tflops, 1), "tflops_best": round(2.0 * m * n * k / (t["min_ms"] * 1e-3) / 1e12, 1),
                    "bound": "mfma" if m > 16 else "hbm", "frac_mfma_peak": round(tflops / MFMA_F16_PEAK_TFLOPS, 4),
                    "kernel": tl.gemm_kernel(m, n, k), "max_rel_sampled": rel}
+            if t_dense is not None:
+                row["dense_fp16_us"] = round(t_dense["mean_ms"] * 1e3, 2)
+                row["dense_fp16_tflops"] = round(2.0 * m * n * k / (t_dense["mean_ms"] * 1e-3) / 1e12, 1)
+                row["vs_dense_fp16"] = round(t_dense["mean_ms"] / t["mean_ms"], 3)
             if m <= 16:
                 gb = packed_bytes(n, k) / (t["mean_ms"] * 1e-3) / 1e9
                 row["GBps"] = round(gb, 1)
                 row["frac_hbm_peak"] = round(gb / HBM_PEAK_GBS, 4)
             rows.append(row)
             del a, c, full
+        del dense
         del nz, sg, sc
     return rows
 
@@ -628,7 +652,8 @@ def main():
                 agg = sum(2.0 * c["M"] * c["N"] * c["K"] for c in m512) / sum(c["us"] for c in m512) / 1e6
                 out["gemm_m512"] = {"tflops_both_shapes": round(agg, 1), "frac_mfma_peak": round(agg / MFMA_F16_PEAK_TFLOPS, 4),
                                     "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s (2*M*N*K)",
-                                    "per_shape": [{k: c[k] for k in ("N", "K", "us", "tflops", "frac_mfma_peak")} for c in m512]}
+                                    "per_shape": [{k: c[k] for k in ("N", "K", "us", "tflops", "frac_mfma_peak", "kernel", "dense_fp16_us", "vs_dense_fp16")
+                                                   if k in c} for c in m512]}
         if not args.no_single_calls and headline:
             out["single_calls"] = single_call_rows(torch, tl, timer, problems, "llama8b", 32)
         if 5 in want:

@@ -848,11 +848,11 @@ __global__ __launch_bounds__(kPpThreads, 1) void gemm_pp_kernel(
     }
 }
 
-// ---- The row-split kernel: eight waves that split the weight rows, weights decoded straight into MFMA operand
+// ---- The row-split kernel: the waves of a workgroup split the weight rows, weights decoded straight into MFMA operand
 // registers.
 //
-// A workgroup computes 256 weight rows x 32 MF activation rows; wave w owns weight rows 32 w .. 32 w + 31 (one A-operand
-// fragment) and all the activation rows (MF accumulator fragments). What this changes against the kernels above:
+// A workgroup computes 256 weight rows x 32 MF activation rows; a wave owns NF A-operand fragments of 32 weight rows and
+// all the activation rows (NF x MF accumulator fragments). What this changes against the kernels above:
 //   * decoded weights never pass through LDS (its write port was the slowest unit of those kernels): lane (li, lq) of wave
 //     w loads the mask words of its own row, and the byte of a word IS the eight weights of one MFMA operand: one
 //     v_perm puts byte t of the even-weight and odd-weight codes into the two halves of a dword, then a packed shift,
@@ -871,18 +871,24 @@ __global__ __launch_bounds__(kPpThreads, 1) void gemm_pp_kernel(
 // Tiles that do not fill the last round of workgroups over the CUs are split along K between several workgroups
 // (`splits`), which exchange fp32 sums through memory like the kernels above; the tiles before them (`full_tiles`)
 // run whole. The workgroups of one XCD take consecutive work items of both kinds.
+//
+// Two shapes of workgroup compute the same 256 x 128 tile. NF = 1: eight waves (two per SIMD) with one weight fragment
+// each: one workgroup per CU, the fastest when there are not enough tiles for two workgroups per CU. NF = 2: four waves
+// (one per SIMD) with two weight fragments each, so that every activation fragment read from LDS feeds two MFMAs, and
+// two workgroups per CU: the waves that share a SIMD then belong to different workgroups and do not wait for each
+// other at barriers, and one workgroup's first loads and last stores hide behind the other's MFMAs.
 constexpr int kNsBN = 256;
-constexpr int kNsThreads = 512;
 constexpr int kNsPitch = 2 * kNsBN + 16;  // bytes per activation row of the output tile in LDS
 
-template <int MF>
-__global__ __launch_bounds__(kNsThreads, 1) void gemm_ns_kernel(
+template <int MF, int NF>
+__global__ __launch_bounds__(512 / NF) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_ns_kernel(
     const uint16_t *__restrict__ A, const uint32_t *__restrict__ nzB, const uint32_t *__restrict__ sgB,
     const uint16_t *__restrict__ scB, uint16_t *__restrict__ C, int M, int N, int K, int full_tiles, int splits,
     float *__restrict__ partial, unsigned *__restrict__ arrivals) {
     constexpr int BM = 32 * MF;
-    constexpr int kChunk = 4 * MF * 1024;  // bytes of one chunk: four steps of MF fragments
-    constexpr int kDma = MF / 2;           // 1 KB pieces per wave and chunk
+    constexpr int kWaves = 8 / NF, kNsThreads = 64 * kWaves;
+    constexpr int kChunk = 4 * MF * 1024;    // bytes of one chunk: four steps of MF fragments
+    constexpr int kDma = MF * 4 / kWaves;    // 1 KB pieces per wave and chunk
     static_assert(MF == 4, "the ring of four chunks is addressed with 16-bit offsets: 4 x 16 KB");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     typedef __attribute__((address_space(3))) unsigned char LB;
@@ -918,10 +924,15 @@ __global__ __launch_bounds__(kNsThreads, 1) void gemm_ns_kernel(
     const int b_begin = is_split ? (int)((long)blocks * split / splits) : 0;
     const int b_end = is_split ? (int)((long)blocks * (split + 1) / splits) : blocks;
 
-    const int row = min(n0 + 32 * wave + li, N - 1);
-    GB *nz_g = (GB *)nzB + ((size_t)row * words + 4 * lq) * 4;
-    GB *sg_g = (GB *)sgB + ((size_t)row * words + 4 * lq) * 4;
-    GB *sc_g = (GB *)scB + (size_t)row * groups * 2;  // two scales per block: one aligned dword (groups is even)
+    // fragment f of wave w: weight rows n0 + 32 (NF w + f) .. + 31
+    GB *nz_g[NF], *sg_g[NF], *sc_g[NF];
+#pragma unroll
+    for (int f = 0; f < NF; f++) {
+        const int row = min(n0 + 32 * (NF * wave + f) + li, N - 1);
+        nz_g[f] = (GB *)nzB + ((size_t)row * words + 4 * lq) * 4;
+        sg_g[f] = (GB *)sgB + ((size_t)row * words + 4 * lq) * 4;
+        sc_g[f] = (GB *)scB + (size_t)row * groups * 2;  // two scales per block: one aligned dword (groups is even)
+    }
 
     // activation pieces this wave copies per chunk: piece p = wave * kDma + i covers fragment j = p / 4, rows
     // 16 h .. 16 h + 15 of it (h = (p / 2) % 2), column half q = p % 2; lane L of the copy fetches step L / 16 of row
@@ -949,66 +960,78 @@ __global__ __launch_bounds__(kNsThreads, 1) void gemm_ns_kernel(
         for (int i = 0; i < kDma; i++)
             __builtin_amdgcn_global_load_lds(TLLM_GPTR(a_src[i] + off), TLLM_LPTR(lds_l + slot * kChunk + a_dst[i]), 16, 0, 0);
     };
-    u4 nx_nz = {0u, 0u, 0u, 0u}, nx_sg = {0u, 0u, 0u, 0u};
-    uint32_t nx_sc = 0;
+    u4 nx_nz[NF], nx_sg[NF];
+    uint32_t nx_sc[NF];
+#pragma unroll
+    for (int f = 0; f < NF; f++) {
+        nx_nz[f] = u4{0u, 0u, 0u, 0u};
+        nx_sg[f] = u4{0u, 0u, 0u, 0u};
+        nx_sc[f] = 0;
+    }
     auto load_masks = [&](int b) {
         const int bb = min(b, blocks - 1);
-        GB *p0 = nz_g + (size_t)bb * 32;
-        GB *p1 = sg_g + (size_t)bb * 32;
-        GB *p2 = sc_g + (size_t)bb * 4;
-        asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(nx_nz) : "v"(p0) : "memory");
-        asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(nx_sg) : "v"(p1) : "memory");
-        asm volatile("global_load_dword %0, %1, off" : "+v"(nx_sc) : "v"(p2) : "memory");
+#pragma unroll
+        for (int f = 0; f < NF; f++) {
+            GB *p0 = nz_g[f] + (size_t)bb * 32;
+            GB *p1 = sg_g[f] + (size_t)bb * 32;
+            GB *p2 = sc_g[f] + (size_t)bb * 4;
+            asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(nx_nz[f]) : "v"(p0) : "memory");
+            asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(nx_sg[f]) : "v"(p1) : "memory");
+            asm volatile("global_load_dword %0, %1, off" : "+v"(nx_sc[f]) : "v"(p2) : "memory");
+        }
     };
 
-    f16v acc[MF];
+    f16v acc[NF][MF];
 #pragma unroll
-    for (int j = 0; j < MF; j++)
+    for (int f = 0; f < NF; f++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) acc[j][r] = 0.f;
+        for (int j = 0; j < MF; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[f][j][r] = 0.f;
 
-    uint32_t cu_nz[4], cu_sg[4];  // mask word 2 u + lq of the current block
-    h2 sp2[2];                    // its two scales, each in both halves
+    uint32_t cu_nz[NF][4], cu_sg[NF][4];  // mask word 2 u + lq of the current block
+    h2 sp2[NF][2];                        // its two scales, each in both halves
     u4 Bv[2][MF];
 #pragma unroll
     for (int q = 0; q < 2; q++)
 #pragma unroll
         for (int j = 0; j < MF; j++) Bv[q][j] = u4{0u, 0u, 0u, 0u};
-    u4 av[2];
-    uint32_t t0 = 0, t1 = 0, qn = 0;
-    h2 sp = {};
-    auto codes = [&](int u) {  // the two-bit codes (negative, non-zero) of mask word u: even weights in t0, odd weights in t1
-        const uint32_t m_nz = cu_nz[u], m_sg = cu_sg[u];
-        sp = sp2[u >> 1];
+    u4 av[2][NF];
+    uint32_t t0[NF] = {}, t1[NF] = {}, qn[NF] = {};
+    h2 sp[NF] = {};
+    auto codes = [&](int f, int u) {  // the two-bit codes (negative, non-zero) of mask word u: even weights in t0, odd weights in t1
+        const uint32_t m_nz = cu_nz[f][u], m_sg = cu_sg[f][u];
+        sp[f] = sp2[f][u >> 1];
         const uint32_t neg = m_nz & ~m_sg;
-        t0 = __builtin_amdgcn_bitop3_b32(neg << 1, m_nz, 0xAAAAAAAAu, 0xE4);
-        t1 = __builtin_amdgcn_bitop3_b32(neg, m_nz >> 1, 0xAAAAAAAAu, 0xE4);
+        t0[f] = __builtin_amdgcn_bitop3_b32(neg << 1, m_nz, 0xAAAAAAAAu, 0xE4);
+        t1[f] = __builtin_amdgcn_bitop3_b32(neg, m_nz >> 1, 0xAAAAAAAAu, 0xE4);
     };
-    auto pick = [&](int t) {  // byte t of the even codes into the low half, of the odd codes into the high half
-        qn = __builtin_amdgcn_perm(t1, t0, 0x0C000C00u | (uint32_t)t | ((uint32_t)(4 + t) << 16));
+    auto pick = [&](int f, int t) {  // byte t of the even codes into the low half, of the odd codes into the high half
+        qn[f] = __builtin_amdgcn_perm(t1[f], t0[f], 0x0C000C00u | (uint32_t)t | ((uint32_t)(4 + t) << 16));
     };
-    auto pair = [&](int e) -> uint32_t {  // weights 2 e, 2 e + 1 of the byte as +-2 scale / 0
-        us2 v = __builtin_bit_cast(us2, qn);
+    auto pair = [&](int f, int e) -> uint32_t {  // weights 2 e, 2 e + 1 of the byte as +-2 scale / 0
+        us2 v = __builtin_bit_cast(us2, qn[f]);
         v = v << (uint16_t)(14 - 2 * e);
         uint32_t top = __builtin_bit_cast(uint32_t, v);
         if (e > 0) top &= 0xC000C000u;  // (for e = 0 the shift leaves nothing below the field)
-        return __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, top) * sp);
+        return __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, top) * sp[f]);
     };
     auto take_masks = [&]() {  // the loads into nx_* are complete where this is called
-        asm volatile("" : "+v"(nx_nz), "+v"(nx_sg), "+v"(nx_sc));
-        // v_permlane32_swap(a, b): a keeps its lower half-wave and takes b's lower half-wave as its upper one; b takes
-        // a's upper half-wave as its lower one and keeps its upper one
-        const auto s01 = __builtin_amdgcn_permlane32_swap(nx_nz[0], nx_nz[1], false, false);
-        const auto s23 = __builtin_amdgcn_permlane32_swap(nx_nz[2], nx_nz[3], false, false);
-        const auto g01 = __builtin_amdgcn_permlane32_swap(nx_sg[0], nx_sg[1], false, false);
-        const auto g23 = __builtin_amdgcn_permlane32_swap(nx_sg[2], nx_sg[3], false, false);
-        cu_nz[0] = s01[0]; cu_nz[2] = s01[1]; cu_nz[1] = s23[0]; cu_nz[3] = s23[1];
-        cu_sg[0] = g01[0]; cu_sg[2] = g01[1]; cu_sg[1] = g23[0]; cu_sg[3] = g23[1];
-        sp2[0] = __builtin_bit_cast(h2, __builtin_amdgcn_perm(nx_sc, nx_sc, 0x01000100u));
-        sp2[1] = __builtin_bit_cast(h2, __builtin_amdgcn_perm(nx_sc, nx_sc, 0x03020302u));
 #pragma unroll
-        for (int u = 0; u < 4; u++) asm volatile("" : "+v"(cu_nz[u]), "+v"(cu_sg[u]));
-        asm volatile("" : "+v"(sp2[0]), "+v"(sp2[1]));
+        for (int f = 0; f < NF; f++) {
+            asm volatile("" : "+v"(nx_nz[f]), "+v"(nx_sg[f]), "+v"(nx_sc[f]));
+            const auto s01 = __builtin_amdgcn_permlane32_swap(nx_nz[f][0], nx_nz[f][1], false, false);
+            const auto s23 = __builtin_amdgcn_permlane32_swap(nx_nz[f][2], nx_nz[f][3], false, false);
+            const auto g01 = __builtin_amdgcn_permlane32_swap(nx_sg[f][0], nx_sg[f][1], false, false);
+            const auto g23 = __builtin_amdgcn_permlane32_swap(nx_sg[f][2], nx_sg[f][3], false, false);
+            cu_nz[f][0] = s01[0]; cu_nz[f][2] = s01[1]; cu_nz[f][1] = s23[0]; cu_nz[f][3] = s23[1];
+            cu_sg[f][0] = g01[0]; cu_sg[f][2] = g01[1]; cu_sg[f][1] = g23[0]; cu_sg[f][3] = g23[1];
+            sp2[f][0] = __builtin_bit_cast(h2, __builtin_amdgcn_perm(nx_sc[f], nx_sc[f], 0x01000100u));
+            sp2[f][1] = __builtin_bit_cast(h2, __builtin_amdgcn_perm(nx_sc[f], nx_sc[f], 0x03020302u));
+#pragma unroll
+            for (int u = 0; u < 4; u++) asm volatile("" : "+v"(cu_nz[f][u]), "+v"(cu_sg[f][u]));
+            asm volatile("" : "+v"(sp2[f][0]), "+v"(sp2[f][1]));
+        }
     };
 
     // ---- prologue: masks of the first two blocks, the first four chunks; operands of the first step.
@@ -1028,9 +1051,12 @@ __global__ __launch_bounds__(kNsThreads, 1) void gemm_ns_kernel(
     TLLM_FENCE();
 #pragma unroll
     for (int j = 0; j < MF; j++) TLLM_LDS_READ128(Bv[0][j], b_rd, j * 4096);
-    codes(0);
-    pick(0);
-    av[0] = u4{pair(0), pair(1), pair(2), pair(3)};
+#pragma unroll
+    for (int f = 0; f < NF; f++) {
+        codes(f, 0);
+        pick(f, 0);
+        av[0][f] = u4{pair(f, 0), pair(f, 1), pair(f, 2), pair(f, 3)};
+    }
     TLLM_FENCE();
 
     // One step: the MFMAs of step s = (chunk c in ring slot u, t) with the decode of step s + 1 between them; the
@@ -1045,7 +1071,7 @@ __global__ __launch_bounds__(kNsThreads, 1) void gemm_ns_kernel(
         constexpr int ru = t == 3 ? ((u + 1) & 3) : u, rt = (t + 1) & 3;
         if (t == 3) {
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            if (u < 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kDma + 3) : "memory");
+            if (u < 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kDma + 3 * NF) : "memory");
             else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kDma) : "memory");
             __builtin_amdgcn_s_barrier();
             TLLM_FENCE();
@@ -1061,22 +1087,26 @@ __global__ __launch_bounds__(kNsThreads, 1) void gemm_ns_kernel(
         if (t != 3) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(MF) : "memory");
         TLLM_FENCE();
         u4(&R)[MF] = Bv[cur];
-        u4 &a_cur = av[cur];
-        uint32_t an[4];
+        u4(&a_cur)[NF] = av[cur];
+        uint32_t an[NF][4];
 #pragma unroll
-        for (int j = 0; j < MF; j++) {
-            asm volatile("" : "+v"(R[j]));
-            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, a_cur), __builtin_bit_cast(h8, R[j]), acc[j], 0, 0, 0);
-            TLLM_FENCE();
-            if (j == 0) {
-                if (t == 3) codes(ru);
-                pick(rt);
+        for (int f = 0; f < NF; f++)
+#pragma unroll
+            for (int j = 0; j < MF; j++) {
+                if (f == 0) asm volatile("" : "+v"(R[j]));
+                acc[f][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, a_cur[f]), __builtin_bit_cast(h8, R[j]), acc[f][j], 0, 0, 0);
+                TLLM_FENCE();
+                // the decode of fragment f of step s + 1 behind the MFMAs of fragment f
+                if (j == 0) {
+                    if (t == 3) codes(f, ru);
+                    pick(f, rt);
+                }
+                an[f][j] = pair(f, j);
+                asm volatile("" : "+v"(an[f][j]));  // computed here, between the MFMAs, not where it is used
+                TLLM_FENCE();
             }
-            an[j] = pair(j);
-            asm volatile("" : "+v"(an[j]));  // computed here, between the MFMAs, not where it is used
-            TLLM_FENCE();
-        }
-        av[nxt] = u4{an[0], an[1], an[2], an[3]};
+#pragma unroll
+        for (int f = 0; f < NF; f++) av[nxt][f] = u4{an[f][0], an[f][1], an[f][2], an[f][3]};
     };
     std::integral_constant<int, 0> i0;
     std::integral_constant<int, 1> i1;
@@ -1100,18 +1130,20 @@ __global__ __launch_bounds__(kNsThreads, 1) void gemm_ns_kernel(
 #undef TLLM_LPTR
 
     if (is_split) {
-        // fp32 sums of this part into its slot (element (j, g, tid, e) at ((j * 4 + g) * 512 + tid) * 4 + e), written
-        // through to memory; the last part of a tile to arrive adds all slots in part order, its own sums from its
-        // registers in their place of that order
+        // fp32 sums of this part into its slot (quad g of fragment (f, j) of thread tid at
+        // (((f * MF + j) * 4 + g) * threads + tid) * 4), written through to memory; the last part of a tile to arrive adds
+        // all slots in part order, its own included (read back: a second register set for its own sums would not fit),
+        // so the bits do not depend on which part arrives last
         constexpr int kSlot = BM * kNsBN;
         const int st = tile - full_tiles;
         float *mine = partial + ((size_t)st * splits + split) * kSlot + tid * 4;
 #pragma unroll
-        for (int j = 0; j < MF; j++)
+        for (int fj = 0; fj < NF * MF; fj++)
 #pragma unroll
             for (int g = 0; g < 4; g++) {
-                const f4 v = {acc[j][4 * g], acc[j][4 * g + 1], acc[j][4 * g + 2], acc[j][4 * g + 3]};
-                float *dst = mine + (size_t)(j * 4 + g) * kNsThreads * 4;
+                const f16v &a = acc[fj / MF][fj % MF];
+                const f4 v = {a[4 * g], a[4 * g + 1], a[4 * g + 2], a[4 * g + 3]};
+                float *dst = mine + (size_t)(fj * 4 + g) * kNsThreads * 4;
                 // (two idle issue slots: a store of more than 8 bytes still reads its data registers after it has issued)
                 asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(dst), "v"(v) : "memory");
             }
@@ -1127,69 +1159,64 @@ __global__ __launch_bounds__(kNsThreads, 1) void gemm_ns_kernel(
         if (!last_arrival_ns) return;
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
         const float *slots = partial + (size_t)st * splits * kSlot + tid * 4;
-        f16v own[MF];
 #pragma unroll
-        for (int j = 0; j < MF; j++) {
-            own[j] = acc[j];
+        for (int fj = 0; fj < NF * MF; fj++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) acc[j][r] = 0.f;
-        }
+            for (int r = 0; r < 16; r++) acc[fj / MF][fj % MF][r] = 0.f;
         for (int q = 0; q < splits; q++) {
-            if (q == split) {
-#pragma unroll
-                for (int j = 0; j < MF; j++) acc[j] += own[j];
-                continue;
-            }
             const float *slot = slots + (size_t)q * kSlot;
 #pragma unroll
-            for (int j = 0; j < MF; j++) {
+            for (int fj = 0; fj < NF * MF; fj++) {
                 f4 v[4];
 #pragma unroll
-                for (int g = 0; g < 4; g++) v[g] = *reinterpret_cast<const f4 *>(slot + (size_t)(j * 4 + g) * kNsThreads * 4);
+                for (int g = 0; g < 4; g++) v[g] = *reinterpret_cast<const f4 *>(slot + (size_t)(fj * 4 + g) * kNsThreads * 4);
+                f16v &a = acc[fj / MF][fj % MF];
 #pragma unroll
                 for (int g = 0; g < 4; g++)
 #pragma unroll
-                    for (int e = 0; e < 4; e++) acc[j][4 * g + e] += v[g][e];
+                    for (int e = 0; e < 4; e++) a[4 * g + e] += v[g][e];
             }
         }
     }
 
-    // ---- store. Register 4 g + v of fragment j is weight row n0 + 32 wave + 8 g + 4 lq + v for activation row
+    // ---- store. Register 4 g + v of fragment (f, j) is weight row n0 + 32 (NF wave + f) + 8 g + 4 lq + v for activation row
     // m0 + 32 j + li: stored as they are these are 8-byte pieces in 32 different lines per instruction. The tile goes
     // through LDS instead (the ring is free now) and leaves as whole 512-byte rows, two rows per instruction.
     const bool wide_store = (N & 7) == 0 && (reinterpret_cast<uintptr_t>(C) & 15) == 0;
     if (wide_store) {
         __syncthreads();  // every wave is done with the ring
 #pragma unroll
-        for (int j = 0; j < MF; j++)
+        for (int fj = 0; fj < NF * MF; fj++)
 #pragma unroll
             for (int g = 0; g < 4; g++) {
+                const int f = fj / MF, j = fj % MF;
                 uint16_t hv[4];
 #pragma unroll
-                for (int v = 0; v < 4; v++) hv[v] = f2h(acc[j][4 * g + v] * 0.5f);
-                *reinterpret_cast<uint2 *>(lds + (32 * j + li) * kNsPitch + (32 * wave + 8 * g + 4 * lq) * 2) =
+                for (int v = 0; v < 4; v++) hv[v] = f2h(acc[f][j][4 * g + v] * 0.5f);
+                *reinterpret_cast<uint2 *>(lds + (32 * j + li) * kNsPitch + (32 * (NF * wave + f) + 8 * g + 4 * lq) * 2) =
                     uint2{(uint32_t)hv[0] | ((uint32_t)hv[1] << 16), (uint32_t)hv[2] | ((uint32_t)hv[3] << 16)};
             }
         __syncthreads();
         const int piece = lane & 31;
         const int n = n0 + piece * 8;
 #pragma unroll
-        for (int r = 0; r < BM / 16; r++) {
-            const int ml = wave * (BM / 8) + 2 * r + lq;
+        for (int r = 0; r < BM / (2 * kWaves); r++) {
+            const int ml = wave * (BM / kWaves) + 2 * r + lq;
             const int m = m0 + ml;
             if (m < M && n < N) *reinterpret_cast<u4 *>(C + (size_t)m * N + n) = *reinterpret_cast<const u4 *>(lds + ml * kNsPitch + piece * 16);
         }
     } else {
 #pragma unroll
-        for (int j = 0; j < MF; j++) {
+        for (int fj = 0; fj < NF * MF; fj++) {
+            const int f = fj / MF, j = fj % MF;
             const int m = m0 + j * 32 + li;
             if (m >= M) continue;
 #pragma unroll
             for (int g = 0; g < 4; g++) {
-                const int n = n0 + 32 * wave + 8 * g + 4 * lq;
+                const int n = n0 + 32 * (NF * wave + f) + 8 * g + 4 * lq;
 #pragma unroll
                 for (int v = 0; v < 4; v++)
-                    if (n + v < N) C[(size_t)m * N + n + v] = f2h(acc[j][4 * g + v] * 0.5f);
+                    if (n + v < N) C[(size_t)m * N + n + v] = f2h(acc[f][j][4 * g + v] * 0.5f);
             }
         }
     }
@@ -1281,6 +1308,7 @@ struct GemmConfig {
     float us;     // estimated time
     bool rowsplit = false;  // the row-split kernel (256 weight rows x 128 activation rows per workgroup)
     int full_tiles = 0;     // row-split kernel: tiles computed by one workgroup each
+    int frags = 1;          // row-split kernel: weight fragments per wave (1: eight waves, one workgroup per CU; 2: four waves, two per CU)
 };
 GemmConfig choose_config(const Problem &p, size_t workspace_floats);
 
@@ -1348,8 +1376,9 @@ hipError_t launch_pingpong(const Problem &p, float *workspace, hipStream_t s) {
     return hipGetLastError();
 }
 
+template <int NF>
 hipError_t launch_rowsplit(const Problem &p, const GemmConfig &c, float *partial, unsigned *arrivals, hipStream_t s) {
-    constexpr int MF = 4, BM = 32 * MF;
+    constexpr int MF = 4, BM = 32 * MF, kNsThreads = 512 / NF;
     static std::mutex attr_mutex;
     static bool attr_set[64] = {};
     int dev = 0;
@@ -1360,7 +1389,7 @@ hipError_t launch_rowsplit(const Problem &p, const GemmConfig &c, float *partial
     if (dev >= 0 && dev < 64) {
         std::lock_guard<std::mutex> lock(attr_mutex);
         if (!attr_set[dev]) {
-            if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_ns_kernel<MF>),
+            if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_ns_kernel<MF, NF>),
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
                 return e;
             attr_set[dev] = true;
@@ -1369,7 +1398,7 @@ hipError_t launch_rowsplit(const Problem &p, const GemmConfig &c, float *partial
     const int tiles = ((p.batch + BM - 1) / BM) * ((p.rows + kNsBN - 1) / kNsBN);
     const int parts = (tiles - c.full_tiles) * c.splits;
     const int wgs = 8 * ((c.full_tiles + 7) / 8 + (parts + 7) / 8);
-    gemm_ns_kernel<MF><<<wgs, kNsThreads, lds, s>>>(p.x, p.nz, p.sg, p.scales, p.y, p.batch, p.rows, p.cols, c.full_tiles,
+    gemm_ns_kernel<MF, NF><<<wgs, kNsThreads, lds, s>>>(p.x, p.nz, p.sg, p.scales, p.y, p.batch, p.rows, p.cols, c.full_tiles,
                                                     c.splits, partial, arrivals);
     return hipGetLastError();
 }
@@ -1427,11 +1456,11 @@ GemmConfig choose_config(const Problem &p, size_t limit_floats) {
     // CUs are split along K (at most as far as the CUs reach, two blocks per part at least, and while the slots fit the
     // workspace) when that is cheaper than a last round of whole tiles; an exchange costs about 6 us + 1.5 us per part
     // (fitted to 4096 x 14336 at M = 128 ... 512). Tiles are 128 activation rows high: not for fewer than 96.
-    const char *env_rs = getenv("TLLM_GEMM_ROWSPLIT");  // 0: never, 1: whenever the shape allows (read at every call)
+    const char *env_rs = getenv("TLLM_GEMM_ROWSPLIT");  // 0: never, 1 / 2: whenever the shape allows, in its eight-wave / four-wave form (read at every call)
     const int forced_rs = env_rs ? atoi(env_rs) : -1;
     const bool rs_ok = p.cols % 256 == 0 && !((reinterpret_cast<uintptr_t>(p.x) | reinterpret_cast<uintptr_t>(p.nz) |
                                                 reinterpret_cast<uintptr_t>(p.sg)) & 15);
-    if (forced_rs != 0 && rs_ok && forced != 1 && (forced_rs == 1 || p.batch >= 96)) {
+    if (forced_rs != 0 && rs_ok && forced != 1 && (forced_rs >= 1 || p.batch >= 96)) {
         const int blocks = p.cols / 256;
         const int tiles = ((p.batch + 127) / 128) * ((p.rows + kNsBN - 1) / kNsBN);
         const float block_us = 3.3f, fixed_us = 9.0f;
@@ -1456,7 +1485,18 @@ GemmConfig choose_config(const Problem &p, size_t limit_floats) {
                 }
             }
         }
-        if (forced_rs == 1 || rs.us < best.us) best = rs;
+        // Two workgroups of four waves per CU: a workgroup alone on its CU takes 3.7 us per block, two together 5.3 us
+        // each; pays when there are more tiles than CUs. (No K split in this form.) TLLM_GEMM_ROWSPLIT=2 forces it.
+        if (tiles > n_cu || forced_rs == 2) {
+            const int slots = 2 * n_cu, last = tiles % slots;
+            GemmConfig two = rs;
+            two.frags = 2;
+            two.splits = 1;
+            two.full_tiles = tiles;
+            two.us = (float)(tiles / slots) * (float)blocks * 5.3f + (last > n_cu ? 5.3f : last > 0 ? 3.7f : 0.f) * (float)blocks + fixed_us;
+            if (forced_rs == 2 || (forced_rs != 1 && two.us < rs.us)) rs = two;
+        }
+        if (forced_rs >= 1 || rs.us < best.us) best = rs;
     }
     return best;
 }
@@ -1468,7 +1508,8 @@ float gemm_mfma_cost_us(const Problem &p) { return choose_config(p, kStaticSlotF
 
 const char *gemm_mfma_kernel_name(const Problem &p) {
     const GemmConfig c = choose_config(p, kStaticSlotFloats);
-    if (c.rowsplit) return c.splits > 1 ? "tllm::gemm_ns_kernel<4>, last tiles K split" : "tllm::gemm_ns_kernel<4>";
+    if (c.rowsplit && c.frags == 2) return "tllm::gemm_ns_kernel<4, 2>";
+    if (c.rowsplit) return c.splits > 1 ? "tllm::gemm_ns_kernel<4, 1>, last tiles K split" : "tllm::gemm_ns_kernel<4, 1>";
     if (c.pingpong) return "tllm::gemm_pp_kernel<2> after tllm::tile_acts_kernel";
     if (c.height == 1) return c.splits > 1 ? "tllm::gemm_mfma_kernel<2>, K split" : "tllm::gemm_mfma_kernel<2>";
     return c.splits > 1 ? "tllm::gemm_mfma_kernel<1>, K split" : "tllm::gemm_mfma_kernel<1>";
@@ -1476,7 +1517,7 @@ const char *gemm_mfma_kernel_name(const Problem &p) {
 
 namespace {
 hipError_t launch_config(const Problem &p, const GemmConfig &c, float *workspace, unsigned *arrivals, hipStream_t s) {
-    if (c.rowsplit) return launch_rowsplit(p, c, workspace, arrivals, s);
+    if (c.rowsplit) return c.frags == 2 ? launch_rowsplit<2>(p, c, workspace, arrivals, s) : launch_rowsplit<1>(p, c, workspace, arrivals, s);
     if (c.pingpong) return launch_pingpong(p, workspace, s);
     return c.height == 1 ? launch<2>(p, c.splits, workspace, arrivals, s) : launch<1>(p, c.splits, workspace, arrivals, s);
 }

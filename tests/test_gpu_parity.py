@@ -294,16 +294,18 @@ def test_gemm_row_split_kernel_edges(dev, oracle, M, N, K):
     nz, sg, s, _ = synth.problem(M * 5 + N + K, N, K, dontcare_sign=True)
     A = synth.acts_f16(np.random.default_rng(M + K + 9), M, K)
     ref = oracle.gemm_f64(A.view(np.uint16), nz, sg, s.view(np.uint16))
-    with gemm_forced(rowsplit=1):
-        assert "gemm_ns_kernel" in tl.gemm_kernel(M, N, K)
-        assert ("K split" in tl.gemm_kernel(M, N, K)) == (K == 6144)
-        got = run_gemm(dev, A, nz, sg, s)
-        again = run_gemm(dev, A, nz, sg, s)
     with gemm_forced(pingpong=0, rowsplit=0):
         other = run_gemm(dev, A, nz, sg, s)
-    assert_close(oracle, got, ref, what=f"row-split gemm {M}x{N}x{K}")
-    assert np.array_equal(got, again), "the row-split kernel must give the same bits on every call"
-    assert_close(oracle, got, other, tol=2e-3, what=f"row-split against four-wave {M}x{N}x{K}")
+    for form in (1, 2):  # eight waves with one weight fragment each / four waves with two
+        with gemm_forced(rowsplit=form):
+            name = tl.gemm_kernel(M, N, K)
+            assert f"gemm_ns_kernel<4, {form}>" in name
+            assert ("K split" in name) == (K == 6144 and form == 1)
+            got = run_gemm(dev, A, nz, sg, s)
+            again = run_gemm(dev, A, nz, sg, s)
+        assert_close(oracle, got, ref, what=f"row-split gemm, form {form}, {M}x{N}x{K}")
+        assert np.array_equal(got, again), "the row-split kernel must give the same bits on every call"
+        assert_close(oracle, got, other, tol=2e-3, what=f"row-split form {form} against four-wave {M}x{N}x{K}")
 
 
 @pytest.mark.parametrize("group,M", [(32, 3), (64, 20), (256, 5)])
@@ -1241,8 +1243,8 @@ def test_gemm_every_output_against_dense_product(dev, oracle, M, N, K):
     multiplied by the activations in fp32 (torch), which is itself checked against the fp64 oracle on sampled
     rows and columns. A fault confined to a few lanes and registers of one exchange step (1 output in 256)
     passes a sampled check more often than not; this test is the one that sees it. Each shape runs as the
-    library chooses, with the eight-wave kernel forced, with the row-split kernel forced and with the four-wave
-    kernels only."""
+    library chooses, with the eight-wave kernel forced, with the row-split kernel forced in both its forms and with
+    the four-wave kernels only."""
     torch, tl = dev
     gen = torch.Generator(device="cuda")
     gen.manual_seed(7000 + M + N + K)
@@ -1253,7 +1255,7 @@ def test_gemm_every_output_against_dense_product(dev, oracle, M, N, K):
     del W
     _check_sampled(oracle, torch, A, nz, sg, sc, ref, 4, 40, M + K, f"dense fp32 product {M}x{N}x{K}")
     tau = float(torch.sqrt(torch.mean(ref * ref)).item()) / 64.0
-    for force in ({}, {"pingpong": 1, "rowsplit": 0}, {"rowsplit": 1}, {"pingpong": 0, "rowsplit": 0}):
+    for force in ({}, {"pingpong": 1, "rowsplit": 0}, {"rowsplit": 1}, {"rowsplit": 2}, {"pingpong": 0, "rowsplit": 0}):
         with gemm_forced(**force):
             for rep in range(2):
                 Cm = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")

@@ -99,11 +99,11 @@ int tllm_quantize_absmax_i8(const uint16_t *input, int8_t *output, float *scale,
  * Replaces ternary::ternary_gemm, reference include/kernels.cuh:37-40
  * (kernels/ternary_gemm.cu:33-195). Any M >= 1 is accepted.
  * Allocation: none per call, with one exception: a workspace that belongs to (device, stream). Two kinds
- * of shapes use it. Shapes with few weight tiles (M > 16 and N * M small against the chip) split K over
- * several workgroups per tile, which exchange fp32 partial sums through it; tall shapes (M of about 512 and
- * more on wide matrices) run a kernel that reads the activations from a copy in matrix-core fragment order,
- * which a small kernel writes there first (M rounded up to 32, times K, times 2 bytes; such a shape is only
- * chosen while that stays within TLLM_GEMM_STATIC_SCRATCH_BYTES). The first such call on a stream creates
+ * of shapes use it. Shapes whose output tiles do not fill the chip, or not its last round (M > 16), split K
+ * over several workgroups per tile, which exchange fp32 partial sums through it (at most 32 MiB); tall shapes
+ * whose K is not a multiple of 256 run a kernel that reads the activations from a copy in matrix-core
+ * fragment order, which a small kernel writes there first (M rounded up to 32, times K, times 2 bytes; such
+ * a shape is only chosen while that stays within TLLM_GEMM_STATIC_SCRATCH_BYTES). The first such call on a stream creates
  * the workspace (and a call with a larger need grows it: stream synchronisation, free, allocation).
  * tllm_gemm_workspace_reserve does that ahead of time. While `stream` is being captured into a graph
  * nothing is allocated: a call whose workspace is missing or too small then runs the kernel that needs

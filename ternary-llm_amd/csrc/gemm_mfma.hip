@@ -5,7 +5,10 @@
 // Here the product scale * w is formed exactly in fp16 (w in {-1,0,+1}), so the only difference to
 // the reference is the order of the fp32 additions.
 //
-// Tiling. A workgroup (4 waves, one per SIMD) computes 128 weight rows x BM activation rows; every wave
+// Three kernels, chosen per shape by a cost model (choose_config): the four-wave kernel described next, the eight-wave
+// ping-pong kernel (gemm_pp_kernel) and the row-split kernel (gemm_ns_kernel), each described where it is defined.
+//
+// Tiling of the four-wave kernel. A workgroup (4 waves, one per SIMD) computes 128 weight rows x BM activation rows; every wave
 // owns all 128 weight rows and BM/4 activation rows of its own. Per stage of 64 columns of K:
 //   * weights: each thread decodes one 32-bit mask word pair of one weight row into LDS. One
 //     v_bitop3 puts the 2-bit field (negative, non-zero) of every even/odd weight in place, two

@@ -43,7 +43,10 @@ constexpr int kImageBytes = 16 * kSliceCols * 2;             // operands of one 
 struct BatchSched {
     const Problem *table;    // device table, or nullptr: use the by-value problem
     const int *unit_prefix;  // [count + 1] first block of each problem
-    const int *wg_first;     // [grid + 1] first block of each workgroup, then [grid] the problem that block is in
+    // [grid + 1] first position of each workgroup in `order`, then [grid] the problem its first block is in, then
+    // `order`: [pool_begin] the block at each position. A workgroup walks consecutive positions; the blocks there ascend
+    // and are chosen by the host so that the workgroups of an XCD work on neighbouring blocks at about the same time.
+    const int *wg_first;
     // Blocks [pool_begin, pool_end) belong to no workgroup: whoever has finished its own blocks takes
     // them one at a time through counters[0]. counters[1] counts the workgroups that have left; the
     // last one sets both back to zero for the next launch (launches of one plan must not overlap).
@@ -95,15 +98,18 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
     const int li = lane & 15;  // MFMA A row / D column (activation row)
     const int lq = lane >> 4;  // MFMA k quarter / D row quad
 
-    int u = 0, u_end = 0, pi = 0;
+    // pos walks positions (plan: of `order`; single problem: the blocks themselves), u is the block there
+    int pos = 0, pos_end = 0, pi = 0;
+    const int *order = nullptr;
     if (sc.table) {
-        u = sc.wg_first[blockIdx.x];
-        u_end = sc.wg_first[blockIdx.x + 1];
-        pi = sc.wg_first[gridDim.x + 1 + blockIdx.x];  // no scan over the problems before this span
+        pos = sc.wg_first[blockIdx.x];
+        pos_end = sc.wg_first[blockIdx.x + 1];
+        pi = sc.wg_first[gridDim.x + 1 + blockIdx.x];  // no scan over the problems before the first block
+        order = sc.wg_first + 2 * gridDim.x + 1;
     } else {
         const int total = (single.rows + kBlockRows - 1) / kBlockRows;
-        u = (int)((int64_t)total * blockIdx.x / gridDim.x);
-        u_end = (int)((int64_t)total * (blockIdx.x + 1) / gridDim.x);
+        pos = (int)((int64_t)total * blockIdx.x / gridDim.x);
+        pos_end = (int)((int64_t)total * (blockIdx.x + 1) / gridDim.x);
     }
 
     // operands of an all-zero weight row (every code = 1)
@@ -112,20 +118,25 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
 
     Problem p = single;
     __shared__ int pool_block;
-    for (;; u++) {
-        if (u >= u_end) {
+    bool in_pool = false;
+    for (;; pos++) {
+        if (pos >= pos_end) {
             // own blocks done: go on with the pool block asked for while the last block was running
             // (the barriers that end a block separate the write of pool_block, this read, and the
             // next write)
             if (!sc.counters) break;
             const int t = __builtin_amdgcn_readfirstlane(pool_block);
             if (t >= sc.pool_end - sc.pool_begin) break;
-            u = sc.pool_begin + t;
-            u_end = u + 1;
+            pos = sc.pool_begin + t;
+            pos_end = pos + 1;
             pi = sc.pool_problem[t];
+            in_pool = true;
         }
+        // the pool's blocks come after all others and are their own positions; the blocks of a workgroup's own
+        // positions ascend, so the scan for the problem below only moves forward
+        const int u = order && !in_pool ? order[pos] : pos;
         // the last block of the span, or a pool block: ask for the next pool block
-        const bool request = sc.counters != nullptr && u + 1 >= u_end && tid == 0;
+        const bool request = sc.counters != nullptr && pos + 1 >= pos_end && tid == 0;
         int requested = 0;
         if (request) requested = __hip_atomic_fetch_add(sc.counters, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         int first_unit = 0;

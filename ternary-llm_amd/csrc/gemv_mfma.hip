@@ -1093,18 +1093,37 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
             units = units < 4 * wgs ? 4 * wgs : units;
         }
         const int grid = units < wgs ? units : wgs;
-        int64_t total_w = 0;
-        for (int t = 0; t < units; t++) total_w += weight[t];
-        wg_first.assign(grid + 1, units);
-        wg_first[0] = 0;
-        int64_t acc = 0;  // weight of blocks [0, t)
-        int t = 0;
-        for (int g = 1; g < grid; g++) {
-            const int lo = wg_first[g - 1] + 1, hi = units - (grid - g);
-            while (t < hi && (t < lo || acc * grid < total_w * g)) acc += weight[t++];
-            wg_first[g] = t;
+        // List scheduling on the host, in the order the blocks lie in memory: chunks of as many consecutive blocks as an
+        // XCD has workgroups go to the XCD with the least work so far (workgroup ids w, w + 8, ... share an XCD), and
+        // inside the XCD each block to the workgroup with the least work so far. At run time the workgroups of an XCD
+        // are then on the same chunk at about the same time, which is mostly one matrix: its activation rows come from
+        // HBM once per XCD and from that XCD's L2 afterwards, not once per block. A workgroup's blocks ascend.
+        const int n_xcd = grid % 8 == 0 ? 8 : 1, per_xcd = grid / n_xcd;
+        std::vector<std::vector<int>> mine(grid);
+        std::vector<int64_t> wg_load(grid, 0), xcd_load(n_xcd, 0);
+        for (int b0 = 0; b0 < units; b0 += per_xcd) {
+            int x = 0;
+            for (int i = 1; i < n_xcd; i++)
+                if (xcd_load[i] < xcd_load[x]) x = i;
+            for (int b = b0; b < units && b < b0 + per_xcd; b++) {
+                int w = x;
+                for (int i = 1; i < per_xcd; i++)
+                    if (wg_load[x + n_xcd * i] < wg_load[w]) w = x + n_xcd * i;
+                mine[w].push_back(b);
+                wg_load[w] += weight[b];
+                xcd_load[x] += weight[b];
+            }
         }
-        for (int g = 0; g < grid; g++) wg_first.push_back(block_problem[wg_first[g]]);
+        std::vector<int> order, first_problem;
+        wg_first.assign(grid + 1, 0);
+        for (int w = 0; w < grid; w++) {
+            wg_first[w] = (int)order.size();
+            first_problem.push_back(mine[w].empty() ? 0 : block_problem[mine[w][0]]);
+            order.insert(order.end(), mine[w].begin(), mine[w].end());
+        }
+        wg_first[grid] = (int)order.size();
+        wg_first.insert(wg_first.end(), first_problem.begin(), first_problem.end());
+        wg_first.insert(wg_first.end(), order.begin(), order.end());
         pool_first.assign(block_problem.begin() + units, block_problem.end());
         d.pool_begin = units;
         d.pool_end = all_units;

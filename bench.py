@@ -287,6 +287,39 @@ def plan_rows(torch, tl, orc, timer, label, model, layers, batches, p_zero, lo, 
     return rows, sets[0]
 
 
+def int8_sweep_row(torch, tl, orc, timer, label, problems, steps, warmup):
+    """The same sweep on INT8 activations (the reference's decode path, ternary_gemv_int8 per linear): every input
+    vector quantised once by quantize_absmax_int8 outside the timed region, then one plan launch per step over the
+    int8 vectors and their device-resident scales. Sampled rows against the oracle's integer arithmetic."""
+    probs, scales = [], []
+    for (nz, sg, sc, x, y, rows, cols, _) in problems:
+        q = torch.zeros(cols, dtype=torch.int8, device="cuda")
+        qs = torch.zeros(1, dtype=torch.float32, device="cuda")
+        tl.quantize_absmax_int8(x, q, qs, cols)
+        probs.append((nz, sg, sc, q, torch.zeros((1, rows), dtype=torch.float16, device="cuda"), rows, cols, 1))
+        scales.append(qs)
+    torch.cuda.synchronize()
+    plan = tl.LinearPlan(probs, input_scales=scales)
+    t = timer.run(plan.launch, steps, warmup)
+    nbytes = sum(packed_bytes(p[5], p[6]) for p in probs)
+    rng = np.random.default_rng(3)
+    worst = 0.0
+    n = len(probs)
+    for i in sorted(set([0, 1, 4, 6, n - 1, n // 2])):
+        nz, sg, sc, q, y, rows, cols, _ = probs[i]
+        pick = np.sort(rng.choice(rows, size=min(64, rows), replace=False))
+        ref = orc.gemv_i8_f64(nz[pick].cpu().numpy().view(np.uint32), sg[pick].cpu().numpy().view(np.uint32),
+                              sc[pick].cpu().numpy().view(np.uint16), q.cpu().numpy(), float(scales[i].item()))
+        full = y.float()
+        tau = float((full * full).mean().sqrt().item()) / 64.0
+        got = y[0, pick].cpu().numpy().astype(np.float64)
+        worst = max(worst, float((np.abs(got - ref) / np.maximum(np.abs(ref), tau)).max()))
+    row = hbm_row(label, t, nbytes, plan.kernel + " on int8 activations", worst)
+    row["matrices_per_launch"] = n
+    plan.close()
+    return row
+
+
 def gemm_rows(torch, tl, orc, timer, seed, m_list, p_zero, calls, warm):
     """Prefill GEMM (cfg4): LLaMA-3-8B gate/up 14336x4096 and down 4096x14336, M tokens each; dense-equivalent
     2*M*N*K flops against the FP16 matrix peak (M = 16 is HBM-bound and also gets its weight-stream rate).
@@ -643,6 +676,8 @@ def main():
             r, _ = plan_rows(torch, tl, orc, timer, "cfg3: llama8b 32-layer sweep", "llama8b", 32, extra, 0.42, 0.01, 0.03,
                              args.seed, cfg_steps, 20, problems=problems)
             cfgs += r
+            cfgs.append(int8_sweep_row(torch, tl, orc, timer, "cfg3: llama8b 32-layer sweep, batch 1, int8 activations (plan of ternary_gemv_int8)",
+                                       problems, cfg_steps, 20))
         if 4 in want:
             gemm_m = [int(v) for v in args.gemm_m.split(",") if v.strip()]
             g = gemm_rows(torch, tl, orc, timer, args.seed, gemm_m, 0.42, args.gemm_calls, args.gemm_warm)

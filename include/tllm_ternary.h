@@ -258,6 +258,19 @@ int tllm_linear_plan_create(tllm_linear_plan **plan, const tllm_linear_problem *
 int tllm_linear_plan_create_normed(tllm_linear_plan **plan, const tllm_linear_problem *problems,
                                    const uint16_t *const *norm_weights, float eps, int count,
                                    int group_size);
+/*
+ * The same on INT8 activations: problem i's `input` points at int8 [cols] (cast to the field's type; 16-byte
+ * aligned) and input_scales[i] (HOST array of `count` DEVICE pointers) at the float tllm_quantize_absmax_i8
+ * wrote for that vector; batch 1, flags 0. Every output is what tllm_ternary_gemv_i8_dscale gives for that
+ * matrix, bit for bit:
+ *   output[r] = fp16( *input_scales[i] * sum_g float(scales[r,g]) * float(sum_{k in g} w[r,k] * input_int8[k]) ).
+ * One launch then replaces the ternary_gemv_int8 calls of a decode step that do not depend on each other
+ * (reference src/transformer.cpp:132-142 per linear, 199-217 and 264-278 for the groups). Shapes that the
+ * matrix-core kernel does not serve (cols below 512 or not a multiple of 128) are rejected with
+ * TLLM_ERR_BAD_PLAN: issue those with tllm_ternary_gemv_i8.
+ */
+int tllm_linear_plan_create_i8(tllm_linear_plan **plan, const tllm_linear_problem *problems,
+                               const float *const *input_scales, int count, int group_size);
 /* One launch over every problem of the plan. Allocation-free. Besides the outputs a launch uses two device
  * counters that deal the tail of a large plan out to the workgroups (the kernel resets them when it ends, so
  * replays of a captured graph need no clearing). The plan holds 16 such pairs and launches take them in turn:

@@ -219,7 +219,8 @@ int tllm_read_stream(const void *src, size_t bytes, uint32_t *sink, tllm_stream_
 }
 
 static int create_plan(tllm_linear_plan **plan, const tllm_linear_problem *problems,
-                       const uint16_t *const *norm_weights, float eps, int count, int group_size) {
+                       const uint16_t *const *norm_weights, float eps, int count, int group_size,
+                       const float *const *input_scales = nullptr) {
     if (!plan || !problems) return TLLM_ERR_NULL_POINTER;
     *plan = nullptr;
     if (count < 1) return TLLM_ERR_BAD_PLAN;
@@ -243,7 +244,19 @@ static int create_plan(tllm_linear_plan **plan, const tllm_linear_problem *probl
         if (q.flags & TLLM_PROBLEM_SWIGLU_GATE) {
             if (i + 1 >= count || q.batch != 1) return TLLM_ERR_BAD_PLAN;
         }
-        if (int e = tllm::check_linear(host[i], group_size)) return e;
+        if (input_scales) {
+            // int8 activations: `input` points at int8 [cols]; one row, no pairs; the scale lives on the device
+            if (q.batch != 1 || q.flags) return TLLM_ERR_BAD_PLAN;
+            if (!input_scales[i] || !q.input || !q.output) return TLLM_ERR_NULL_POINTER;
+            if (int e = tllm::check_weight(host[i].nz, host[i].sg, host[i].scales, q.rows, q.cols, group_size)) return e;
+            if (tllm::misaligned(q.input, 16) || tllm::misaligned(q.output, 2) || tllm::misaligned(input_scales[i], 4))
+                return TLLM_ERR_MISALIGNED;
+            if (tllm::overlaps(q.input, (size_t)q.cols, q.output, (size_t)q.rows * 2)) return TLLM_ERR_ALIAS;
+            host[i].flags |= tllm::kProblemInt8Input;
+            host[i].x_scale = input_scales[i];
+        } else if (int e = tllm::check_linear(host[i], group_size)) {
+            return e;
+        }
         if (norm_weights && norm_weights[i]) {
             // RMSNorm prologue: batch 1, a row that the one-pass staging holds, 16-byte aligned weights
             if (q.batch != 1 || q.cols > 16384 || !(eps >= 0.0f)) return TLLM_ERR_BAD_PLAN;
@@ -260,7 +273,7 @@ static int create_plan(tllm_linear_plan **plan, const tllm_linear_problem *probl
     if (!pl) return TLLM_ERR_TOO_LARGE;
     if (hipError_t e = tllm::plan_device_create(pl->host, &pl->dev)) {
         delete pl;
-        return (int)e;
+        return input_scales && e == hipErrorInvalidValue ? TLLM_ERR_BAD_PLAN : (int)e;  // a shape the int8 plan kernel does not serve
     }
     if (pl->dev.extras && !pl->dev.use_mfma) {  // a shape that only the general kernel serves: no pairs, no prologue
         tllm::plan_device_destroy(&pl->dev);
@@ -281,6 +294,12 @@ int tllm_linear_plan_create_normed(tllm_linear_plan **plan, const tllm_linear_pr
                                    int group_size) {
     if (!norm_weights) return TLLM_ERR_NULL_POINTER;
     return create_plan(plan, problems, norm_weights, eps, count, group_size);
+}
+
+int tllm_linear_plan_create_i8(tllm_linear_plan **plan, const tllm_linear_problem *problems,
+                               const float *const *input_scales, int count, int group_size) {
+    if (!input_scales) return TLLM_ERR_NULL_POINTER;
+    return create_plan(plan, problems, nullptr, 0.0f, count, group_size, input_scales);
 }
 
 int tllm_linear_plan_launch(const tllm_linear_plan *plan, tllm_stream_t stream) {

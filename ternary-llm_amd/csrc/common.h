@@ -30,14 +30,20 @@ struct Problem {
     int32_t rows;
     int32_t cols;
     int32_t batch;
-    int32_t flags;  // kProblemSwigluGate
-    // optional prologue (plans only): x is RMS-normalised with these weights before it is used
-    const uint16_t *norm_w;
+    int32_t flags;  // kProblemSwigluGate, kProblemInt8Input
+    union {
+        // optional prologue (plans only): x is RMS-normalised with these weights before it is used
+        const uint16_t *norm_w;
+        // plans on int8 activations (kProblemInt8Input: x points at int8 values, batch 1): the activation scale in
+        // device memory, as tllm_quantize_absmax_i8 writes it
+        const float *x_scale;
+    };
     float eps;
     int32_t pad;
 };
 static_assert(sizeof(Problem) == sizeof(tllm_linear_problem) + 16, "tllm_linear_problem, then the prologue");
 constexpr int kProblemSwigluGate = TLLM_PROBLEM_SWIGLU_GATE;
+constexpr int kProblemInt8Input = 0x100;  // set by tllm_linear_plan_create_i8, not a public flag
 
 // CU count of the current device, asked once per device (256 if the runtime cannot tell). Safe to
 // call from several host threads.
@@ -155,6 +161,7 @@ struct PlanDevice {
     int pair_stride = 0;  // floats between the two partial-sum areas of a SwiGLU pair (0: no pairs)
     bool fine = false;    // units of 16 rows (decode-size plans that would leave most workgroup slots empty)
     bool extras = false;  // SwiGLU pairs or RMSNorm prologues present: the kernel instance that knows them
+    bool x_is_i8 = false; // every problem reads int8 activations and its own device-resident scale
     int image_bytes = 0;
     int lds_bytes = 0;
 };

@@ -319,7 +319,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                 else if (m) ex = (int)((__builtin_bit_cast(uint32_t, h2f((uint16_t)m)) >> 23) & 0xFF) - 127;
                 if (tid == 0) {
                     float f = m ? __builtin_bit_cast(float, (uint32_t)(127 + ex + 10) << 23) : 0.0f;
-                    if (sc.x_is_i8) f *= sc.i8_scale_dev ? *sc.i8_scale_dev : sc.i8_scale;
+                    if (sc.x_is_i8) f *= sc.table ? *p.x_scale : (sc.i8_scale_dev ? *sc.i8_scale_dev : sc.i8_scale);
                     fscale[b] = f;
                 }
                 return ex;
@@ -1134,8 +1134,16 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
     bool has_pairs = false, has_norm = false;
     for (const Problem &p : host) {
         has_pairs = has_pairs || (p.flags & kProblemSwigluGate);
-        has_norm = has_norm || p.norm_w != nullptr;
+        has_norm = has_norm || (p.norm_w != nullptr && !(p.flags & kProblemInt8Input));
     }
+    // int8 activations: all problems or none, batch 1 (the caller has checked), MFMA kernel only
+    bool any_i8 = false, all_i8 = true;
+    for (const Problem &p : host) {
+        any_i8 = any_i8 || (p.flags & kProblemInt8Input);
+        all_i8 = all_i8 && (p.flags & kProblemInt8Input);
+    }
+    if (any_i8 && (!all_i8 || max_batch != 1 || has_pairs)) return hipErrorInvalidValue;
+    d.x_is_i8 = any_i8;
     // SwiGLU pairs and RMSNorm prologues exist in the wide-tile MFMA GEMV kernel only (batch 1)
     d.extras = has_pairs || has_norm;
     bool all_batch = max_batch >= 2 && !d.extras;
@@ -1179,6 +1187,7 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
     } else {
         d.wide = all_wide;
         d.use_mfma = d.extras ? all_wide : all_wide || all_tall;
+        if (d.x_is_i8 && !d.use_mfma) return hipErrorInvalidValue;  // the table kernel for general shapes is fp16 only
         if (d.wide) {  // decode-size plans: fine-grained units
             int64_t coarse = 0;
             int whole = 0;  // largest image of a whole row: the fine-grained instances do not stage in segments
@@ -1259,6 +1268,7 @@ hipError_t plan_device_launch(const PlanDevice &plan, hipStream_t s) {
     sc.pool_first = plan.pool_first;
     sc.pool_count = plan.pool_count;
     sc.counters = counters;
+    sc.x_is_i8 = plan.x_is_i8 ? 1 : 0;
     sc.count = plan.count;
     sc.pair_stride = plan.pair_stride;
     sc.max_units = plan.max_units;

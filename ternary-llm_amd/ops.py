@@ -16,7 +16,7 @@ ABI_SYMBOLS = (
     "tllm_error_string", "tllm_abi_version", "tllm_ternary_gemv_f16", "tllm_ternary_gemv_i8",
     "tllm_ternary_gemv_i8_dscale", "tllm_quantize_absmax_i8", "tllm_ternary_gemm_f16",
     "tllm_linear_plan_create", "tllm_linear_plan_launch", "tllm_linear_plan_weight_bytes",
-    "tllm_linear_plan_destroy", "tllm_rmsnorm_f16", "tllm_silu_mul_f16", "tllm_linear_plan_create_normed",
+    "tllm_linear_plan_destroy", "tllm_rmsnorm_f16", "tllm_silu_mul_f16", "tllm_linear_plan_create_normed", "tllm_linear_plan_create_i8",
     "tllm_add_f16", "tllm_rope_f16", "tllm_embedding_lookup_f16", "tllm_copy_to_kv_cache_f16",
     "tllm_linear_plan_kernel", "tllm_gemm_workspace_reserve", "tllm_gemm_workspace_release",
     "tllm_ternary_gemm_f16_static", "tllm_read_stream", "tllm_ternary_gemm_kernel",
@@ -84,6 +84,7 @@ def lib():
     L.tllm_gemm_workspace_release.restype = None
     L.tllm_linear_plan_create.argtypes = [C.POINTER(vp), C.POINTER(_Problem), i, i]
     L.tllm_linear_plan_create_normed.argtypes = [C.POINTER(vp), C.POINTER(_Problem), C.POINTER(vp), f, i, i]
+    L.tllm_linear_plan_create_i8.argtypes = [C.POINTER(vp), C.POINTER(_Problem), C.POINTER(vp), i, i]
     L.tllm_linear_plan_launch.argtypes = [vp, vp]
     L.tllm_linear_plan_weight_bytes.argtypes = [vp]
     L.tllm_linear_plan_weight_bytes.restype = C.c_int64
@@ -233,7 +234,7 @@ SWIGLU_GATE = 1  # TLLM_PROBLEM_SWIGLU_GATE
 class LinearPlan:
     """Several independent ternary linears issued as one launch."""
 
-    def __init__(self, problems, group_size=128, norm_weights=None, eps=1e-5):
+    def __init__(self, problems, group_size=128, norm_weights=None, eps=1e-5, input_scales=None):
         """problems: iterable of (nz, sign, scales, input, output, rows, cols, batch[, flags]);
         flags = SWIGLU_GATE marks the gate of a pair whose up projection is the next problem
         (output may be None there): the pair stores silu(gate) * up in the gate's output."""
@@ -246,7 +247,13 @@ class LinearPlan:
             arr[k] = _Problem(nz.data_ptr(), sg.data_ptr(), sc.data_ptr(), x.data_ptr(),
                               y.data_ptr() if y is not None else 0, rows, cols, batch, flags)
         self._h = C.c_void_p(0)
-        if norm_weights is None:
+        if input_scales is not None:
+            # int8 activations: every problem's input is an int8 tensor, input_scales[k] the float32 device tensor
+            # that quantize_absmax_int8 wrote for it
+            self._keep_scales = list(input_scales)
+            ptrs = (C.c_void_p * max(len(problems), 1))(*[t.data_ptr() for t in self._keep_scales])
+            check(lib().tllm_linear_plan_create_i8(C.byref(self._h), arr, ptrs, len(problems), group_size))
+        elif norm_weights is None:
             check(lib().tllm_linear_plan_create(C.byref(self._h), arr, len(problems), group_size))
         else:
             # one fp16 weight tensor (or None) per problem: RMSNorm prologue on that problem's input

@@ -798,6 +798,67 @@ def test_linear_plan_matches_single_calls(dev, oracle):
     plan.close()
 
 
+def test_linear_plan_on_int8_activations(dev, oracle):
+    """A plan whose problems read int8 activations and their device-resident scales (the reference's decode path,
+    quantize_absmax_int8 + ternary_gemv_int8 per linear): every output must equal, bit for bit, what the single-call
+    operator gives for that matrix, and agree with the oracle's integer arithmetic; a plan that mixes shapes the
+    matrix-core kernel does not serve is rejected."""
+    torch, tl = dev
+    shapes = [(2048, 2048), (512, 2048), (2048, 8192), (4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336)]
+    probs, scales, refs = [], [], []
+    for k, (rows, cols) in enumerate(shapes * 3):
+        nz, sg, s, x = synth.problem(8100 + k, rows, cols, unit_rms=True)
+        dx = up(torch, x)
+        q = torch.zeros(cols, dtype=torch.int8, device="cuda")
+        qs = torch.zeros(1, dtype=torch.float32, device="cuda")
+        tl.quantize_absmax_int8(dx, q, qs, cols)
+        y = torch.full((1, rows), float("nan"), dtype=torch.float16, device="cuda")
+        probs.append((up(torch, nz), up(torch, sg), up(torch, s), q, y, rows, cols, 1))
+        scales.append(qs)
+        torch.cuda.synchronize()
+        if k < len(shapes):
+            refs.append(oracle.gemv_i8_f64(nz, sg, s.view(np.uint16), q.cpu().numpy(), float(qs.item())))
+    plan = tl.LinearPlan(probs, input_scales=scales)
+    assert "gemv_mfma_kernel" in plan.kernel
+    for launch in range(2):
+        for p in probs:
+            p[4].fill_(float("nan"))
+        plan.launch()
+        torch.cuda.synchronize()
+        for k, (dnz, dsg, ds, q, y, rows, cols, _) in enumerate(probs):
+            single = torch.full((rows,), float("nan"), dtype=torch.float16, device="cuda")
+            tl.ternary_gemv_int8(dnz, dsg, ds, q, scales[k], single, rows, cols, 128)
+            torch.cuda.synchronize()
+            assert torch.equal(y[0], single), f"int8 plan, problem {k} ({rows}x{cols}), launch {launch}: differs from the single call"
+            if k < len(shapes):
+                assert_close(oracle, y[0].cpu().numpy().astype(np.float64), refs[k], what=f"int8 plan {rows}x{cols}")
+    plan.close()
+    # shorter rows (below the 2048 columns of the wide tiles): the plan runs the tall tiles, checked against the oracle
+    tall, tall_scales, tall_refs = [], [], []
+    for k, (rows, cols) in enumerate([(100, 1536), (64, 512), (300, 1152)]):
+        nz, sg, s, x = synth.problem(8150 + k, rows, cols, unit_rms=True)
+        q = torch.zeros(cols, dtype=torch.int8, device="cuda")
+        qs = torch.zeros(1, dtype=torch.float32, device="cuda")
+        tl.quantize_absmax_int8(up(torch, x), q, qs, cols)
+        torch.cuda.synchronize()
+        tall.append((up(torch, nz), up(torch, sg), up(torch, s), q, torch.full((1, rows), float("nan"), dtype=torch.float16, device="cuda"),
+                     rows, cols, 1))
+        tall_scales.append(qs)
+        tall_refs.append(oracle.gemv_i8_f64(nz, sg, s.view(np.uint16), q.cpu().numpy(), float(qs.item())))
+    plan = tl.LinearPlan(tall, input_scales=tall_scales)
+    plan.launch()
+    torch.cuda.synchronize()
+    for p, ref in zip(tall, tall_refs):
+        assert_close(oracle, p[4][0].cpu().numpy().astype(np.float64), ref, what=f"int8 plan, tall tiles, {p[5]}x{p[6]}")
+    plan.close()
+    # 384 columns are fewer than the matrix-core kernel takes: such a plan is refused, not run some other way
+    nz, sg, s, x = synth.problem(8199, 64, 256 + 128, unit_rms=True)
+    small = (up(torch, nz), up(torch, sg), up(torch, s), torch.zeros(384, dtype=torch.int8, device="cuda"),
+             torch.zeros((1, 64), dtype=torch.float16, device="cuda"), 64, 384, 1)
+    with pytest.raises(Exception):
+        tl.LinearPlan([probs[0], small], input_scales=[scales[0], scales[0]])
+
+
 def test_linear_plan_model_sweep_every_row(dev, oracle):
     """A LLaMA-1B-shaped sweep (8 layers x 7 matrices in one launch): every output row of every
     problem must equal what the single-call operator gives for that matrix (same kernel, fixed

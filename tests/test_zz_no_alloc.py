@@ -81,6 +81,30 @@ def test_static_gemm_matches_the_allocating_entry_point(oracle):
             os.environ.pop("TLLM_GEMM_PINGPONG", None)
         else:
             os.environ["TLLM_GEMM_PINGPONG"] = old
+    # the row-split kernel's exchange slots live in the same fixed array: tiles split eight ways, then a smaller shape
+    old = os.environ.get("TLLM_GEMM_ROWSPLIT")
+    os.environ["TLLM_GEMM_ROWSPLIT"] = "1"
+    try:
+        for k, (M, N, K) in enumerate([(260, 300, 6144), (130, 256, 4096)]):
+            assert "K split" in tl.gemm_kernel(M, N, K)
+            nz, sg, s, _ = synth.problem(9600 + k, N, K, dontcare_sign=True)
+            A = synth.acts_f16(np.random.default_rng(9700 + k), M, K)
+            rows = np.unique(np.random.default_rng(k).integers(0, M, 6))
+            ref = oracle.gemm_f64(A[rows].view(np.uint16), nz, sg, s.view(np.uint16))
+            case = (M, N, K, _up(torch, A), _up(torch, nz), _up(torch, sg), _up(torch, s), None, None)
+            got = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+            want = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+            call(L.tllm_ternary_gemm_f16_static, case, got)
+            call(L.tllm_ternary_gemm_f16, case, want)
+            torch.cuda.synchronize()
+            assert torch.equal(got.view(torch.int16), want.view(torch.int16)), f"row-split kernel {M}x{N}x{K}: differs from tllm_ternary_gemm_f16"
+            rep_err = oracle.error_report(got.cpu().numpy().astype(np.float64)[rows], ref)
+            assert rep_err["max_rel"] <= 1e-3, f"row-split kernel {M}x{N}x{K}: {rep_err}"
+    finally:
+        if old is None:
+            os.environ.pop("TLLM_GEMM_ROWSPLIT", None)
+        else:
+            os.environ["TLLM_GEMM_ROWSPLIT"] = old
     # same argument checks as the allocating entry point
     M, N, K, dA, dnz, dsg, ds, _, _ = cases[0]
     out = torch.zeros((M, N), dtype=torch.float16, device="cuda")

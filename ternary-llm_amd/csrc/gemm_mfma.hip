@@ -1450,10 +1450,10 @@ GemmConfig choose_config(const Problem &p, size_t limit_floats) {
             if (workspace_floats(p, cand) > limit_floats) break;
             const long wgs = tiles * splits;
             const float stages = (float)((groups + splits - 1) / splits * 2);
-            // the exchange: all workgroups write their fp32 tile at once (about 5.5 us with the
-            // hand-over), then the last one of a tile reads the `splits` slots on its own, at about
-            // 29 GB/s (fitted to 14336x4096 and 4096x14336 at M = 128: 10 us with 2, 23.5 us with 8)
-            const float exchange = splits > 1 ? 5.5f + (float)splits * (float)(bm * kBN * 4) / 29.0e3f : 0.0f;
+            // the exchange: all workgroups write their fp32 tile at once, then the last one of a tile reads the
+            // `splits` slots on its own: 2 us + 0.7 us per slot + 25 ns per workgroup of the launch for 64 KB slots
+            // (fitted to fifteen shapes between 100 x 2048 x 2048 and 512 x 8192 x 28672)
+            const float exchange = splits > 1 ? (2.0f + 0.7f * (float)splits + 0.025f * (float)(tiles * splits)) * (float)(bm / 128) : 0.0f;
             const float us = (float)((wgs + n_cu - 1) / n_cu) * stages * stage_us[c] + 5.0f + exchange;
             if (best.us == 0.f || us < best.us) best = GemmConfig{c, splits, false, us};
         }
@@ -1495,8 +1495,11 @@ GemmConfig choose_config(const Problem &p, size_t limit_floats) {
             while (splits > 1 && (size_t)rem * splits * 128 * kNsBN > limit_floats) splits--;
             if (splits > 1) {
                 const float exchange = 6.0f + 1.5f * (float)splits;
-                const float us = (float)(tiles / n_cu) * (float)blocks * block_us + (float)((blocks + splits - 1) / splits) * block_us +
-                                 exchange + fixed_us;
+                // (a launch that leaves CUs idle runs its blocks and its exchange faster: down to 3/4 of the time)
+                const float parts = (float)rem * (float)splits;
+                const float thin = tiles < n_cu ? 0.75f + 0.25f * std::min(1.0f, parts / (float)n_cu) : 1.0f;
+                const float us = (float)(tiles / n_cu) * (float)blocks * block_us +
+                                 thin * ((float)((blocks + splits - 1) / splits) * block_us + exchange + fixed_us);
                 if (us < rs.us) {
                     rs.splits = splits;
                     rs.full_tiles = tiles - rem;

@@ -1101,11 +1101,12 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
         const int n_xcd = grid % 8 == 0 ? 8 : 1, per_xcd = grid / n_xcd;
         std::vector<std::vector<int>> mine(grid);
         std::vector<int64_t> wg_load(grid, 0), xcd_load(n_xcd, 0);
-        for (int b0 = 0; b0 < units; b0 += per_xcd) {
+        const int chunk = per_xcd;
+        for (int b0 = 0; b0 < units; b0 += chunk) {
             int x = 0;
             for (int i = 1; i < n_xcd; i++)
                 if (xcd_load[i] < xcd_load[x]) x = i;
-            for (int b = b0; b < units && b < b0 + per_xcd; b++) {
+            for (int b = b0; b < units && b < b0 + chunk; b++) {
                 int w = x;
                 for (int i = 1; i < per_xcd; i++)
                     if (wg_load[x + n_xcd * i] < wg_load[w]) w = x + n_xcd * i;
@@ -1114,11 +1115,21 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
                 xcd_load[x] += weight[b];
             }
         }
+        // The kernel asks for its first run-time block while it works on its last own one: every workgroup needs a
+        // block of its own. The first chunks go to the XCDs that have none yet and fill all their workgroups, so none is
+        // left empty as long as there are at least `grid` blocks; should weights ever defeat that, deal the blocks out
+        // in turn instead.
+        bool some_empty = false;
+        for (int w = 0; w < grid; w++) some_empty = some_empty || mine[w].empty();
+        if (some_empty) {
+            for (int w = 0; w < grid; w++) mine[w].clear();
+            for (int b = 0; b < units; b++) mine[b % grid].push_back(b);
+        }
         std::vector<int> order, first_problem;
         wg_first.assign(grid + 1, 0);
         for (int w = 0; w < grid; w++) {
             wg_first[w] = (int)order.size();
-            first_problem.push_back(mine[w].empty() ? 0 : block_problem[mine[w][0]]);
+            first_problem.push_back(block_problem[mine[w][0]]);
             order.insert(order.end(), mine[w].begin(), mine[w].end());
         }
         wg_first[grid] = (int)order.size();

@@ -1093,15 +1093,18 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
             units = units < 4 * wgs ? 4 * wgs : units;
         }
         const int grid = units < wgs ? units : wgs;
-        // List scheduling on the host, in the order the blocks lie in memory: chunks of as many consecutive blocks as an
-        // XCD has workgroups go to the XCD with the least work so far (workgroup ids w, w + 8, ... share an XCD), and
+        // List scheduling on the host, in the order the blocks lie in memory: chunks of consecutive blocks
+        // go to the XCD with the least work so far (workgroup ids w, w + 8, ... share an XCD), and
         // inside the XCD each block to the workgroup with the least work so far. At run time the workgroups of an XCD
         // are then on the same chunk at about the same time, which is mostly one matrix: its activation rows come from
         // HBM once per XCD and from that XCD's L2 afterwards, not once per block. A workgroup's blocks ascend.
         const int n_xcd = grid % 8 == 0 ? 8 : 1, per_xcd = grid / n_xcd;
         std::vector<std::vector<int>> mine(grid);
         std::vector<int64_t> wg_load(grid, 0), xcd_load(n_xcd, 0);
-        const int chunk = per_xcd;
+        // (chunks of 8: whole XCD-loads of 32 neighbouring blocks put all of an XCD's workgroups into the same phase of
+        // their blocks and cost 3 % on the 8B sweep at sixteen rows; with 8 an XCD is in four places at a time, the
+        // activation rows of four matrices still fit its L2, and the 70B sweep keeps its + 4 %)
+        const int chunk = per_xcd < 8 ? per_xcd : 8;
         for (int b0 = 0; b0 < units; b0 += chunk) {
             int x = 0;
             for (int i = 1; i < n_xcd; i++)

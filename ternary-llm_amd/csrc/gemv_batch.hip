@@ -14,7 +14,8 @@
 // group, the 2-bit codes are cut out with one AND per two weights (gemv_layout.h) and 4 x 4
 // v_mfma_f32_16x16x32_f16 give one 16 x 16 result per scale group: rows x activation rows. The fp32
 // group scales multiply whole result tiles; results stay in registers over all slices (every wave
-// owns its rows for the whole of K), so there is no reduction between waves and no atomics.
+// owns its rows for the whole of K, the two waves that share a tile add up once at the end), so
+// there are no atomics.
 // The "+1" of the code c = w + 1 is removed by subtracting the product of an all-zero weight row,
 // computed once per slice with the same instructions (exact zeros stay exact).
 #include "common.h"
@@ -57,9 +58,7 @@ struct BatchSched {
 
 struct Tile {
     u4 nz, sg;
-};
-struct Scales {
-    u2 sc[4];  // scales of rows 4*lq + v, groups 4*slice .. +3 (fp16 x 4)
+    u2 sc;  // scales of row 4*lq + (li & 3), groups 4*slice .. +3 (fp16 x 4)
 };
 
 __device__ __forceinline__ f4 mfma16(const uint32_t *o, u4 b, f4 c) {
@@ -67,13 +66,33 @@ __device__ __forceinline__ f4 mfma16(const uint32_t *o, u4 b, f4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a), __builtin_bit_cast(h8, b), c, 0, 0, 0);
 }
 
-// Lanes i, i+16, i+32, i+48 hold row q of a 4 x 4 matrix in a[0..3]; afterwards they hold column q.
-__device__ __forceinline__ void transpose4(u4 &a) {
-    auto s0 = __builtin_amdgcn_permlane32_swap(a[0], a[2], false, false);
-    auto s1 = __builtin_amdgcn_permlane32_swap(a[1], a[3], false, false);
-    auto t0 = __builtin_amdgcn_permlane16_swap(s0[0], s1[0], false, false);
-    auto t1 = __builtin_amdgcn_permlane16_swap(s0[1], s1[1], false, false);
-    a = u4{t0[0], t0[1], t1[0], t1[1]};
+// Lanes i, i+16, i+32, i+48 hold row q of a 4 x 4 matrix in a[0..3] (and of another in b[0..3]); afterwards they hold
+// column q. The swaps work in place on the registers they are given; written through the builtins, which return new
+// values, the same sequence cost 13 register copies per tile. The compiler does not see inside the block: a vector
+// instruction that writes one of these registers must be two wait states away from the swap that reads it, hence
+// the leading s_nop (the swaps themselves are interleaved so that each is two instructions behind its producer).
+__device__ __forceinline__ void transpose4x2(u4 &a, u4 &b) {
+    uint32_t a0 = a[0], a1 = a[1], a2 = a[2], a3 = a[3], b0 = b[0], b1 = b[1], b2 = b[2], b3 = b[3];
+    asm volatile(
+        "s_nop 1\n\t"
+        "v_permlane32_swap_b32 %0, %2\n\t"
+        "v_permlane32_swap_b32 %1, %3\n\t"
+        "v_permlane32_swap_b32 %4, %6\n\t"
+        "v_permlane32_swap_b32 %5, %7\n\t"
+        "v_permlane16_swap_b32 %0, %1\n\t"
+        "v_permlane16_swap_b32 %2, %3\n\t"
+        "v_permlane16_swap_b32 %4, %5\n\t"
+        "v_permlane16_swap_b32 %6, %7\n\t"
+        "s_nop 1"
+        : "+v"(a0), "+v"(a1), "+v"(a2), "+v"(a3), "+v"(b0), "+v"(b1), "+v"(b2), "+v"(b3));
+    a = u4{a0, a1, a2, a3};
+    b = u4{b0, b1, b2, b3};
+}
+
+// The value lane `kFrom` of each quad holds, in all four lanes of the quad.
+template <int kFrom>
+__device__ __forceinline__ uint32_t quad_broadcast(uint32_t x) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, kFrom * 0x55, 0xF, 0xF, true);
 }
 
 // kTilesPerWave: 4 for long streams (256-row blocks amortise the per-slice operand build best);
@@ -163,21 +182,23 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
             return rbe;
         };
         const uint32_t lane_mask_off = ((uint32_t)li * words + 4u * lq) * 4u;
-        const uint32_t lane_scale_off = (uint32_t)(4 * lq) * groups * 2u;
+        // Scales: a lane holds the results of rows 4*lq + v, v = 0..3 (MFMA D layout). It loads the scales of row
+        // 4*lq + (li & 3) only, so that the four lanes of every quad of lane quarter lq hold rows 4*lq .. 4*lq + 3, and
+        // takes the other three from its quad neighbours (one DPP move per register): one load per tile whose 64 lanes
+        // ask for 16 different addresses, four neighbouring lanes for four neighbouring rows. (With the MFMA operands
+        // exchanged a lane would need the scales of one row only and no DPP moves, but its load, 16 different rows in
+        // 16 neighbouring lanes, cost more than the moves save: 3 % slower at 5 and 8 activation rows.) They travel
+        // with the masks of the same tile and slice, a whole step ahead: the loads of a wave return in order, and a
+        // scale load asked for later than the masks it belongs to would make its tile wait for every mask load issued
+        // before it.
+        const uint32_t lane_scale_off = (uint32_t)(4 * lq + (li & 3)) * groups * 2u;
         auto load_tile = [&](int k, int slice) -> Tile {
             Tile t;
-            const size_t base = (size_t)tile_first_row(k, nullptr) * words * 4 + (size_t)slice * 64;
+            const int first = tile_first_row(k, nullptr);
+            const size_t base = (size_t)first * words * 4 + (size_t)slice * 64;
             t.nz = *reinterpret_cast<const GU4 *>(nz_g + base + lane_mask_off);
             t.sg = *reinterpret_cast<const GU4 *>(sg_g + base + lane_mask_off);
-            return t;
-        };
-        // the scales (8 bytes per row and slice, mostly cache hits) are asked for one tile ahead only
-        auto load_scales = [&](int k, int slice) -> Scales {
-            Scales t;
-            const size_t base = (size_t)tile_first_row(k, nullptr) * groups * 2 + (size_t)slice * 8;
-#pragma unroll
-            for (int v = 0; v < 4; v++)
-                t.sc[v] = *reinterpret_cast<const GU2 *>(sc_g + base + (size_t)(v * groups) * 2 + lane_scale_off);
+            t.sc = *reinterpret_cast<const GU2 *>(sc_g + (size_t)first * groups * 2 + (size_t)slice * 8 + lane_scale_off);
             return t;
         };
 
@@ -185,15 +206,18 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
         const int xpar = tid >> 8, xj = (tid >> 4) & 15, xseg = tid & 15;
         const bool x_live = xj < p.batch;
         const GU4 *x_src = (const GU4 *)(p.x + (size_t)(x_live ? xj : 0) * p.cols) + xseg * 4;
-        // a slice past the end of an odd number of slices is built as zeros
+        // Every thread loads, also where the image is to be zeros (an activation row past the batch, the slice past
+        // the end of an odd number of slices): loads under a branch would leave the number of loads in flight unknown
+        // to the compiler, which then waits for all of them before a tile's masks are used.
         auto load_x = [&](u4 (&xr)[4], int slice) {
+            const int sl = min(slice, slices - 1);
 #pragma unroll
-            for (int i = 0; i < 4; i++)
-                xr[i] = x_live && slice < slices ? x_src[slice * (kSliceCols / 8) + i] : u4{0u, 0u, 0u, 0u};
+            for (int i = 0; i < 4; i++) xr[i] = x_src[sl * (kSliceCols / 8) + i];
         };
         // builds the operands of one slice: element (chunk c, word q, step t, row j, e) at
         // ((c*4 + t)*64 + q*16 + j)*16 + 2e bytes: lane (j, q) of MFMA (c, t) reads 16 contiguous bytes
-        auto build_image = [&](const u4 (&xr)[4], int buf) {
+        // (`dead`: write zeros whatever was loaded)
+        auto build_image = [&](const u4 (&xr)[4], int buf, bool dead) {
             // largest magnitude of the activation row inside the slice: packed unsigned maximum of the
             // sign-stripped halves, then across the 16 threads of the row (one DPP row rotation each)
             us2 m2 = {0, 0};
@@ -207,6 +231,9 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
             m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x124, 0xF, 0xF, true));  // row_ror:4
             m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x122, 0xF, 0xF, true));  // row_ror:2
             m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x121, 0xF, 0xF, true));  // row_ror:1
+            if (dead) m = 0;
+            // byte selectors of the permutes below; selector 0x0C yields a zero byte
+            const uint32_t sel_lo = dead ? 0x0C0C0C0Cu : 0x05040100u, sel_hi = dead ? 0x0C0C0C0Cu : 0x07060302u;
             // amax in [2^ex, 2^(ex+1)); x'' = x * 2^(14-ex) stays below 2^15
             int ex = 0;
             if (m >= 0x7C00u) ex = 15;  // inf/nan present: they propagate to the outputs
@@ -233,7 +260,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
                 for (int dq = 0; dq < 4; dq++) {
                     const int mm = 4 * h + dq;
                     const uint32_t lo = mm == 0 ? src[8] : src[mm], hi = mm == 0 ? src[0] : src[mm + 8];
-                    const uint32_t pair = __builtin_amdgcn_perm(hi, lo, z ? 0x07060302u : 0x05040100u);
+                    const uint32_t pair = __builtin_amdgcn_perm(hi, lo, z ? sel_hi : sel_lo);
                     const uint16_t cbits = (uint16_t)((29 - exl - code_shift(mm)) << 10);
                     const h2 mult = __builtin_bit_cast(h2, (uint32_t)cbits | ((uint32_t)cbits << 16));
                     v[dq] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, pair) * mult);
@@ -250,16 +277,20 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
         auto my_slice = [&](int step) -> int { return min(2 * step + parity, slices - 1); };  // weights: clamped
         u4 xr[4];
         load_x(xr, xpar);
+        // The first loads are issued in the order the loop issues them (activations, then tile by tile): the
+        // compiler's count of loads in flight at the top of the loop is the worse of the two ways into it.
+        __builtin_amdgcn_sched_barrier(0);
         Tile ring[kTilesPerWave];
 #pragma unroll
-        for (int k = 0; k < kTilesPerWave; k++) ring[k] = load_tile(k, my_slice(0));
-        Scales sc_next = load_scales(0, my_slice(0));
+        for (int k = 0; k < kTilesPerWave; k++) {
+            ring[k] = load_tile(k, my_slice(0));
+            __builtin_amdgcn_sched_barrier(0);
+        }
 
         for (int st = 0; st < steps; st++) {
             const int buf = st & 1;
-            const int s = my_slice(st);
-            build_image(xr, buf);
-            if (st + 1 < steps) load_x(xr, 2 * (st + 1) + xpar);
+            build_image(xr, buf, !x_live || 2 * st + xpar >= slices);
+            load_x(xr, 2 * (st + 1) + xpar);
             // one barrier per step: it publishes buffer `buf`; the other buffer is rewritten only in
             // the next iteration, after every wave has passed this barrier and so has finished
             // reading it into registers.
@@ -284,13 +315,16 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
 #pragma unroll
             for (int k = 0; k < kTilesPerWave; k++) {
                 Tile t = ring[k];
-                const Scales ts = sc_next;
-                // order matters: loads return in order, so the scales (needed by the next tile) are
-                // asked for before the masks of the next slice (needed four tiles from now)
-                sc_next = k + 1 < kTilesPerWave ? load_scales(k + 1, s) : load_scales(0, s_next);
-                ring[k] = load_tile(k, s_next);
-                transpose4(t.nz);
-                transpose4(t.sg);
+                transpose4x2(t.nz, t.sg);
+                // sq[v][h]: scales of row 4*lq + v, groups 2h and 2h + 1 of the slice
+                uint32_t sq[4][2];
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    sq[0][h] = quad_broadcast<0>(t.sc[h]);
+                    sq[1][h] = quad_broadcast<1>(t.sc[h]);
+                    sq[2][h] = quad_broadcast<2>(t.sc[h]);
+                    sq[3][h] = quad_broadcast<3>(t.sc[h]);
+                }
                 f4 r = {0.f, 0.f, 0.f, 0.f};
                 // the MFMAs of chunk c + 1 are issued before the results of chunk c are touched
                 f4 da[2];  // one chain of four MFMAs per scale group; two groups in flight
@@ -306,7 +340,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
                     const f4 d = da[c & 1] - bias[c];
 #pragma unroll
                     for (int v = 0; v < 4; v++) {
-                        const uint16_t sbits = (uint16_t)(ts.sc[v][c >> 1] >> (16 * (c & 1)));
+                        const uint16_t sbits = (uint16_t)(sq[v][c >> 1] >> (16 * (c & 1)));
                         r[v] += h2f(sbits) * d[v];
                     }
                 };
@@ -319,6 +353,13 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
                 __builtin_amdgcn_sched_barrier(0);
                 retire(1);
                 issue(3);
+                __builtin_amdgcn_sched_barrier(0);
+                // The next slice of this tile is asked for only now that the registers of this one are dead (the masks,
+                // in which the swaps above worked in place; the scales went to their quads at the top), so that the
+                // loads write the registers the loop carries: a request placed earlier loads into other registers, and
+                // the copies into the carried ones at the end of the step wait for every load in flight.
+                __builtin_amdgcn_sched_barrier(0);
+                ring[k] = load_tile(k, s_next);
                 __builtin_amdgcn_sched_barrier(0);
                 retire(2);
                 retire(3);

@@ -98,9 +98,11 @@ int tllm_quantize_absmax_i8(const uint16_t *input, int8_t *output, float *scale,
  * A fp16 [M,K] row-major, packed weight [N,K], C fp16 [M,N] row-major.
  * Replaces ternary::ternary_gemm, reference include/kernels.cuh:37-40
  * (kernels/ternary_gemm.cu:33-195). Any M >= 1 is accepted.
- * Allocation: none per call, with one exception: a workspace that belongs to (device, stream). Two kinds
+ * Allocation: none per call, with one exception: a workspace that belongs to (device, stream). Three kinds
  * of shapes use it. Shapes whose output tiles do not fill the chip, or not its last round (M > 16), split K
- * over several workgroups per tile, which exchange fp32 partial sums through it (at most 32 MiB); tall shapes
+ * over several workgroups per tile, which exchange fp32 partial sums through it (at most 32 MiB); so do shapes
+ * of 2 to 16 activation rows (and wider ones that run as passes of 16) with so few weight rows that their
+ * 64-row blocks would leave half the chip idle (N <= 64 * CUs / 2, K >= 4096: at most 1 MiB); tall shapes
  * whose K is not a multiple of 256 run a kernel that reads the activations from a copy in matrix-core
  * fragment order, which a small kernel writes there first (M rounded up to 32, times K, times 2 bytes; such
  * a shape is only chosen while that stays within TLLM_GEMM_STATIC_SCRATCH_BYTES). The first such call on a stream creates

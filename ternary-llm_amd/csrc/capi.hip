@@ -106,8 +106,7 @@ int tllm_gemm_workspace_reserve(int M, int N, int K, int group_size, tllm_stream
     if ((int64_t)M * K > INT32_MAX || (int64_t)M * N > INT32_MAX) return TLLM_ERR_TOO_LARGE;
     // only the shape matters here: the pointers are never dereferenced
     Problem p{nullptr, nullptr, nullptr, nullptr, nullptr, N, K, M, 0};
-    if (group_size != 128 || M <= 16) return TLLM_OK;  // paths that never split K
-    return (int)tllm::gemm_mfma_reserve(p, (hipStream_t)stream);
+    return (int)tllm::dispatch_reserve(p, group_size, (hipStream_t)stream);
 }
 
 void tllm_gemm_workspace_release(void) { tllm::gemm_mfma_release_all(); }

@@ -107,7 +107,12 @@ hipError_t launch_gemv_mfma_i8(const Problem &p, float scale_value, const float 
 
 // 128-group MFMA kernel for 2..16 activation rows, K a multiple of 512 (gemv_batch.hip).
 bool gemv_batch_supports(const Problem &p, int group);
-hipError_t launch_gemv_batch(const Problem &p, hipStream_t s);
+// fixed_scratch: a launch that shares out K among workgroups exchanges its sums through the library's fixed device
+// array instead of the stream's workspace (no allocation, ever).
+hipError_t launch_gemv_batch(const Problem &p, hipStream_t s, bool fixed_scratch = false);
+// Creates (or grows) the exchange workspace of stream s for this shape, if its launch would share out K at all.
+hipError_t gemv_batch_reserve(const Problem &p, hipStream_t s);
+const char *gemv_batch_kernel_name(const Problem &p);  // what launch_gemv_batch would run, given exchange memory (static string)
 int gemv_batch_block_rows();
 float gemv_batch_cost_us(const Problem &p);  // rough time of one launch_gemv_batch
 hipError_t launch_gemv_batch_table(const Problem *table, const int *unit_prefix, const int *wg_first, int grid,
@@ -119,6 +124,13 @@ bool gemm_mfma_supports(const Problem &p, int group);
 hipError_t launch_gemm_mfma(const Problem &p, hipStream_t s);
 float gemm_mfma_cost_us(const Problem &p);
 const char *gemm_mfma_kernel_name(const Problem &p);  // the kernel launch_gemm_mfma would run (static string)  // rough time of launch_gemm_mfma, to choose between kernels
+// Exchange memory for launches that share out K among workgroups (gemm_mfma.hip): `floats` fp32 slots and
+// kSplitArrivalSlots arrival counters that are zero between launches. fixed: the library's fixed device array
+// (*partial stays null if it is too small); else the workspace of (device, stream s), created or grown unless the
+// stream is being captured (then *partial stays null when what exists is too small). Launches on one stream run in
+// order and so may share it.
+constexpr int kSplitArrivalSlots = 1024;
+hipError_t split_exchange_memory(hipStream_t s, size_t floats, bool fixed, float **partial, unsigned **arrivals);
 // Creates (or grows) the split-K workspace of stream s for this shape, if the shape splits K at all.
 hipError_t gemm_mfma_reserve(const Problem &p, hipStream_t s);
 void gemm_mfma_release_all();  // frees every split-K workspace (nothing may still be running on them)
@@ -127,8 +139,10 @@ bool gemm_mfma_static_fits(const Problem &p);
 hipError_t launch_gemm_mfma_static(const Problem &p, hipStream_t s);
 
 // Picks the kernel for one linear (fast 128-group paths when they apply, else the row-wave kernel).
-// static_scratch: a GEMM that splits K exchanges its partial sums through the fixed device array.
+// static_scratch: a launch that splits K exchanges its partial sums through the fixed device array.
 hipError_t dispatch_linear(const Problem &p, int group, hipStream_t s, bool static_scratch = false);
+// Creates (or grows) the exchange workspace of stream s that dispatch_linear would use for this shape, if any.
+hipError_t dispatch_reserve(const Problem &p, int group, hipStream_t s);
 // True if dispatch_linear would run the prefill GEMM kernel (the only path that may need exchange memory).
 bool dispatch_takes_gemm(const Problem &p, int group);
 // Name of the kernel dispatch_linear would launch for this shape (static string; pointers may be null).

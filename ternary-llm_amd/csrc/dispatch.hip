@@ -51,7 +51,7 @@ hipError_t dispatch_linear(const Problem &p, int group, hipStream_t s, bool stat
             q.batch = p.batch - b0 < kBatchRows ? p.batch - b0 : kBatchRows;
             q.x = p.x + (size_t)b0 * p.cols;
             q.y = p.y + (size_t)b0 * p.rows;
-            if (hipError_t e = launch_gemv_batch(q, s)) return e;
+            if (hipError_t e = launch_gemv_batch(q, s, static_scratch)) return e;
         }
         return hipSuccess;
     }
@@ -72,10 +72,25 @@ hipError_t dispatch_linear(const Problem &p, int group, hipStream_t s, bool stat
 }
 
 
+hipError_t dispatch_reserve(const Problem &p, int group, hipStream_t s) {
+    if (group != 128 || (p.batch == 1 && gemv_mfma_supports(p, group))) return hipSuccess;
+    if (streams_in_passes(p, group)) {
+        Problem q = p;
+        q.batch = p.batch < kBatchRows ? p.batch : kBatchRows;
+        return gemv_batch_reserve(q, s);
+    }
+    if (gemv_mfma_supports(p, group) || !gemm_mfma_supports(p, group)) return hipSuccess;
+    return gemm_mfma_reserve(p, s);
+}
+
 const char *dispatch_kernel_name(const Problem &p, int group) {
     if (group != 128) return "tllm::gemv_rowwave_f16_kernel";
     if (p.batch == 1 && gemv_mfma_supports(p, group)) return "tllm::gemv_mfma_kernel";
-    if (streams_in_passes(p, group)) return "tllm::gemv_batch_kernel";
+    if (streams_in_passes(p, group)) {
+        Problem q = p;
+        q.batch = p.batch < kBatchRows ? p.batch : kBatchRows;
+        return gemv_batch_kernel_name(q);
+    }
     if (gemv_mfma_supports(p, group)) return "tllm::gemv_mfma_kernel<Tall>";
     if (gemm_mfma_supports(p, group)) return gemm_mfma_kernel_name(p);
     return "tllm::gemv_mfma_kernel<Tall>, passes";

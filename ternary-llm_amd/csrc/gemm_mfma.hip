@@ -1242,7 +1242,7 @@ struct SplitWorkspace {
     size_t floats = 0;
     unsigned *arrivals = nullptr;
 };
-constexpr size_t kArrivalSlots = 1024;  // tiles of a split launch (at most one per CU pair)
+constexpr size_t kArrivalSlots = kSplitArrivalSlots;  // tiles of a split launch (at most one per CU pair)
 std::mutex g_ws_mutex;
 std::vector<SplitWorkspace> g_ws;
 
@@ -1544,6 +1544,22 @@ hipError_t launch_config(const Problem &p, const GemmConfig &c, float *workspace
     return c.height == 1 ? launch<2>(p, c.splits, workspace, arrivals, s) : launch<1>(p, c.splits, workspace, arrivals, s);
 }
 }  // namespace
+
+hipError_t split_exchange_memory(hipStream_t s, size_t floats, bool fixed, float **partial, unsigned **arrivals) {
+    *partial = nullptr;
+    *arrivals = nullptr;
+    if (fixed) {
+        if (floats > kStaticSlotFloats) return hipSuccess;
+        unsigned char *base = nullptr;
+        if (hipError_t e = static_scratch(&base)) return e;
+        *arrivals = reinterpret_cast<unsigned *>(base);
+        *partial = reinterpret_cast<float *>(base) + kArrivalSlots;
+        return hipSuccess;
+    }
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipError_t e = hipStreamIsCapturing(s, &cap)) return e;
+    return split_workspace(s, floats, cap == hipStreamCaptureStatusNone, partial, arrivals);
+}
 
 hipError_t launch_gemm_mfma(const Problem &p, hipStream_t s) {
     GemmConfig c = choose_config(p, kStaticSlotFloats);

@@ -18,6 +18,8 @@
 // there are no atomics.
 // The "+1" of the code c = w + 1 is removed by subtracting the product of an all-zero weight row,
 // computed once per slice with the same instructions (exact zeros stay exact).
+#include <stdlib.h>
+
 #include "common.h"
 #include "gemv_layout.h"
 
@@ -54,6 +56,13 @@ struct BatchSched {
     int pool_begin, pool_end;
     const int *pool_problem;  // [pool_end - pool_begin] the problem each pool block is in
     int *counters;            // nullptr: no pool
+    // One problem with few rows and a long K: k_parts workgroups per block, each under its share of the steps
+    // (workgroup b works on block b / k_parts, part b % k_parts). Each part leaves its fp32 sums in its slot of
+    // `partial`; the part that arrives last at the block's counter in `arrivals` (zero before the launch, zero again
+    // after it) adds all slots in part order, its own included, so the bits do not depend on the order of arrival.
+    int k_parts;
+    float *partial;
+    unsigned *arrivals;
 };
 
 struct Tile {
@@ -125,11 +134,16 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
         pos_end = sc.wg_first[blockIdx.x + 1];
         pi = sc.wg_first[gridDim.x + 1 + blockIdx.x];  // no scan over the problems before the first block
         order = sc.wg_first + 2 * gridDim.x + 1;
+    } else if (sc.k_parts > 1) {
+        pos = blockIdx.x / sc.k_parts;
+        pos_end = pos + 1;
     } else {
         const int total = (single.rows + kBlockRows - 1) / kBlockRows;
         pos = (int)((int64_t)total * blockIdx.x / gridDim.x);
         pos_end = (int)((int64_t)total * (blockIdx.x + 1) / gridDim.x);
     }
+    const int k_parts = sc.k_parts > 1 ? sc.k_parts : 1;
+    const int k_part = sc.k_parts > 1 ? (int)(blockIdx.x % sc.k_parts) : 0;
 
     // operands of an all-zero weight row (every code = 1)
     uint32_t zero_o[16];
@@ -274,20 +288,21 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
         for (int k = 0; k < kTilesPerWave; k++) acc[k] = f4{0.f, 0.f, 0.f, 0.f};
 
         const int steps = (slices + 1) / 2;
+        const int st_begin = steps * k_part / k_parts, st_end = steps * (k_part + 1) / k_parts;
         auto my_slice = [&](int step) -> int { return min(2 * step + parity, slices - 1); };  // weights: clamped
         u4 xr[4];
-        load_x(xr, xpar);
+        load_x(xr, 2 * st_begin + xpar);
         // The first loads are issued in the order the loop issues them (activations, then tile by tile): the
         // compiler's count of loads in flight at the top of the loop is the worse of the two ways into it.
         __builtin_amdgcn_sched_barrier(0);
         Tile ring[kTilesPerWave];
 #pragma unroll
         for (int k = 0; k < kTilesPerWave; k++) {
-            ring[k] = load_tile(k, my_slice(0));
+            ring[k] = load_tile(k, my_slice(st_begin));
             __builtin_amdgcn_sched_barrier(0);
         }
 
-        for (int st = 0; st < steps; st++) {
+        for (int st = st_begin; st < st_end; st++) {
             const int buf = st & 1;
             build_image(xr, buf, !x_live || 2 * st + xpar >= slices);
             load_x(xr, 2 * (st + 1) + xpar);
@@ -311,7 +326,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
                 d0 = mfma16(zero_o + 12, B[4 * c + 3], d0);
                 bias[c] = d0;
             }
-            const int s_next = my_slice(min(st + 1, steps - 1));
+            const int s_next = my_slice(min(st + 1, st_end - 1));
 #pragma unroll
             for (int k = 0; k < kTilesPerWave; k++) {
                 Tile t = ring[k];
@@ -379,8 +394,50 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
                 for (int v = 0; v < 4; v++) hand[(k * 4 + v) * kWave + lane] = acc[k][v];
         }
         __syncthreads();
+        if (parity == 0) {
+#pragma unroll
+            for (int k = 0; k < kTilesPerWave; k++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) acc[k][v] += hand[(k * 4 + v) * kWave + lane];
+        }
+        bool stores = true;
+        if (k_parts > 1) {  // (the same for the whole workgroup)
+            // this part's sums into its slot, written through to memory: quad k of lane `lane` of wave `wave` at
+            // ((wave * kTilesPerWave + k) * 64 + lane) * 4 floats
+            constexpr int kSlot = 4 * kTilesPerWave * kWave * 4;
+            float *slots = sc.partial + (size_t)u * k_parts * kSlot + ((size_t)wave * kTilesPerWave * kWave + lane) * 4;
+            if (parity == 0) {
+#pragma unroll
+                for (int k = 0; k < kTilesPerWave; k++) {
+                    float *dst = slots + (size_t)k_part * kSlot + k * kWave * 4;
+                    const f4 v = acc[k];
+                    // (two idle issue slots: a store of more than 8 bytes still reads its data registers after it
+                    // has issued, and the compiler does not see inside the block)
+                    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(dst), "v"(v) : "memory");
+                }
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            }
+            __shared__ unsigned last_part;
+            __syncthreads();
+            if (tid == 0) {
+                const unsigned before = __hip_atomic_fetch_add(&sc.arrivals[u], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                last_part = before == (unsigned)k_parts - 1;
+                if (last_part) __hip_atomic_store(&sc.arrivals[u], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            __syncthreads();
+            stores = last_part != 0;
+            if (stores && parity == 0) {
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+#pragma unroll
+                for (int k = 0; k < kTilesPerWave; k++) acc[k] = f4{0.f, 0.f, 0.f, 0.f};
+                for (int q = 0; q < k_parts; q++)
+#pragma unroll
+                    for (int k = 0; k < kTilesPerWave; k++)
+                        acc[k] += *reinterpret_cast<const f4 *>(slots + (size_t)q * kSlot + k * kWave * 4);
+            }
+        }
         // lane (lq, li) holds rows first + 4*lq + v of activation row li
-        if (parity == 0 && li < p.batch) {
+        if (stores && parity == 0 && li < p.batch) {
 #pragma unroll
             for (int k = 0; k < kTilesPerWave; k++) {
                 if (4 * k + wave >= n_tiles) continue;
@@ -388,8 +445,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
                 const int first = tile_first_row(k, &skip);
 #pragma unroll
                 for (int v = 0; v < 4; v++)
-                    if (4 * lq + v >= skip)
-                        p.y[(size_t)li * p.rows + first + 4 * lq + v] = f2h(acc[k][v] + hand[(k * 4 + v) * kWave + lane]);
+                    if (4 * lq + v >= skip) p.y[(size_t)li * p.rows + first + 4 * lq + v] = f2h(acc[k][v]);
             }
         }
         if (request) pool_block = requested;
@@ -430,11 +486,15 @@ static hipError_t prepare_kernel() {
 }
 
 template <int T>
-static hipError_t launch_single(const Problem &p, int wgs, hipStream_t s) {
+static hipError_t launch_single(const Problem &p, int wgs, int k_parts, float *partial, unsigned *arrivals, hipStream_t s) {
     if (hipError_t e = prepare_kernel<T>()) return e;
     const int blocks = (p.rows + 64 * T - 1) / (64 * T);
-    BatchSched sc{nullptr, nullptr, nullptr};
-    gemv_batch_kernel<T><<<blocks < wgs ? blocks : wgs, kThreads, kLdsBytes, s>>>(p, sc);
+    BatchSched sc{};
+    sc.k_parts = k_parts;
+    sc.partial = partial;
+    sc.arrivals = arrivals;
+    const int grid = k_parts > 1 ? blocks * k_parts : blocks < wgs ? blocks : wgs;
+    gemv_batch_kernel<T><<<grid, kThreads, kLdsBytes, s>>>(p, sc);
     return hipGetLastError();
 }
 
@@ -445,26 +505,80 @@ static int single_tiles(const Problem &p, int cus) {
     return 1;
 }
 
-hipError_t launch_gemv_batch(const Problem &p, hipStream_t s) {
+// Time of one matrix alone in 64-row blocks whose steps are shared out among `parts` workgroups each, in us, fitted to
+// eleven shapes of 512 to 8192 rows and 4096 to 28672 columns (within 1.5 us on all of them): 3 us of launch and
+// ramp, 1.78 us per step of 1024 columns, and for the exchange 1.5 us + 0.2 us per part + 0.027 us per workgroup of the
+// launch (256 workgroups start and arrive noticeably later than 64).
+static float single_split_us(int blocks, int steps, int parts) {
+    const float chain = 3.0f + 1.78f * (float)((steps + parts - 1) / parts);
+    return parts > 1 ? chain + 1.5f + 0.2f * (float)parts + 0.027f * (float)(blocks * parts) : chain;
+}
+
+// Workgroups per 64-row block along K for one matrix alone: with so few rows that CUs would stay without a block,
+// the steps of a block may be shared out among up to 8 workgroups, as many as the estimate above likes best.
+static int single_k_parts(const Problem &p, int cus) {
+    if (single_tiles(p, cus) != 1) return 1;
+    const int blocks = (p.rows + 63) / 64;
+    const int steps = (p.cols / kSliceCols + 1) / 2;
+    int most = cus / blocks;
+    if (most > steps) most = steps;
+    if (most > 8) most = 8;
+    if (most < 2 || blocks > kSplitArrivalSlots) return 1;
+    // TLLM_BATCH_K_PARTS=n (a tuning aid, read at every call): n parts where they fit, 1 = never share out K
+    const char *env = getenv("TLLM_BATCH_K_PARTS");
+    const int forced = env ? atoi(env) : 0;
+    if (forced > 0) return forced < most ? forced : most;
+    int best = 1;
+    for (int parts = 2; parts <= most; parts++)
+        if (single_split_us(blocks, steps, parts) < single_split_us(blocks, steps, best)) best = parts;
+    return best;
+}
+static size_t single_exchange_floats(const Problem &p, int parts) {
+    return (size_t)((p.rows + 63) / 64) * parts * (4 * kWave * 4);
+}
+
+hipError_t launch_gemv_batch(const Problem &p, hipStream_t s, bool fixed_scratch) {
     const int cus = device_cus();  // one workgroup of 8 waves per CU
-    switch (single_tiles(p, cus)) {
-        case 4: return launch_single<4>(p, cus, s);
-        case 2: return launch_single<2>(p, cus, s);
-        default: return launch_single<1>(p, cus, s);
+    int parts = single_k_parts(p, cus);
+    float *partial = nullptr;
+    unsigned *arrivals = nullptr;
+    if (parts > 1) {
+        // (no exchange memory to be had, e.g. under stream capture without a reserved workspace: one workgroup per block)
+        if (hipError_t e = split_exchange_memory(s, single_exchange_floats(p, parts), fixed_scratch, &partial, &arrivals)) return e;
+        if (!partial) parts = 1;
     }
+    switch (single_tiles(p, cus)) {
+        case 4: return launch_single<4>(p, cus, 1, nullptr, nullptr, s);
+        case 2: return launch_single<2>(p, cus, 1, nullptr, nullptr, s);
+        default: return launch_single<1>(p, cus, parts, partial, arrivals, s);
+    }
+}
+
+const char *gemv_batch_kernel_name(const Problem &p) {
+    return single_k_parts(p, device_cus()) > 1 ? "tllm::gemv_batch_kernel, K shared out" : "tllm::gemv_batch_kernel";
+}
+
+hipError_t gemv_batch_reserve(const Problem &p, hipStream_t s) {
+    const int parts = single_k_parts(p, device_cus());
+    float *partial = nullptr;
+    unsigned *arrivals = nullptr;
+    return parts > 1 ? split_exchange_memory(s, single_exchange_floats(p, parts), false, &partial, &arrivals) : hipSuccess;
 }
 
 float gemv_batch_cost_us(const Problem &p) {
     // measured on single matrices: 3 us of launch and ramp, then the larger of the streaming time
     // (a workgroup moves about 17 bytes of packed weights per ns with 256-row blocks, 13 with 64-row
-    // blocks) and the latency chain of the K loop (1.8 us per step of 1024 columns)
+    // blocks) and the latency chain of the K loop (1.8 us per step of 1024 columns; single_split_us when
+    // the steps of a block are shared out)
     const int cus = device_cus();
     const int t = single_tiles(p, cus);
+    const int parts = single_k_parts(p, cus);
     const int blocks = (p.rows + 64 * t - 1) / (64 * t);
-    const float rate = (t == 4 ? 17.0e3f : t == 2 ? 15.0e3f : 13.0e3f) * (float)(blocks < cus ? blocks : cus);
-    const float stream = 0.265625f * (float)p.rows * (float)p.cols / rate;
-    const float chain = 1.8f * (float)((p.cols / kSliceCols + 1) / 2);
-    return 3.0f + (stream > chain ? stream : chain);
+    const int wgs = blocks * parts;
+    const float rate = (t == 4 ? 17.0e3f : t == 2 ? 15.0e3f : 13.0e3f) * (float)(wgs < cus ? wgs : cus);
+    const float stream = 3.0f + 0.265625f * (float)p.rows * (float)p.cols / rate;
+    const float chain = single_split_us(blocks, (p.cols / kSliceCols + 1) / 2, parts);
+    return stream > chain ? stream : chain;
 }
 
 int gemv_batch_block_rows() { return 64 * kMaxTilesPerWave; }
@@ -474,7 +588,7 @@ hipError_t launch_gemv_batch_table(const Problem *table, const int *unit_prefix,
                                    hipStream_t s) {
     if (hipError_t e = prepare_kernel<kMaxTilesPerWave>()) return e;
     BatchSched sc{table, unit_prefix, wg_first, pool_begin, pool_end, pool_problem,
-                  pool_end > pool_begin ? counters : nullptr};
+                  pool_end > pool_begin ? counters : nullptr, 1, nullptr, nullptr};
     Problem none{};
     gemv_batch_kernel<kMaxTilesPerWave><<<grid, kThreads, kLdsBytes, s>>>(none, sc);
     return hipGetLastError();

@@ -429,8 +429,9 @@ def test_batched_decode_special_cases(dev, oracle):
 def test_batched_plan_8b_layer_batch4_and_16(dev, oracle):
     """One LLaMA-3-8B-shaped layer (7 projections, rows cut to keep the oracle fast) as a plan at
     batch 2, 3, 4 and 16: sampled rows == oracle; at batch 16 the plan runs the kernel of the single
-    call, so its output equals the single call's bit for bit (up to 4 the plan takes the tall-tile
-    kernel, which stages the 14336-column rows in segments)."""
+    call, so its output equals the single call's bit for bit, unless the single call shares out K among
+    workgroups, which adds the fp32 sums in another order (up to 4 the plan takes the tall-tile kernel,
+    which stages the 14336-column rows in segments)."""
     torch, tl = dev
     shapes = [(512, 4096), (128, 4096), (128, 4096), (512, 4096), (1800, 4096), (1800, 4096), (520, 14336)]
     for batch in (2, 3, 4, 16):
@@ -450,7 +451,7 @@ def test_batched_plan_8b_layer_batch4_and_16(dev, oracle):
             for k, (pr, (nz, sg, s, x)) in enumerate(zip(probs, host)):
                 got = pr[4].cpu().numpy()
                 single = run_gemm(dev, x, nz, sg, s)
-                if batch > 4:
+                if batch > 4 and "shared out" not in tl.gemm_kernel(batch, pr[5], pr[6]):
                     assert np.array_equal(got.astype(np.float64), single), f"batch {batch} problem {k}: plan != single call"
                 rows_s = np.unique(np.random.default_rng(k).integers(0, nz.shape[0], 64))
                 ref = oracle.gemm_f64(x.view(np.uint16), nz[rows_s], sg[rows_s], s[rows_s].view(np.uint16))
@@ -1327,6 +1328,68 @@ def test_gemm_every_output_against_dense_product(dev, oracle, M, N, K):
                 bad = int((~(rel <= TOL)).sum().item())
                 assert bad == 0, (f"gemm {M}x{N}x{K} ({tl.gemm_kernel(M, N, K)}, forced={force}, repetition {rep}): "
                                   f"{bad} of {M * N} outputs beyond {TOL}, max_rel {float(rel.max()):.3e}")
+
+
+@pytest.mark.parametrize("M,N,K", [
+    (16, 4096, 14336),   # 64 blocks of 64 rows, four workgroups each
+    (9, 1000, 4096),     # ragged last block, two parts of two steps
+    (16, 192, 6144),     # three parts
+    (5, 64, 28672),      # one block, eight parts
+    (16, 320, 3584),     # an odd number of 512-column slices
+    (24, 128, 8192),     # more than 16 activation rows: passes of the same launch, or the prefill kernel (the library's choice)
+])
+def test_batched_decode_k_shared_out_every_output(dev, oracle, M, N, K):
+    """Few weight rows under a long K: the steps of a 64-row block are shared out among several workgroups, which
+    exchange fp32 sums through the stream's workspace. Every output against the fp32 product of the expanded
+    weights (itself sampled against the fp64 oracle); repeated calls give the same bits (the sums are added in part
+    order whichever part arrives last); the entry point with the fixed exchange array gives the same bits; a
+    captured graph without a reserved workspace (no exchange: one workgroup per block) stays within tolerance."""
+    torch, tl = dev
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(7300 + M + N + K)
+    nz, sg, sc = _device_problem(torch, N, K, 0.42, 0.01, 0.03, gen)
+    nz[N // 2] = 0  # a row without weights: exact zeros from every part
+    A = torch.randn((M, K), device="cuda", generator=gen).to(torch.float16)
+    W = _dense_weights(torch, nz, sg, sc)
+    ref = A.float() @ W.t()
+    del W
+    _check_sampled(oracle, torch, A, nz, sg, sc, ref, 4, 40, M + K, f"dense fp32 product {M}x{N}x{K}")
+    if M <= 16:
+        assert "K shared out" in tl.gemm_kernel(M, N, K)
+    tau = float(torch.sqrt(torch.mean(ref * ref)).item()) / 64.0
+
+    def check(Cm, what):
+        rel = (Cm.float() - ref).abs() / torch.clamp(ref.abs(), min=tau)
+        bad = int((~(rel <= TOL)).sum().item())
+        assert bad == 0, f"{what} {M}x{N}x{K}: {bad} of {M * N} outputs beyond {TOL}, max_rel {float(rel.max()):.3e}"
+        assert bool((Cm[:, N // 2] == 0).all()), f"{what}: a row without weights must give exact zeros"
+
+    outs = []
+    for rep in range(3):
+        Cm = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+        tl.ternary_gemm(A, nz, sg, sc, Cm, M, N, K, 128)
+        torch.cuda.synchronize()
+        check(Cm, f"call {rep}")
+        outs.append(Cm.view(torch.int16).clone())
+    assert all(bool((o == outs[0]).all()) for o in outs[1:]), "repeated calls differ in bits"
+    Cs = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    tl.ternary_gemm_static(A, nz, sg, sc, Cs, M, N, K, 128)
+    torch.cuda.synchronize()
+    assert bool((Cs.view(torch.int16) == outs[0]).all()), "fixed exchange array: bits differ from the workspace's"
+    # under capture on a stream that has no workspace nothing may be allocated: the launch takes no exchange
+    st = torch.cuda.Stream()
+    Cg = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(st):
+        with torch.cuda.graph(g, stream=st):
+            tl.ternary_gemm(A, nz, sg, sc, Cg, M, N, K, 128, stream=st)
+    torch.cuda.synchronize()
+    for rep in range(2):
+        Cg.fill_(float("nan"))
+        g.replay()
+        torch.cuda.synchronize()
+        check(Cg, f"graph replay {rep} without a workspace")
 
 
 @pytest.mark.parametrize("batch", [1, 2, 4, 16])

@@ -341,33 +341,36 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
                     sq[3][h] = quad_broadcast<3>(t.sc[h]);
                 }
                 f4 r = {0.f, 0.f, 0.f, 0.f};
-                // the MFMAs of chunk c + 1 are issued before the results of chunk c are touched
-                f4 da[2];  // one chain of four MFMAs per scale group; two groups in flight
-                auto issue = [&](int c) {
-                    uint32_t o[16];
-                    decode_word(t.nz[c], t.sg[c], o);
-                    da[c & 1] = mfma16(o + 0, B[4 * c + 0], f4{0.f, 0.f, 0.f, 0.f});
-                    da[c & 1] = mfma16(o + 4, B[4 * c + 1], da[c & 1]);
-                    da[c & 1] = mfma16(o + 8, B[4 * c + 2], da[c & 1]);
-                    da[c & 1] = mfma16(o + 12, B[4 * c + 3], da[c & 1]);
+                // One chain of four MFMAs per scale group. The chains of two groups are issued alternately, so that an
+                // MFMA never follows the one it depends on directly, and the results of the first pair are touched only
+                // after the second pair has been issued (+ 1 % against one chain after the other).
+                f4 da[2], db[2];
+                auto issue_pair = [&](int c, f4 (&d)[2]) {
+                    uint32_t o0[16], o1[16];
+                    decode_word(t.nz[c], t.sg[c], o0);
+                    decode_word(t.nz[c + 1], t.sg[c + 1], o1);
+                    d[0] = mfma16(o0 + 0, B[4 * c + 0], f4{0.f, 0.f, 0.f, 0.f});
+                    d[1] = mfma16(o1 + 0, B[4 * c + 4], f4{0.f, 0.f, 0.f, 0.f});
+                    d[0] = mfma16(o0 + 4, B[4 * c + 1], d[0]);
+                    d[1] = mfma16(o1 + 4, B[4 * c + 5], d[1]);
+                    d[0] = mfma16(o0 + 8, B[4 * c + 2], d[0]);
+                    d[1] = mfma16(o1 + 8, B[4 * c + 6], d[1]);
+                    d[0] = mfma16(o0 + 12, B[4 * c + 3], d[0]);
+                    d[1] = mfma16(o1 + 12, B[4 * c + 7], d[1]);
                 };
-                auto retire = [&](int c) {
-                    const f4 d = da[c & 1] - bias[c];
+                auto retire = [&](int c, const f4 &dc) {
+                    const f4 d = dc - bias[c];
 #pragma unroll
                     for (int v = 0; v < 4; v++) {
                         const uint16_t sbits = (uint16_t)(sq[v][c >> 1] >> (16 * (c & 1)));
                         r[v] += h2f(sbits) * d[v];
                     }
                 };
-                issue(0);
+                issue_pair(0, da);
                 __builtin_amdgcn_sched_barrier(0);
-                issue(1);
-                __builtin_amdgcn_sched_barrier(0);
-                retire(0);
-                issue(2);
-                __builtin_amdgcn_sched_barrier(0);
-                retire(1);
-                issue(3);
+                issue_pair(2, db);
+                retire(0, da[0]);
+                retire(1, da[1]);
                 __builtin_amdgcn_sched_barrier(0);
                 // The next slice of this tile is asked for only now that the registers of this one are dead (the masks,
                 // in which the swaps above worked in place; the scales went to their quads at the top), so that the
@@ -376,8 +379,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
                 __builtin_amdgcn_sched_barrier(0);
                 ring[k] = load_tile(k, s_next);
                 __builtin_amdgcn_sched_barrier(0);
-                retire(2);
-                retire(3);
+                retire(2, db[0]);
+                retire(3, db[1]);
                 acc[k] += r * scale_j;
                 __builtin_amdgcn_sched_barrier(0);
             }

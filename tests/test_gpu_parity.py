@@ -1390,6 +1390,22 @@ def test_batched_decode_k_shared_out_every_output(dev, oracle, M, N, K):
         g.replay()
         torch.cuda.synchronize()
         check(Cg, f"graph replay {rep} without a workspace")
+    # with a workspace reserved for the capture stream the captured launch shares out K like the eager one
+    st2 = torch.cuda.Stream()
+    tl.gemm_workspace_reserve(M, N, K, 128, stream=st2)
+    Ch = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    torch.cuda.synchronize()
+    g2 = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(st2):
+        with torch.cuda.graph(g2, stream=st2):
+            tl.ternary_gemm(A, nz, sg, sc, Ch, M, N, K, 128, stream=st2)
+    torch.cuda.synchronize()
+    for rep in range(3):
+        Ch.fill_(float("nan"))
+        torch.cuda.synchronize()
+        g2.replay()
+        torch.cuda.synchronize()
+        assert bool((Ch.view(torch.int16) == outs[0]).all()), f"graph replay {rep} with a reserved workspace: bits differ"
 
 
 @pytest.mark.parametrize("batch", [1, 2, 4, 16])

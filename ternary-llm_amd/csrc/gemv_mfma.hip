@@ -901,7 +901,7 @@ constexpr int64_t kPoolTaskWeights = TLLM_POOL_TASK_WEIGHTS;
 double block_pool_fraction() {
     static const double f = [] {
         const char *e = getenv("TLLM_BLOCK_POOL_FRACTION");
-        const double v = e ? atof(e) : 0.25;
+        const double v = e ? atof(e) : 0.4;
         return v < 0.0 ? 0.0 : v > 0.9 ? 0.9 : v;
     }();
     return f;

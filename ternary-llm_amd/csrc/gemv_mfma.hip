@@ -54,19 +54,17 @@ constexpr int kSegSlices = 8;
 __host__ __device__ constexpr int tall_seg_slices(int batch) { return 8192 / 512 / batch; }
 constexpr int kThreads = kNW * kWave;
 constexpr int kMaxBatch = 4;  // activation rows the tall tiles carry
-#ifndef TLLM_TILES_AHEAD
-#define TLLM_TILES_AHEAD 3
-#endif
-constexpr int kTilesAhead = TLLM_TILES_AHEAD;  // tile loads in flight per wave (register ring, unrolled)
-
+// kAhead of a tile geometry: tile loads in flight per wave (register ring, unrolled). Wide tiles: two, three and four
+// give the same rate. Tall tiles: two are 9 - 11 % faster than three on the 8B sweep at two and four activation rows
+// (and four 8 % slower): their units and chunks are then 128 rows instead of 192, and the ring takes 16 registers less.
 struct Wide {
-    static constexpr int kCols = 2048, kRows = 4, kChunks = 16, kScales = 1, kWgPerCu = 3;
+    static constexpr int kCols = 2048, kRows = 4, kChunks = 16, kScales = 1, kWgPerCu = 3, kAhead = 3;
 };
 struct Tall {
-    static constexpr int kCols = 512, kRows = 16, kChunks = 4, kScales = 4, kWgPerCu = 3;
+    static constexpr int kCols = 512, kRows = 16, kChunks = 4, kScales = 4, kWgPerCu = 3, kAhead = 2;
 };
 
-// Work is counted in units of kNW * kRows * kTilesAhead rows of one matrix. A workgroup owns a
+// Work is counted in units of kNW * kRows * kAhead rows of one matrix. A workgroup owns a
 // contiguous span of units (of about equal weight, cut by the host) and processes it in tasks of
 // up to max_units units that stay inside one matrix.
 struct Sched {
@@ -157,7 +155,7 @@ __device__ __forceinline__ f4 tile_product(const u4 nz, const u4 sg, const u4 (&
 
 // kExtras: the table may hold SwiGLU pairs and RMSNorm prologues (a separate instance, so that plans
 // without them keep the register allocation of the plain kernel).
-// kFine: units of one tile per wave (16 rows for wide tiles) instead of kTilesAhead, for launches
+// kFine: units of one tile per wave (16 rows for wide tiles) instead of kAhead, for launches
 // that would otherwise leave most of the chip's workgroup slots empty; the tile ring then runs
 // across the walks of a wave and the B operands are reloaded for every tile.
 template <class G, bool kExtras = false, bool kFine = false>
@@ -179,7 +177,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
     const int li = lane & 15;  // MFMA A row / D column
     const int lq = lane >> 4;  // MFMA k quarter / D row quad
 
-    constexpr int kUnitRows = kNW * G::kRows * (kFine ? 1 : kTilesAhead);
+    constexpr int kUnitRows = kNW * G::kRows * (kFine ? 1 : G::kAhead);
     int u = 0, u_end = 0, pi = 0;
     if (sc.table) {
         u = sc.wg_first[blockIdx.x];
@@ -487,7 +485,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
         // the waves round-robin, so at any time the waves of a workgroup work on neighbouring
         // slices of the same rows: the cache lines of a row (masks and, above all, the 2-byte
         // scales) are fetched from HBM once and shared, not once per slice.
-        // chunk size: a quarter of the rows that exist, rounded up to whole groups of kTilesAhead tiles
+        // chunk size: a quarter of the rows that exist, rounded up to whole groups of G::kAhead tiles
         const int chunk_rows = ((r_end - r_begin + kNW - 1) / kNW + kUnitRows / kNW - 1) / (kUnitRows / kNW) * (kUnitRows / kNW);
         const int n_walks = kNW * seg_n;
         const int my_walks = seg_n;  // walks wave, wave + kNW, ...
@@ -564,15 +562,15 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
         };
 
         // rows of chunk c that exist, as a number of tiles; slots round that up to whole groups of
-        // kTilesAhead (slots past the live tiles re-read the last one, their results are dropped)
+        // G::kAhead (slots past the live tiles re-read the last one, their results are dropped)
         auto chunk_tiles = [&](int c) -> int {
             const int rows_c = max(0, min(r_end - (r_begin + c * chunk_rows), chunk_rows));
             return (rows_c + G::kRows - 1) / G::kRows;
         };
-        const int n_slots = chunk_rows / G::kRows;  // a multiple of kTilesAhead
+        const int n_slots = chunk_rows / G::kRows;  // a multiple of G::kAhead
 
         {
-            // Load cursor over this wave's walks; it runs kTilesAhead slots ahead of the compute
+            // Load cursor over this wave's walks; it runs G::kAhead slots ahead of the compute
             // loop, across walks. Walks of chunks without rows are skipped by both cursors alike.
             int l_walk = wave, l_slot = 0;
             auto next_load = [&]() -> Tile<G> {
@@ -584,9 +582,9 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                 if (++l_slot == n_slots) { l_slot = 0; l_walk += kNW; }
                 return t;
             };
-            Tile<G> ring[kTilesAhead];
+            Tile<G> ring[G::kAhead];
 #pragma unroll
-            for (int k = 0; k < kTilesAhead; k++) {
+            for (int k = 0; k < G::kAhead; k++) {
                 ring[k] = next_load();
                 __builtin_amdgcn_sched_barrier(0);  // same issue order as in the loop below
             }
@@ -663,9 +661,9 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                 float bias_sel = 0.0f;
                 int wi = 0, j = 0, c_begin = 0, n_rb = 0;
                 const int total = my_walks * n_slots;
-                for (int t0 = 0; t0 < total; t0 += kTilesAhead) {
+                for (int t0 = 0; t0 < total; t0 += G::kAhead) {
 #pragma unroll
-                    for (int k = 0; k < kTilesAhead; k++) {
+                    for (int k = 0; k < G::kAhead; k++) {
                         if (t0 + k < total) {
                             if (j == 0) {
                                 const int walk = wave + wi * kNW;
@@ -708,10 +706,10 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                 auto process = [&](const Tile<G> &t, int rb, bool live) { process_tile(t, rb, live, B, bias, bias_sel); };
 
                 // No branch surrounds a load or an MFMA, so the wait counters stay exact and
-                // kTilesAhead - 1 tiles remain in flight while one is consumed.
-                for (int j = 0; j < n_slots; j += kTilesAhead) {
+                // G::kAhead - 1 tiles remain in flight while one is consumed.
+                for (int j = 0; j < n_slots; j += G::kAhead) {
 #pragma unroll
-                    for (int k = 0; k < kTilesAhead; k++) {
+                    for (int k = 0; k < G::kAhead; k++) {
                         process(ring[k], c_begin + min(j + k, max(n_rb, 1) - 1) * G::kRows, j + k < n_rb);
                         ring[k] = next_load();
                         // keep the scheduler from interleaving whole tiles: that would need the
@@ -813,8 +811,8 @@ int resident_wgs(size_t lds_bytes) {
 }
 
 template <class G>
-constexpr int range_unit() {  // rows: every wave walks whole groups of kTilesAhead tiles
-    return kNW * G::kRows * kTilesAhead;
+constexpr int range_unit() {  // rows: every wave walks whole groups of G::kAhead tiles
+    return kNW * G::kRows * G::kAhead;
 }
 constexpr int kFineUnit = kNW * Wide::kRows;  // rows of a unit of the fine-grained instances: one tile per wave
 constexpr int kTallFineUnit = kNW * Tall::kRows;
@@ -1174,7 +1172,7 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
     // (both variables are read at every plan creation, not once per process)
     const char *env_batch = getenv("TLLM_TALL_MAX_BATCH");
     const int tall_max_batch = env_batch ? atoi(env_batch) : 4;
-    // ... for plans large enough: its units (192 rows of one matrix) are what spans are cut in, and a
+    // ... for plans large enough: its units (128 rows of one matrix) are what spans are cut in, and a
     // unit of a long-row matrix must not outweigh a workgroup's share of the plan by much (8B shapes:
     // the tall tiles win from 12 layers on, share 1.2, and lose at 8; 70B: lose at 8 layers, share
     // 1.6, win at 20, share 4). TLLM_TALL_MIN_SHARE overrides the ratio.

@@ -54,11 +54,13 @@ constexpr int kSegSlices = 8;
 __host__ __device__ constexpr int tall_seg_slices(int batch) { return 8192 / 512 / batch; }
 constexpr int kThreads = kNW * kWave;
 constexpr int kMaxBatch = 4;  // activation rows the tall tiles carry
-// kAhead of a tile geometry: tile loads in flight per wave (register ring, unrolled). Wide tiles: two, three and four
-// give the same rate. Tall tiles: two are 9 - 11 % faster than three on the 8B sweep at two and four activation rows
-// (and four 8 % slower): their units and chunks are then 128 rows instead of 192, and the ring takes 16 registers less.
+// kAhead of a tile geometry: tile loads in flight per wave (register ring, unrolled) = tiles per wave in a unit of work.
+// Wide tiles: two, three and four give the same rate on long plans (8B sweep within 0.5 %); two make units of 32 rows
+// instead of 48 and leave more registers to the rest, which takes 6 % off a single call and 5 % off the 16-layer 1B
+// plan. Tall tiles: two are 9 - 11 % faster than three on the 8B sweep at two and four activation rows (one 13 % and
+// four 8 % slower): units of 128 rows, and the kernel fits its 168 registers without spilling.
 struct Wide {
-    static constexpr int kCols = 2048, kRows = 4, kChunks = 16, kScales = 1, kWgPerCu = 3, kAhead = 3;
+    static constexpr int kCols = 2048, kRows = 4, kChunks = 16, kScales = 1, kWgPerCu = 3, kAhead = 2;
 };
 struct Tall {
     static constexpr int kCols = 512, kRows = 16, kChunks = 4, kScales = 4, kWgPerCu = 3, kAhead = 2;
@@ -816,10 +818,12 @@ constexpr int range_unit() {  // rows: every wave walks whole groups of G::kAhea
 }
 constexpr int kFineUnit = kNW * Wide::kRows;  // rows of a unit of the fine-grained instances: one tile per wave
 constexpr int kTallFineUnit = kNW * Tall::kRows;
-// A launch with fewer than six 48-row units per workgroup slot of the chip runs in units of 16 rows
-// instead: the spans end closer together (8B shapes, one launch for 1 / 2 / 4 layers: 24.9 -> 21.1,
-// 37.4 -> 33.2, 57.5 -> 49.2 us; at 8 layers, nine units per slot, the coarse units win again).
-bool wants_fine(int64_t coarse_units, int slots) { return coarse_units <= 6 * (int64_t)slots; }
+// A launch with no more 32-row units than the chip has workgroup slots runs in units of 16 rows instead (one tile per
+// wave): a single matrix of the 8B shapes takes 9.2 us per call so against 9.6 us. Beyond one unit per slot the coarse
+// units win (8B shapes, one plan launch for 2 / 3 / 4 / 6 / 8 layers, i.e. 3.5 to 14 units per slot: 32.2 / 46.0 / 51.0 /
+// 67.7 / 90.0 us against 35.9 / 49.9 / 57.8 / 78.9 / 99.1 us in units of 16 rows; the gate/up plan of a decode step,
+// 1.2 units per slot, 4 us faster; only one whole layer, 1.75 per slot, loses 0.5 us of 22).
+bool wants_fine(int64_t coarse_units, int slots) { return coarse_units <= (int64_t)slots; }
 
 template <class G>
 int image_bytes_of(int cols, int batch, bool segmented = true) {

@@ -1176,13 +1176,13 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
     // (both variables are read at every plan creation, not once per process)
     const char *env_batch = getenv("TLLM_TALL_MAX_BATCH");
     const int tall_max_batch = env_batch ? atoi(env_batch) : 4;
-    // ... for plans large enough: its units (128 rows of one matrix) are what spans are cut in, and a
-    // unit of a long-row matrix must not outweigh a workgroup's share of the plan by much (8B shapes:
-    // the tall tiles win from 12 layers on, share 1.2, and lose at 8; 70B: lose at 8 layers, share
-    // 1.6, win at 20, share 4). TLLM_TALL_MIN_SHARE overrides the ratio.
-    // Medium plans take the tall tiles in units of 64 rows (one tile per wave) when a share is at least
-    // 3.5 of those (8B shapes at 12 layers, share 3.7: +16 % at two rows, +9 % at three; 70B at 8
-    // layers, share 4.9: +18 % / +8 %; shares of 2.5 and less lose against the batched kernel).
+    // ... for plans large enough: its units (128 rows of one matrix) are what spans are cut in, and a unit of a
+    // long-row matrix must not outweigh a workgroup's share of the plan: the tall tiles are taken from a share of one
+    // unit on (TLLM_TALL_MIN_SHARE overrides the ratio), and in units of 64 rows (one tile per wave) from a share of
+    // 1.75 of those. One plan launch, us, batched kernel / tall tiles, at four activation rows: 8B shapes 2, 4, 6, 8, 12
+    // layers (shares 0.3 to 1.8): 77 / 93, 97 / 119, 155 / 154, 178 / 165, 246 / 212; 70B 1, 2, 4, 8 layers (0.3 to
+    // 2.4): 142 / 177, 211 / 234, 345 / 332, 587 / 563. At two rows the tall tiles win from 6 layers of 8B (154 / 133)
+    // and 2 of 70B (211 / 198) on.
     bool tall_pays = all_tall && max_batch <= tall_max_batch, tall_fine = false;
     if (tall_pays) {
         int64_t total = 0;
@@ -1192,7 +1192,7 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
             max_cols = std::max(max_cols, (int)p.cols);
         }
         const char *env_share = getenv("TLLM_TALL_MIN_SHARE");
-        const double min_share = env_share ? atof(env_share) : 2.0;
+        const double min_share = env_share ? atof(env_share) : 1.0;
         const double share = (double)total / (Tall::kWgPerCu * di->cus);
         tall_pays = share >= min_share * (double)range_unit<Tall>() * max_cols;
         if (!tall_pays) tall_pays = tall_fine = share >= 1.75 * min_share * (double)kTallFineUnit * max_cols;

@@ -493,13 +493,13 @@ def test_tall_tile_plan_with_batch_columns(dev, oracle, batch, monkeypatch):
 
 def test_tall_tile_plan_in_fine_units(dev, oracle, monkeypatch):
     """A plan of two activation rows sized so that the tall tiles run in units of 64 rows (a share
-    per workgroup of more than 3.5 and less than 4 such units, i.e. less than two of the ordinary
+    per workgroup of more than 1.75 and less than 2 such units, i.e. less than one of the ordinary
     units of 128 rows): sampled rows against the oracle."""
     torch, tl = dev
     gen = torch.Generator(device="cuda")
     gen.manual_seed(99)
     batch, probs = 2, []
-    for rows, cols in [(20000, 4096)] * 12 + [(9000, 14336)] * 6 + [(20000, 4096)] * 12:
+    for rows, cols in [(5600, 4096)] * 12 + [(9000, 14336)] * 6 + [(5600, 4096)] * 12:
         w = _rand_weight(torch, gen, rows, cols)
         x = torch.randn((batch, cols), device="cuda", generator=gen).to(torch.float16)
         y = torch.full((batch, rows), float("nan"), dtype=torch.float16, device="cuda")

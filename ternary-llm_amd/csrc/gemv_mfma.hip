@@ -884,13 +884,15 @@ double span_share(int wg, int cus, int grid) {
 // Part of a large plan's weights that is kept out of the spans and dealt out at run time in pieces
 // of about kPoolTaskWeights weights: spans of the right average size still do not end together
 // (+-4 % from workgroup to workgroup and launch to launch), and the last workgroup sets the time.
-// Measured on the 8B sweep in steady state: 0 -> 5375 GB/s, 0.10 -> 5495, 0.15 -> 5517, 0.30 slower
-// again (a pool task of 768 K weights spends a quarter of its 25 us on staging and hand-over).
+// Measured on the 8B sweep in steady state with units of 48 rows: 0 -> 5375 GB/s, 0.10 -> 5495, 0.15 -> 5517, 0.30
+// slower again (a pool task of 768 K weights spends a quarter of its 25 us on staging and hand-over); with the
+// units of 32 rows the spans end closer together and a smaller pool is enough: 0 -> 5766, 0.03 -> 5816, 0.05 -> 5865,
+// 0.07 -> 5830, 0.10 -> 5817, 0.15 -> 5770, 0.30 -> 5648 (70B, 80 layers: 0.15 -> 5865, 0.05 -> 5895).
 // TLLM_POOL_FRACTION overrides it (0 switches the pool off).
 double pool_fraction() {
     static const double f = [] {
         const char *e = getenv("TLLM_POOL_FRACTION");
-        const double v = e ? atof(e) : 0.15;
+        const double v = e ? atof(e) : 0.05;
         return v < 0.0 ? 0.0 : v > 0.5 ? 0.5 : v;
     }();
     return f;

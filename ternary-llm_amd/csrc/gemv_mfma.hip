@@ -888,14 +888,24 @@ double span_share(int wg, int cus, int grid) {
 // slower again (a pool task of 768 K weights spends a quarter of its 25 us on staging and hand-over); with the
 // units of 32 rows the spans end closer together and a smaller pool is enough: 0 -> 5766, 0.03 -> 5816, 0.05 -> 5865,
 // 0.07 -> 5830, 0.10 -> 5817, 0.15 -> 5770, 0.30 -> 5648 (70B, 80 layers: 0.15 -> 5865, 0.05 -> 5895).
-// TLLM_POOL_FRACTION overrides it (0 switches the pool off).
-double pool_fraction() {
-    static const double f = [] {
-        const char *e = getenv("TLLM_POOL_FRACTION");
-        const double v = e ? atof(e) : 0.05;
-        return v < 0.0 ? 0.0 : v > 0.5 ? 0.5 : v;
-    }();
-    return f;
+// Plans of two to four activation rows (units of 128 rows, four times the work per unit) keep the larger pool:
+// 8B sweep at four rows 0 -> 3938 GB/s, 0.05 -> 3885, 0.10 -> 4003, 0.15 -> 4040, 0.25 -> 3989; at two rows
+// 0 -> 3982, 0.05 -> 3916, 0.10 -> 4220, 0.15 -> 4240, 0.25 -> 4284; on a faster box 0.15 / 0.20 / 0.25 at four
+// rows 4136 / 4114 / 4084, at three 4021 / 4167 / 4120, at two 4254 / 4440 / 4336.
+// TLLM_POOL_FRACTION and TLLM_TALL_POOL_FRACTION override them (0 switches the pool off).
+double pool_fraction(bool wide) {
+    static const double f[2] = {
+        [] {
+            const char *e = getenv("TLLM_TALL_POOL_FRACTION");
+            const double v = e ? atof(e) : 0.2;
+            return v < 0.0 ? 0.0 : v > 0.5 ? 0.5 : v;
+        }(),
+        [] {
+            const char *e = getenv("TLLM_POOL_FRACTION");
+            const double v = e ? atof(e) : 0.05;
+            return v < 0.0 ? 0.0 : v > 0.5 ? 0.5 : v;
+        }()};
+    return f[wide ? 1 : 0];
 }
 #ifndef TLLM_POOL_TASK_WEIGHTS
 #define TLLM_POOL_TASK_WEIGHTS (768 * 1024)
@@ -985,7 +995,7 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
     // cost) in proportion to the workgroup's share; at least one unit per workgroup. With
     // max_task_units > 0 and enough work, the last problems with short rows (staging x is cheap
     // there) go to the shared pool instead, cut into small tasks inside one problem each.
-    auto partition = [&](int unit, int wgs, int max_task_units) {
+    auto partition = [&](int unit, int wgs, int max_task_units, bool wide) {
         const int n = (int)host.size();
         // the up half of a SwiGLU pair has no units: its rows are done with the gate's
         auto is_up = [&](const std::vector<Problem> &v, int i) { return i > 0 && (v[i - 1].flags & kProblemSwigluGate); };
@@ -1003,7 +1013,7 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
         // the workgroups would then end with one more task than the rest (1B shapes, 16 layers: 54 us
         // without the pool, 60.5 us with it; 8B shapes, 8 layers: 100 / 99 us)
         if (max_task_units > 0 && all_units >= 8 * wgs && (double)all_w / wgs >= 2.3 * (double)kPoolTaskWeights) {
-            const int64_t want = (int64_t)((double)all_w * pool_fraction());
+            const int64_t want = (int64_t)((double)all_w * pool_fraction(wide));
             int64_t got = 0;
             int left_units = all_units;
             for (int pass = 0; pass < 2 && got < want; pass++)
@@ -1235,7 +1245,7 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
                                : d.wide           ? resident_wgs<Wide>(d.lds_bytes)
                                : d.fine           ? resident_wgs<Tall, false, true>(d.lds_bytes)
                                                   : resident_wgs<Tall>(d.lds_bytes);
-            partition(unit, per_cu * di->cus, max_units);
+            partition(unit, per_cu * di->cus, max_units, d.wide);
             d.max_units = max_units;
             d.image_bytes = max_image;
         }

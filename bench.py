@@ -40,7 +40,7 @@ HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense FP16 matrix peak
 # HBM bytes one launch of the headline workload moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
 # copy kernel of known size (profiles/gemv_mfma_wide__llama8b_sweep_b1.md); valid for that workload only.
-HEADLINE_TRAFFIC_BYTES = 1954977907
+HEADLINE_TRAFFIC_BYTES = 1923342227
 HEADLINE_TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this workload (profiles/gemv_mfma_wide__llama8b_sweep_b1.md), not read in this run"
 
 SHAPES = {

@@ -18,7 +18,8 @@
 // Two tile geometries:
 //   Wide (batch 1):   4 rows x 2048 columns. Lanes 4a..4a+3 read 64 contiguous bytes of row a, so
 //                     the loads coalesce; result column j is scale group j of the slice.
-//   Tall (batch 1-4): 16 rows x 512 columns. Result column j is group j % 4 of batch column j / 4.
+//   Tall (batch 1-4): 16 rows x 512 columns. Result column j is group j % 4 of batch column j / 4. The four
+//                     scales of (row, slice) come as one 8-byte load and are transposed inside the lane quad.
 #include <cstdio>
 #include <cstdlib>
 #include <mutex>
@@ -39,6 +40,9 @@ typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(1))) const uint32_t GU32;
 typedef __attribute__((address_space(1))) const uint16_t GU16;
 typedef __attribute__((address_space(1))) const u4 GU4;
+typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+// (a row of scales starts on any even byte when the number of groups is odd)
+typedef __attribute__((address_space(1))) const u2 __attribute__((aligned(2))) GU2;
 #define GB __attribute__((address_space(1)))
 template <class T>
 __device__ __forceinline__ __attribute__((address_space(1))) const T *as_global(const T *p) {
@@ -58,12 +62,14 @@ constexpr int kMaxBatch = 4;  // activation rows the tall tiles carry
 // Wide tiles: two, three and four give the same rate on long plans (8B sweep within 0.5 %); two make units of 32 rows
 // instead of 48 and leave more registers to the rest, which takes 6 % off a single call and 5 % off the 16-layer 1B
 // plan. Tall tiles: two are 9 - 11 % faster than three on the 8B sweep at two and four activation rows (one 13 % and
-// four 8 % slower): units of 128 rows, and the kernel fits its 168 registers without spilling.
+// four 8 % slower): units of 128 rows, and the kernel fits its 168 registers without spilling. (Since the scales of a
+// tall tile come as one 8-byte load the kernel needs 157 registers and three tiles fit without spills too: still 7 - 10 %
+// slower than two at two to four rows.)
 struct Wide {
-    static constexpr int kCols = 2048, kRows = 4, kChunks = 16, kScales = 1, kWgPerCu = 3, kAhead = 2;
+    static constexpr int kCols = 2048, kRows = 4, kChunks = 16, kWgPerCu = 3, kAhead = 2;
 };
 struct Tall {
-    static constexpr int kCols = 512, kRows = 16, kChunks = 4, kScales = 4, kWgPerCu = 3, kAhead = 2;
+    static constexpr int kCols = 512, kRows = 16, kChunks = 4, kWgPerCu = 3, kAhead = 2;
 };
 
 // Work is counted in units of kNW * kRows * kAhead rows of one matrix. A workgroup owns a
@@ -93,10 +99,20 @@ struct Sched {
     const float *i8_scale_dev;
 };
 
+// The scales that travel with a tile. Wide: the one scale of the lane's (row, group). Tall: the four scales (one
+// slice) of row 4 * lq + (li & 3) as one 8-byte load; the lane needs the scale of its own group li & 3 for each of the
+// rows 4 * lq + v instead, which is the 4 x 4 transpose of these halfwords inside the quad (quad_scales).
 template <class G>
-struct Tile {
+struct Tile;
+template <>
+struct Tile<Wide> {
     u4 nz, sg;
-    uint16_t sc[G::kScales];
+    uint16_t sc[1];
+};
+template <>
+struct Tile<Tall> {
+    u4 nz, sg;
+    uint32_t sc[2];
 };
 
 template <int kCtrl>
@@ -116,6 +132,22 @@ __device__ __forceinline__ float lane_select(float a, float b, uint64_t mask) {
     float r;
     asm("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "s"(mask));
     return r;
+}
+
+// 4 x 4 transpose of 16-bit values inside every quad of lanes. In: lane q of a quad holds a0 = (e0 | e1 << 16),
+// a1 = (e2 | e3 << 16), the four elements of its row q. Out: t0 = (element q of row 0 | element q of row 1 << 16),
+// t1 = the same of rows 2 and 3. Step 1 trades halfwords with lane q ^ 1 (sel: 0x05040100 in even lanes = own low half,
+// partner's low half; 0x03020706 in odd lanes = partner's high half, own high half; v_perm bytes 0-3 come from the
+// second operand, 4-7 from the first), step 2 trades one word with lane q ^ 2 (hi: the lanes with q >= 2).
+__device__ __forceinline__ void quad_scales(uint32_t a0, uint32_t a1, uint32_t sel, uint64_t hi, uint32_t &t0, uint32_t &t1) {
+    const uint32_t p0 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)a0, kQuadSwap1, 0xF, 0xF, true);
+    const uint32_t p1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)a1, kQuadSwap1, 0xF, 0xF, true);
+    const uint32_t d0 = __builtin_amdgcn_perm(p0, a0, sel);  // rows {q & ~1, q | 1}, element (q & 1)
+    const uint32_t d1 = __builtin_amdgcn_perm(p1, a1, sel);  // the same rows, element 2 + (q & 1)
+    const uint32_t send = __builtin_bit_cast(uint32_t, lane_select(__builtin_bit_cast(float, d1), __builtin_bit_cast(float, d0), hi));
+    const uint32_t got = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)send, kQuadSwap2, 0xF, 0xF, true);
+    t0 = __builtin_bit_cast(uint32_t, lane_select(__builtin_bit_cast(float, d0), __builtin_bit_cast(float, got), hi));
+    t1 = __builtin_bit_cast(uint32_t, lane_select(__builtin_bit_cast(float, got), __builtin_bit_cast(float, d1), hi));
 }
 
 __device__ __forceinline__ f4 mfma16(const uint32_t *o, u4 b, f4 c) {
@@ -533,13 +565,8 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
         const char GB *sg_g = reinterpret_cast<const char GB *>(as_global(w_sg));
         const char GB *sc_g = reinterpret_cast<const char GB *>(as_global(w_sc));
         const uint32_t lane_a = ((uint32_t)a_row * words + 4u * a_chunk) * 4u;
-        uint32_t lane_s[G::kScales];
-        if constexpr (G::kRows == 4) {
-            lane_s[0] = ((uint32_t)lq * groups + li) * 2u;
-        } else {
-#pragma unroll
-            for (int v = 0; v < 4; v++) lane_s[v] = ((uint32_t)(4 * lq + v) * groups + (li & 3)) * 2u;
-        }
+        const uint32_t lane_s = G::kRows == 4 ? ((uint32_t)lq * groups + li) * 2u
+                                              : (uint32_t)(4 * lq + (li & 3)) * groups * 2u;
 
         auto load_tile = [&](int slice, int rb) -> Tile<G> {
             Tile<G> t;
@@ -557,9 +584,14 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                 t.nz = *reinterpret_cast<const GU4 *>(nz_g + base_a + lane_a);
                 t.sg = *reinterpret_cast<const GU4 *>(sg_g + base_a + lane_a);
             }
-#pragma unroll
-            for (int v = 0; v < G::kScales; v++)
-                t.sc[v] = *reinterpret_cast<const GU16 *>(sc_g + base_s + lane_s[v]);
+            if constexpr (G::kRows == 4) {
+                t.sc[0] = *reinterpret_cast<const GU16 *>(sc_g + base_s + lane_s);
+            } else {
+                // (a slice starts on a multiple of four groups: 8-byte aligned when the scale array is)
+                const u2 w = *reinterpret_cast<const GU2 *>(sc_g + base_s + lane_s);
+                t.sc[0] = w[0];
+                t.sc[1] = w[1];
+            }
             return t;
         };
 
@@ -595,6 +627,9 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
             // lanes whose result row (li & 3) is odd / is 2 or 3 (wide tiles pick one of four D rows)
             const uint64_t odd_lanes = __builtin_amdgcn_ballot_w64((li & 1) != 0);
             const uint64_t hi_lanes = __builtin_amdgcn_ballot_w64((li & 2) != 0);
+            // tall tiles, transpose of the scales: byte selector of the first step, lanes of the second
+            const uint32_t quad_sel = (li & 1) ? 0x03020706u : 0x05040100u;
+            const uint64_t quad_hi = hi_lanes;
             // tall tiles: the lane adds the results of rows 4 lq + v, batch column bcol, if it is the first of its quad
             const bool adds = (li & 3) == 0 && bcol < p.batch;
             float *part_lane = my_part + 4 * lq * p.batch + bcol;
@@ -618,9 +653,12 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                     if (li == 0 && lq >= sh && live) my_part[rb - sh - r_begin + lq] += x;
                 } else {
                     float r[4];
+                    uint32_t rows01, rows23;  // this lane's group of rows 4 lq, 4 lq + 1 and of rows 4 lq + 2, 4 lq + 3
+                    quad_scales(t.sc[0], t.sc[1], quad_sel, quad_hi, rows01, rows23);
 #pragma unroll
                     for (int v = 0; v < 4; v++) {
-                        float x = h2f(t.sc[v]) * (d[v] - bias[v]);
+                        const uint32_t pair = v < 2 ? rows01 : rows23;
+                        float x = h2f((uint16_t)((v & 1) ? pair >> 16 : pair)) * (d[v] - bias[v]);
                         x = dpp_add<kQuadSwap1>(x);
                         x = dpp_add<kQuadSwap2>(x);
                         r[v] = x;

@@ -545,6 +545,38 @@ def test_tall_tile_plan_with_mixed_batch_sizes(dev, oracle, monkeypatch):
     plan.close()
 
 
+def test_tall_tile_plan_scales_on_any_halfword(dev, oracle, monkeypatch):
+    """The tall tiles fetch the four scales of a (row, slice) as one 8-byte load. The boundary asks
+    for 2-byte alignment of a scale array only, and with an odd number of groups every second row
+    starts on an odd halfword: arrays that begin one halfword past an aligned address, group counts
+    of 9, 32 and 145, every output against the oracle."""
+    torch, tl = dev
+    monkeypatch.setenv("TLLM_TALL_MIN_SHARE", "0")
+    batch = 3
+    shapes = [(300, 1152), (520, 4096), (200, 18560), (64, 512)]
+    probs, host = [], []
+    for k, (rows, cols) in enumerate(shapes):
+        nz, sg, s, _ = synth.problem(9500 + k, rows, cols, dontcare_sign=True)
+        x = synth.acts_f16(np.random.default_rng(9600 + k), batch, cols)
+        y = torch.full((batch, rows), float("nan"), dtype=torch.float16, device="cuda")
+        s_dev = up(torch, s)
+        shifted = torch.zeros(s_dev.numel() + 1, dtype=s_dev.dtype, device="cuda")
+        shifted[1:] = s_dev.reshape(-1)
+        s_odd = shifted[1:].view(s_dev.shape)
+        assert s_odd.data_ptr() % 4 == 2
+        probs.append((up(torch, nz), up(torch, sg), s_odd, up(torch, x), y, rows, cols, batch))
+        host.append((nz, sg, s, x, shifted))
+    plan = tl.LinearPlan(probs)
+    assert plan.kernel == "tllm::gemv_mfma_kernel<Tall>"
+    plan.launch()
+    torch.cuda.synchronize()
+    for k, (pr, (nz, sg, s, x, _)) in enumerate(zip(probs, host)):
+        got = pr[4].cpu().numpy().astype(np.float64)
+        ref = oracle.gemm_f64(x.view(np.uint16), nz, sg, s.view(np.uint16))
+        assert_close(oracle, got, ref, what=f"tall plan, shifted scales, problem {k}")
+    plan.close()
+
+
 # ------------------------------------------------------------- element-wise
 def _half_out(oracle, ref):
     """fp16 rounding of an fp64 reference, as float64 (for a 1-ulp comparison)."""

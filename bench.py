@@ -42,6 +42,9 @@ MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense FP16 matrix peak
 # copy kernel of known size (profiles/gemv_mfma_wide__llama8b_sweep_b1.md); valid for that workload only.
 HEADLINE_TRAFFIC_BYTES = 1923342227
 HEADLINE_TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this workload (profiles/gemv_mfma_wide__llama8b_sweep_b1.md), not read in this run"
+# The same for the 8B sweep with 4 and with 16 activation rows (profiles/gemv_batch__llama8b_sweep_b4_b16.md): bytes per launch.
+BATCH_SWEEP_TRAFFIC_BYTES = {4: 2297534500, 16: 2050618752}
+BATCH_SWEEP_TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this workload (profiles/gemv_batch__llama8b_sweep_b4_b16.md), not read in this run"
 
 SHAPES = {
     # name: (hidden, q_dim, kv_dim, ffn, layers)
@@ -675,6 +678,11 @@ def main():
             extra = [int(v) for v in args.also_batch.split(",") if v.strip()]
             r, _ = plan_rows(torch, tl, orc, timer, "cfg3: llama8b 32-layer sweep", "llama8b", 32, extra, 0.42, 0.01, 0.03,
                              args.seed, cfg_steps, 20, problems=problems)
+            for row, b in zip(r, extra):
+                if b in BATCH_SWEEP_TRAFFIC_BYTES:
+                    row["traffic"] = BATCH_SWEEP_TRAFFIC_BYTES[b]
+                    row["traffic_over_algorithmic"] = round(BATCH_SWEEP_TRAFFIC_BYTES[b] / sweep_bytes, 3)
+                    row["traffic_source"] = BATCH_SWEEP_TRAFFIC_SOURCE
             cfgs += r
             cfgs.append(int8_sweep_row(torch, tl, orc, timer, "cfg3: llama8b 32-layer sweep, batch 1, int8 activations (plan of ternary_gemv_int8)",
                                        problems, cfg_steps, 20))

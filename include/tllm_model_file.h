@@ -31,7 +31,8 @@ enum {
  * entries (0 for an all-zero group), stored as fp16 (round to nearest even).
  * Replaces ternarize_tensor + pack_ternary_to_bitmasks, reference ternarize/pack.py:41-101,
  * 120-169 (the reference's default threshold_factor is 0.7). Sums are taken in fp32 in column
- * order. cols % group_size must be 0 and group_size % 32 must be 0 (the reference pads the input
+ * order (the reference sums in torch's order; on the seeded tensors of its own packing test,
+ * tests/test_packing.py:92-111 and 141-173, masks and fp16 scales agree bit for bit). cols % group_size must be 0 and group_size % 32 must be 0 (the reference pads the input
  * dimension to a multiple of 32 with zero weights, pack.py:24-34; here the caller passes padded
  * matrices). Outputs are HOST arrays: nonzero_masks / sign_masks uint32 [rows, cols/32] (the sign
  * bit of a zero weight is written as 0), scales fp16 bits [rows, cols/group_size].

@@ -37,11 +37,13 @@
  *   quantize_i8 ........ closed forms (absmax=0 -> scale 1 / all zero, +-absmax ->
  *                        +-127, ties to even) and a numpy restatement via np.rint.
  *   gemv_i8_f64 ........ exact integer matmul in numpy int64.
- *   ternarize .......... the two degenerate cases of tests/test_packing.py:177-205
- *                        and a numpy restatement; the fp16 scale VALUES the reference
- *                        would produce for its torch seeds 42/123 are parity unpinned
- *                        (they depend on torch's random stream; only shape/dtype/value-set
- *                        properties are asserted by the reference for those seeds).
+ *   ternarize .......... the two degenerate cases of tests/test_packing.py:177-205,
+ *                        a numpy restatement, and tests/golden/pack_seed42.json /
+ *                        pack_seed123.json: inputs and outputs of the reference's own
+ *                        ternarize_tensor + pack_ternary_to_bitmasks on the two seeded
+ *                        tensors of tests/test_packing.py:92-111, 141-173 (written by
+ *                        tests/golden/make_pack_fixtures.py); masks, ternary values and
+ *                        fp16 scales are reproduced bit for bit.
  *   rmsnorm_f64 ........ the reference holds no test or fixture for it; pinned by closed
  *                        forms (constant row -> c/sqrt(c^2+eps); unit RMS of the output at
  *                        eps=0, w=1; invariance under x -> a*x at eps=0; linearity in w;

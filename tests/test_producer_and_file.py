@@ -63,6 +63,39 @@ def test_ternarize_pack_matches_oracle_bit_for_bit(oracle, rows, cols, group):
     assert np.array_equal(sc.view(np.uint16).ravel(), np.asarray(s).view(np.uint16).ravel())
 
 
+def _pack_fixture(name):
+    import json
+    with open(os.path.join(os.path.dirname(__file__), "golden", name + ".json")) as f:
+        fx = json.load(f)
+    rows, cols = fx["rows"], fx["cols"]
+    w = np.array([int(v, 16) for v in fx["weight_f32"]], np.uint32).view(np.float32).reshape(rows, cols)
+    t = np.array(["-0+".index(c) - 1 for c in fx["ternary"]], np.int8).reshape(rows, cols)
+    nz = np.array([int(v, 16) for v in fx["nz"]], np.uint32).reshape(rows, cols // 32)
+    sg = np.array([int(v, 16) for v in fx["sign"]], np.uint32).reshape(rows, cols // 32)
+    sc = np.array([int(v, 16) for v in fx["scales"]], np.uint16).reshape(rows, cols // fx["group"])
+    return fx, w, t, nz, sg, sc
+
+
+@pytest.mark.parametrize("name", ["pack_seed42", "pack_seed123"])
+def test_producer_reproduces_the_reference_producer(oracle, name):
+    """tests/golden/pack_seed*.json hold what the reference's ternarize_tensor + pack_ternary_to_bitmasks
+    (ternarize/pack.py:41-101, 120-169) gave for the two seeded tensors of its own packing test
+    (tests/test_packing.py:92-111, 141-173), written by tests/golden/make_pack_fixtures.py. The C++ producer
+    and the oracle's restatement must give the same masks AND the same fp16 scales, bit for bit (the
+    reference sums a group in torch's order, both restatements left to right: on these 320 groups the
+    fp32 sums round to the same fp16 value)."""
+    fx, w, t, rnz, rsg, rsc = _pack_fixture(name)
+    nz, sg, sc = tl.ternarize_pack(w, group_size=fx["group"], threshold_factor=fx["threshold_factor"])
+    assert np.array_equal(nz, rnz) and np.array_equal(sg, rsg)
+    assert np.array_equal(sc.view(np.uint16), rsc)
+    ot, os_ = oracle.ternarize(w, group=fx["group"], factor=fx["threshold_factor"])
+    assert np.array_equal(ot.reshape(t.shape), t)
+    assert np.array_equal(np.asarray(os_).view(np.uint16).reshape(rsc.shape), rsc)
+    onz, osg = oracle.pack(t)
+    assert np.array_equal(onz, rnz) and np.array_equal(osg, rsg)
+    assert np.array_equal(synth.unpack_np(rnz, rsg), t)      # the independent unpack of tests/synth.py
+
+
 def test_ternarize_rejects_bad_shapes():
     with pytest.raises(tl.TllmError):
         tl.ternarize_pack(np.zeros((2, 100), np.float32))          # cols % 32

@@ -16,6 +16,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include <cstdint>
+#include <atomic>
 #include <cstdio>
 #include <cstdlib>
 
@@ -34,15 +35,19 @@ inline error_handler_t &error_handler() {
     return h;
 }
 
-// First non-zero code since the caller last set it to 0 (negative: TLLM_ERR_*, positive: hipError_t).
-inline int &last_error() {
-    static int e = 0;
+// First non-zero code since the caller last set it to 0 (negative: TLLM_ERR_*, positive: hipError_t). One atomic for
+// the whole process, shared by every thread and stream: the first rejected call wins (compare-and-swap from 0), later
+// ones leave it alone, `ternary::last_error() = 0` clears it. A caller that needs to know WHICH call failed installs
+// an error_handler, which receives the operator's name with every code.
+inline std::atomic<int> &last_error() {
+    static std::atomic<int> e{0};
     return e;
 }
 
 inline void report(const char *op, int code) {
     if (code == 0) return;
-    if (!last_error()) last_error() = code;
+    int none = 0;
+    last_error().compare_exchange_strong(none, code, std::memory_order_relaxed);
     if (error_handler()) error_handler()(op, code);
 #ifdef TERNARY_ABORT_ON_ERROR
     std::abort();

@@ -106,9 +106,12 @@ int tllm_quantize_absmax_i8(const uint16_t *input, int8_t *output, float *scale,
  * whose K is not a multiple of 256 run a kernel that reads the activations from a copy in matrix-core
  * fragment order, which a small kernel writes there first (M rounded up to 32, times K, times 2 bytes; such
  * a shape is only chosen while that stays within TLLM_GEMM_STATIC_SCRATCH_BYTES). The first such call on a stream creates
- * the workspace (and a call with a larger need grows it: stream synchronisation, free, allocation).
- * tllm_gemm_workspace_reserve does that ahead of time. While `stream` is being captured into a graph
- * nothing is allocated: a call whose workspace is missing or too small then runs the kernel that needs
+ * the workspace: ONE allocation of TLLM_GEMM_STATIC_SCRATCH_BYTES (the most any shape is allowed to need: the kernel
+ * choice works under that limit), with its arrival counters cleared before the call returns (one device
+ * synchronisation, that once). It is never grown, moved or freed afterwards, except by tllm_gemm_workspace_release:
+ * a graph captured on the stream keeps pointing at valid memory whatever shapes run on the stream later.
+ * tllm_gemm_workspace_reserve creates it ahead of time. While `stream` is being captured into a graph
+ * nothing is allocated: a call whose stream has no workspace yet then runs the kernel that needs
  * none (same result up to the order of the fp32 additions, slower). Calls that use one stream's workspace
  * must not overlap in time: replays of a captured graph on another stream count as calls on the stream
  * the graph was captured on.
@@ -143,11 +146,13 @@ int tllm_ternary_gemm_f16_static(const uint16_t *A, const uint32_t *nz_B, const 
 const char *tllm_ternary_gemm_kernel(int M, int N, int K, int group_size);
 
 /*
- * Creates, or grows, the split-K workspace of `stream` for the GEMM shape (M, N, K) so that later
- * tllm_ternary_gemm_f16 calls of that shape (or a smaller need) on that stream allocate nothing, e.g.
- * before capturing them into a graph. May synchronise the stream. No counterpart in the reference (its
- * GEMM needs no workspace). tllm_gemm_workspace_release frees every workspace of the process; no GEMM
- * call may be in flight.
+ * Creates the workspace of `stream` if the GEMM shape (M, N, K) uses one and the stream has none yet, so that
+ * later tllm_ternary_gemm_f16 calls on that stream allocate nothing, e.g. before capturing them into a graph
+ * (the workspace has one size, so reserving for any shape that needs it serves every shape). May synchronise
+ * the device, once per stream. No counterpart in the reference (its GEMM needs no workspace).
+ * tllm_gemm_workspace_release frees every workspace of the process: no GEMM call may be in flight, and a
+ * graph that was captured with a call that used a workspace must not be replayed afterwards (it holds the
+ * freed address): destroy such graphs first, or never release.
  */
 int tllm_gemm_workspace_reserve(int M, int N, int K, int group_size, tllm_stream_t stream);
 void tllm_gemm_workspace_release(void);
@@ -296,6 +301,19 @@ void tllm_linear_plan_destroy(tllm_linear_plan *plan);
  * reference operators; its benchmark prints a copy bandwidth for the same purpose (tests/benchmark.cu:87-95).
  */
 int tllm_read_stream(const void *src, size_t bytes, uint32_t *sink, tllm_stream_t stream);
+
+/*
+ * Testing and tuning aid: the kernel-choice switches of the library. Each is read from its environment variable
+ * once per process (TLLM_GEMM_PATH, TLLM_GEMM_ROWSPLIT, TLLM_GEMM_PINGPONG, TLLM_BATCH_K_PARTS, TLLM_TALL_MAX_BATCH,
+ * TLLM_TALL_MIN_SHARE, TLLM_READ_SHAPE) when the library first needs one; no operator call reads the environment.
+ * These two calls change and read them afterwards, by name: "gemm_path" (0 cost model, 1 prefill GEMM, 2 passes of
+ * the decode kernel), "gemm_rowsplit" / "gemm_pingpong" (-1 cost model, 0 never, 1 or 2 forced), "batch_k_parts",
+ * "tall_max_batch", "tall_min_share_milli", "read_wgs_per_cu", "read_in_flight". An unknown name returns
+ * TLLM_ERR_BAD_SHAPE. Results never depend on them beyond the order of fp32 additions. Not for concurrent use
+ * with operator calls whose choice should be stable. No counterpart in the reference.
+ */
+int tllm_debug_set_tuning(const char *name, int value);
+int tllm_debug_get_tuning(const char *name, int *value);
 
 #ifdef __cplusplus
 }

@@ -210,6 +210,20 @@ int tllm_copy_to_kv_cache_f16(const uint16_t *k, const uint16_t *v, uint16_t *k_
                                               max_seq_len, (hipStream_t)stream);
 }
 
+int tllm_debug_set_tuning(const char *name, int value) {
+    std::atomic<int> *v = tllm::tuning_by_name(name);
+    if (!v) return TLLM_ERR_BAD_SHAPE;
+    v->store(value, std::memory_order_relaxed);
+    return TLLM_OK;
+}
+
+int tllm_debug_get_tuning(const char *name, int *value) {
+    std::atomic<int> *v = tllm::tuning_by_name(name);
+    if (!v || !value) return v ? TLLM_ERR_NULL_POINTER : TLLM_ERR_BAD_SHAPE;
+    *value = v->load(std::memory_order_relaxed);
+    return TLLM_OK;
+}
+
 int tllm_read_stream(const void *src, size_t bytes, uint32_t *sink, tllm_stream_t stream) {
     if (!src) return TLLM_ERR_NULL_POINTER;
     if (bytes < 16) return TLLM_ERR_BAD_SHAPE;
@@ -272,7 +286,8 @@ static int create_plan(tllm_linear_plan **plan, const tllm_linear_problem *probl
     if (!pl) return TLLM_ERR_TOO_LARGE;
     if (hipError_t e = tllm::plan_device_create(pl->host, &pl->dev)) {
         delete pl;
-        return input_scales && e == hipErrorInvalidValue ? TLLM_ERR_BAD_PLAN : (int)e;  // a shape the int8 plan kernel does not serve
+        // (invalid value: a shape that only the general kernel serves, which knows neither int8 activations nor pairs nor prologues)
+        return e == hipErrorInvalidValue ? TLLM_ERR_BAD_PLAN : (int)e;
     }
     if (pl->dev.extras && !pl->dev.use_mfma) {  // a shape that only the general kernel serves: no pairs, no prologue
         tllm::plan_device_destroy(&pl->dev);

@@ -45,6 +45,22 @@ static_assert(sizeof(Problem) == sizeof(tllm_linear_problem) + 16, "tllm_linear_
 constexpr int kProblemSwigluGate = TLLM_PROBLEM_SWIGLU_GATE;
 constexpr int kProblemInt8Input = 0x100;  // set by tllm_linear_plan_create_i8, not a public flag
 
+// Tuning switches. Each is read from its environment variable ONCE, when the library first asks for any of them;
+// afterwards only tllm_debug_set_tuning changes them (tests force kernel choices through it). No call path reads the
+// environment again.
+struct Tuning {
+    std::atomic<int> gemm_path{0};              // TLLM_GEMM_PATH=mfma|stream: 1 | 2 forces prefill GEMM | passes of the batched decode kernel for M > 16
+    std::atomic<int> gemm_rowsplit{-1};         // TLLM_GEMM_ROWSPLIT: 0 never, 1 / 2 whenever the shape allows (eight-wave / four-wave form)
+    std::atomic<int> gemm_pingpong{-1};         // TLLM_GEMM_PINGPONG: 0 never, 1 whenever the shape allows
+    std::atomic<int> batch_k_parts{0};          // TLLM_BATCH_K_PARTS: n parts where they fit, 1 never share out K
+    std::atomic<int> tall_max_batch{4};         // TLLM_TALL_MAX_BATCH: most activation rows of a plan on the tall-tile kernel
+    std::atomic<int> tall_min_share_milli{1000};  // TLLM_TALL_MIN_SHARE (x 1000): share of the plan per workgroup, in units, from which tall tiles run
+    std::atomic<int> read_wgs_per_cu{8};        // TLLM_READ_SHAPE="wgs_per_cu,loads_in_flight" of tllm_read_stream
+    std::atomic<int> read_in_flight{8};
+};
+Tuning &tuning();
+std::atomic<int> *tuning_by_name(const char *name);  // nullptr: no such switch
+
 // CU count of the current device, asked once per device (256 if the runtime cannot tell). Safe to
 // call from several host threads.
 inline int current_device_cus() {

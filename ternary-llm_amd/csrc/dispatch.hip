@@ -1,24 +1,55 @@
 // Kernel selection for one linear.
+#include <stdio.h>
 #include <stdlib.h>
+#include <string.h>
 
 #include "common.h"
 
 namespace tllm {
 
+Tuning &tuning() {
+    static Tuning t;
+    static const bool from_env = [] {
+        if (const char *e = getenv("TLLM_GEMM_PATH")) t.gemm_path = e[0] == 'm' ? 1 : e[0] == 's' ? 2 : 0;
+        if (const char *e = getenv("TLLM_GEMM_ROWSPLIT")) t.gemm_rowsplit = atoi(e);
+        if (const char *e = getenv("TLLM_GEMM_PINGPONG")) t.gemm_pingpong = atoi(e);
+        if (const char *e = getenv("TLLM_BATCH_K_PARTS")) t.batch_k_parts = atoi(e);
+        if (const char *e = getenv("TLLM_TALL_MAX_BATCH")) t.tall_max_batch = atoi(e);
+        if (const char *e = getenv("TLLM_TALL_MIN_SHARE")) t.tall_min_share_milli = (int)(atof(e) * 1000.0 + 0.5);
+        if (const char *e = getenv("TLLM_READ_SHAPE")) {
+            int a = 8, b = 8;
+            if (sscanf(e, "%d,%d", &a, &b) == 2) {
+                t.read_wgs_per_cu = a;
+                t.read_in_flight = b;
+            }
+        }
+        return true;
+    }();
+    (void)from_env;
+    return t;
+}
+
+std::atomic<int> *tuning_by_name(const char *name) {
+    Tuning &t = tuning();
+    const struct {
+        const char *name;
+        std::atomic<int> *value;
+    } all[] = {{"gemm_path", &t.gemm_path},           {"gemm_rowsplit", &t.gemm_rowsplit},
+               {"gemm_pingpong", &t.gemm_pingpong},   {"batch_k_parts", &t.batch_k_parts},
+               {"tall_max_batch", &t.tall_max_batch}, {"tall_min_share_milli", &t.tall_min_share_milli},
+               {"read_wgs_per_cu", &t.read_wgs_per_cu}, {"read_in_flight", &t.read_in_flight}};
+    for (const auto &e : all)
+        if (name && !strcmp(name, e.name)) return e.value;
+    return nullptr;
+}
+
 namespace {
 constexpr int kTallBatch = 4;    // activation rows per pass of the batch-1 family's tall tiles
 constexpr int kBatchRows = 16;   // activation rows per pass of the batched decode kernel
 
-// TLLM_GEMM_PATH=mfma|stream forces the choice between the prefill GEMM and passes of the batched
-// decode kernel for M > 16 (a tuning aid; unset: the cost model decides)
-int forced_path() {
-    static int v = -1;
-    if (v < 0) {
-        const char *e = getenv("TLLM_GEMM_PATH");
-        v = !e ? 0 : (e[0] == 'm' ? 1 : e[0] == 's' ? 2 : 0);
-    }
-    return v;
-}
+// gemm_path 1 | 2 forces the choice between the prefill GEMM and passes of the batched decode kernel for M > 16
+// (a tuning aid; 0: the cost model decides)
+int forced_path() { return tuning().gemm_path.load(std::memory_order_relaxed); }
 }  // namespace
 
 namespace {

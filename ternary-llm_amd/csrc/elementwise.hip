@@ -321,9 +321,9 @@ __global__ __launch_bounds__(256) void read_stream_kernel(const u4v *__restrict_
 }
 
 hipError_t launch_read_stream(const void *src, size_t bytes, uint32_t *sink, hipStream_t s) {
-    // TLLM_READ_SHAPE="wgs_per_cu,loads_in_flight" (tuning aid); default 8 workgroups per CU, 8 loads per thread
-    int per_cu = 8, flight = 8;
-    if (const char *e = getenv("TLLM_READ_SHAPE")) sscanf(e, "%d,%d", &per_cu, &flight);
+    // launch shape from the tuning switches (TLLM_READ_SHAPE="wgs_per_cu,loads_in_flight"); default 8 workgroups per CU, 8 loads per thread
+    const int per_cu = tuning().read_wgs_per_cu.load(std::memory_order_relaxed);
+    const int flight = tuning().read_in_flight.load(std::memory_order_relaxed);
     const int grid = current_device_cus() * (per_cu < 1 ? 1 : per_cu > 64 ? 64 : per_cu);
     const u4v *p = reinterpret_cast<const u4v *>(src);
     if (flight >= 16) read_stream_kernel<16><<<grid, 256, 0, s>>>(p, bytes / 16, sink);

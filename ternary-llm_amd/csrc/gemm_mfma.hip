@@ -1231,54 +1231,48 @@ __global__ __launch_bounds__(512 / NF) __attribute__((amdgpu_waves_per_eu(2, 2))
 
 // ---- split-K exchange memory: fp32 slots and one arrival counter per tile.
 //
-// Ordinary calls use a workspace per (device, stream), created by tllm_gemm_workspace_reserve or by the
-// first call that needs it and grown on demand; calls on one stream run in order and so may share it.
-// Nothing is allocated, freed or synchronised while the stream is being captured into a graph: a call
-// that would have to falls back to one workgroup per tile (no exchange).
+// Ordinary calls use a workspace per (device, stream), created by tllm_gemm_workspace_reserve or by the first call
+// that needs one. It is allocated ONCE, at the largest size any configuration is allowed to need (the limit the
+// kernel choice works under, kStaticSlotFloats), and lives at that address until tllm_gemm_workspace_release: a graph
+// captured on the stream keeps pointing at valid memory whatever shapes run on the stream afterwards. Calls on one
+// stream run in order and so may share it. Nothing is allocated or synchronised while the stream is being captured
+// into a graph: a call that would have to falls back to one workgroup per tile (no exchange).
 struct SplitWorkspace {
     int device = -1;
     hipStream_t stream = nullptr;
     float *partial = nullptr;
-    size_t floats = 0;
     unsigned *arrivals = nullptr;
 };
 constexpr size_t kArrivalSlots = kSplitArrivalSlots;  // tiles of a split launch (at most one per CU pair)
+constexpr size_t kWorkspaceFloats = (size_t)TLLM_GEMM_STATIC_SCRATCH_BYTES / 4 - kArrivalSlots;
 std::mutex g_ws_mutex;
 std::vector<SplitWorkspace> g_ws;
 
-__global__ void clear_arrivals_kernel(unsigned *arrivals, int n) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) arrivals[i] = 0u;
-}
-
-// may_allocate = false: only hands out what exists. *partial stays null when the workspace is too small.
+// may_allocate = false: only hands out what exists. *partial stays null when there is none (or the need exceeds
+// what a workspace ever holds).
 hipError_t split_workspace(hipStream_t s, size_t floats, bool may_allocate, float **partial, unsigned **arrivals) {
+    if (floats > kWorkspaceFloats) return hipSuccess;
     int dev = 0;
     if (hipError_t e = hipGetDevice(&dev)) return e;
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     SplitWorkspace *w = nullptr;
     for (SplitWorkspace &c : g_ws)
         if (c.device == dev && c.stream == s) w = &c;
-    if ((!w || w->floats < floats) && !may_allocate) return hipSuccess;
     if (!w) {
-        g_ws.push_back(SplitWorkspace{});
-        w = &g_ws.back();
-        w->device = dev;
-        w->stream = s;
-    }
-    if (w->floats < floats) {
-        if (hipError_t e = hipStreamSynchronize(s)) return e;  // earlier launches may still use the old buffers
-        if (w->partial) (void)hipFree(w->partial);
-        w->partial = nullptr;
-        w->floats = 0;
-        if (hipError_t e = hipMalloc(reinterpret_cast<void **>(&w->partial), floats * sizeof(float))) return e;
-        w->floats = floats;
-        if (!w->arrivals) {
-            if (hipError_t e = hipMalloc(reinterpret_cast<void **>(&w->arrivals), kArrivalSlots * sizeof(unsigned))) return e;
-            // cleared once, in stream order; every launch leaves the counters at zero again
-            clear_arrivals_kernel<<<(int)(kArrivalSlots / 256), 256, 0, s>>>(w->arrivals, (int)kArrivalSlots);
-            if (hipError_t e = hipGetLastError()) return e;
+        if (!may_allocate) return hipSuccess;
+        // counters first, then the slots: one allocation. The counters are cleared here, synchronously, so that they
+        // are zero for whichever stream a launch (or the replay of a graph) that uses them runs on; every launch
+        // leaves them at zero again.
+        unsigned char *base = nullptr;
+        if (hipError_t e = hipMalloc(reinterpret_cast<void **>(&base), (kArrivalSlots + kWorkspaceFloats) * 4)) return e;
+        hipError_t e = hipMemset(base, 0, kArrivalSlots * sizeof(unsigned));
+        if (!e) e = hipDeviceSynchronize();
+        if (e) {
+            (void)hipFree(base);
+            return e;
         }
+        g_ws.push_back(SplitWorkspace{dev, s, reinterpret_cast<float *>(base) + kArrivalSlots, reinterpret_cast<unsigned *>(base)});
+        w = &g_ws.back();
     }
     *partial = w->partial;
     *arrivals = w->arrivals;
@@ -1288,7 +1282,7 @@ hipError_t split_workspace(hipStream_t s, size_t floats, bool may_allocate, floa
 // The exchange memory of tllm_ternary_gemm_f16_static: a fixed array in device memory, one copy per GPU,
 // held until the process ends. Arrival counters first (zero when the module is loaded, left at zero by
 // every launch), then the fp32 slots.
-constexpr size_t kStaticSlotFloats = (size_t)TLLM_GEMM_STATIC_SCRATCH_BYTES / 4 - kArrivalSlots;
+constexpr size_t kStaticSlotFloats = kWorkspaceFloats;
 static __device__ __align__(256) unsigned char scratch[TLLM_GEMM_STATIC_SCRATCH_BYTES];
 
 // Device address of `scratch` on the current device, asked once per device.
@@ -1461,8 +1455,7 @@ GemmConfig choose_config(const Problem &p, size_t limit_floats) {
     // The eight-wave kernel: 0.85 us per stage (0.69 - 0.92 measured, the clock falls with the load), 9 us of
     // start, first loads, pair exchange and stores, and the copy of the activations into fragment order
     // (read + write at about 4 TB/s behind 2.5 us of its own start).
-    const char *env = getenv("TLLM_GEMM_PINGPONG");  // 0: never, 1: whenever the shape allows (read at every call: tests switch it)
-    const int forced = env ? atoi(env) : -1;
+    const int forced = tuning().gemm_pingpong.load(std::memory_order_relaxed);  // 0: never, 1: whenever the shape allows
     const GemmConfig pp{1, 1, true, 0.f};
     if (forced != 0 && workspace_floats(p, pp) <= limit_floats) {
         const long tiles = (long)n_tiles * ((p.batch + 255) / 256);
@@ -1475,8 +1468,7 @@ GemmConfig choose_config(const Problem &p, size_t limit_floats) {
     // CUs are split along K (at most as far as the CUs reach, two blocks per part at least, and while the slots fit the
     // workspace) when that is cheaper than a last round of whole tiles; an exchange costs about 6 us + 1.5 us per part
     // (fitted to 4096 x 14336 at M = 128 ... 512). Tiles are 128 activation rows high: not for fewer than 96.
-    const char *env_rs = getenv("TLLM_GEMM_ROWSPLIT");  // 0: never, 1 / 2: whenever the shape allows, in its eight-wave / four-wave form (read at every call)
-    const int forced_rs = env_rs ? atoi(env_rs) : -1;
+    const int forced_rs = tuning().gemm_rowsplit.load(std::memory_order_relaxed);  // 0: never, 1 / 2: whenever the shape allows, in its eight-wave / four-wave form
     const bool rs_ok = p.cols % 256 == 0 && !((reinterpret_cast<uintptr_t>(p.x) | reinterpret_cast<uintptr_t>(p.nz) |
                                                 reinterpret_cast<uintptr_t>(p.sg)) & 15);
     if (forced_rs != 0 && rs_ok && forced != 1 && (forced_rs >= 1 || p.batch >= 96)) {
@@ -1588,8 +1580,7 @@ void gemm_mfma_release_all() {
     (void)hipGetDevice(&dev);
     for (SplitWorkspace &w : g_ws) {
         (void)hipSetDevice(w.device);
-        if (w.partial) (void)hipFree(w.partial);
-        if (w.arrivals) (void)hipFree(w.arrivals);
+        if (w.arrivals) (void)hipFree(w.arrivals);  // the one allocation: counters, then slots
     }
     g_ws.clear();
     (void)hipSetDevice(dev);

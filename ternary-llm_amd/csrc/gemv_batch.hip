@@ -527,9 +527,8 @@ static int single_k_parts(const Problem &p, int cus) {
     if (most > steps) most = steps;
     if (most > 8) most = 8;
     if (most < 2 || blocks > kSplitArrivalSlots) return 1;
-    // TLLM_BATCH_K_PARTS=n (a tuning aid, read at every call): n parts where they fit, 1 = never share out K
-    const char *env = getenv("TLLM_BATCH_K_PARTS");
-    const int forced = env ? atoi(env) : 0;
+    // tuning switch batch_k_parts = n: n parts where they fit, 1 = never share out K
+    const int forced = tuning().batch_k_parts.load(std::memory_order_relaxed);
     if (forced > 0) return forced < most ? forced : most;
     int best = 1;
     for (int parts = 2; parts <= most; parts++)

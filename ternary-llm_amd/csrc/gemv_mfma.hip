@@ -1222,13 +1222,11 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
         all_tall = all_tall && addressable && tall_ok(p);
     }
     // Up to this many activation rows the tall-tile MFMA kernel is the faster of the two (8B and 70B
-    // sweeps: +17 % at two rows, +13 % at three, +5 % at four). TLLM_TALL_MAX_BATCH overrides.
-    // (both variables are read at every plan creation, not once per process)
-    const char *env_batch = getenv("TLLM_TALL_MAX_BATCH");
-    const int tall_max_batch = env_batch ? atoi(env_batch) : 4;
+    // sweeps: +17 % at two rows, +13 % at three, +5 % at four). The tuning switch tall_max_batch overrides.
+    const int tall_max_batch = tuning().tall_max_batch.load(std::memory_order_relaxed);
     // ... for plans large enough: its units (128 rows of one matrix) are what spans are cut in, and a unit of a
     // long-row matrix must not outweigh a workgroup's share of the plan: the tall tiles are taken from a share of one
-    // unit on (TLLM_TALL_MIN_SHARE overrides the ratio), and in units of 64 rows (one tile per wave) from a share of
+    // unit on (the tuning switch tall_min_share_milli overrides the ratio), and in units of 64 rows (one tile per wave) from a share of
     // 1.75 of those. One plan launch, us, batched kernel / tall tiles, at four activation rows: 8B shapes 2, 4, 6, 8, 12
     // layers (shares 0.3 to 1.8): 77 / 93, 97 / 119, 155 / 154, 178 / 165, 246 / 212; 70B 1, 2, 4, 8 layers (0.3 to
     // 2.4): 142 / 177, 211 / 234, 345 / 332, 587 / 563. At two rows the tall tiles win from 6 layers of 8B (154 / 133)
@@ -1241,8 +1239,7 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
             total += (int64_t)p.rows * p.cols;
             max_cols = std::max(max_cols, (int)p.cols);
         }
-        const char *env_share = getenv("TLLM_TALL_MIN_SHARE");
-        const double min_share = env_share ? atof(env_share) : 1.0;
+        const double min_share = tuning().tall_min_share_milli.load(std::memory_order_relaxed) / 1000.0;
         const double share = (double)total / (Tall::kWgPerCu * di->cus);
         tall_pays = share >= min_share * (double)range_unit<Tall>() * max_cols;
         if (!tall_pays) tall_pays = tall_fine = share >= 1.75 * min_share * (double)kTallFineUnit * max_cols;
@@ -1274,6 +1271,9 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
         const int mats = has_pairs ? 2 : 1;
         const int max_units = max_units_for(max_image, max_batch, unit, mats, d.wide ? kLdsLimit : kTallLdsLimit);
         if (max_units < 1) d.use_mfma = false;
+        // (again, after the demotion: the table kernel for general shapes reads fp16 activations and knows neither
+        // SwiGLU pairs nor RMSNorm prologues)
+        if ((d.x_is_i8 || d.extras) && !d.use_mfma) return hipErrorInvalidValue;
         if (d.use_mfma) {
             d.pair_stride = has_pairs ? kNW * max_units * unit * max_batch : 0;
             d.lds_bytes = max_image + kNW * max_units * unit * max_batch * 4 * mats;
@@ -1321,6 +1321,10 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
 }
 
 hipError_t plan_device_launch(const PlanDevice &plan, hipStream_t s) {
+    // the schedule, the table and the counters live on the device the plan was created on
+    int dev = -1;
+    if (hipError_t e = hipGetDevice(&dev)) return e;
+    if (dev != plan.device) return hipErrorInvalidDevice;
     int *counters = plan.counters + 2 * (plan.next_slot->fetch_add(1, std::memory_order_relaxed) % kPlanSlots);
     if (plan.batch_kernel)
         return launch_gemv_batch_table(plan.problems, plan.unit_prefix, plan.wg_first, plan.grid, plan.pool_begin,

@@ -20,6 +20,7 @@ ABI_SYMBOLS = (
     "tllm_add_f16", "tllm_rope_f16", "tllm_embedding_lookup_f16", "tllm_copy_to_kv_cache_f16",
     "tllm_linear_plan_kernel", "tllm_gemm_workspace_reserve", "tllm_gemm_workspace_release",
     "tllm_ternary_gemm_f16_static", "tllm_read_stream", "tllm_ternary_gemm_kernel",
+    "tllm_debug_set_tuning", "tllm_debug_get_tuning",
 )
 # include/tllm_model_file.h
 FILE_ABI_SYMBOLS = (
@@ -81,6 +82,8 @@ def lib():
     L.tllm_gemm_workspace_reserve.argtypes = [i, i, i, i, vp]
     L.tllm_read_stream.argtypes = [vp, C.c_size_t, vp, vp]
     L.tllm_gemm_workspace_release.argtypes = []
+    L.tllm_debug_set_tuning.argtypes = [C.c_char_p, i]
+    L.tllm_debug_get_tuning.argtypes = [C.c_char_p, C.POINTER(i)]
     L.tllm_gemm_workspace_release.restype = None
     L.tllm_linear_plan_create.argtypes = [C.POINTER(vp), C.POINTER(_Problem), i, i]
     L.tllm_linear_plan_create_normed.argtypes = [C.POINTER(vp), C.POINTER(_Problem), C.POINTER(vp), f, i, i]
@@ -177,6 +180,35 @@ def ternary_gemm_static(A, nz_B, sign_B, scales_B, Cout, M, N, K, group_size=128
 def read_stream(buf, stream=None):
     """Measurement aid: one read-only pass over a device tensor (the streaming ceiling of the GPU)."""
     check(lib().tllm_read_stream(_ptr(buf), buf.numel() * buf.element_size(), None, _stream(stream)))
+
+
+def set_tuning(name, value):
+    """Testing aid: sets one kernel-choice switch of the library (include/tllm_ternary.h, tllm_debug_set_tuning)."""
+    check(lib().tllm_debug_set_tuning(name.encode(), int(value)))
+
+
+def get_tuning(name):
+    v = C.c_int(0)
+    check(lib().tllm_debug_get_tuning(name.encode(), C.byref(v)))
+    return v.value
+
+
+class tuning:
+    """with tuning(gemm_rowsplit=1, ...): the switches are set inside the block and put back afterwards."""
+
+    def __init__(self, **kw):
+        self.want = kw
+
+    def __enter__(self):
+        self.old = {k: get_tuning(k) for k in self.want}
+        for k, v in self.want.items():
+            set_tuning(k, v)
+        return self
+
+    def __exit__(self, *exc):
+        for k, v in self.old.items():
+            set_tuning(k, v)
+        return False
 
 
 def gemm_kernel(M, N, K, group_size=128):

@@ -20,3 +20,20 @@ def oracle():
         orc.build()
     orc.load()
     return orc
+
+
+@pytest.fixture
+def tuned():
+    """tuned(name=value, ...) sets kernel-choice switches of the library (tllm_debug_set_tuning) for the rest of
+    the test; they are put back when it ends."""
+    import ternary_llm_amd as tl
+    entered = []
+
+    def apply(**kw):
+        ctx = tl.tuning(**kw)
+        ctx.__enter__()
+        entered.append(ctx)
+
+    yield apply
+    for ctx in reversed(entered):
+        ctx.__exit__(None, None, None)

@@ -63,28 +63,22 @@ def assert_close(oracle, got, ref, tol=TOL, what=""):
 
 
 class gemm_forced:
-    """Forces the GEMM kernel choice through the environment switches the library reads at every call:
+    """Forces the GEMM kernel choice through the library's tuning switches (tllm_debug_set_tuning):
     gemm_forced(pingpong=1), gemm_forced(rowsplit=1), gemm_forced(pingpong=0, rowsplit=0), gemm_forced() for the
-    library's own choice."""
-    NAMES = {"pingpong": "TLLM_GEMM_PINGPONG", "rowsplit": "TLLM_GEMM_ROWSPLIT"}
+    library's own choice. The switches are put back on exit."""
+    NAMES = {"pingpong": "gemm_pingpong", "rowsplit": "gemm_rowsplit"}
 
     def __init__(self, **kw):
-        self.want = {self.NAMES[k]: str(v) for k, v in kw.items()}
+        self.want = {name: -1 for name in self.NAMES.values()}
+        self.want.update({self.NAMES[k]: int(v) for k, v in kw.items()})
 
     def __enter__(self):
-        self.old = {n: os.environ.get(n) for n in self.NAMES.values()}
-        for n in self.NAMES.values():
-            os.environ.pop(n, None)
-        os.environ.update(self.want)
+        self.ctx = tl.tuning(**self.want)
+        self.ctx.__enter__()
         return self
 
     def __exit__(self, *exc):
-        for n, v in self.old.items():
-            if v is None:
-                os.environ.pop(n, None)
-            else:
-                os.environ[n] = v
-        return False
+        return self.ctx.__exit__(*exc)
 
 
 # -------------------------------------------------------------------- GEMV
@@ -461,12 +455,12 @@ def test_batched_plan_8b_layer_batch4_and_16(dev, oracle):
 
 
 @pytest.mark.parametrize("batch", [2, 3, 4])
-def test_tall_tile_plan_with_batch_columns(dev, oracle, batch, monkeypatch):
+def test_tall_tile_plan_with_batch_columns(dev, oracle, batch, tuned):
     """Plans of two to four activation rows on the tall-tile MFMA kernel (large plans take it by
     themselves; a small one is made to here): several batch columns in one operand image, rows of
     14336 and 36864 columns staged in segments, rows that are not whole slices, two launches."""
     torch, tl = dev
-    monkeypatch.setenv("TLLM_TALL_MIN_SHARE", "0")
+    tuned(tall_min_share_milli=0)
     shapes = [(700, 4096), (128, 4096), (1800, 4096), (520, 14336), (100, 36864), (300, 1152), (64, 512)]
     probs, host = [], []
     for k, (rows, cols) in enumerate(shapes):
@@ -491,7 +485,7 @@ def test_tall_tile_plan_with_batch_columns(dev, oracle, batch, monkeypatch):
     plan.close()
 
 
-def test_tall_tile_plan_in_fine_units(dev, oracle, monkeypatch):
+def test_tall_tile_plan_in_fine_units(dev, oracle, tuned):
     """A plan of two activation rows sized so that the tall tiles run in units of 64 rows (a share
     per workgroup of more than 1.75 and less than 2 such units, i.e. less than one of the ordinary
     units of 128 rows): sampled rows against the oracle."""
@@ -520,11 +514,11 @@ def test_tall_tile_plan_in_fine_units(dev, oracle, monkeypatch):
     plan.close()
 
 
-def test_tall_tile_plan_with_mixed_batch_sizes(dev, oracle, monkeypatch):
+def test_tall_tile_plan_with_mixed_batch_sizes(dev, oracle, tuned):
     """One plan whose problems carry one to four activation rows each, on the tall-tile kernel: the
     segment length and the operand image depend on the problem's own batch size."""
     torch, tl = dev
-    monkeypatch.setenv("TLLM_TALL_MIN_SHARE", "0")
+    tuned(tall_min_share_milli=0)
     shapes = [(700, 4096, 1), (300, 14336, 3), (520, 8192, 4), (200, 36864, 2), (64, 512, 4), (900, 18432, 1)]
     probs, host = [], []
     for k, (rows, cols, batch) in enumerate(shapes):
@@ -545,13 +539,13 @@ def test_tall_tile_plan_with_mixed_batch_sizes(dev, oracle, monkeypatch):
     plan.close()
 
 
-def test_tall_tile_plan_scales_on_any_halfword(dev, oracle, monkeypatch):
+def test_tall_tile_plan_scales_on_any_halfword(dev, oracle, tuned):
     """The tall tiles fetch the four scales of a (row, slice) as one 8-byte load. The boundary asks
     for 2-byte alignment of a scale array only, and with an odd number of groups every second row
     starts on an odd halfword: arrays that begin one halfword past an aligned address, group counts
     of 9, 32 and 145, every output against the oracle."""
     torch, tl = dev
-    monkeypatch.setenv("TLLM_TALL_MIN_SHARE", "0")
+    tuned(tall_min_share_milli=0)
     batch = 3
     shapes = [(300, 1152), (520, 4096), (200, 18560), (64, 512)]
     probs, host = [], []
@@ -1559,3 +1553,49 @@ def test_gemm_split_k_under_graph_capture(dev, oracle):
                 tl.ternary_gemm(dA, dnz, dsg, ds, eager, M, N, K, 128)
                 torch.cuda.synchronize()
         del graph
+
+
+def test_captured_split_gemm_survives_later_larger_shapes(dev, oracle):
+    """A stream's exchange workspace never moves: a graph captured with a small split shape on a stream whose
+    workspace was reserved for that shape, then eager calls on the same stream whose exchange is many times larger,
+    then the graph again: every replay gives the bits of the eager small call."""
+    torch, tl = dev
+    small, large = (130, 256, 4096), (512, 1024, 14336)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    cases = {}
+    for k, (M, N, K) in enumerate((small, large)):
+        nz, sg, s, _ = synth.problem(9800 + k, N, K, dontcare_sign=True)
+        A = synth.acts_f16(np.random.default_rng(9810 + k), M, K)
+        cases[(M, N, K)] = (up(torch, A), up(torch, nz), up(torch, sg), up(torch, s), A, nz, sg, s)
+    for shape in (small, large):
+        assert "K split" in tl.gemm_kernel(*shape), f"{shape}: the test needs shapes that exchange partial sums"
+    M, N, K = small
+    dA, dnz, dsg, ds, A, nz, sg, s = cases[small]
+    rows = np.unique(np.random.default_rng(2).integers(0, M, 6))
+    ref = oracle.gemm_f64(A[rows].view(np.uint16), nz, sg, s.view(np.uint16))
+    out = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    eager = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        tl.gemm_workspace_reserve(M, N, K, 128, stream=side)
+        tl.ternary_gemm(dA, dnz, dsg, ds, eager, M, N, K, 128, stream=side)
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            tl.ternary_gemm(dA, dnz, dsg, ds, out, M, N, K, 128, stream=side)
+    torch.cuda.synchronize()
+    assert_close(oracle, eager.cpu().numpy().astype(np.float64)[rows], ref, what="eager small split")
+    Ml, Nl, Kl = large
+    lA, lnz, lsg, ls = cases[large][:4]
+    big = torch.zeros((Ml, Nl), dtype=torch.float16, device="cuda")
+    for replay in range(3):
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), eager.view(torch.int16)), f"replay {replay}: differs from the eager call"
+        with torch.cuda.stream(side):      # a larger exchange on the capture stream, and another reserve
+            tl.ternary_gemm(lA, lnz, lsg, ls, big, Ml, Nl, Kl, 128, stream=side)
+            tl.gemm_workspace_reserve(Ml, Nl, Kl, 128, stream=side)
+        torch.cuda.synchronize()
+    del graph

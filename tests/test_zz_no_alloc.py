@@ -59,9 +59,8 @@ def test_static_gemm_matches_the_allocating_entry_point(oracle):
             assert rep_err["max_rel"] <= 1e-3, f"{case[:3]} round {rep}: {rep_err}"
     # the kernel for tall problems keeps its fragment-ordered copy of the activations in the same fixed array:
     # forced onto a small ragged shape, then a smaller one
-    import os
-    old = os.environ.get("TLLM_GEMM_PINGPONG")
-    os.environ["TLLM_GEMM_PINGPONG"] = "1"
+    forced = tl.tuning(gemm_pingpong=1)
+    forced.__enter__()
     try:
         for k, (M, N, K) in enumerate([(600, 520, 640), (70, 136, 384)]):
             nz, sg, s, _ = synth.problem(9400 + k, N, K, dontcare_sign=True)
@@ -77,13 +76,10 @@ def test_static_gemm_matches_the_allocating_entry_point(oracle):
             rep_err = oracle.error_report(got.cpu().numpy().astype(np.float64), ref)
             assert rep_err["max_rel"] <= 1e-3, f"tall kernel {M}x{N}x{K}: {rep_err}"
     finally:
-        if old is None:
-            os.environ.pop("TLLM_GEMM_PINGPONG", None)
-        else:
-            os.environ["TLLM_GEMM_PINGPONG"] = old
+        forced.__exit__(None, None, None)
     # the row-split kernel's exchange slots live in the same fixed array: tiles split eight ways, then a smaller shape
-    old = os.environ.get("TLLM_GEMM_ROWSPLIT")
-    os.environ["TLLM_GEMM_ROWSPLIT"] = "1"
+    forced = tl.tuning(gemm_rowsplit=1)
+    forced.__enter__()
     try:
         for k, (M, N, K) in enumerate([(260, 300, 6144), (130, 256, 4096)]):
             assert "K split" in tl.gemm_kernel(M, N, K)
@@ -101,10 +97,7 @@ def test_static_gemm_matches_the_allocating_entry_point(oracle):
             rep_err = oracle.error_report(got.cpu().numpy().astype(np.float64)[rows], ref)
             assert rep_err["max_rel"] <= 1e-3, f"row-split kernel {M}x{N}x{K}: {rep_err}"
     finally:
-        if old is None:
-            os.environ.pop("TLLM_GEMM_ROWSPLIT", None)
-        else:
-            os.environ["TLLM_GEMM_ROWSPLIT"] = old
+        forced.__exit__(None, None, None)
     # same argument checks as the allocating entry point
     M, N, K, dA, dnz, dsg, ds, _, _ = cases[0]
     out = torch.zeros((M, N), dtype=torch.float16, device="cuda")

@@ -49,14 +49,17 @@ int tllm_abi_version(void);
  * y[r] = fp16( sum_g float(scales[r,g]) * sum_{k in g} w[r,k] * float(input[k]) ),  fp32 accumulation.
  * Replaces ternary::ternary_gemv, reference include/kernels.cuh:11-14
  * (kernels/ternary_gemv.cu:27-100). input fp16 [cols], output fp16 [rows].
- * Two documented deviations (group_size 128, the matrix-core kernels; they also hold for the int8 variant,
- * tllm_ternary_gemm_f16 with M <= 16 and the plans):
- *  - Inf or NaN in `input` makes EVERY output of that activation row non-finite (the reference: only the rows
- *    with a non-zero weight on that column).
- *  - Dynamic range of one activation vector: a row's result carries an absolute error of about 2^-22 of the
- *    vector's largest magnitude. Outputs keep the 1e-3 relative bar as long as no element is more than about
- *    2^10 times the typical one; beyond that, rows with a ZERO weight on the outlier column lose accuracy
- *    (the reference accumulates term by term in fp32 and has no such limit).
+ * Inf, NaN and outliers in `input` (group_size 128, the matrix-core kernels; the same holds for the int8 variant,
+ * tllm_ternary_gemm_f16 with M <= 16 and the plans): as in the reference, which adds term by term
+ * (kernels/ternary_gemv.cu:60-82), a non-finite activation makes exactly the rows non-finite that hold a non-zero
+ * weight on its column, and an activation of any magnitude leaves the accuracy of the rows that hold none
+ * untouched. (The kernels meet weights and activations in a matrix multiply, where every activation enters the
+ * fp32 sums of every row; an activation that is non-finite, or more than 2^8 times the typical magnitude of its
+ * 128-column group, is therefore kept out of the operand and added afterwards, scale * w * x in fp32, to the rows
+ * that hold a weight there.) Limit: a workgroup holds 64 such activations per vector (128 for all activation rows
+ * of a 2..16-row call together); further ones stay inside the matrix operand, where a finite one costs the rows
+ * that do not use it about 2^-21 of its magnitude and a non-finite one makes every output of that activation row
+ * non-finite.
  */
 int tllm_ternary_gemv_f16(const uint32_t *nonzero_masks, const uint32_t *sign_masks,
                           const uint16_t *scales, const uint16_t *input, uint16_t *output,

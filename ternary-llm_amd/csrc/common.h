@@ -82,6 +82,15 @@ __device__ __forceinline__ uint16_t f2h(float v) {  // round to nearest even
     return __builtin_bit_cast(uint16_t, (_Float16)v);
 }
 
+// fp16(v) of an fp32 value the compiler must take as it is: without this it may fold the multiplication that
+// produced v into a mixed-precision instruction that rounds the exact product once, straight to fp16, and whether it
+// does depends on the code around. Two kernels that promise the same bits (RMSNorm on its own and as a prologue)
+// round twice, fp32 then fp16, like the reference's __float2half of an fp32 product (kernels/rmsnorm.cu:20-106).
+__device__ __forceinline__ uint16_t f2h_of_rounded(float v) {
+    asm("" : "+v"(v));
+    return f2h(v);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);

@@ -45,7 +45,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(const uint16_t *i
         float v;
         if (r) v = ro ? h2f(ro[i]) : h2f(x[i]) + h2f(r[i]);
         else v = h2f(x[i]);
-        output[row + i] = f2h(v * inv * h2f(weight[i]));
+        output[row + i] = f2h_of_rounded(v * inv * h2f(weight[i]));
     }
 }
 
@@ -84,7 +84,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_rows_kernel(const uint16
             }
         }
 #pragma unroll
-        for (int j = 0; j < 8; j++) ss += v[c][j] * v[c][j];
+        for (int j = 0; j < 8; j++) ss = __builtin_fmaf(v[c][j], v[c][j], ss);  // (written out: the prologue of the plan kernel takes the same sums in the same order)
         if (residual && residual_out) {
             uint32_t o[4];
 #pragma unroll
@@ -113,8 +113,8 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_rows_kernel(const uint16
         uint32_t o[4];
 #pragma unroll
         for (int j = 0; j < 4; j++)
-            o[j] = (uint32_t)f2h(v[c][2 * j] * inv * h2f((uint16_t)ww[j])) |
-                   (uint32_t)f2h(v[c][2 * j + 1] * inv * h2f((uint16_t)(ww[j] >> 16))) << 16;
+            o[j] = (uint32_t)f2h_of_rounded(v[c][2 * j] * inv * h2f((uint16_t)ww[j])) |
+                   (uint32_t)f2h_of_rounded(v[c][2 * j + 1] * inv * h2f((uint16_t)(ww[j] >> 16))) << 16;
         *(uint4 *)(output + row + (size_t)chunk * 8) = make_uint4(o[0], o[1], o[2], o[3]);
     }
 }

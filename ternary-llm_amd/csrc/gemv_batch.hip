@@ -6,7 +6,7 @@
 //
 // Dataflow. A workgroup of 4 waves owns a block of up to 256 weight rows and walks K in slices of
 // 512 columns. Per slice the workgroup turns x[0..16, slice] into ready-made MFMA B operands in LDS
-// (power-of-two normalised per activation row and slice, laid out in the element order of the
+// (power-of-two normalised per activation row and scale group, laid out in the element order of the
 // decode below), every wave copies them into 64 registers, and then each wave streams its own tiles
 // of 16 rows x 512 columns: lane (row i, chunk q) loads 16 bytes of each mask plane (one scale group
 // of one row), four lane-row swaps transpose the 4 x 4 (chunk, word) block held by lanes i, i+16,
@@ -42,6 +42,7 @@ constexpr int kSliceCols = 512;                 // 4 scale groups
 constexpr int kTileRows = 16;
 constexpr int kMaxTilesPerWave = 4;             // tiles of one wave per slice = loads in flight
 constexpr int kImageBytes = 16 * kSliceCols * 2;             // operands of one slice, 16 activation rows
+constexpr int kMaxOutliers = 128;  // outlier activations a workgroup can hold per block of rows (all activation rows together); more stay in the image
 
 struct BatchSched {
     const Problem *table;    // device table, or nullptr: use the by-value problem
@@ -112,8 +113,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
     // [buffer][slice parity]: the operands of two neighbouring slices are built per step
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     unsigned char (*image)[2][kImageBytes] = reinterpret_cast<unsigned char (*)[2][kImageBytes]>(lds_raw);
-    // per activation row: 2^(ex + 10) of the slice, 0 for an all-zero slice
-    float (*pow2)[2][16] = reinterpret_cast<float (*)[2][16]>(lds_raw + 4 * kImageBytes);
+    // per scale group of the slice and activation row: 2^(ex + 10) of the group, 0 for an all-zero group
+    float (*pow2)[2][4][16] = reinterpret_cast<float (*)[2][4][16]>(lds_raw + 4 * kImageBytes);
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -148,6 +149,14 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
     // operands of an all-zero weight row (every code = 1)
     uint32_t zero_o[16];
     decode_word(0u, 0u, zero_o);
+
+    // Activations that stay out of the operand images (see build_image): column, fp16 bits | activation row << 16.
+    // The list is rebuilt for every block of weight rows, since every block walks the whole of its K range.
+    __shared__ int n_outliers;
+    __shared__ int out_col[kMaxOutliers];
+    __shared__ uint32_t out_val[kMaxOutliers];
+    if (tid == 0) n_outliers = 0;
+    __syncthreads();
 
     Problem p = single;
     __shared__ int pool_block;
@@ -231,9 +240,11 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
         // builds the operands of one slice: element (chunk c, word q, step t, row j, e) at
         // ((c*4 + t)*64 + q*16 + j)*16 + 2e bytes: lane (j, q) of MFMA (c, t) reads 16 contiguous bytes
         // (`dead`: write zeros whatever was loaded)
-        auto build_image = [&](const u4 (&xr)[4], int buf, bool dead) {
-            // largest magnitude of the activation row inside the slice: packed unsigned maximum of the
-            // sign-stripped halves, then across the 16 threads of the row (one DPP row rotation each)
+        auto build_image = [&](const u4 (&xr)[4], int buf, bool dead, int slice) {
+            // largest magnitude of the activation row inside the thread's SCALE GROUP (128 columns: the four threads
+            // of a quad): packed unsigned maximum of the sign-stripped halves, then across the quad (two DPP swaps).
+            // Every group is normalised by itself, so an outlier activation costs precision only inside its own
+            // group; 2^(ex+10) of the group meets the group's result tile beside its fp32 scale.
             us2 m2 = {0, 0};
 #pragma unroll
             for (int i = 0; i < 4; i++)
@@ -241,11 +252,41 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
                 for (int e = 0; e < 4; e++)
                     m2 = __builtin_elementwise_max(m2, __builtin_bit_cast(us2, xr[i][e] & 0x7FFF7FFFu));
             uint32_t m = max((uint32_t)m2[0], (uint32_t)m2[1]);
-            m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x128, 0xF, 0xF, true));  // row_ror:8
-            m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x124, 0xF, 0xF, true));  // row_ror:4
-            m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x122, 0xF, 0xF, true));  // row_ror:2
-            m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x121, 0xF, 0xF, true));  // row_ror:1
             if (dead) m = 0;
+            uint32_t src[16];
+#pragma unroll
+            for (int d = 0; d < 16; d++) src[d] = xr[d >> 2][d & 3];
+            // Outliers first. The matrix product sees the codes w + 1, so an activation also enters the fp32 sums of the
+            // rows whose weight on its column is ZERO, to be cancelled against the all-zero-row product: that costs every
+            // such row about 2^-21 of the activation's magnitude, and would carry an Inf or NaN into every row. An element
+            // more than 2^8 times the smallest non-zero thread maximum of its group (a robust "typical magnitude"; Inf and
+            // NaN always) stays OUT of the image: it goes to a short list, and the end of the block adds scale * w * x
+            // for it to the rows that hold a weight there, term by term in fp32 like the reference
+            // (kernels/ternary_gemm.cu:131-155). When the list is full the element stays in the image.
+            uint32_t t = m ? m : 0xFFFFu;
+            t = min(t, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)t, 0xB1, 0xF, 0xF, true));  // quad_perm [1,0,3,2]
+            t = min(t, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)t, 0x4E, 0xF, 0xF, true));  // quad_perm [2,3,0,1]
+            const uint32_t limit = min(t + (8u << 10), 0x7BFFu);  // fp16 bits: 2^8 times t, at most the largest finite number
+            if (m > limit) {
+                m = 0;
+#pragma unroll
+                for (int d = 0; d < 16; d++)
+#pragma unroll
+                    for (int h = 0; h < 2; h++) {
+                        const uint32_t bits = (src[d] >> (16 * h)) & 0xFFFFu;
+                        if ((bits & 0x7FFFu) > limit) {
+                            const int slot = __hip_atomic_fetch_add(&n_outliers, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                            if (slot < kMaxOutliers) {
+                                out_col[slot] = slice * kSliceCols + xseg * 32 + 2 * d + h;
+                                out_val[slot] = bits | (uint32_t)xj << 16;
+                                src[d] &= ~(0xFFFFu << (16 * h));
+                            }
+                        }
+                        m = max(m, (src[d] >> (16 * h)) & 0x7FFFu);
+                    }
+            }
+            m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0xB1, 0xF, 0xF, true));  // quad_perm [1,0,3,2]
+            m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x4E, 0xF, 0xF, true));  // quad_perm [2,3,0,1]
             // byte selectors of the permutes below; selector 0x0C yields a zero byte
             const uint32_t sel_lo = dead ? 0x0C0C0C0Cu : 0x05040100u, sel_hi = dead ? 0x0C0C0C0Cu : 0x07060302u;
             // amax in [2^ex, 2^(ex+1)); x'' = x * 2^(14-ex) stays below 2^15
@@ -256,10 +297,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
             // a smaller maximum are normalised as if it were 2^-3: their multipliers are then >= 2^7,
             // and multiplying an fp16 number by a power of two >= 1 is exact (no overflow: |x| < 2^-2).
             const int exl = max(ex, -3);
-            if (xseg == 0) pow2[buf][xpar][xj] = m ? __builtin_bit_cast(float, (uint32_t)(127 + exl + 10) << 23) : 0.0f;
-            uint32_t src[16];
-#pragma unroll
-            for (int d = 0; d < 16; d++) src[d] = xr[d >> 2][d & 3];
+            if ((xseg & 3) == 0) pow2[buf][xpar][xseg >> 2][xj] = m ? __builtin_bit_cast(float, (uint32_t)(127 + exl + 10) << 23) : 0.0f;
             const int c = xseg >> 2, q = xseg & 3;
             // Operand t = 2z + h, dword d' holds the elements of decode dword m = 4h + d' (gemv_layout.h):
             // column 2m + z in its low half, column 2(m + 8) + z in its high half (m = 0: the other
@@ -304,7 +342,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
 
         for (int st = st_begin; st < st_end; st++) {
             const int buf = st & 1;
-            build_image(xr, buf, !x_live || 2 * st + xpar >= slices);
+            build_image(xr, buf, !x_live || 2 * st + xpar >= slices, 2 * st + xpar);
             load_x(xr, 2 * (st + 1) + xpar);
             // one barrier per step: it publishes buffer `buf`; the other buffer is rewritten only in
             // the next iteration, after every wave has passed this barrier and so has finished
@@ -313,18 +351,21 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
             u4 B[16];
 #pragma unroll
             for (int k = 0; k < 16; k++) B[k] = *reinterpret_cast<const u4 *>(&image[buf][parity][(k * 64 + lane) * 16]);
-            const float scale_j = pow2[buf][parity][li];
             // the product of an all-zero weight row (the "+1" of every code), formed exactly like a
-            // tile's own product, so that subtracting it leaves exact zeros where the weights are zero
+            // tile's own product, so that subtracting it leaves exact zeros where the weights are zero; both meet
+            // the group's factor 2^(ex+10) of this lane's activation row in one fused multiply-add (the product of
+            // the bias and a power of two is exact)
+            float pg[4];
             f4 bias[4];
 #pragma unroll
             for (int c = 0; c < 4; c++) {
+                pg[c] = pow2[buf][parity][c][li];
                 f4 d0 = {0.f, 0.f, 0.f, 0.f};
                 d0 = mfma16(zero_o + 0, B[4 * c + 0], d0);
                 d0 = mfma16(zero_o + 4, B[4 * c + 1], d0);
                 d0 = mfma16(zero_o + 8, B[4 * c + 2], d0);
                 d0 = mfma16(zero_o + 12, B[4 * c + 3], d0);
-                bias[c] = d0;
+                bias[c] = d0 * pg[c];
             }
             const int s_next = my_slice(min(st + 1, st_end - 1));
 #pragma unroll
@@ -359,11 +400,10 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
                     d[1] = mfma16(o1 + 12, B[4 * c + 7], d[1]);
                 };
                 auto retire = [&](int c, const f4 &dc) {
-                    const f4 d = dc - bias[c];
 #pragma unroll
                     for (int v = 0; v < 4; v++) {
                         const uint16_t sbits = (uint16_t)(sq[v][c >> 1] >> (16 * (c & 1)));
-                        r[v] += h2f(sbits) * d[v];
+                        r[v] += h2f(sbits) * __builtin_fmaf(dc[v], pg[c], -bias[c][v]);
                     }
                 };
                 issue_pair(0, da);
@@ -381,7 +421,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
                 __builtin_amdgcn_sched_barrier(0);
                 retire(2, db[0]);
                 retire(3, db[1]);
-                acc[k] += r * scale_j;
+                acc[k] += r;
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -396,12 +436,36 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
 #pragma unroll
                 for (int v = 0; v < 4; v++) hand[(k * 4 + v) * kWave + lane] = acc[k][v];
         }
+        // (the list is complete: every append lies before the barrier above; it is cleared for the next block behind
+        // the barrier below, so every thread takes its length here)
+        const int n_out = min(n_outliers, kMaxOutliers);
         __syncthreads();
         if (parity == 0) {
 #pragma unroll
             for (int k = 0; k < kTilesPerWave; k++)
 #pragma unroll
                 for (int v = 0; v < 4; v++) acc[k][v] += hand[(k * 4 + v) * kWave + lane];
+        }
+        // what the activations that stayed out of the images add: scale * (+-x) to the rows that hold a weight on the
+        // column (lane (lq, li) holds rows first + 4 lq + v of activation row li)
+        if (n_out && parity == 0) {
+            for (int o = 0; o < n_out; o++) {
+                const uint32_t vb = out_val[o];
+                if ((int)(vb >> 16) != li) continue;
+                const int col = out_col[o];
+                const uint32_t bit = 1u << (col & 31);
+                const float xv = h2f((uint16_t)vb);
+#pragma unroll
+                for (int k = 0; k < kTilesPerWave; k++) {
+                    const int first = tile_first_row(k, nullptr);
+#pragma unroll
+                    for (int v = 0; v < 4; v++) {
+                        const size_t row = (size_t)(first + 4 * lq + v);
+                        const size_t at = row * words + (col >> 5);
+                        if (p.nz[at] & bit) acc[k][v] += h2f(p.scales[row * groups + (col >> 7)]) * ((p.sg[at] & bit) ? xv : -xv);
+                    }
+                }
+            }
         }
         bool stores = true;
         if (k_parts > 1) {  // (the same for the whole workgroup)
@@ -452,6 +516,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemv_batch_kernel(Problem single,
             }
         }
         if (request) pool_block = requested;
+        if (tid == 0) n_outliers = 0;  // (every thread took the length before the second barrier of the hand-over)
         __syncthreads();  // the next block rewrites the image buffers
     }
     if (sc.counters && tid == 0) {
@@ -473,7 +538,7 @@ bool gemv_batch_supports(const Problem &p, int group) {
            (size_t)p.rows * (p.cols / 8) < ((size_t)1 << 32) && (size_t)p.rows * (p.cols / 128) * 2 < ((size_t)1 << 32);
 }
 
-constexpr size_t kLdsBytes = 4 * kImageBytes + 2 * 2 * 16 * sizeof(float);
+constexpr size_t kLdsBytes = 4 * kImageBytes + 2 * 2 * 4 * 16 * sizeof(float);
 
 template <int T>
 static hipError_t prepare_kernel() {

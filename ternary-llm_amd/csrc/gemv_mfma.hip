@@ -58,6 +58,8 @@ constexpr int kSegSlices = 8;
 __host__ __device__ constexpr int tall_seg_slices(int batch) { return 8192 / 512 / batch; }
 constexpr int kThreads = kNW * kWave;
 constexpr int kMaxBatch = 4;  // activation rows the tall tiles carry
+// Outlier activations a workgroup can hold per staged row (all batch columns together); more stay in the image.
+constexpr int kMaxOutliers = 64;
 // kAhead of a tile geometry: tile loads in flight per wave (register ring, unrolled) = tiles per wave in a unit of work.
 // Wide tiles: two, three and four give the same rate on long plans (8B sweep within 0.5 %); two make units of 32 rows
 // instead of 48 and leave more registers to the rest, which takes 6 % off a single call and 5 % off the 16-layer 1B
@@ -195,12 +197,18 @@ __device__ __forceinline__ f4 tile_product(const u4 nz, const u4 sg, const u4 (&
 template <class G, bool kExtras = false, bool kFine = false>
 __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma_kernel(Problem single, Sched sc) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    uint16_t *image = reinterpret_cast<uint16_t *>(lds);
+    // [group factors | operand image | partial sums]: image_bytes counts the first two, 1 : 64 (one float per 128
+    // two-byte image elements)
+    float *gfac = reinterpret_cast<float *>(lds);
+    uint16_t *image = reinterpret_cast<uint16_t *>(lds + sc.image_bytes / 65);
     float *partial = reinterpret_cast<float *>(lds + sc.image_bytes);
-    __shared__ uint32_t red_amax[kNW][kMaxBatch];
     __shared__ float red_ss[kNW];
     __shared__ float fscale[kMaxBatch];
     __shared__ u4 zero_operand;  // what the idle lanes of a B operand read
+    // Activations that stay out of the operand image (see stage_piece): column, fp16 bits | batch column << 16
+    __shared__ int n_outliers;
+    __shared__ int out_col[kMaxOutliers];
+    __shared__ uint32_t out_val[kMaxOutliers];
     if (threadIdx.x == 0) zero_operand = u4{0u, 0u, 0u, 0u};
 
     const int tid = threadIdx.x;
@@ -226,7 +234,6 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
     int cur = -1;      // problem whose activations are staged
     int cur_seg = -1;  // and which segment of its columns
     constexpr int kSegBatch = G::kRows == 4 ? 1 : kMaxBatch;
-    int cur_ex[kSegBatch] = {};  // exponents of that problem's largest activations (rows staged in segments)
     Problem p = single;
     int slices = 0, groups = 0, words = 0, img_stride = 0;
     int seg_lo = 0, seg_n = 0;  // slices of the staged segment
@@ -281,6 +288,9 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
         for (int seg = 0; seg < n_seg; seg++) {
         if (seg != cur_seg) {
             // ------------------------------------------------ stage the activations of problem pi
+            // (the list of outliers belongs to the whole row: it starts again with the row's first segment; the
+            // barrier that ended the task before lies between its last reader and this write)
+            if (seg == 0 && tid == 0) n_outliers = 0;
             __syncthreads();  // every wave is done with the image that was staged before
             cur_seg = seg;
             seg_lo = seg * seg_len;
@@ -297,7 +307,10 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                 return uint4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
             };
             // Image element (slice, t, chunk, e) = fp16(x[col] * 2^(14-ex-p)), where 2^ex is the power
-            // of two at or below the largest magnitude of the batch column. The last slice of a row
+            // of two at or below the largest magnitude of the element's SCALE GROUP (its 128-column chunk): every
+            // group is normalised by itself, so an outlier activation costs precision only inside its own group (a
+            // result column of the matrix product collects exactly one group, and 2^(ex+10) of the group joins its
+            // fp32 scale when the column is taken out of the accumulators). The last slice of a row
             // that is not a whole number of slices is moved left so that it ends with the row; the
             // chunks it then shares with the slice before it are zero in the image. Eight-element
             // pieces are numbered in image order; piece_of() loads the activations of one.
@@ -340,22 +353,63 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                     dst[image_index(s.t, chunk, s.e, G::kChunks)] = f2h(h2f(hx) * mult);
                 }
             };
-            // amax bits -> exponent; also sets the output scale of the column
-            auto exponent_of = [&](int b) -> int {
-                uint32_t m = 0;
+            // One piece into the image. The 16 pieces of a 128-column group are held by 16 neighbouring threads
+            // (one DPP row), whatever the staging path.
+            // Outliers first. The matrix product sees the codes w + 1, so an activation also enters the fp32 sums of
+            // the rows whose weight on its column is ZERO, to be cancelled against the all-zero-row product later:
+            // that costs every such row about 2^-21 of the activation's magnitude, too much once it is some hundred
+            // times the magnitude of its neighbours, and it would carry an Inf or NaN into every row. An element more
+            // than 2^8 times the smallest non-zero piece maximum of its group (a robust "typical magnitude"; Inf and
+            // NaN always) therefore stays OUT of the image: it goes to a short list, and the epilogue adds
+            // scale * w * x for it to the rows that hold a weight there, term by term in fp32 like the reference
+            // (kernels/ternary_gemv.cu:60-82). When the list is full the element stays in the image.
+            // Then the exponent of the group's largest remaining magnitude; 2^(ex+10) goes to the table of group
+            // factors (the image of an all-zero group is zero whatever the exponent).
+            auto stage_piece = [&](int b, int c8, uint4 v) {
+                uint32_t m = magnitude(0u, v);
+                uint32_t t = m ? m : 0xFFFFu;
+                t = min(t, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)t, 0x128, 0xF, 0xF, true));  // row_ror:8
+                t = min(t, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)t, 0x124, 0xF, 0xF, true));  // row_ror:4
+                t = min(t, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)t, 0x122, 0xF, 0xF, true));  // row_ror:2
+                t = min(t, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)t, 0x121, 0xF, 0xF, true));  // row_ror:1
+                const uint32_t limit = min(t + (8u << 10), 0x7BFFu);  // fp16 bits: 2^8 times t, at most the largest finite number
+                if (m > limit) {
+                    const int slice = seg_lo + (c8 * 8) / G::kCols;
+                    const int chunk = ((c8 * 8) % G::kCols) / kChunkCols;
+                    const int col0 = (min(slice * G::kChunks, groups - G::kChunks) + chunk) * kChunkCols + (c8 * 8) % kChunkCols;
+                    uint32_t w4[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-                for (int w = 0; w < kNW; w++) m = max(m, red_amax[w][b]);
-                // amax in [2^ex, 2^(ex+1)); x'' = x * 2^(14-ex) stays below 2^15
-                int ex = 0;                 // all-zero activations: the image is zero whatever the exponent
-                if (m >= 0x7C00u) ex = 15;  // inf/nan present: they propagate to the outputs
-                else if (m) ex = (int)((__builtin_bit_cast(uint32_t, h2f((uint16_t)m)) >> 23) & 0xFF) - 127;
-                if (tid == 0) {
-                    float f = m ? __builtin_bit_cast(float, (uint32_t)(127 + ex + 10) << 23) : 0.0f;
-                    if (sc.x_is_i8) f *= sc.table ? *p.x_scale : (sc.i8_scale_dev ? *sc.i8_scale_dev : sc.i8_scale);
-                    fscale[b] = f;
+                    for (int e = 0; e < 8; e++) {
+                        const uint32_t bits = (w4[e >> 1] >> (16 * (e & 1))) & 0xFFFFu;
+                        if ((bits & 0x7FFFu) > limit) {
+                            const int slot = __hip_atomic_fetch_add(&n_outliers, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                            if (slot < kMaxOutliers) {
+                                out_col[slot] = col0 + e;
+                                out_val[slot] = bits | (uint32_t)b << 16;
+                                w4[e >> 1] &= ~(0xFFFFu << (16 * (e & 1)));
+                            }
+                        }
+                    }
+                    v = uint4{w4[0], w4[1], w4[2], w4[3]};
+                    m = magnitude(0u, v);
                 }
-                return ex;
+                m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x128, 0xF, 0xF, true));
+                m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x124, 0xF, 0xF, true));
+                m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x122, 0xF, 0xF, true));
+                m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x121, 0xF, 0xF, true));
+                // amax in [2^ex, 2^(ex+1)); x'' = x * 2^(14-ex) stays below 2^15
+                int ex = 0;
+                if (m >= 0x7C00u) ex = 15;  // inf/nan left in the image (full list): they propagate to every output
+                else if (m) ex = (int)((__builtin_bit_cast(uint32_t, h2f((uint16_t)m)) >> 23) & 0xFF) - 127;
+                if ((c8 & 15) == 0) gfac[b * (pieces / 16) + c8 / 16] = __builtin_bit_cast(float, (uint32_t)(127 + ex + 10) << 23);
+                write_piece(image + (size_t)b * img_stride, c8, v, ex);
             };
+            // what every output of a batch column is multiplied with at the end: the activation scale of int8 input
+            if (tid < kMaxBatch) {
+                float f = 1.0f;
+                if (sc.x_is_i8) f = sc.table ? *p.x_scale : (sc.i8_scale_dev ? *sc.i8_scale_dev : sc.i8_scale);
+                fscale[tid] = f;
+            }
             // The piece addresses depend on the thread index only; hidden behind an empty asm they are
             // worked out here, each time, instead of living in registers across the whole kernel.
             int stid = tid;
@@ -364,7 +418,6 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
             if (n_seg == 1 && p.batch == 1 && pieces <= kKeep * kThreads) {
                 // one pass over x: all loads are issued together and kept for the image
                 uint4 keep[kKeep];
-                uint32_t m = 0;
 #pragma unroll
                 for (int k = 0; k < kKeep; k++) {
                     const int c8 = stid + k * kThreads;
@@ -381,8 +434,8 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
 #pragma unroll
                         for (int e = 0; e < 4; e++) {
                             const float lo = h2f((uint16_t)w4[e]), hi = h2f((uint16_t)(w4[e] >> 16));
-                            ss += lo * lo;
-                            ss += hi * hi;
+                            ss = __builtin_fmaf(lo, lo, ss);
+                            ss = __builtin_fmaf(hi, hi, ss);
                         }
                         __builtin_amdgcn_sched_barrier(0);  // piece by piece: few registers
                     }
@@ -411,43 +464,27 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                             uint32_t o[4];
 #pragma unroll
                             for (int e = 0; e < 4; e++)
-                                o[e] = (uint32_t)f2h(h2f((uint16_t)x4[e]) * inv * h2f((uint16_t)n4[e])) |
-                                       (uint32_t)f2h(h2f((uint16_t)(x4[e] >> 16)) * inv * h2f((uint16_t)(n4[e] >> 16))) << 16;
+                                o[e] = (uint32_t)f2h_of_rounded(h2f((uint16_t)x4[e]) * inv * h2f((uint16_t)n4[e])) |
+                                       (uint32_t)f2h_of_rounded(h2f((uint16_t)(x4[e] >> 16)) * inv * h2f((uint16_t)(n4[e] >> 16))) << 16;
                             x = uint4{o[0], o[1], o[2], o[3]};
                             __builtin_amdgcn_sched_barrier(0);
                         }
                     }
                 }
 #pragma unroll
-                for (int k = 0; k < kKeep; k++) m = magnitude(m, keep[k]);
-#pragma unroll
-                for (int off = 32; off > 0; off >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, off, kWave));
-                if (lane == 0) red_amax[wave][0] = m;
-                __syncthreads();
-                const int ex = exponent_of(0);
-#pragma unroll
                 for (int k = 0; k < kKeep; k++) {
                     const int c8 = stid + k * kThreads;
-                    if (c8 < pieces) write_piece(image, c8, keep[k], ex);
+                    if (c8 < pieces) stage_piece(0, c8, keep[k]);
                     __builtin_amdgcn_sched_barrier(0);  // one piece at a time: keeps the register need low
                 }
             } else if constexpr (kFine && G::kRows == 4) {
                 // a whole row too long for the registers (the fine-grained instances do not stage in
-                // segments): one pass for the magnitude, one for the image, piece by piece
-                uint32_t m = 0;
-                for (int c8 = stid; c8 < pieces; c8 += kThreads) m = magnitude(m, piece_of(0, c8));
-#pragma unroll
-                for (int off = 32; off > 0; off >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, off, kWave));
-                if (lane == 0) red_amax[wave][0] = m;
-                __syncthreads();
-                const int ex = exponent_of(0);
-                for (int c8 = stid; c8 < pieces; c8 += kThreads) write_piece(image, c8, piece_of(0, c8), ex);
+                // segments): piece by piece (the trip count is the same for the 16 threads of a group)
+                for (int c8 = stid; c8 < pieces; c8 += kThreads) stage_piece(0, c8, piece_of(0, c8));
             } else {
-                // Long rows or several batch columns: one pass for the magnitudes, one for the image.
-                // The (column, piece) pairs are numbered column-major and taken kFlat * kThreads at a
-                // time, so that a thread has kFlat loads in flight whatever the shape. A row staged in
-                // segments gets its exponents from one pass over the whole row, made when the problem
-                // is first seen; its segments are then written with those.
+                // Long rows or several batch columns. The (column, piece) pairs are numbered column-major and
+                // taken kFlat * kThreads at a time, so that a thread has kFlat loads in flight whatever the shape
+                // (the pieces of a column are a multiple of 16, so the 16 threads of a DPP row always hold one group).
                 constexpr int kFlat = G::kRows == 4 ? kKeep / 2 : kKeep;  // loads in flight per thread (wide tiles: fewer registers to spare)
                 auto column_of = [&](int item, int per_col) -> int {  // item / per_col for at most kSegBatch columns
                     int b = 0;
@@ -455,41 +492,6 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                     for (int c = 1; c < kSegBatch; c++) b += item >= c * per_col;
                     return b;
                 };
-                if (n_seg == 1 || (fresh && seg == 0)) {
-                    const bool whole_row = n_seg > 1;
-                    const int per_col = whole_row ? p.cols / 8 : pieces;
-                    const int items = per_col * p.batch;
-                    uint32_t m[kSegBatch] = {};
-                    for (int base = 0; base < items; base += kFlat * kThreads) {
-                        uint4 kp[kFlat];
-                        int kb[kFlat];
-#pragma unroll
-                        for (int k = 0; k < kFlat; k++) {
-                            const int item = base + stid + k * kThreads;
-                            const int b = column_of(item, per_col);
-                            kb[k] = item < items ? b : -1;
-                            kp[k] = item >= items ? uint4{0u, 0u, 0u, 0u}
-                                    : whole_row   ? load8(b, item - b * per_col)
-                                                  : piece_of(b, item - b * per_col);
-                        }
-#pragma unroll
-                        for (int k = 0; k < kFlat; k++)
-#pragma unroll
-                            for (int c = 0; c < kSegBatch; c++)
-                                if (kb[k] == c) m[c] = magnitude(m[c], kp[k]);
-                    }
-#pragma unroll
-                    for (int c = 0; c < kSegBatch; c++) {
-#pragma unroll
-                        for (int off = 32; off > 0; off >>= 1)
-                            m[c] = max(m[c], (uint32_t)__shfl_xor((int)m[c], off, kWave));
-                        if (lane == 0) red_amax[wave][c] = m[c];
-                    }
-                    __syncthreads();
-#pragma unroll
-                    for (int c = 0; c < kSegBatch; c++)
-                        if (c < p.batch) cur_ex[c] = exponent_of(c);
-                }
                 const int items = pieces * p.batch;
                 for (int base = 0; base < items; base += kFlat * kThreads) {
                     uint4 kp[kFlat];
@@ -503,10 +505,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                     for (int k = 0; k < kFlat; k++) {
                         const int item = base + stid + k * kThreads;
                         const int b = column_of(item, pieces);
-                        int ex = cur_ex[0];
-#pragma unroll
-                        for (int c = 1; c < kSegBatch; c++) ex = b == c ? cur_ex[c] : ex;
-                        if (item < items) write_piece(image + (size_t)b * img_stride, item - b * pieces, kp[k], ex);
+                        if (item < items) stage_piece(b, item - b * pieces, kp[k]);
                         __builtin_amdgcn_sched_barrier(0);
                     }
                 }
@@ -633,8 +632,9 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
             // tall tiles: the lane adds the results of rows 4 lq + v, batch column bcol, if it is the first of its quad
             const bool adds = (li & 3) == 0 && bcol < p.batch;
             float *part_lane = my_part + 4 * lq * p.batch + bcol;
+            // bias, bias_sel: the all-zero-row product of the slice, already multiplied by the group factor gf
             auto process_tile = [&](const Tile<G> &t, int rb, bool live, const u4 (&B)[kMfmaPerTile], const f4 &bias,
-                                    float bias_sel) {
+                                    float bias_sel, float gf) {
                 f4 d0, d1;
                 tile_product2(t.nz, t.sg, B, d0, d1);
                 const f4 d = d0 + d1;
@@ -642,10 +642,11 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                 if constexpr (G::kRows == 4) {
                     // lane (row quad lq, column li): only D row 4*lq + (li & 3) pairs this column's
                     // chunk with the row that loaded it; it is group li of row rb - sh + lq.
-                    // (bias_sel was formed the same way, so an all-zero row still gives exactly 0)
+                    // (bias_sel was formed the same way and its product with the power of two gf is exact, so an
+                    // all-zero row still gives exactly 0)
                     const float dv = lane_select(lane_select(d[0], d[1], odd_lanes),
                                                  lane_select(d[2], d[3], odd_lanes), hi_lanes);
-                    float x = h2f(t.sc[0]) * (dv - bias_sel);
+                    float x = h2f(t.sc[0]) * __builtin_fmaf(dv, gf, -bias_sel);
                     x = dpp_add<kQuadSwap1>(x);
                     x = dpp_add<kQuadSwap2>(x);
                     x = dpp_add<kRowHalfMirror>(x);
@@ -658,7 +659,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
 #pragma unroll
                     for (int v = 0; v < 4; v++) {
                         const uint32_t pair = v < 2 ? rows01 : rows23;
-                        float x = h2f((uint16_t)((v & 1) ? pair >> 16 : pair)) * (d[v] - bias[v]);
+                        float x = h2f((uint16_t)((v & 1) ? pair >> 16 : pair)) * __builtin_fmaf(d[v], gf, -bias[v]);
                         x = dpp_add<kQuadSwap1>(x);
                         x = dpp_add<kQuadSwap2>(x);
                         r[v] = x;
@@ -680,7 +681,10 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
             };
 
             // the B operands of a slice, and what an all-zero weight row gives with them
-            auto load_operands = [&](int slice, u4 (&B)[kMfmaPerTile], f4 &bias, float &bias_sel) {
+            // this lane's result column collects one scale group of one batch column: the factor 2^(ex+10) of that
+            // group, from the table the staging left
+            const float *gfac_lane = gfac + (G::kRows == 4 ? li : min(bcol, p.batch - 1) * (seg_n * G::kChunks) + (li & 3));
+            auto load_operands = [&](int slice, u4 (&B)[kMfmaPerTile], f4 &bias, float &bias_sel, float &gf) {
                 // Every lane reads (no branch): the idle lanes read the zero operand with stride 0.
                 const u4 *src = b_active ? reinterpret_cast<const u4 *>(image + (size_t)bcol * img_stride +
                                                                         slice * G::kCols) + b_chunk
@@ -688,17 +692,19 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                 const int stride = b_active ? G::kChunks : 0;
 #pragma unroll
                 for (int k = 0; k < kMfmaPerTile; k++) B[k] = src[k * stride];
+                gf = gfac_lane[slice * G::kChunks];
                 // an all-zero weight row gives the "+1" term of the code, to be subtracted
                 bias = tile_product(zero4, zero4, B);
                 // wide tiles: the one bias entry this lane uses
-                bias_sel = lane_select(lane_select(bias[0], bias[1], odd_lanes),
-                                       lane_select(bias[2], bias[3], odd_lanes), hi_lanes);
+                bias_sel = gf * lane_select(lane_select(bias[0], bias[1], odd_lanes),
+                                            lane_select(bias[2], bias[3], odd_lanes), hi_lanes);
+                bias = bias * gf;
             };
             if constexpr (kFine) {
                 // one flat sequence of (walk, slot) pairs, three at a time through the ring
                 u4 B[kMfmaPerTile];
                 f4 bias;
-                float bias_sel = 0.0f;
+                float bias_sel = 0.0f, gf = 0.0f;
                 int wi = 0, j = 0, c_begin = 0, n_rb = 0;
                 const int total = my_walks * n_slots;
                 for (int t0 = 0; t0 < total; t0 += G::kAhead) {
@@ -710,9 +716,9 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                                 const int chunk = walk / seg_n, slice = walk - chunk * seg_n;
                                 c_begin = r_begin + chunk * chunk_rows;
                                 n_rb = chunk_tiles(chunk);
-                                load_operands(slice, B, bias, bias_sel);
+                                load_operands(slice, B, bias, bias_sel, gf);
                             }
-                            process_tile(ring[k], c_begin + min(j, max(n_rb, 1) - 1) * G::kRows, j < n_rb, B, bias, bias_sel);
+                            process_tile(ring[k], c_begin + min(j, max(n_rb, 1) - 1) * G::kRows, j < n_rb, B, bias, bias_sel, gf);
                             if (++j == n_slots) {
                                 j = 0;
                                 wi++;
@@ -728,22 +734,13 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                 const int chunk = walk / seg_n, slice = walk - chunk * seg_n;
                 const int c_begin = r_begin + chunk * chunk_rows;
                 const int n_rb = chunk_tiles(chunk);  // live tiles of this walk (0: nothing to add)
-                // this slice's activations become the B operands. Every lane reads (no branch): the
-                // idle lanes read the zero operand with stride 0.
+                // this slice's activations become the B operands
                 u4 B[kMfmaPerTile];
-                const u4 *src = b_active ? reinterpret_cast<const u4 *>(image + (size_t)bcol * img_stride +
-                                                                        slice * G::kCols) + b_chunk
-                                         : &zero_operand;
-                const int stride = b_active ? G::kChunks : 0;
-#pragma unroll
-                for (int k = 0; k < kMfmaPerTile; k++) B[k] = src[k * stride];
-                // an all-zero weight row gives the "+1" term of the code, to be subtracted
-                const f4 bias = tile_product(zero4, zero4, B);
-                // wide tiles: the one bias entry this lane uses
-                const float bias_sel = lane_select(lane_select(bias[0], bias[1], odd_lanes),
-                                                   lane_select(bias[2], bias[3], odd_lanes), hi_lanes);
+                f4 bias;
+                float bias_sel, gf;
+                load_operands(slice, B, bias, bias_sel, gf);
 
-                auto process = [&](const Tile<G> &t, int rb, bool live) { process_tile(t, rb, live, B, bias, bias_sel); };
+                auto process = [&](const Tile<G> &t, int rb, bool live) { process_tile(t, rb, live, B, bias, bias_sel, gf); };
 
                 // No branch surrounds a load or an MFMA, so the wait counters stay exact and
                 // G::kAhead - 1 tiles remain in flight while one is consumed.
@@ -771,11 +768,30 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
         // ------------------------------------------------ add the waves' partial sums in wave order, store fp16
         {
             const int nrows = r_end - r_begin;
+            // what the activations that stayed out of the image add to a row: scale * (+-x) where the row holds a
+            // weight on the column, nothing where it holds none
+            const int n_out = min(n_outliers, kMaxOutliers);
+            auto outlier_sum = [&](const uint32_t *w_nz, const uint32_t *w_sg, const uint16_t *w_sc, int row, int b) -> float {
+                float corr = 0.0f;
+                for (int o = 0; o < n_out; o++) {
+                    const uint32_t vb = out_val[o];
+                    if ((int)(vb >> 16) != b) continue;
+                    const int col = out_col[o];
+                    const size_t at = (size_t)row * words + (col >> 5);
+                    const uint32_t bit = 1u << (col & 31);
+                    if (w_nz[at] & bit) {
+                        const float xv = h2f((uint16_t)vb);
+                        corr += h2f(w_sc[(size_t)row * groups + (col >> 7)]) * ((w_sg[at] & bit) ? xv : -xv);
+                    }
+                }
+                return corr;
+            };
             for (int idx = tid; idx < nrows * p.batch; idx += kThreads) {
                 const int b = idx / nrows, rl = idx - b * nrows;
                 float sum = 0.0f;
 #pragma unroll
                 for (int w = 0; w < kNW; w++) sum += partial[w * wave_stride + (size_t)rl * p.batch + b];
+                if (n_out) sum += outlier_sum(p.nz, p.sg, p.scales, r_begin + rl, b);
                 uint16_t out = f2h(sum * fscale[b]);
                 if (pair) {
                     // out = silu(gate) * up on the fp16-rounded projections, in fp32: what the two
@@ -784,6 +800,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
 #pragma unroll
                     for (int w = 0; w < kNW; w++)
                         sum_up += partial[sc.pair_stride + w * wave_stride + (size_t)rl * p.batch + b];
+                    if (n_out) sum_up += outlier_sum(sc.table[pi + 1].nz, sc.table[pi + 1].sg, sc.table[pi + 1].scales, r_begin + rl, b);
                     const float g = h2f(out), up = h2f(f2h(sum_up * fscale[b]));
                     out = f2h(g / (1.0f + expf(-g)) * up);
                 }
@@ -871,7 +888,8 @@ int image_bytes_of(int cols, int batch, bool segmented = true) {
         const int n_seg = (slices + seg_max - 1) / seg_max;
         slices = (slices + n_seg - 1) / n_seg;
     }
-    return slices * G::kCols * 2 * batch;
+    const int image = slices * G::kCols * 2 * batch;
+    return image + image / 64;  // and one fp32 factor per 128-column group
 }
 
 // Geometry limits: a tile must fit inside the matrix (edge tiles are moved back, not clipped).

@@ -73,6 +73,7 @@ class gemm_forced:
         self.want.update({self.NAMES[k]: int(v) for k, v in kw.items()})
 
     def __enter__(self):
+        import ternary_llm_amd as tl
         self.ctx = tl.tuning(**self.want)
         self.ctx.__enter__()
         return self

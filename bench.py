@@ -12,8 +12,8 @@ The same run measures every other benchmark configuration and reports them in `c
   cfg2  the LLaMA-1B layer set x 16 layers as one plan (cache-resident 258 MB, and rotated over 775 MB)
   cfg3  the 8B sweep at batch 1 (the headline), 4 and 16
   cfg4  the prefill GEMM, M in {16, 128, 512, 2048} x {gate/up 14336 x 4096, down 4096 x 14336}
-  cfg5  LLaMA-70B, all 80 layers resident (18.2 GB packed), batch 1 and 16 (--sparsity-sweep adds
-        P(0) = 0.2 and 0.7)
+  cfg5  LLaMA-70B, all 80 layers resident (18.2 GB packed), batch 1 and 16, at P(0) = 0.42, 0.2 and 0.7
+  lm_head  the ternary output head (128256 x 4096 and 128256 x 8192), one GEMV per call
 plus `single_calls` (the reference's own call pattern, one operator call per matrix, replayed from a
 captured HIP graph so that no host time is in the figure: fp16 and int8 activations, and the dependent
 chain of a decode step), `copy_ceiling` (what this GPU streams with a plain read / copy kernel) and
@@ -38,13 +38,31 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense FP16 matrix peak
-# HBM bytes one launch of the headline workload moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
-# copy kernel of known size (profiles/gemv_mfma_wide__llama8b_sweep_b1.md); valid for that workload only.
-HEADLINE_TRAFFIC_BYTES = 1923342227
-HEADLINE_TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this workload (profiles/gemv_mfma_wide__llama8b_sweep_b1.md), not read in this run"
-# The same for the 8B sweep with 4 and with 16 activation rows (profiles/gemv_batch__llama8b_sweep_b4_b16.md): bytes per launch.
-BATCH_SWEEP_TRAFFIC_BYTES = {4: 2297534500, 16: 2050618752}
-BATCH_SWEEP_TRAFFIC_SOURCE = "rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this workload (profiles/gemv_batch__llama8b_sweep_b4_b16.md), not read in this run"
+# HBM bytes one launch moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a copy kernel of known size
+# (the profile named beside each figure); valid for that workload only, and only for the kernel source it was
+# profiled on: `sha256_16` is the first 16 hex digits of the sha256 of that csrc file then. The bench recomputes the
+# hash and marks the figure `traffic_stale` when the file has changed since.
+TRAFFIC = {
+    "headline": {"bytes": 1923342227, "file": "gemv_mfma.hip", "sha256_16": "PENDING",
+                 "source": "rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this workload (profiles/gemv_mfma_wide__llama8b_sweep_b1.md), not read in this run"},
+    4: {"bytes": 2297534500, "file": "gemv_mfma.hip", "sha256_16": "PENDING",
+        "source": "rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this workload (profiles/gemv_batch__llama8b_sweep_b4_b16.md), not read in this run"},
+    16: {"bytes": 2050618752, "file": "gemv_batch.hip", "sha256_16": "PENDING",
+         "source": "rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this workload (profiles/gemv_batch__llama8b_sweep_b4_b16.md), not read in this run"},
+}
+
+
+def traffic_fields(key, algorithmic_bytes):
+    """The profiled HBM bytes per launch of a workload, with the check that the kernel source is still the one profiled."""
+    import hashlib
+    t = TRAFFIC[key]
+    path = os.path.join(ROOT, "ternary-llm_amd", "csrc", t["file"])
+    with open(path, "rb") as f:
+        now = hashlib.sha256(f.read()).hexdigest()[:16]
+    return {"traffic": t["bytes"], "traffic_over_algorithmic": round(t["bytes"] / algorithmic_bytes, 3),
+            "traffic_source": t["source"], "traffic_profiled_on": f"{t['file']} sha256 {t['sha256_16']}",
+            "traffic_stale": now != t["sha256_16"]}
+
 
 SHAPES = {
     # name: (hidden, q_dim, kv_dim, ffn, layers)
@@ -490,6 +508,25 @@ def decode_chain(torch, tl, problems, model, layers):
                          ("RMSNorm prologue + SwiGLU pair: 4 per layer", four, 4)), "close": close}
 
 
+def lm_head_rows(torch, tl, orc, timer, seed):
+    """The ternary output head of a .tllm model (reference src/transformer.cpp:308-311: ternary_linear on
+    vocab x hidden): one batch-1 GEMV per call on 128256 x 4096 (8B) and 128256 x 8192 (70B), back-to-back calls."""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(seed + 77)
+    out = []
+    for rows, cols in ((128256, 4096), (128256, 8192)):
+        nz, sg = gen_masks(torch, rows, cols, 0.42, gen)
+        sc = (torch.rand((rows, cols // 128), device="cuda", generator=gen) * 0.02 + 0.01).to(torch.float16)
+        x = torch.randn((1, cols), device="cuda", generator=gen).to(torch.float16)
+        y = torch.zeros((1, rows), dtype=torch.float16, device="cuda")
+        t = timer.run(lambda: tl.ternary_gemv(nz, sg, sc, x, y, rows, cols, 128), 100, 10)
+        parity = check_sample(orc, [(nz, sg, sc, x, y, rows, cols, 1)], [0])
+        out.append(hbm_row(f"lm_head: {rows}x{cols} GEMV, one call", t, packed_bytes(rows, cols), "tllm::gemv_mfma_kernel<Wide>", parity,
+                           "the same matrix every call: " + ("fits" if packed_bytes(rows, cols) < 256 * 2 ** 20 else "exceeds") + " the 256 MB Infinity Cache"))
+        del nz, sg, sc
+    return out
+
+
 def copy_ceiling(torch, tl, timer):
     """What this GPU moves with nothing to compute: a read-only pass over 4 GiB (the library's streaming kernel:
     16-byte non-temporal loads; a few launch shapes are tried and the best is kept) and a device-to-device copy of
@@ -497,12 +534,15 @@ def copy_ceiling(torch, tl, timer):
     src = torch.ones(1 << 30, dtype=torch.int32, device="cuda")
     best = None
     for shape in ("3,16", "8,8", "24,4", "32,8"):   # workgroups per CU, loads in flight per thread
-        os.environ["TLLM_READ_SHAPE"] = shape
+        per_cu, flight = (int(v) for v in shape.split(","))
+        tl.set_tuning("read_wgs_per_cu", per_cu)
+        tl.set_tuning("read_in_flight", flight)
         t = timer.run(lambda: tl.read_stream(src), 20, 3)
         rate = src.numel() * 4 / (t["mean_ms"] * 1e-3) / 1e9
         if best is None or rate > best[0]:
             best = (rate, src.numel() * 4 / (t["min_ms"] * 1e-3) / 1e9, shape)
-    os.environ.pop("TLLM_READ_SHAPE", None)
+    tl.set_tuning("read_wgs_per_cu", 8)
+    tl.set_tuning("read_in_flight", 8)
     half = src[: 1 << 29]
     dst = torch.empty_like(half)
     t2 = timer.run(lambda: dst.copy_(half), 20, 3)
@@ -578,7 +618,7 @@ def main():
     ap.add_argument("--gemm-m", default="16,128,512,2048", help="token counts M of configuration 4")
     ap.add_argument("--gemm-calls", type=int, default=200, help="timed launches per GEMM case")
     ap.add_argument("--gemm-warm", type=int, default=20, help="untimed launches before them (after the settle phase)")
-    ap.add_argument("--sparsity-sweep", action="store_true", help="configuration 5 also at P(0) = 0.2 and 0.7")
+    ap.add_argument("--no-sparsity-sweep", action="store_true", help="configuration 5 at P(0) = 0.42 only (default: also 0.2 and 0.7)")
     ap.add_argument("--no-single-calls", action="store_true")
     ap.add_argument("--seed", type=int, default=20240611)
     args = ap.parse_args()
@@ -654,8 +694,7 @@ def main():
             "bound": "hbm", "achieved": round(gbps, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(gbps / HBM_PEAK_GBS, 4),
             "frac_best_group": round(sweep_bytes / (t["min_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-            "traffic": HEADLINE_TRAFFIC_BYTES if headline else None,
-            "traffic_source": HEADLINE_TRAFFIC_SOURCE if headline else None,
+            **(traffic_fields("headline", sweep_bytes) if headline else {"traffic": None}),
             "kernel": plan.kernel if args.mode == "plan" else "per-matrix launches",
             "bytes_per_launch": sweep_bytes // launches_per_step,
         },
@@ -679,10 +718,8 @@ def main():
             r, _ = plan_rows(torch, tl, orc, timer, "cfg3: llama8b 32-layer sweep", "llama8b", 32, extra, 0.42, 0.01, 0.03,
                              args.seed, cfg_steps, 20, problems=problems)
             for row, b in zip(r, extra):
-                if b in BATCH_SWEEP_TRAFFIC_BYTES:
-                    row["traffic"] = BATCH_SWEEP_TRAFFIC_BYTES[b]
-                    row["traffic_over_algorithmic"] = round(BATCH_SWEEP_TRAFFIC_BYTES[b] / sweep_bytes, 3)
-                    row["traffic_source"] = BATCH_SWEEP_TRAFFIC_SOURCE
+                if b in TRAFFIC:
+                    row.update(traffic_fields(b, sweep_bytes))
             cfgs += r
             cfgs.append(int8_sweep_row(torch, tl, orc, timer, "cfg3: llama8b 32-layer sweep, batch 1, int8 activations (plan of ternary_gemv_int8)",
                                        problems, cfg_steps, 20))
@@ -700,11 +737,18 @@ def main():
         if not args.no_single_calls and headline:
             out["single_calls"] = single_call_rows(torch, tl, timer, problems, "llama8b", 32)
         if 5 in want:
-            zs = [0.42] + ([0.2, 0.7] if args.sparsity_sweep else [])
+            zs = [0.42] + ([] if args.no_sparsity_sweep else [0.2, 0.7])
             for pz in zs:
                 r, _ = plan_rows(torch, tl, orc, timer, f"cfg5: llama70b 80-layer sweep resident, P(0)={pz}", "llama70b", 80, [1, 16],
                                  pz, 0.005, 0.02, args.seed + 5, 40, 5)
                 cfgs += r
+        if 3 in want and headline:
+            cfgs += lm_head_rows(torch, tl, orc, timer, args.seed)
+            # the headline once more from idle clocks: no settle phase, the driver's own warm-up and step counts
+            cold = Timer(torch, 0.0).run(step, 20, 5)
+            out["cold_start"] = {"ms_per_step": round(cold["mean_ms"], 5), "GBps": round(sweep_bytes / (cold["mean_ms"] * 1e-3) / 1e9, 1),
+                                 "frac_hbm_peak": round(sweep_bytes / (cold["mean_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                                 "what": "the headline step with settle_ms 0, warmup 5, steps 20, measured right after host-side work (clocks not settled)"}
         out["configs"] = cfgs
         out["copy_ceiling"] = copy_ceiling(torch, tl, timer)
     if not args.no_cpu_baseline:

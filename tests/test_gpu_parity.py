@@ -1600,3 +1600,45 @@ def test_captured_split_gemm_survives_later_larger_shapes(dev, oracle):
             tl.gemm_workspace_reserve(Ml, Nl, Kl, 128, stream=side)
         torch.cuda.synchronize()
     del graph
+
+
+@pytest.mark.parametrize("cols", [4096, 8192])
+def test_lm_head_shape_every_output(dev, oracle, cols):
+    """The ternary output head of a .tllm model (reference src/transformer.cpp:308-311, src/model.cpp lm_head branch):
+    128256 rows, far more than any projection. Batch 1 (single call and int8 pair), 4 and 16 activation rows, every
+    output against the fp32 product of the expanded weights, which is itself checked against the fp64 oracle on
+    samples."""
+    torch, tl = dev
+    rows = 128256
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(8800 + cols)
+    nz, sg, sc = _device_problem(torch, rows, cols, 0.42, 0.01, 0.03, gen)
+    W = _dense_weights(torch, nz, sg, sc)
+    for batch in (1, 4, 16):
+        x = torch.randn((batch, cols), device="cuda", generator=gen).to(torch.float16)
+        ref = x.float() @ W.t()
+        y = torch.full((batch, rows), float("nan"), dtype=torch.float16, device="cuda")
+        if batch == 1:
+            tl.ternary_gemv(nz, sg, sc, x[0], y[0], rows, cols, 128)
+        else:
+            tl.ternary_gemm(x, nz, sg, sc, y, batch, rows, cols, 128)
+        torch.cuda.synchronize()
+        if batch == 1:
+            _check_sampled(oracle, torch, x, nz, sg, sc, ref, 1, 48, cols, f"dense fp32 product {rows}x{cols}")
+        tau = float(torch.sqrt(torch.mean(ref * ref)).item()) / 64.0
+        rel = (y.float() - ref).abs() / torch.clamp(ref.abs(), min=tau)
+        bad = int((~(rel <= TOL)).sum().item())
+        assert bad == 0, f"lm_head {rows}x{cols} batch {batch}: {bad} outputs beyond {TOL}, max_rel {float(rel.max()):.3e}"
+        del ref, rel
+    # the reference's decode path: quantise, then the int8 GEMV with the device-resident scale
+    x = torch.randn((1, cols), device="cuda", generator=gen).to(torch.float16)
+    q = torch.zeros(cols, dtype=torch.int8, device="cuda")
+    qs = torch.zeros(1, dtype=torch.float32, device="cuda")
+    yi = torch.full((1, rows), float("nan"), dtype=torch.float16, device="cuda")
+    tl.quantize_absmax_int8(x, q, qs, cols)
+    tl.ternary_gemv_int8(nz, sg, sc, q, qs, yi[0], rows, cols, 128)
+    torch.cuda.synchronize()
+    ref = (q.float() * qs) @ W.t()
+    tau = float(torch.sqrt(torch.mean(ref * ref)).item()) / 64.0
+    rel = (yi[0].float() - ref).abs() / torch.clamp(ref.abs(), min=tau)
+    assert float(rel.max()) <= TOL, f"lm_head int8 {rows}x{cols}: max_rel {float(rel.max()):.3e}"

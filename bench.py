@@ -424,7 +424,13 @@ def single_call_rows(torch, tl, timer, problems, model, layers):
             tl.quantize_absmax_int8(x, q8[cols], qs[cols], cols)
             tl.ternary_gemv_int8(nz, sg, sc, q8[cols], qs[cols], y, rows, cols, 128)
 
+    def i8_fused_calls():   # the same linear as ONE launch: quantised inside the GEMV, bit-identical to the pair
+        for nz, sg, sc, x, y, rows, cols, _ in problems:
+            tl.ternary_linear_int8(nz, sg, sc, x, y, rows, cols, 128)
+
     for name, fn, kernel in ((f"single calls, fp16 activations: {n} x ternary_gemv from one graph", f16_calls, "tllm::gemv_mfma_kernel<Wide, fine>"),
+                             (f"single calls, int8 linear in one launch: {n} x ternary_linear_int8 (quantised inside the GEMV) from one graph", i8_fused_calls,
+                              "tllm::gemv_mfma_kernel<Wide, fine>, input quantised in the staging pass"),
                              (f"single calls, int8 activations: {n} x (quantize_absmax_int8 + ternary_gemv_int8) from one graph", i8_calls,
                               "tllm::gemv_mfma_kernel<Wide, fine> on int8 activations")):
         graph = capture(torch, fn)

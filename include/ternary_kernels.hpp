@@ -84,6 +84,19 @@ inline void quantize_absmax_int8(const half *input, int8_t *output, float *scale
            tllm_quantize_absmax_i8(reinterpret_cast<const uint16_t *>(input), output, scale, n, stream));
 }
 
+// The reference's INT8 linear as one call (no counterpart in include/kernels.cuh: there it is the member function
+// Transformer::ternary_linear_int8, src/transformer.cpp:126-143, which quantises, copies the scale to the host and
+// calls ternary_gemv_int8). Same result bit for bit; no int8 buffer, no scale, no copy.
+inline void ternary_linear_int8(const uint32_t *nonzero_masks, const uint32_t *sign_masks,
+                                const half *weight_scales, const half *input, half *output, int rows,
+                                int cols, int group_size, hipStream_t stream = 0) {
+    report("ternary_linear_int8",
+           tllm_ternary_linear_int8_f16(nonzero_masks, sign_masks,
+                                        reinterpret_cast<const uint16_t *>(weight_scales),
+                                        reinterpret_cast<const uint16_t *>(input),
+                                        reinterpret_cast<uint16_t *>(output), rows, cols, group_size, stream));
+}
+
 // Reference include/kernels.cuh:37-40.
 inline void ternary_gemm(const half *A, const uint32_t *nz_B, const uint32_t *sign_B,
                          const half *scales_B, half *C, int M, int N, int K, int group_size,

@@ -77,6 +77,16 @@ int tllm_ternary_gemv_i8(const uint32_t *nonzero_masks, const uint32_t *sign_mas
                          tllm_stream_t stream);
 
 /*
+ * The reference's whole INT8 linear in one launch: absmax-quantises the fp16 `input` (as tllm_quantize_absmax_i8
+ * does) inside the GEMV and multiplies (as tllm_ternary_gemv_i8 does); `output` holds, bit for bit, what the two
+ * calls store. No int8 buffer, no scale, no device-to-host copy. Replaces Transformer::ternary_linear_int8,
+ * reference src/transformer.cpp:126-143 (kernels/activations.cu:88-151 + kernels/ternary_gemv.cu:116-216).
+ */
+int tllm_ternary_linear_int8_f16(const uint32_t *nonzero_masks, const uint32_t *sign_masks,
+                                 const uint16_t *weight_scales, const uint16_t *input, uint16_t *output,
+                                 int rows, int cols, int group_size, tllm_stream_t stream);
+
+/*
  * Same as tllm_ternary_gemv_i8 but reads the activation scale from DEVICE memory
  * (the float written by tllm_quantize_absmax_i8), so a decode step needs no
  * device-to-host copy between the two calls. No counterpart in the reference, which
@@ -234,7 +244,7 @@ typedef struct tllm_linear_problem {
     int32_t rows;
     int32_t cols;
     int32_t batch; /* 1..TLLM_MAX_PLAN_BATCH */
-    int32_t flags; /* 0, or TLLM_PROBLEM_SWIGLU_GATE */
+    int32_t flags; /* 0, TLLM_PROBLEM_SWIGLU_GATE or TLLM_PROBLEM_QUANTIZE_INPUT */
 } tllm_linear_problem;
 
 enum { TLLM_MAX_PLAN_BATCH = 16 };
@@ -249,6 +259,15 @@ enum { TLLM_MAX_PLAN_BATCH = 16 };
  * half, src/transformer.cpp:266-286 (gate GEMV, up GEMV, silu_mul_forward).
  */
 enum { TLLM_PROBLEM_SWIGLU_GATE = 1 };
+
+/*
+ * Flag of a problem whose fp16 input the launch quantises to int8 itself before it multiplies (batch 1, not with
+ * a SwiGLU pair or an RMSNorm prologue): the output is what tllm_quantize_absmax_i8 followed by
+ * tllm_ternary_gemv_i8_dscale stores for that matrix, bit for bit, without the int8 vector and its scale ever being
+ * written. Replaces the reference's ternary_linear_int8 (src/transformer.cpp:126-143: quantise, copy the scale to
+ * the host, int8 GEMV) for every linear of a group in one launch.
+ */
+enum { TLLM_PROBLEM_QUANTIZE_INPUT = 2 };
 
 typedef struct tllm_linear_plan tllm_linear_plan;
 

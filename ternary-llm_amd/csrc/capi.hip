@@ -141,6 +141,15 @@ int tllm_ternary_gemv_i8(const uint32_t *nonzero_masks, const uint32_t *sign_mas
                           nullptr, output, rows, cols, group_size, stream);
 }
 
+int tllm_ternary_linear_int8_f16(const uint32_t *nonzero_masks, const uint32_t *sign_masks,
+                                 const uint16_t *weight_scales, const uint16_t *input, uint16_t *output,
+                                 int rows, int cols, int group_size, tllm_stream_t stream) {
+    Problem p{nonzero_masks, sign_masks, weight_scales, input, output, rows, cols, 1, tllm::kProblemQuantInput};
+    if (int e = tllm::check_linear(p, group_size)) return e;
+    if (group_size == 128 && tllm::gemv_mfma_supports(p, group_size)) return (int)tllm::launch_gemv_mfma(p, (hipStream_t)stream);
+    return (int)tllm::launch_gemv_rowwave_q8(p, group_size, (hipStream_t)stream);
+}
+
 int tllm_ternary_gemv_i8_dscale(const uint32_t *nonzero_masks, const uint32_t *sign_masks,
                                 const uint16_t *weight_scales, const int8_t *input_int8,
                                 const float *input_scale_device, uint16_t *output, int rows,
@@ -245,7 +254,12 @@ static int create_plan(tllm_linear_plan **plan, const tllm_linear_problem *probl
         host[i] = Problem{q.nonzero_masks, q.sign_masks, q.scales, q.input, q.output,
                           q.rows, q.cols, q.batch, q.flags};
         if (q.batch < 1 || q.batch > TLLM_MAX_PLAN_BATCH) return TLLM_ERR_BAD_PLAN;
-        if (q.flags & ~TLLM_PROBLEM_SWIGLU_GATE) return TLLM_ERR_BAD_PLAN;
+        if (q.flags & ~(TLLM_PROBLEM_SWIGLU_GATE | TLLM_PROBLEM_QUANTIZE_INPUT)) return TLLM_ERR_BAD_PLAN;
+        if (q.flags & TLLM_PROBLEM_QUANTIZE_INPUT) {
+            // quantised inside the launch: one activation row, fp16 input, neither pair nor prologue
+            if (q.batch != 1 || (q.flags & TLLM_PROBLEM_SWIGLU_GATE) || input_scales || (norm_weights && norm_weights[i]))
+                return TLLM_ERR_BAD_PLAN;
+        }
         const bool is_up = i > 0 && (problems[i - 1].flags & TLLM_PROBLEM_SWIGLU_GATE);
         if (is_up) {
             // the up half of a SwiGLU pair: same shape and activations as its gate, no output of its own

@@ -30,7 +30,7 @@ struct Problem {
     int32_t rows;
     int32_t cols;
     int32_t batch;
-    int32_t flags;  // kProblemSwigluGate, kProblemInt8Input
+    int32_t flags;  // kProblemSwigluGate, kProblemQuantInput, kProblemInt8Input
     union {
         // optional prologue (plans only): x is RMS-normalised with these weights before it is used
         const uint16_t *norm_w;
@@ -44,6 +44,9 @@ struct Problem {
 static_assert(sizeof(Problem) == sizeof(tllm_linear_problem) + 16, "tllm_linear_problem, then the prologue");
 constexpr int kProblemSwigluGate = TLLM_PROBLEM_SWIGLU_GATE;
 constexpr int kProblemInt8Input = 0x100;  // set by tllm_linear_plan_create_i8, not a public flag
+// fp16 activations that the kernel quantises to int8 itself (absmax, reference kernels/activations.cu:88-142) before it
+// multiplies: quantize_absmax_int8 + ternary_gemv_int8 in one launch, bit for bit (batch 1)
+constexpr int kProblemQuantInput = TLLM_PROBLEM_QUANTIZE_INPUT;
 
 // Tuning switches. Each is read from its environment variable ONCE, when the library first asks for any of them;
 // afterwards only tllm_debug_set_tuning changes them (tests force kernel choices through it). No call path reads the
@@ -107,6 +110,8 @@ hipError_t launch_gemv_rowwave_i8(const uint32_t *nz, const uint32_t *sg, const 
                                   uint16_t *y, int rows, int cols, int group, hipStream_t s);
 hipError_t launch_quantize_absmax_i8(const uint16_t *x, int8_t *q, float *scale, int n,
                                      hipStream_t s);
+// quantize_absmax_int8 + ternary_gemv_int8 in one launch for the shapes the matrix-core kernel does not serve
+hipError_t launch_gemv_rowwave_q8(const Problem &p, int group, hipStream_t s);
 
 // Element-wise neighbours of the linears (elementwise.hip).
 hipError_t launch_rmsnorm(const uint16_t *input, const uint16_t *weight, uint16_t *output, const uint16_t *residual,

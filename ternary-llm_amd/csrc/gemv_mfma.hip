@@ -123,6 +123,22 @@ __device__ __forceinline__ float dpp_add(float v) {
     const int r = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), kCtrl, 0xF, 0xF, true);
     return v + __builtin_bit_cast(float, r);
 }
+// The largest value any lane of the wave holds, as a wave-uniform number: four DPP rotations inside the rows of 16
+// lanes, then one lane of each row read into a scalar (much shorter than a butterfly of cross-lane permutes).
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t m) {
+    m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x128, 0xF, 0xF, true));  // row_ror:8
+    m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x124, 0xF, 0xF, true));  // row_ror:4
+    m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x122, 0xF, 0xF, true));  // row_ror:2
+    m = max(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x121, 0xF, 0xF, true));  // row_ror:1
+    const uint32_t a = (uint32_t)__builtin_amdgcn_readlane((int)m, 0), b = (uint32_t)__builtin_amdgcn_readlane((int)m, 16);
+    const uint32_t c = (uint32_t)__builtin_amdgcn_readlane((int)m, 32), d = (uint32_t)__builtin_amdgcn_readlane((int)m, 48);
+    return max(max(a, b), max(c, d));
+}
+// fp16 bits -> magnitude bits for a maximum that skips NaN the way fmaxf does (Inf counts)
+__device__ __forceinline__ uint32_t finite_magnitude(uint32_t half_bits) {
+    const uint32_t mag = half_bits & 0x7FFFu;
+    return mag > 0x7C00u ? 0u : mag;
+}
 constexpr int kQuadSwap1 = 0xB1;       // quad_perm [1,0,3,2]
 constexpr int kQuadSwap2 = 0x4E;       // quad_perm [2,3,0,1]
 constexpr int kRowHalfMirror = 0x141;  // lane k <-> 7-k inside each 8 lanes
@@ -203,6 +219,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
     uint16_t *image = reinterpret_cast<uint16_t *>(lds + sc.image_bytes / 65);
     float *partial = reinterpret_cast<float *>(lds + sc.image_bytes);
     __shared__ float red_ss[kNW];
+    __shared__ float q_inv, q_scale;  // absmax quantisation of the staged problem's activations (kProblemQuantInput)
     __shared__ float fscale[kMaxBatch];
     __shared__ u4 zero_operand;  // what the idle lanes of a B operand read
     // Activations that stay out of the operand image (see stage_piece): column, fp16 bits | batch column << 16
@@ -296,9 +313,54 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
             seg_lo = seg * seg_len;
             seg_n = min(seg_len, slices - seg_lo);
             img_stride = seg_n * G::kCols;
+            // Activations that the launch quantises itself (reference kernels/activations.cu:100-141): the largest
+            // magnitude of the whole row first (one pass, also for rows staged in segments: when the row's first
+            // segment is staged), then every element becomes the integer the quantisation gives it, as an fp16
+            // number, and the kernel goes on as for int8 input.
+            const bool quant = (p.flags & kProblemQuantInput) != 0;
+            // (rows that the one-pass staging below keeps in registers find their maximum there, without a second read)
+            const bool quant_from_registers = quant && n_seg == 1 && p.batch == 1 && img_stride / 8 <= 8 * kThreads;
+            if (quant && seg == 0 && !quant_from_registers) {
+                // (the magnitudes compare as their fp16 bit patterns; NaN is skipped, as fmaxf skips it)
+                uint32_t m = 0;
+                for (int c8 = tid; c8 < p.cols / 8; c8 += kThreads) {
+                    const uint4 v = reinterpret_cast<const uint4 *>(p.x)[c8];
+                    const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                    for (int e = 0; e < 4; e++) m = max(m, max(finite_magnitude(w4[e]), finite_magnitude(w4[e] >> 16)));
+                }
+                m = wave_max_u32(m);
+                if (lane == 0) red_ss[wave] = h2f((uint16_t)m);
+                __syncthreads();
+                if (tid == 0) {
+                    float amax = 0.0f;
+#pragma unroll
+                    for (int w = 0; w < kNW; w++) amax = fmaxf(amax, red_ss[w]);
+                    q_inv = amax > 0.0f ? 127.0f / amax : 0.0f;
+                    q_scale = amax > 0.0f ? amax / 127.0f : 1.0f;
+                }
+                __syncthreads();
+            }
+            const float quant_inv = quant && !quant_from_registers ? q_inv : 0.0f;
+            // eight fp16 activations -> the integers the quantisation gives them, as fp16 numbers (exact)
+            auto quantised = [](const uint4 &v, float inv) -> uint4 {
+                const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
+                uint32_t h[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    // (no clamp needed: |x| <= amax and inv = fl(127 / amax) keep the product within 127 (1 + 2^-23), which
+                    // rounds to 127; a non-finite x gives NaN here and the conversion to int makes it 0, as in the quantiser)
+                    const int r = (int)rintf(h2f((uint16_t)(w4[e >> 1] >> (16 * (e & 1)))) * inv);
+                    h[e] = f2h((float)r);
+                }
+                return uint4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
+            };
             // eight consecutive activations as fp16 bits; int8 values convert exactly
             auto load8 = [&](int b, int c8) -> uint4 {
-                if (!sc.x_is_i8) return reinterpret_cast<const uint4 *>(p.x + (size_t)b * p.cols)[c8];
+                if (!sc.x_is_i8) {
+                    const uint4 v = reinterpret_cast<const uint4 *>(p.x + (size_t)b * p.cols)[c8];
+                    return quant && !quant_from_registers ? quantised(v, quant_inv) : v;
+                }
                 const uint2 q = reinterpret_cast<const uint2 *>(p.x)[c8];
                 const uint32_t w2[2] = {q.x, q.y};
                 uint32_t h[8];
@@ -408,7 +470,8 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
             if (tid < kMaxBatch) {
                 float f = 1.0f;
                 if (sc.x_is_i8) f = sc.table ? *p.x_scale : (sc.i8_scale_dev ? *sc.i8_scale_dev : sc.i8_scale);
-                fscale[tid] = f;
+                if (quant && !quant_from_registers) f = q_scale;
+                fscale[tid] = f;  // (rows quantised from registers: set there)
             }
             // The piece addresses depend on the thread index only; hidden behind an empty asm they are
             // worked out here, each time, instead of living in registers across the whole kernel.
@@ -469,6 +532,30 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                             x = uint4{o[0], o[1], o[2], o[3]};
                             __builtin_amdgcn_sched_barrier(0);
                         }
+                    }
+                }
+                if (quant_from_registers) {
+                    // absmax quantisation of the kept pieces (pieces a moved-back last slice repeats are zeros here
+                    // and their originals are among the others: the maximum is the row's)
+                    uint32_t m = 0;
+#pragma unroll
+                    for (int k = 0; k < kKeep; k++) {
+                        const uint32_t w4[4] = {keep[k].x, keep[k].y, keep[k].z, keep[k].w};
+#pragma unroll
+                        for (int e = 0; e < 4; e++) m = max(m, max(finite_magnitude(w4[e]), finite_magnitude(w4[e] >> 16)));
+                    }
+                    m = wave_max_u32(m);
+                    if (lane == 0) red_ss[wave] = h2f((uint16_t)m);
+                    __syncthreads();
+                    float amax = 0.0f;
+#pragma unroll
+                    for (int w = 0; w < kNW; w++) amax = fmaxf(amax, red_ss[w]);
+                    const float inv = amax > 0.0f ? 127.0f / amax : 0.0f;
+                    if (tid == 0) fscale[0] = amax > 0.0f ? amax / 127.0f : 1.0f;
+#pragma unroll
+                    for (int k = 0; k < kKeep; k++) {
+                        if (stid + k * kThreads < pieces) keep[k] = quantised(keep[k], inv);
+                        __builtin_amdgcn_sched_barrier(0);
                     }
                 }
 #pragma unroll
@@ -1215,10 +1302,11 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
     };
 
     // several activation rows: the batched kernel if every problem fits it
-    bool has_pairs = false, has_norm = false;
+    bool has_pairs = false, has_norm = false, has_quant = false;
     for (const Problem &p : host) {
         has_pairs = has_pairs || (p.flags & kProblemSwigluGate);
         has_norm = has_norm || (p.norm_w != nullptr && !(p.flags & kProblemInt8Input));
+        has_quant = has_quant || (p.flags & kProblemQuantInput);  // (batch 1, no pair, no prologue: the caller has checked)
     }
     // int8 activations: all problems or none, batch 1 (the caller has checked), MFMA kernel only
     bool any_i8 = false, all_i8 = true;
@@ -1230,7 +1318,7 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
     d.x_is_i8 = any_i8;
     // SwiGLU pairs and RMSNorm prologues exist in the wide-tile MFMA GEMV kernel only (batch 1)
     d.extras = has_pairs || has_norm;
-    bool all_batch = max_batch >= 2 && !d.extras;
+    bool all_batch = max_batch >= 2 && !d.extras && !has_quant;  // (only the batch-1 family quantises its input itself)
     for (const Problem &p : host) all_batch = all_batch && gemv_batch_supports(p, 128);
     // one geometry per launch otherwise: wide tiles if every problem allows them, else tall ones
     bool all_wide = true, all_tall = true;
@@ -1291,7 +1379,7 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
         if (max_units < 1) d.use_mfma = false;
         // (again, after the demotion: the table kernel for general shapes reads fp16 activations and knows neither
         // SwiGLU pairs nor RMSNorm prologues)
-        if ((d.x_is_i8 || d.extras) && !d.use_mfma) return hipErrorInvalidValue;
+        if ((d.x_is_i8 || d.extras || has_quant) && !d.use_mfma) return hipErrorInvalidValue;
         if (d.use_mfma) {
             d.pair_stride = has_pairs ? kNW * max_units * unit * max_batch : 0;
             d.lds_bytes = max_image + kNW * max_units * unit * max_batch * 4 * mats;

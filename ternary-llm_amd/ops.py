@@ -20,7 +20,7 @@ ABI_SYMBOLS = (
     "tllm_add_f16", "tllm_rope_f16", "tllm_embedding_lookup_f16", "tllm_copy_to_kv_cache_f16",
     "tllm_linear_plan_kernel", "tllm_gemm_workspace_reserve", "tllm_gemm_workspace_release",
     "tllm_ternary_gemm_f16_static", "tllm_read_stream", "tllm_ternary_gemm_kernel",
-    "tllm_debug_set_tuning", "tllm_debug_get_tuning",
+    "tllm_debug_set_tuning", "tllm_debug_get_tuning", "tllm_ternary_linear_int8_f16",
 )
 # include/tllm_model_file.h
 FILE_ABI_SYMBOLS = (
@@ -75,6 +75,7 @@ def lib():
     L.tllm_abi_version.restype = i
     L.tllm_ternary_gemv_f16.argtypes = [vp, vp, vp, vp, vp, i, i, i, vp]
     L.tllm_ternary_gemv_i8.argtypes = [vp, vp, vp, vp, f, vp, i, i, i, vp]
+    L.tllm_ternary_linear_int8_f16.argtypes = [vp, vp, vp, vp, vp, i, i, i, vp]
     L.tllm_ternary_gemv_i8_dscale.argtypes = [vp, vp, vp, vp, vp, vp, i, i, i, vp]
     L.tllm_quantize_absmax_i8.argtypes = [vp, vp, vp, i, vp]
     L.tllm_ternary_gemm_f16.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, vp]
@@ -158,6 +159,13 @@ def ternary_gemv_int8(nonzero_masks, sign_masks, weight_scales, input_int8, inpu
                                              _ptr(input_scale), _ptr(output), rows, cols,
                                              group_size, _stream(stream))
     check(code)
+
+
+def ternary_linear_int8(nonzero_masks, sign_masks, weight_scales, input, output, rows, cols, group_size=128, stream=None):
+    """The reference's INT8 linear (Transformer::ternary_linear_int8, src/transformer.cpp:126-143) in one launch:
+    fp16 input, quantised inside the kernel; bit for bit quantize_absmax_int8 + ternary_gemv_int8."""
+    check(lib().tllm_ternary_linear_int8_f16(_ptr(nonzero_masks), _ptr(sign_masks), _ptr(weight_scales), _ptr(input),
+                                             _ptr(output), rows, cols, group_size, _stream(stream)))
 
 
 def quantize_absmax_int8(input, output, scale, n, stream=None):
@@ -261,6 +269,7 @@ def copy_to_kv_cache(k, v, k_cache, v_cache, batch, n_kv_heads, head_dim, seq_le
 
 
 SWIGLU_GATE = 1  # TLLM_PROBLEM_SWIGLU_GATE
+QUANTIZE_INPUT = 2  # TLLM_PROBLEM_QUANTIZE_INPUT
 
 
 class LinearPlan:

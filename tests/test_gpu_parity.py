@@ -1642,3 +1642,73 @@ def test_lm_head_shape_every_output(dev, oracle, cols):
     tau = float(torch.sqrt(torch.mean(ref * ref)).item()) / 64.0
     rel = (yi[0].float() - ref).abs() / torch.clamp(ref.abs(), min=tau)
     assert float(rel.max()) <= TOL, f"lm_head int8 {rows}x{cols}: max_rel {float(rel.max()):.3e}"
+
+
+@pytest.mark.parametrize("rows,cols,group", [(1024, 1024, 128), (4096, 4096, 128), (300, 11008, 128), (14336, 4096, 128),
+                                             (4096, 14336, 128), (64, 28672, 128), (200, 36864, 128), (100, 256, 128),
+                                             (50, 384, 64), (8, 128, 32)])
+def test_fused_int8_linear_equals_the_pair(dev, oracle, rows, cols, group):
+    """tllm_ternary_linear_int8_f16 (fp16 in, quantised inside the GEMV) stores the bits of quantize_absmax_int8 +
+    ternary_gemv_int8 (reference src/transformer.cpp:126-143), on the matrix-core kernel (one segment, rows staged
+    in segments) and on the general kernel (short rows, other group sizes); and stays within the bar of the
+    oracle's integer arithmetic."""
+    torch, tl = dev
+    nz, sg, s, x = synth.problem(8300 + rows, rows, cols, group=group, dontcare_sign=True)
+    x = (x.astype(np.float32) * 3.7).astype(np.float16)
+    dnz, dsg, ds, dx = up(torch, nz), up(torch, sg), up(torch, s), up(torch, x)
+    q = torch.zeros(cols, dtype=torch.int8, device="cuda")
+    qs = torch.zeros(1, dtype=torch.float32, device="cuda")
+    pair = torch.full((rows,), float("nan"), dtype=torch.float16, device="cuda")
+    fused = torch.full((rows,), float("nan"), dtype=torch.float16, device="cuda")
+    tl.quantize_absmax_int8(dx, q, qs, cols)
+    tl.ternary_gemv_int8(dnz, dsg, ds, q, qs, pair, rows, cols, group)
+    tl.ternary_linear_int8(dnz, dsg, ds, dx, fused, rows, cols, group)
+    torch.cuda.synchronize()
+    assert torch.equal(fused.view(torch.int16), pair.view(torch.int16))
+    qo, so = oracle.quantize_i8(x.view(np.uint16))
+    ref = oracle.gemv_i8_f64(nz, sg, s.view(np.uint16), qo, np.float32(so), group)
+    assert_close(oracle, fused.cpu().numpy().astype(np.float64), ref, what=f"fused int8 linear {rows}x{cols} g{group}")
+
+
+def test_fused_int8_linear_special_inputs(dev, oracle):
+    """All-zero activations (scale 1, outputs exactly 0), one non-zero element, and a plan of three problems that
+    quantise their shared input themselves (the q/k/v group of a decode step) against the three pairs."""
+    torch, tl = dev
+    rows, cols = 512, 4096
+    nz, sg, s, x = synth.problem(8400, rows, cols, dontcare_sign=True)
+    dnz, dsg, ds = up(torch, nz), up(torch, sg), up(torch, s)
+    y = torch.full((rows,), float("nan"), dtype=torch.float16, device="cuda")
+    tl.ternary_linear_int8(dnz, dsg, ds, torch.zeros(cols, dtype=torch.float16, device="cuda"), y, rows, cols, 128)
+    torch.cuda.synchronize()
+    assert bool((y.view(torch.int16) == 0).all())
+    one = np.zeros(cols, np.float16)
+    one[1234] = np.float16(-0.37)
+    tl.ternary_linear_int8(dnz, dsg, ds, up(torch, one), y, rows, cols, 128)
+    torch.cuda.synchronize()
+    w = synth.unpack_np(nz, sg)[:, 1234].astype(np.float64)
+    amax = np.float32(abs(np.float16(-0.37)))                       # the element quantises to -127, the scale is amax / 127
+    want = w * s[:, 1234 // 128].astype(np.float64) * -127.0 * float(amax / np.float32(127.0))
+    np.testing.assert_allclose(y.cpu().numpy().astype(np.float64), want, rtol=1e-3, atol=0)
+    shapes = [(4096, cols), (1024, cols), (1024, cols)]
+    dx = up(torch, x)
+    probs, pairs = [], []
+    q = torch.zeros(cols, dtype=torch.int8, device="cuda")
+    qs = torch.zeros(1, dtype=torch.float32, device="cuda")
+    tl.quantize_absmax_int8(dx, q, qs, cols)
+    for k, (r, c) in enumerate(shapes):
+        a, b, sc_, _ = synth.problem(8410 + k, r, c, dontcare_sign=True)
+        wdev = (up(torch, a), up(torch, b), up(torch, sc_))
+        out = torch.full((1, r), float("nan"), dtype=torch.float16, device="cuda")
+        probs.append((*wdev, dx.view(1, -1), out, r, c, 1, tl.QUANTIZE_INPUT))
+        ref = torch.zeros(r, dtype=torch.float16, device="cuda")
+        tl.ternary_gemv_int8(*wdev, q, qs, ref, r, c, 128)
+        pairs.append(ref)
+    plan = tl.LinearPlan(probs)
+    plan.launch()
+    torch.cuda.synchronize()
+    for pr, ref in zip(probs, pairs):
+        assert torch.equal(pr[4][0].view(torch.int16), ref.view(torch.int16))
+    plan.close()
+    with pytest.raises(tl.TllmError):      # not together with a SwiGLU pair
+        tl.LinearPlan([(*probs[1][:3], dx.view(1, -1), probs[1][4], 1024, cols, 1, tl.QUANTIZE_INPUT | tl.SWIGLU_GATE),
+                       (*probs[2][:3], dx.view(1, -1), None, 1024, cols, 1)])

@@ -36,7 +36,8 @@ enum {
     TLLM_ERR_BAD_PLAN = -6,     /* plan handle is NULL, count < 1, batch out of range, or a pair / prologue rule is broken */
     TLLM_ERR_MISALIGNED = -7,   /* masks/activations not 16-byte aligned, scales/outputs not 2-byte aligned */
     /* -8 and -9 belong to tllm_model_file.h */
-    TLLM_ERR_SCRATCH_TOO_SMALL = -10 /* tllm_ternary_gemm_f16_static: the shape needs more exchange memory than the fixed scratch */
+    TLLM_ERR_SCRATCH_TOO_SMALL = -10, /* tllm_ternary_gemm_f16_static: the shape needs more exchange memory than the fixed scratch */
+    TLLM_ERR_STAGE_TIMEOUT = -11      /* tllm_linear_plan_status: a launch of a staged plan gave up waiting between two stages */
 };
 
 /* Human-readable text for a negative TLLM_ERR_* code (host pointer, static storage). */
@@ -300,6 +301,34 @@ int tllm_linear_plan_create_normed(tllm_linear_plan **plan, const tllm_linear_pr
  */
 int tllm_linear_plan_create_i8(tllm_linear_plan **plan, const tllm_linear_problem *problems,
                                const float *const *input_scales, int count, int group_size);
+/*
+ * A plan whose problems DEPEND on each other, run in stages inside ONE launch: stages[i] (HOST array, ascending from 0,
+ * at most 8 stages) says after which problems problem i runs; the problems of one stage are independent, and every
+ * problem of stage s + 1 may read what stage s stored. Between two stages the workgroups of the launch wait for each
+ * other at a counter in device memory instead of ending the kernel, which saves the start, the drain and the launch gap
+ * of a kernel per stage. Replaces the dependent launches of a decode step, reference src/transformer.cpp:239-296, e.g.
+ *   stage 0  o_proj, residuals[0] = the residual stream (output = stream + projection, in place allowed)
+ *   stage 1  gate / up as a SwiGLU pair with norm_weights = the FFN norm: reads the stream through RMSNorm
+ *   stage 2  down_proj on the pair's output, residuals = the stream again
+ *   stage 3  q / k / v of the next layer with that layer's attention norm
+ * Every output equals, bit for bit, what the separate launches store (tllm_ternary_gemv_f16, tllm_add_f16, the
+ * normed / paired plans). residuals[i] (HOST array of DEVICE pointers, entries or the array itself may be NULL) is
+ * fp16 [rows]: the problem then stores fp16(residual[r] + fp16(projection)), the reference's add_forward behind the
+ * projection; it may be the problem's own output, not its input. norm_weights as in
+ * tllm_linear_plan_create_normed (may be NULL). Every problem: batch 1, group_size 128, cols a multiple of 128 between
+ * 2048 and 28672, rows >= 16 (else TLLM_ERR_BAD_PLAN). TLLM_PROBLEM_QUANTIZE_INPUT is allowed where the other plans allow it.
+ * The launch is sized so that all its workgroups are resident together; should they not be (the GPU is shared
+ * with kernels that hold its CUs for long), a workgroup gives up after about a second of waiting, every workgroup
+ * ends normally, outputs are then incomplete, and tllm_linear_plan_status reports it.
+ */
+int tllm_linear_plan_create_staged(tllm_linear_plan **plan, const tllm_linear_problem *problems,
+                                   const uint16_t *const *norm_weights, const uint16_t *const *residuals,
+                                   const int32_t *stages, float eps, int count, int group_size);
+/* TLLM_OK, or TLLM_ERR_STAGE_TIMEOUT if a launch of this staged plan gave up waiting since the last call (the flag
+ * is read from the device and cleared; synchronise the launches you ask about first). Until it is cleared, further
+ * launches of the plan do not wait either. Plans without stages: always TLLM_OK. */
+int tllm_linear_plan_status(const tllm_linear_plan *plan);
+
 /* One launch over every problem of the plan. Allocation-free. Besides the outputs a launch uses two device
  * counters that deal the tail of a large plan out to the workgroups (the kernel resets them when it ends, so
  * replays of a captured graph need no clearing). The plan holds 16 such pairs and launches take them in turn:

@@ -66,6 +66,8 @@ const char *tllm_error_string(int code) {
         case TLLM_ERR_MISALIGNED: return "pointer alignment: masks/activations need 16 bytes, fp16 arrays 2";
         case -8: return "file cannot be opened, is truncated, or a write failed";   // TLLM_ERR_IO
         case -9: return "not a .tllm file of a supported version, or a header field is out of range";  // TLLM_ERR_BAD_FILE
+        case TLLM_ERR_STAGE_TIMEOUT:
+            return "a launch of a staged plan gave up waiting for a stage (its workgroups were not all running at the same time)";
         case TLLM_ERR_SCRATCH_TOO_SMALL:
             return "the split-K exchange of this GEMM shape needs more than the fixed device scratch of "
                    "tllm_ternary_gemm_f16_static (TLLM_GEMM_STATIC_SCRATCH_BYTES): use tllm_ternary_gemm_f16";
@@ -242,7 +244,8 @@ int tllm_read_stream(const void *src, size_t bytes, uint32_t *sink, tllm_stream_
 
 static int create_plan(tllm_linear_plan **plan, const tllm_linear_problem *problems,
                        const uint16_t *const *norm_weights, float eps, int count, int group_size,
-                       const float *const *input_scales = nullptr) {
+                       const float *const *input_scales = nullptr, const uint16_t *const *residuals = nullptr,
+                       const int32_t *stages = nullptr) {
     if (!plan || !problems) return TLLM_ERR_NULL_POINTER;
     *plan = nullptr;
     if (count < 1) return TLLM_ERR_BAD_PLAN;
@@ -294,11 +297,24 @@ static int create_plan(tllm_linear_plan **plan, const tllm_linear_problem *probl
         } else if (is_up && norm_weights && norm_weights[i - 1]) {
             return TLLM_ERR_BAD_PLAN;  // the halves of a pair see the same activations
         }
+        if (stages) {
+            // staged plans: one activation row; an up problem shares its gate's stage; the residual of the epilogue is
+            // fp16 [rows] and may be the output itself, but not the input
+            if (q.batch != 1 || stages[i] < 0 || stages[i] >= tllm::kMaxStages) return TLLM_ERR_BAD_PLAN;
+            if (is_up && stages[i] != stages[i - 1]) return TLLM_ERR_BAD_PLAN;
+            host[i].stage = stages[i];
+            if (residuals && residuals[i]) {
+                if (is_up || (q.flags & TLLM_PROBLEM_SWIGLU_GATE)) return TLLM_ERR_BAD_PLAN;
+                if (tllm::misaligned(residuals[i], 2)) return TLLM_ERR_MISALIGNED;
+                if (tllm::overlaps(residuals[i], (size_t)q.rows * 2, q.input, (size_t)q.cols * 2)) return TLLM_ERR_ALIAS;
+                host[i].residual = residuals[i];
+            }
+        }
         bytes += (int64_t)q.rows * (q.cols / 32) * 8 + (int64_t)q.rows * (q.cols / group_size) * 2;
     }
     tllm_linear_plan *pl = new (std::nothrow) tllm_linear_plan{std::move(host), {}, group_size, bytes};
     if (!pl) return TLLM_ERR_TOO_LARGE;
-    if (hipError_t e = tllm::plan_device_create(pl->host, &pl->dev)) {
+    if (hipError_t e = stages ? tllm::plan_device_create_staged(pl->host, &pl->dev) : tllm::plan_device_create(pl->host, &pl->dev)) {
         delete pl;
         // (invalid value: a shape that only the general kernel serves, which knows neither int8 activations nor pairs nor prologues)
         return e == hipErrorInvalidValue ? TLLM_ERR_BAD_PLAN : (int)e;
@@ -330,6 +346,25 @@ int tllm_linear_plan_create_i8(tllm_linear_plan **plan, const tllm_linear_proble
     return create_plan(plan, problems, nullptr, 0.0f, count, group_size, input_scales);
 }
 
+int tllm_linear_plan_create_staged(tllm_linear_plan **plan, const tllm_linear_problem *problems,
+                                   const uint16_t *const *norm_weights, const uint16_t *const *residuals,
+                                   const int32_t *stages, float eps, int count, int group_size) {
+    if (!stages) return TLLM_ERR_NULL_POINTER;
+    return create_plan(plan, problems, norm_weights, eps, count, group_size, nullptr, residuals, stages);
+}
+
+int tllm_linear_plan_status(const tllm_linear_plan *plan) {
+    if (!plan) return TLLM_ERR_BAD_PLAN;
+    if (!plan->dev.status) return TLLM_OK;
+    int v = 0;
+    if (hipError_t e = hipMemcpy(&v, plan->dev.status, sizeof v, hipMemcpyDeviceToHost)) return (int)e;
+    if (v != 0) {
+        if (hipError_t e = hipMemset(plan->dev.status, 0, sizeof v)) return (int)e;
+        return TLLM_ERR_STAGE_TIMEOUT;
+    }
+    return TLLM_OK;
+}
+
 int tllm_linear_plan_launch(const tllm_linear_plan *plan, tllm_stream_t stream) {
     if (!plan || plan->host.empty()) return TLLM_ERR_BAD_PLAN;
     return (int)tllm::plan_device_launch(plan->dev, (hipStream_t)stream);
@@ -344,6 +379,7 @@ const char *tllm_linear_plan_kernel(const tllm_linear_plan *plan) {
     const tllm::PlanDevice &d = plan->dev;
     if (d.batch_kernel) return "tllm::gemv_batch_kernel";
     if (!d.use_mfma) return "tllm::gemv_rowwave_f16_table_kernel";
+    if (d.n_stages > 0) return "tllm::gemv_mfma_kernel<Wide, extras, fine>, staged";
     if (!d.wide) return d.fine ? "tllm::gemv_mfma_kernel<Tall, fine>" : "tllm::gemv_mfma_kernel<Tall>";
     if (d.extras) return d.fine ? "tllm::gemv_mfma_kernel<Wide, extras, fine>" : "tllm::gemv_mfma_kernel<Wide, extras>";
     return d.fine ? "tllm::gemv_mfma_kernel<Wide, fine>" : "tllm::gemv_mfma_kernel<Wide>";

@@ -39,9 +39,12 @@ struct Problem {
         const float *x_scale;
     };
     float eps;
-    int32_t pad;
+    int32_t stage;  // staged plans: the problem runs after every problem of the stages before it has stored its output
+    // optional epilogue (staged plans): the output is fp16(residual[r] + fp16(projection)), the reference's add_forward
+    // behind the projection; may point at the output itself (in place)
+    const uint16_t *residual;
 };
-static_assert(sizeof(Problem) == sizeof(tllm_linear_problem) + 16, "tllm_linear_problem, then the prologue");
+static_assert(sizeof(Problem) == sizeof(tllm_linear_problem) + 24, "tllm_linear_problem, then the prologue and the epilogue");
 constexpr int kProblemSwigluGate = TLLM_PROBLEM_SWIGLU_GATE;
 constexpr int kProblemInt8Input = 0x100;  // set by tllm_linear_plan_create_i8, not a public flag
 // fp16 activations that the kernel quantises to int8 itself (absmax, reference kernels/activations.cu:88-142) before it
@@ -58,6 +61,7 @@ struct Tuning {
     std::atomic<int> batch_k_parts{0};          // TLLM_BATCH_K_PARTS: n parts where they fit, 1 never share out K
     std::atomic<int> tall_max_batch{4};         // TLLM_TALL_MAX_BATCH: most activation rows of a plan on the tall-tile kernel
     std::atomic<int> tall_min_share_milli{1000};  // TLLM_TALL_MIN_SHARE (x 1000): share of the plan per workgroup, in units, from which tall tiles run
+    std::atomic<int> stage_spin_limit{0};       // polls a workgroup of a staged plan waits for a stage (0: the plan's own limit); tests force a wait to expire with 1
     std::atomic<int> read_wgs_per_cu{8};        // TLLM_READ_SHAPE="wgs_per_cu,loads_in_flight" of tllm_read_stream
     std::atomic<int> read_in_flight{8};
 };
@@ -208,8 +212,19 @@ struct PlanDevice {
     bool x_is_i8 = false; // every problem reads int8 activations and its own device-resident scale
     int image_bytes = 0;
     int lds_bytes = 0;
+    // staged plans: the spans of stage s start at wg_first + s * (2 * grid + 1); between two stages every workgroup
+    // waits for all workgroups at a counter (n_stages counters and a "workgroups that have left" counter per launch
+    // slot, after the hand-out counters), for at most spin_limit polls; a wait that expires sets *status
+    int n_stages = 0;
+    int *stage_counters = nullptr;
+    int *status = nullptr;
+    int spin_limit = 0;
 };
 hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out);
+// A plan whose problems run in stages inside one launch (Problem::stage, ascending); batch 1, shapes the wide-tile
+// kernel serves with whole rows in LDS. hipErrorInvalidValue for a plan that does not qualify.
+hipError_t plan_device_create_staged(const std::vector<Problem> &host, PlanDevice *out);
+constexpr int kMaxStages = 8;
 hipError_t plan_device_launch(const PlanDevice &plan, hipStream_t s);
 void plan_device_destroy(PlanDevice *plan);
 

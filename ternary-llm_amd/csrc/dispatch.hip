@@ -37,7 +37,8 @@ std::atomic<int> *tuning_by_name(const char *name) {
     } all[] = {{"gemm_path", &t.gemm_path},           {"gemm_rowsplit", &t.gemm_rowsplit},
                {"gemm_pingpong", &t.gemm_pingpong},   {"batch_k_parts", &t.batch_k_parts},
                {"tall_max_batch", &t.tall_max_batch}, {"tall_min_share_milli", &t.tall_min_share_milli},
-               {"read_wgs_per_cu", &t.read_wgs_per_cu}, {"read_in_flight", &t.read_in_flight}};
+               {"read_wgs_per_cu", &t.read_wgs_per_cu}, {"read_in_flight", &t.read_in_flight},
+               {"stage_spin_limit", &t.stage_spin_limit}};
     for (const auto &e : all)
         if (name && !strcmp(name, e.name)) return e.value;
     return nullptr;

@@ -99,6 +99,16 @@ struct Sched {
     int x_is_i8;
     float i8_scale;
     const float *i8_scale_dev;
+    // Staged plans (kExtras instances): n_stages > 0; the spans of stage s start at wg_first + s * (2 * grid + 1).
+    // A workgroup that has stored the last output of its span of stage s adds one to stage_counters[s] and waits
+    // until all gridDim.x workgroups have (every workgroup is resident: the host sizes the grid for that), for at
+    // most spin_limit polls; a wait that expires sets *status to the stage's number + 1 and the workgroup leaves,
+    // and so do the others when they see it. stage_counters[kMaxStages] counts the workgroups that have left; the
+    // last one sets the counters back to zero for the next launch.
+    int n_stages;
+    int spin_limit;
+    int *stage_counters;
+    int *status;
 };
 
 // The scales that travel with a tile. Wide: the one scale of the lane's (row, group). Tall: the four scales (one
@@ -256,6 +266,16 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
     int seg_lo = 0, seg_n = 0;  // slices of the staged segment
 
     __shared__ int pool_task;
+    __shared__ int stage_reached;
+    const int n_stages = kExtras && sc.n_stages > 0 ? sc.n_stages : 1;
+    const bool staged = kExtras && sc.n_stages > 0;
+    for (int stage = 0; stage < n_stages; stage++) {
+    if (staged) {
+        const int *spans = sc.wg_first + stage * (2 * (int)gridDim.x + 1);
+        u = spans[blockIdx.x];
+        u_end = spans[blockIdx.x + 1];
+        pi = spans[gridDim.x + 1 + blockIdx.x];
+    }
     for (;;) {
         if (u >= u_end) {
             // The span (or pool task) is done: go on with the pool task that was asked for when the
@@ -891,11 +911,53 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                     const float g = h2f(out), up = h2f(f2h(sum_up * fscale[b]));
                     out = f2h(g / (1.0f + expf(-g)) * up);
                 }
-                p.y[(size_t)b * p.rows + r_begin + rl] = out;
+                if (kExtras && p.residual) {
+                    // the reference's add_forward behind the projection (src/transformer.cpp:247-250, 293-296): one
+                    // correctly rounded fp16 add of the residual stream and the fp16-rounded projection
+                    const _Float16 res = __builtin_bit_cast(_Float16, p.residual[r_begin + rl]);
+                    out = __builtin_bit_cast(uint16_t, (_Float16)(res + __builtin_bit_cast(_Float16, out)));
+                }
+                uint16_t *dst = p.y + (size_t)b * p.rows + r_begin + rl;
+                // (staged plans: written through to memory, where the workgroups of the next stage find it whatever
+                // XCD they run on)
+                if (staged) __hip_atomic_store(dst, out, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                else *dst = out;
             }
         }
         if (request) pool_task = requested;
         __syncthreads();
+    }
+    if (staged && stage + 1 < n_stages) {
+        // ---- between two stages: every output of this workgroup's span has reached memory, then count and wait
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) {
+            __hip_atomic_fetch_add(sc.stage_counters + stage, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            int reached = 0;
+            for (int spins = 0; spins < sc.spin_limit; spins++) {
+                if (__hip_atomic_load(sc.stage_counters + stage, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= (int)gridDim.x) {
+                    reached = 1;
+                    break;
+                }
+                // (another workgroup has given up: the counter will never fill)
+                if ((spins & 15) == 15 && __hip_atomic_load(sc.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
+                __builtin_amdgcn_s_sleep(8);
+            }
+            if (!reached) __hip_atomic_store(sc.status, stage + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            stage_reached = reached;
+        }
+        __syncthreads();
+        if (!stage_reached) break;  // (the same for the whole workgroup: every wave leaves through the code below)
+        // what the stage before wrote is read from memory, not from a stale line of this XCD's cache
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        cur = -1;
+    }
+    }  // stages
+    if (staged && tid == 0) {
+        const int left = __hip_atomic_fetch_add(sc.stage_counters + kMaxStages, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (left == (int)gridDim.x - 1) {  // every other workgroup is past its last wait
+            for (int i = 0; i <= kMaxStages; i++) __hip_atomic_store(sc.stage_counters + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
     if (sc.pool_count != 0 && tid == 0) {
         const int left = __hip_atomic_fetch_add(sc.counters + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1426,12 +1488,129 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
     return hipSuccess;
 }
 
+// ------------------------------------------------------------------ staged plan
+// The dependent linears of a decode step in ONE launch (reference src/transformer.cpp:239-296: o_proj, residual add,
+// RMSNorm, gate/up, SiLU * up, down_proj, residual add, and the RMSNorm + q/k/v of the next layer): the problems of a
+// stage are spread over all workgroups of the launch in units of 16 rows, and between two stages the workgroups wait
+// for each other at a device counter instead of ending the kernel. Everything a problem computes is what the
+// single-stage plan computes for it (same kernel instance, same units), so the outputs equal those of separate
+// launches bit for bit.
+hipError_t plan_device_create_staged(const std::vector<Problem> &host, PlanDevice *out) {
+    PlanDevice d;
+    d.count = (int)host.size();
+    if (hipError_t e = hipGetDevice(&d.device)) return e;
+    DeviceInfo *di = nullptr;
+    if (hipError_t e = prepare_device(&di)) return e;
+    const int n = d.count;
+    bool has_pairs = false;
+    int whole = 0, stage = 0;
+    for (int i = 0; i < n; i++) {
+        const Problem &p = host[i];
+        const bool addressable = (size_t)p.rows * (p.cols / 8) < (size_t)1 << 32;
+        if (p.batch != 1 || !addressable || !wide_ok(p) || (p.flags & kProblemInt8Input)) return hipErrorInvalidValue;
+        if (p.stage < stage || p.stage > stage + 1 || p.stage >= kMaxStages || (i == 0 && p.stage != 0)) return hipErrorInvalidValue;
+        stage = p.stage;
+        has_pairs = has_pairs || (p.flags & kProblemSwigluGate);
+        d.max_rows = std::max(d.max_rows, (int)p.rows);
+        whole = std::max(whole, image_bytes_of<Wide>(p.cols, 1, false));
+    }
+    d.n_stages = stage + 1;
+    d.max_batch = 1;
+    const int mats = has_pairs ? 2 : 1;
+    if (whole + kNW * kFineUnit * 4 * mats > kLdsLimit) return hipErrorInvalidValue;  // whole rows in LDS (K <= 28672)
+    const int max_units = max_units_for(whole, 1, kFineUnit, mats);
+    d.use_mfma = d.wide = d.fine = d.extras = true;
+    d.max_units = max_units;
+    d.image_bytes = whole;
+    d.pair_stride = has_pairs ? kNW * max_units * kFineUnit : 0;
+    d.lds_bytes = whole + kNW * max_units * kFineUnit * 4 * mats;
+    // every workgroup of the launch must be resident at the same time: no more than the chip holds
+    const int slots = resident_wgs<Wide, true, true>(d.lds_bytes) * di->cus;
+
+    auto is_up = [&](int i) { return i > 0 && (host[i - 1].flags & kProblemSwigluGate); };
+    auto units_in = [&](int i) { return is_up(i) ? 0 : (host[i].rows + kFineUnit - 1) / kFineUnit; };
+    std::vector<int> prefix(n + 1, 0), stage_begin(d.n_stages + 1, n);
+    for (int i = 0; i < n; i++) {
+        prefix[i + 1] = prefix[i] + units_in(i);
+        if (i == 0 || host[i].stage != host[i - 1].stage) stage_begin[host[i].stage] = i;
+    }
+    stage_begin[d.n_stages] = n;
+    int grid = 1;
+    for (int st = 0; st < d.n_stages; st++) grid = std::max(grid, prefix[stage_begin[st + 1]] - prefix[stage_begin[st]]);
+    grid = std::min(grid, slots);
+    d.grid = grid;
+    // spans of each stage: contiguous, of about equal weight (a unit's weights plus a fixed cost); a stage with
+    // fewer units than workgroups gives one unit each to the first workgroups (the dispatcher hands the first
+    // workgroups of a launch to different CUs)
+    std::vector<int> spans;
+    for (int st = 0; st < d.n_stages; st++) {
+        const int u0 = prefix[stage_begin[st]], u1 = prefix[stage_begin[st + 1]];
+        std::vector<int64_t> weight;
+        for (int i = stage_begin[st]; i < stage_begin[st + 1]; i++)
+            for (int t = 0; t < units_in(i); t++) {
+                const int nr = std::min(kFineUnit, host[i].rows - t * kFineUnit);
+                weight.push_back((int64_t)nr * host[i].cols * ((host[i].flags & kProblemSwigluGate) ? 2 : 1) + 16384);
+            }
+        int64_t total_w = 0;
+        for (int64_t w : weight) total_w += w;
+        std::vector<int> first(grid + 1, u1);
+        first[0] = u0;
+        const int units = u1 - u0;
+        int64_t acc = 0;
+        int t = 0;
+        for (int g = 1; g < grid; g++) {
+            if (units <= grid) {
+                t = std::min(g, units);
+            } else {
+                const int lo = (first[g - 1] - u0) + 1, hi = units - (grid - g);
+                const double want = (double)total_w * g / grid;
+                while (t < hi && (t < lo || (double)acc < want)) acc += weight[t++];
+            }
+            first[g] = u0 + t;
+        }
+        spans.insert(spans.end(), first.begin(), first.end());
+        for (int g = 0, pr = stage_begin[st]; g < grid; g++) {
+            while (pr + 1 < stage_begin[st + 1] && prefix[pr + 1] <= first[g]) pr++;
+            spans.push_back(pr);
+        }
+    }
+
+    auto round16 = [](size_t v) { return (v + 15) / 16 * 16; };
+    const size_t bytes_table = round16(sizeof(Problem) * n), bytes_prefix = round16(sizeof(int) * prefix.size());
+    const size_t bytes_spans = round16(sizeof(int) * spans.size());
+    const size_t bytes_counters = round16(sizeof(int) * (2 * kPlanSlots + kPlanSlots * (kMaxStages + 1) + 1));
+    char *base = nullptr;
+    if (hipError_t e = hipMalloc(&base, bytes_table + bytes_prefix + bytes_spans + bytes_counters)) return e;
+    d.problems = reinterpret_cast<Problem *>(base);
+    d.unit_prefix = reinterpret_cast<int *>(base + bytes_table);
+    d.wg_first = reinterpret_cast<int *>(base + bytes_table + bytes_prefix);
+    d.counters = reinterpret_cast<int *>(base + bytes_table + bytes_prefix + bytes_spans);
+    d.stage_counters = d.counters + 2 * kPlanSlots;
+    d.status = d.stage_counters + kPlanSlots * (kMaxStages + 1);
+    // a poll is an uncached load and a short sleep, a microsecond or two: the wait gives up after about a second
+    d.spin_limit = 500000;
+    hipError_t e = hipMemcpy(d.problems, host.data(), sizeof(Problem) * n, hipMemcpyHostToDevice);
+    if (!e) e = hipMemcpy(d.unit_prefix, prefix.data(), sizeof(int) * prefix.size(), hipMemcpyHostToDevice);
+    if (!e) e = hipMemcpy(d.wg_first, spans.data(), sizeof(int) * spans.size(), hipMemcpyHostToDevice);
+    if (!e) e = hipMemset(d.counters, 0, bytes_counters);
+    d.next_slot = new (std::nothrow) std::atomic<unsigned>(0);
+    if (!e && !d.next_slot) e = hipErrorOutOfMemory;
+    if (e) {
+        (void)hipFree(base);
+        delete d.next_slot;
+        return e;
+    }
+    *out = d;
+    return hipSuccess;
+}
+
 hipError_t plan_device_launch(const PlanDevice &plan, hipStream_t s) {
     // the schedule, the table and the counters live on the device the plan was created on
     int dev = -1;
     if (hipError_t e = hipGetDevice(&dev)) return e;
     if (dev != plan.device) return hipErrorInvalidDevice;
-    int *counters = plan.counters + 2 * (plan.next_slot->fetch_add(1, std::memory_order_relaxed) % kPlanSlots);
+    const unsigned slot = plan.next_slot->fetch_add(1, std::memory_order_relaxed) % kPlanSlots;
+    int *counters = plan.counters + 2 * slot;
     if (plan.batch_kernel)
         return launch_gemv_batch_table(plan.problems, plan.unit_prefix, plan.wg_first, plan.grid, plan.pool_begin,
                                        plan.pool_end, plan.pool_first, counters, s);
@@ -1450,6 +1629,13 @@ hipError_t plan_device_launch(const PlanDevice &plan, hipStream_t s) {
     sc.max_units = plan.max_units;
     sc.max_batch = plan.max_batch;
     sc.image_bytes = plan.image_bytes;
+    if (plan.n_stages > 0) {
+        sc.n_stages = plan.n_stages;
+        sc.stage_counters = plan.stage_counters + slot * (kMaxStages + 1);
+        sc.status = plan.status;
+        const int limit = tuning().stage_spin_limit.load(std::memory_order_relaxed);
+        sc.spin_limit = limit > 0 ? limit : plan.spin_limit;
+    }
     Problem none{};
     if (plan.extras && plan.fine)
         gemv_mfma_kernel<Wide, true, true><<<plan.grid, kThreads, plan.lds_bytes, s>>>(none, sc);

@@ -21,6 +21,7 @@ ABI_SYMBOLS = (
     "tllm_linear_plan_kernel", "tllm_gemm_workspace_reserve", "tllm_gemm_workspace_release",
     "tllm_ternary_gemm_f16_static", "tllm_read_stream", "tllm_ternary_gemm_kernel",
     "tllm_debug_set_tuning", "tllm_debug_get_tuning", "tllm_ternary_linear_int8_f16",
+    "tllm_linear_plan_create_staged", "tllm_linear_plan_status",
 )
 # include/tllm_model_file.h
 FILE_ABI_SYMBOLS = (
@@ -89,6 +90,9 @@ def lib():
     L.tllm_linear_plan_create.argtypes = [C.POINTER(vp), C.POINTER(_Problem), i, i]
     L.tllm_linear_plan_create_normed.argtypes = [C.POINTER(vp), C.POINTER(_Problem), C.POINTER(vp), f, i, i]
     L.tllm_linear_plan_create_i8.argtypes = [C.POINTER(vp), C.POINTER(_Problem), C.POINTER(vp), i, i]
+    L.tllm_linear_plan_create_staged.argtypes = [C.POINTER(vp), C.POINTER(_Problem), C.POINTER(vp), C.POINTER(vp),
+                                                 C.POINTER(C.c_int32), f, i, i]
+    L.tllm_linear_plan_status.argtypes = [vp]
     L.tllm_linear_plan_launch.argtypes = [vp, vp]
     L.tllm_linear_plan_weight_bytes.argtypes = [vp]
     L.tllm_linear_plan_weight_bytes.restype = C.c_int64
@@ -275,7 +279,8 @@ QUANTIZE_INPUT = 2  # TLLM_PROBLEM_QUANTIZE_INPUT
 class LinearPlan:
     """Several independent ternary linears issued as one launch."""
 
-    def __init__(self, problems, group_size=128, norm_weights=None, eps=1e-5, input_scales=None):
+    def __init__(self, problems, group_size=128, norm_weights=None, eps=1e-5, input_scales=None, stages=None,
+                 residuals=None):
         """problems: iterable of (nz, sign, scales, input, output, rows, cols, batch[, flags]);
         flags = SWIGLU_GATE marks the gate of a pair whose up projection is the next problem
         (output may be None there): the pair stores silu(gate) * up in the gate's output."""
@@ -288,7 +293,16 @@ class LinearPlan:
             arr[k] = _Problem(nz.data_ptr(), sg.data_ptr(), sc.data_ptr(), x.data_ptr(),
                               y.data_ptr() if y is not None else 0, rows, cols, batch, flags)
         self._h = C.c_void_p(0)
-        if input_scales is not None:
+        if stages is not None:
+            # dependent problems in one launch: stages[k] ascending; residuals[k] (or None) is added behind problem k's projection
+            n = max(len(problems), 1)
+            self._keep_norm = list(norm_weights) if norm_weights is not None else [None] * len(problems)
+            self._keep_res = list(residuals) if residuals is not None else [None] * len(problems)
+            nw = (C.c_void_p * n)(*[w.data_ptr() if w is not None else None for w in self._keep_norm])
+            rs = (C.c_void_p * n)(*[r.data_ptr() if r is not None else None for r in self._keep_res])
+            st = (C.c_int32 * n)(*[int(v) for v in stages])
+            check(lib().tllm_linear_plan_create_staged(C.byref(self._h), arr, nw, rs, st, float(eps), len(problems), group_size))
+        elif input_scales is not None:
             # int8 activations: every problem's input is an int8 tensor, input_scales[k] the float32 device tensor
             # that quantize_absmax_int8 wrote for it
             self._keep_scales = list(input_scales)
@@ -315,6 +329,10 @@ class LinearPlan:
 
     def launch(self, stream=None):
         check(lib().tllm_linear_plan_launch(self._h, _stream(stream)))
+
+    def status(self):
+        """Staged plans: raises TllmError if a launch gave up waiting between two stages since the last call."""
+        check(lib().tllm_linear_plan_status(self._h))
 
     def close(self):
         if self._h:

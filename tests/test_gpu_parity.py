@@ -1712,3 +1712,161 @@ def test_fused_int8_linear_special_inputs(dev, oracle):
     with pytest.raises(tl.TllmError):      # not together with a SwiGLU pair
         tl.LinearPlan([(*probs[1][:3], dx.view(1, -1), probs[1][4], 1024, cols, 1, tl.QUANTIZE_INPUT | tl.SWIGLU_GATE),
                        (*probs[2][:3], dx.view(1, -1), None, 1024, cols, 1)])
+
+
+def _chain_layer(torch, tl, gen, h, qd, kvd, ffn):
+    """Random weights and norm vectors of one decoder layer (o, gate, up, down of this layer; q, k, v of the next)."""
+    w = {name: _rand_weight(torch, gen, r, c) for name, (r, c) in
+         dict(o=(h, qd), g=(ffn, h), u=(ffn, h), d=(h, ffn), q=(qd, h), k=(kvd, h), v=(kvd, h)).items()}
+    w["n2"] = (torch.randn(h, device="cuda", generator=gen) * 0.1 + 1.0).to(torch.float16)
+    w["n1"] = (torch.randn(h, device="cuda", generator=gen) * 0.1 + 1.0).to(torch.float16)
+    return w
+
+
+def _chain_separate(torch, tl, w, x, att, h, qd, kvd, ffn, eps):
+    """The reference's launches (src/transformer.cpp:239-296 and 193-217 of the next layer), one operator call each."""
+    f16 = dict(dtype=torch.float16, device="cuda")
+    o, xn = torch.zeros((1, h), **f16), torch.zeros((1, h), **f16)
+    g, u, d = torch.zeros((1, ffn), **f16), torch.zeros((1, ffn), **f16), torch.zeros((1, h), **f16)
+    q, k, v = torch.zeros((1, qd), **f16), torch.zeros((1, kvd), **f16), torch.zeros((1, kvd), **f16)
+    xs = x.clone()
+    tl.ternary_gemv(*w["o"], att, o, h, qd, 128)
+    tl.add(xs, o, xs, h)
+    tl.rmsnorm(xs, w["n2"], xn, None, None, 1, h, eps)
+    tl.ternary_gemv(*w["g"], xn, g, ffn, h, 128)
+    tl.ternary_gemv(*w["u"], xn, u, ffn, h, 128)
+    tl.silu_mul(g, u, g, ffn)
+    tl.ternary_gemv(*w["d"], g, d, h, ffn, 128)
+    tl.add(xs, d, xs, h)
+    tl.rmsnorm(xs, w["n1"], xn, None, None, 1, h, eps)
+    tl.ternary_gemv(*w["q"], xn, q, qd, h, 128)
+    tl.ternary_gemv(*w["k"], xn, k, kvd, h, 128)
+    tl.ternary_gemv(*w["v"], xn, v, kvd, h, 128)
+    return xs, g, q, k, v
+
+
+def _chain_staged(torch, tl, w, xs, att, hbuf, q, k, v, h, qd, kvd, ffn, eps):
+    probs = [(*w["o"], att, xs, h, qd, 1),
+             (*w["g"], xs, hbuf, ffn, h, 1, tl.SWIGLU_GATE), (*w["u"], xs, None, ffn, h, 1),
+             (*w["d"], hbuf, xs, h, ffn, 1),
+             (*w["q"], xs, q, qd, h, 1), (*w["k"], xs, k, kvd, h, 1), (*w["v"], xs, v, kvd, h, 1)]
+    norms = [None, w["n2"], w["n2"], None, w["n1"], w["n1"], w["n1"]]
+    residuals = [xs, None, None, xs, None, None, None]
+    return tl.LinearPlan(probs, norm_weights=norms, eps=eps, stages=[0, 1, 1, 2, 3, 3, 3], residuals=residuals)
+
+
+@pytest.mark.parametrize("h,qd,kvd,ffn", [(4096, 4096, 1024, 14336), (2048, 2048, 512, 8192), (2048, 2304, 256, 5632)])
+def test_staged_plan_equals_the_separate_launches(dev, oracle, h, qd, kvd, ffn):
+    """o_proj (+ residual) -> RMSNorm, gate/up, SiLU * up -> down_proj (+ residual) -> RMSNorm, q/k/v of the next
+    layer as ONE launch with waits between the stages: the residual stream, the FFN activation and q, k, v hold the
+    bits of the twelve separate launches, launch after launch; the projection rows are within the bar of the oracle."""
+    torch, tl = dev
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(h + ffn)
+    eps = 1e-5
+    w = _chain_layer(torch, tl, gen, h, qd, kvd, ffn)
+    f16 = dict(dtype=torch.float16, device="cuda")
+    x = torch.randn((1, h), device="cuda", generator=gen).to(torch.float16)
+    att = torch.randn((1, qd), device="cuda", generator=gen).to(torch.float16)
+    want = _chain_separate(torch, tl, w, x, att, h, qd, kvd, ffn, eps)
+    xs, hbuf = x.clone(), torch.full((1, ffn), float("nan"), **f16)
+    q, k, v = torch.full((1, qd), float("nan"), **f16), torch.full((1, kvd), float("nan"), **f16), torch.full((1, kvd), float("nan"), **f16)
+    plan = _chain_staged(torch, tl, w, xs, att, hbuf, q, k, v, h, qd, kvd, ffn, eps)
+    assert "staged" in plan.kernel
+    for launch in range(3):
+        xs.copy_(x)
+        for t in (hbuf, q, k, v):
+            t.fill_(float("nan"))
+        plan.launch()
+        torch.cuda.synchronize()
+        plan.status()
+        for name, got, ref in zip(("residual stream", "silu(gate) * up", "q", "k", "v"), (xs, hbuf, q, k, v), want):
+            assert torch.equal(got.view(torch.int16), ref.view(torch.int16)), f"launch {launch}: {name} differs from the separate launches"
+    # the o_proj rows against the oracle: stream + projection, both fp16-rounded
+    o_ref = oracle.gemv_f64(w["o"][0][:64].cpu().numpy().view(np.uint32), w["o"][1][:64].cpu().numpy().view(np.uint32),
+                            w["o"][2][:64].cpu().numpy().view(np.uint16), att.cpu().numpy().view(np.uint16)[0])
+    plan2 = tl.LinearPlan([(*w["o"], att, xs, h, qd, 1)], stages=[0], residuals=[xs])
+    xs.copy_(x)
+    plan2.launch()
+    torch.cuda.synchronize()
+    got = xs[0, :64].cpu().numpy().astype(np.float64) - x[0, :64].cpu().numpy().astype(np.float64)
+    assert np.abs(got - o_ref).max() <= 2e-3 * max(1.0, np.abs(o_ref).max()) + np.abs(x[0, :64].cpu().numpy().astype(np.float64)).max() * 2.0 ** -10
+    plan.close()
+    plan2.close()
+
+
+def test_staged_plan_in_a_captured_graph_and_on_a_second_stream(dev, oracle):
+    """The staged launch under graph capture (no allocation, counters that reset themselves): replays, with eager
+    launches of the same plan on another stream between them, give the eager bits every time."""
+    torch, tl = dev
+    h, qd, kvd, ffn, eps = 2048, 2048, 512, 8192, 1e-5
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(31)
+    w = _chain_layer(torch, tl, gen, h, qd, kvd, ffn)
+    f16 = dict(dtype=torch.float16, device="cuda")
+    x = torch.randn((1, h), device="cuda", generator=gen).to(torch.float16)
+    att = torch.randn((1, qd), device="cuda", generator=gen).to(torch.float16)
+    want = _chain_separate(torch, tl, w, x, att, h, qd, kvd, ffn, eps)
+    xs, hbuf = x.clone(), torch.zeros((1, ffn), **f16)
+    q, k, v = torch.zeros((1, qd), **f16), torch.zeros((1, kvd), **f16), torch.zeros((1, kvd), **f16)
+    plan = _chain_staged(torch, tl, w, xs, att, hbuf, q, k, v, h, qd, kvd, ffn, eps)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        xs.copy_(x)
+        plan.launch(stream=side)
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            xs.copy_(x)
+            plan.launch(stream=side)
+    torch.cuda.synchronize()
+    for replay in range(4):
+        for t in (hbuf, q, k, v):
+            t.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        plan.status()
+        for name, got, ref in zip(("residual stream", "silu(gate) * up", "q", "k", "v"), (xs, hbuf, q, k, v), want):
+            assert torch.equal(got.view(torch.int16), ref.view(torch.int16)), f"replay {replay}: {name}"
+        xs.copy_(x)            # an eager launch between the replays
+        plan.launch()
+        torch.cuda.synchronize()
+    del graph
+    plan.close()
+
+
+def test_staged_plan_wait_that_expires_is_reported(dev, oracle, tuned):
+    """A wait between two stages is bounded: with the bound forced down to one poll (tuning switch) the workgroups
+    that arrive early give up, every workgroup ends normally, tllm_linear_plan_status reports the timeout once, and
+    the next launch with the ordinary bound is complete and correct."""
+    torch, tl = dev
+    h, qd, kvd, ffn, eps = 2048, 2048, 512, 8192, 1e-5
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(32)
+    w = _chain_layer(torch, tl, gen, h, qd, kvd, ffn)
+    f16 = dict(dtype=torch.float16, device="cuda")
+    x = torch.randn((1, h), device="cuda", generator=gen).to(torch.float16)
+    att = torch.randn((1, qd), device="cuda", generator=gen).to(torch.float16)
+    want = _chain_separate(torch, tl, w, x, att, h, qd, kvd, ffn, eps)
+    xs, hbuf = x.clone(), torch.zeros((1, ffn), **f16)
+    q, k, v = torch.zeros((1, qd), **f16), torch.zeros((1, kvd), **f16), torch.zeros((1, kvd), **f16)
+    plan = _chain_staged(torch, tl, w, xs, att, hbuf, q, k, v, h, qd, kvd, ffn, eps)
+    tl.set_tuning("stage_spin_limit", 1)
+    try:
+        plan.launch()
+        torch.cuda.synchronize()
+        with pytest.raises(tl.TllmError) as err:
+            plan.status()
+        assert err.value.code == -11
+    finally:
+        tl.set_tuning("stage_spin_limit", 0)
+    plan.status()                       # cleared by the call that reported it
+    xs.copy_(x)
+    plan.launch()
+    torch.cuda.synchronize()
+    plan.status()
+    for name, got, ref in zip(("residual stream", "silu(gate) * up", "q", "k", "v"), (xs, hbuf, q, k, v), want):
+        assert torch.equal(got.view(torch.int16), ref.view(torch.int16)), name
+    plan.close()

@@ -505,13 +505,46 @@ def decode_chain(torch, tl, problems, model, layers):
             w["gu_n"].launch()
             tl.ternary_gemv(*w["d"], g, d, h, ffn, 128)
 
+    # Staged plans: the dependent launches of a layer as stages of one launch (waits at device counters between the
+    # stages instead of kernel boundaries); the residual adds ride in the epilogues of o_proj and down_proj.
+    xs = torch.randn((1, h), device="cuda").to(torch.float16)
+    for l, w in enumerate(L):
+        nxt = L[l + 1] if l + 1 < len(L) else None
+        ogd = [(*w["o"], att, xs, h, qd, 1), (*w["g"], xs, g, ffn, h, 1, tl.SWIGLU_GATE), (*w["u"], xs, None, ffn, h, 1),
+               (*w["d"], g, xs, h, ffn, 1)]
+        norms, res, stages = [None, w["n2"], w["n2"], None], [xs, None, None, xs], [0, 1, 1, 2]
+        w["ogd"] = tl.LinearPlan(ogd, norm_weights=norms, eps=eps, stages=stages, residuals=res)
+        if nxt is not None:
+            ogd = ogd + [(*nxt["q"], xs, q, qd, h, 1), (*nxt["k"], xs, k, kvd, h, 1), (*nxt["v"], xs, v, kvd, h, 1)]
+            w["ogdq"] = tl.LinearPlan(ogd, norm_weights=norms + [nxt["n1"]] * 3, eps=eps, stages=stages + [3, 3, 3],
+                                      residuals=res + [None] * 3)
+        else:
+            w["ogdq"] = w["ogd"]
+        w["qkv_s"] = tl.LinearPlan([(*w["q"], xs, q, qd, h, 1), (*w["k"], xs, k, kvd, h, 1), (*w["v"], xs, v, kvd, h, 1)],
+                                   norm_weights=[w["n1"]] * 3, eps=eps)
+
+    def two():
+        for w in L:
+            w["qkv_s"].launch()
+            w["ogd"].launch()
+
+    def one():
+        L[0]["qkv_s"].launch()
+        for w in L:
+            w["ogdq"].launch()
+
     def close():
         for w in L:
-            for key in ("qkv", "gu", "qkv_n", "gu_n"):
+            for key in ("qkv", "gu", "qkv_n", "gu_n", "qkv_s", "ogd"):
                 w[key].close()
+            if w["ogdq"] is not w["ogd"]:
+                w["ogdq"].close()
 
     return {"variants": (("the reference's 10 launches per layer", ten, 10), ("q/k/v and gate/up as plans: 7 per layer", seven, 7),
-                         ("RMSNorm prologue + SwiGLU pair: 4 per layer", four, 4)), "close": close}
+                         ("RMSNorm prologue + SwiGLU pair: 4 per layer", four, 4),
+                         ("staged plan o_proj -> gate/up -> down_proj with the residual adds, q/k/v apart: 2 launches per layer", two, 2),
+                         ("staged plan o_proj -> gate/up -> down_proj -> q/k/v of the next layer: 1 launch per layer", one, 1)),
+            "close": close}
 
 
 def lm_head_rows(torch, tl, orc, timer, seed):

@@ -359,7 +359,8 @@ int tllm_linear_plan_status(const tllm_linear_plan *plan) {
     int v = 0;
     if (hipError_t e = hipMemcpy(&v, plan->dev.status, sizeof v, hipMemcpyDeviceToHost)) return (int)e;
     if (v != 0) {
-        if (hipError_t e = hipMemset(plan->dev.status, 0, sizeof v)) return (int)e;
+        // (the launch that gave up left its barrier half counted: all barriers and the status word start again)
+        if (hipError_t e = hipMemset(plan->dev.stage_counters, 0, plan->dev.barrier_bytes)) return (int)e;
         return TLLM_ERR_STAGE_TIMEOUT;
     }
     return TLLM_OK;

@@ -213,12 +213,13 @@ struct PlanDevice {
     int image_bytes = 0;
     int lds_bytes = 0;
     // staged plans: the spans of stage s start at wg_first + s * (2 * grid + 1); between two stages every workgroup
-    // waits for all workgroups at a counter (n_stages counters and a "workgroups that have left" counter per launch
-    // slot, after the hand-out counters), for at most spin_limit polls; a wait that expires sets *status
+    // waits for all workgroups at a barrier in device memory (stage_counters: one barrier per launch slot), for at
+    // most spin_limit polls; a wait that expires sets *status
     int n_stages = 0;
     int *stage_counters = nullptr;
     int *status = nullptr;
     int spin_limit = 0;
+    size_t barrier_bytes = 0;  // all barriers and the status word: cleared when a timeout is read
 };
 hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out);
 // A plan whose problems run in stages inside one launch (Problem::stage, ascending); batch 1, shapes the wide-tile

@@ -100,16 +100,25 @@ struct Sched {
     float i8_scale;
     const float *i8_scale_dev;
     // Staged plans (kExtras instances): n_stages > 0; the spans of stage s start at wg_first + s * (2 * grid + 1).
-    // A workgroup that has stored the last output of its span of stage s adds one to stage_counters[s] and waits
-    // until all gridDim.x workgroups have (every workgroup is resident: the host sizes the grid for that), for at
-    // most spin_limit polls; a wait that expires sets *status to the stage's number + 1 and the workgroup leaves,
-    // and so do the others when they see it. stage_counters[kMaxStages] counts the workgroups that have left; the
-    // last one sets the counters back to zero for the next launch.
+    // Between two stages the workgroups meet at a barrier in device memory (`barrier`, kBarrierInts ints, one per
+    // launch slot): a workgroup whose outputs of the stage have reached memory adds one to the counter of its group of
+    // kBarrierGroup workgroups; the last of a group adds one to the top counter; the last group sets the counters back
+    // to zero and flips the flag word every other workgroup polls (plain loads, no read-modify-write: hundreds of
+    // atomics on ONE address cost tens of microseconds here, since each is served in turn at the memory side). The flag
+    // alternates from barrier to barrier and across launches; every counter is zero again when a launch ends, so a
+    // replayed graph needs no clearing. Every workgroup is resident (the host sizes the grid for that); a wait gives up
+    // after spin_limit polls, sets *status to the stage's number + 1, and the workgroup leaves; so do the others when
+    // they see it (the host clears the barrier when it reads the status).
     int n_stages;
     int spin_limit;
-    int *stage_counters;
+    int *barrier;
     int *status;
 };
+// Layout of a stage barrier, in ints: [0] the flag, [32] the top counter, [64 + 32 g] the counter of group g: every
+// word that takes atomics from many workgroups sits on a 128-byte line of its own.
+constexpr int kBarrierGroup = 16;
+constexpr int kBarrierMaxGroups = 64;  // grids of up to 1024 workgroups
+constexpr int kBarrierInts = 64 + 32 * kBarrierMaxGroups;
 
 // The scales that travel with a tile. Wide: the one scale of the lane's (row, group). Tall: the four scales (one
 // slice) of row 4 * lq + (li & 3) as one 8-byte load; the lane needs the scale of its own group li & 3 for each of the
@@ -267,6 +276,10 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
 
     __shared__ int pool_task;
     __shared__ int stage_reached;
+    // the flag of the stage barrier as this launch finds it (only thread 0 uses it): no workgroup can flip it before
+    // every workgroup has read it here, because flipping takes the arrival of all of them
+    int barrier_sense = 0;
+    if (kExtras && sc.n_stages > 1 && tid == 0) barrier_sense = __hip_atomic_load(sc.barrier, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const int n_stages = kExtras && sc.n_stages > 0 ? sc.n_stages : 1;
     const bool staged = kExtras && sc.n_stages > 0;
     for (int stage = 0; stage < n_stages; stage++) {
@@ -932,33 +945,47 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         if (tid == 0) {
-            __hip_atomic_fetch_add(sc.stage_counters + stage, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const int want = barrier_sense ^ 1;  // what the flag reads when every workgroup has arrived
+            int *group = sc.barrier + 64 + 32 * ((int)blockIdx.x / kBarrierGroup);
+            const int n_groups = ((int)gridDim.x + kBarrierGroup - 1) / kBarrierGroup;
+            const int in_group = min(kBarrierGroup, (int)gridDim.x - (int)blockIdx.x / kBarrierGroup * kBarrierGroup);
             int reached = 0;
-            for (int spins = 0; spins < sc.spin_limit; spins++) {
-                if (__hip_atomic_load(sc.stage_counters + stage, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= (int)gridDim.x) {
+            bool last = false;
+            if (__hip_atomic_fetch_add(group, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == in_group - 1) {
+                __hip_atomic_store(group, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (__hip_atomic_fetch_add(sc.barrier + 32, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == n_groups - 1) {
+                    __hip_atomic_store(sc.barrier + 32, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    // (the two stores above complete before the flag: nobody passes the barrier, let alone arrives
+                    // at the next one, before the counters are zero)
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    __hip_atomic_store(sc.barrier, want, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    last = true;
+                    reached = 1;
+                }
+            }
+            for (int spins = 0; !last && spins < sc.spin_limit; spins++) {
+                if (__hip_atomic_load(sc.barrier, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == want) {
                     reached = 1;
                     break;
                 }
-                // (another workgroup has given up: the counter will never fill)
+                // (another workgroup has given up: the flag will never flip)
                 if ((spins & 15) == 15 && __hip_atomic_load(sc.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) break;
-                __builtin_amdgcn_s_sleep(8);
+                __builtin_amdgcn_s_sleep(4);
             }
             if (!reached) __hip_atomic_store(sc.status, stage + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             stage_reached = reached;
+            barrier_sense = want;
         }
         __syncthreads();
         if (!stage_reached) break;  // (the same for the whole workgroup: every wave leaves through the code below)
         // what the stage before wrote is read from memory, not from a stale line of this XCD's cache
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+#ifndef TLLM_STAGE_NO_FENCE
+        if (wave == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        __syncthreads();
+#endif
         cur = -1;
     }
     }  // stages
-    if (staged && tid == 0) {
-        const int left = __hip_atomic_fetch_add(sc.stage_counters + kMaxStages, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (left == (int)gridDim.x - 1) {  // every other workgroup is past its last wait
-            for (int i = 0; i <= kMaxStages; i++) __hip_atomic_store(sc.stage_counters + i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-    }
     if (sc.pool_count != 0 && tid == 0) {
         const int left = __hip_atomic_fetch_add(sc.counters + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (left == (int)gridDim.x - 1) {  // every other workgroup has made its last request
@@ -1537,7 +1564,7 @@ hipError_t plan_device_create_staged(const std::vector<Problem> &host, PlanDevic
     stage_begin[d.n_stages] = n;
     int grid = 1;
     for (int st = 0; st < d.n_stages; st++) grid = std::max(grid, prefix[stage_begin[st + 1]] - prefix[stage_begin[st]]);
-    grid = std::min(grid, slots);
+    grid = std::min(std::min(grid, slots), kBarrierGroup * kBarrierMaxGroups);
     d.grid = grid;
     // spans of each stage: contiguous, of about equal weight (a unit's weights plus a fixed cost); a stage with
     // fewer units than workgroups gives one unit each to the first workgroups (the dispatcher hands the first
@@ -1578,15 +1605,17 @@ hipError_t plan_device_create_staged(const std::vector<Problem> &host, PlanDevic
     auto round16 = [](size_t v) { return (v + 15) / 16 * 16; };
     const size_t bytes_table = round16(sizeof(Problem) * n), bytes_prefix = round16(sizeof(int) * prefix.size());
     const size_t bytes_spans = round16(sizeof(int) * spans.size());
-    const size_t bytes_counters = round16(sizeof(int) * (2 * kPlanSlots + kPlanSlots * (kMaxStages + 1) + 1));
+    const size_t bytes_counters = round16(sizeof(int) * (32 + kPlanSlots * kBarrierInts + 32)) + 128;
     char *base = nullptr;
     if (hipError_t e = hipMalloc(&base, bytes_table + bytes_prefix + bytes_spans + bytes_counters)) return e;
     d.problems = reinterpret_cast<Problem *>(base);
     d.unit_prefix = reinterpret_cast<int *>(base + bytes_table);
     d.wg_first = reinterpret_cast<int *>(base + bytes_table + bytes_prefix);
+    // the hand-out counters (unused by staged plans), then, on 128-byte lines, the barriers of the launch slots and the status word
     d.counters = reinterpret_cast<int *>(base + bytes_table + bytes_prefix + bytes_spans);
-    d.stage_counters = d.counters + 2 * kPlanSlots;
-    d.status = d.stage_counters + kPlanSlots * (kMaxStages + 1);
+    d.stage_counters = reinterpret_cast<int *>((reinterpret_cast<uintptr_t>(d.counters + 32) + 127) / 128 * 128);
+    d.status = d.stage_counters + kPlanSlots * kBarrierInts;
+    d.barrier_bytes = sizeof(int) * ((size_t)kPlanSlots * kBarrierInts + 1);
     // a poll is an uncached load and a short sleep, a microsecond or two: the wait gives up after about a second
     d.spin_limit = 500000;
     hipError_t e = hipMemcpy(d.problems, host.data(), sizeof(Problem) * n, hipMemcpyHostToDevice);
@@ -1631,7 +1660,7 @@ hipError_t plan_device_launch(const PlanDevice &plan, hipStream_t s) {
     sc.image_bytes = plan.image_bytes;
     if (plan.n_stages > 0) {
         sc.n_stages = plan.n_stages;
-        sc.stage_counters = plan.stage_counters + slot * (kMaxStages + 1);
+        sc.barrier = plan.stage_counters + slot * kBarrierInts;
         sc.status = plan.status;
         const int limit = tuning().stage_spin_limit.load(std::memory_order_relaxed);
         sc.spin_limit = limit > 0 ? limit : plan.spin_limit;

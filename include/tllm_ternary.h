@@ -112,14 +112,11 @@ int tllm_quantize_absmax_i8(const uint16_t *input, int8_t *output, float *scale,
  * A fp16 [M,K] row-major, packed weight [N,K], C fp16 [M,N] row-major.
  * Replaces ternary::ternary_gemm, reference include/kernels.cuh:37-40
  * (kernels/ternary_gemm.cu:33-195). Any M >= 1 is accepted.
- * Allocation: none per call, with one exception: a workspace that belongs to (device, stream). Three kinds
+ * Allocation: none per call, with one exception: a workspace that belongs to (device, stream). Two kinds
  * of shapes use it. Shapes whose output tiles do not fill the chip, or not its last round (M > 16), split K
  * over several workgroups per tile, which exchange fp32 partial sums through it (at most 32 MiB); so do shapes
  * of 2 to 16 activation rows (and wider ones that run as passes of 16) with so few weight rows that their
- * 64-row blocks would leave half the chip idle (N <= 64 * CUs / 2, K >= 4096: at most 1 MiB); tall shapes
- * whose K is not a multiple of 256 run a kernel that reads the activations from a copy in matrix-core
- * fragment order, which a small kernel writes there first (M rounded up to 32, times K, times 2 bytes; such
- * a shape is only chosen while that stays within TLLM_GEMM_STATIC_SCRATCH_BYTES). The first such call on a stream creates
+ * 64-row blocks would leave half the chip idle (N <= 64 * CUs / 2, K >= 4096: at most 1 MiB). The first such call on a stream creates
  * the workspace: ONE allocation of TLLM_GEMM_STATIC_SCRATCH_BYTES (the most any shape is allowed to need: the kernel
  * choice works under that limit), with its arrival counters cleared before the call returns (one device
  * synchronisation, that once). It is never grown, moved or freed afterwards, except by tllm_gemm_workspace_release:
@@ -137,10 +134,10 @@ int tllm_ternary_gemm_f16(const uint16_t *A, const uint32_t *nz_B, const uint32_
 /*
  * tllm_ternary_gemm_f16 for callers that cannot allocate device memory (code under HIP graph capture,
  * serving loops and harnesses that forbid hipMalloc): same arguments, same kernels, same results bit for
- * bit, but the workspace (split-K exchange or fragment-ordered activations) is a fixed array of
+ * bit, but the workspace (the split-K exchange) is a fixed array of
  * TLLM_GEMM_STATIC_SCRATCH_BYTES in device memory that the library holds on every GPU it runs on until
  * the process ends. The call never allocates, frees or synchronises. Both entry points choose their kernel among those whose workspace
- * fits the array (a split needs at most CUs * 128 KiB; the copy of the activations is used up to 32 MiB),
+ * fits the array (a split needs at most CUs * 128 KiB),
  * so on a 256-CU MI355X every shape runs; a configuration that would not fit is rejected with
  * TLLM_ERR_SCRATCH_TOO_SMALL before anything is launched. All calls on one GPU share the one
  * array: calls that overlap in time on one GPU (two streams, two threads, two graph branches) race on it;
@@ -355,11 +352,11 @@ int tllm_read_stream(const void *src, size_t bytes, uint32_t *sink, tllm_stream_
 
 /*
  * Testing and tuning aid: the kernel-choice switches of the library. Each is read from its environment variable
- * once per process (TLLM_GEMM_PATH, TLLM_GEMM_ROWSPLIT, TLLM_GEMM_PINGPONG, TLLM_BATCH_K_PARTS, TLLM_TALL_MAX_BATCH,
+ * once per process (TLLM_GEMM_PATH, TLLM_GEMM_ROWSPLIT, TLLM_BATCH_K_PARTS, TLLM_TALL_MAX_BATCH,
  * TLLM_TALL_MIN_SHARE, TLLM_READ_SHAPE) when the library first needs one; no operator call reads the environment.
  * These two calls change and read them afterwards, by name: "gemm_path" (0 cost model, 1 prefill GEMM, 2 passes of
- * the decode kernel), "gemm_rowsplit" / "gemm_pingpong" (-1 cost model, 0 never, 1 or 2 forced), "batch_k_parts",
- * "tall_max_batch", "tall_min_share_milli", "read_wgs_per_cu", "read_in_flight". An unknown name returns
+ * the decode kernel), "gemm_rowsplit" (-1 cost model, 0 never, 1 or 2 forced), "batch_k_parts", "tall_max_batch",
+ * "tall_min_share_milli", "stage_spin_limit", "read_wgs_per_cu", "read_in_flight". An unknown name returns
  * TLLM_ERR_BAD_SHAPE. Results never depend on them beyond the order of fp32 additions. Not for concurrent use
  * with operator calls whose choice should be stable. No counterpart in the reference.
  */

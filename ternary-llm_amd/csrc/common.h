@@ -57,7 +57,6 @@ constexpr int kProblemQuantInput = TLLM_PROBLEM_QUANTIZE_INPUT;
 struct Tuning {
     std::atomic<int> gemm_path{0};              // TLLM_GEMM_PATH=mfma|stream: 1 | 2 forces prefill GEMM | passes of the batched decode kernel for M > 16
     std::atomic<int> gemm_rowsplit{-1};         // TLLM_GEMM_ROWSPLIT: 0 never, 1 / 2 whenever the shape allows (eight-wave / four-wave form)
-    std::atomic<int> gemm_pingpong{-1};         // TLLM_GEMM_PINGPONG: 0 never, 1 whenever the shape allows
     std::atomic<int> batch_k_parts{0};          // TLLM_BATCH_K_PARTS: n parts where they fit, 1 never share out K
     std::atomic<int> tall_max_batch{4};         // TLLM_TALL_MAX_BATCH: most activation rows of a plan on the tall-tile kernel
     std::atomic<int> tall_min_share_milli{1000};  // TLLM_TALL_MIN_SHARE (x 1000): share of the plan per workgroup, in units, from which tall tiles run

@@ -12,7 +12,6 @@ Tuning &tuning() {
     static const bool from_env = [] {
         if (const char *e = getenv("TLLM_GEMM_PATH")) t.gemm_path = e[0] == 'm' ? 1 : e[0] == 's' ? 2 : 0;
         if (const char *e = getenv("TLLM_GEMM_ROWSPLIT")) t.gemm_rowsplit = atoi(e);
-        if (const char *e = getenv("TLLM_GEMM_PINGPONG")) t.gemm_pingpong = atoi(e);
         if (const char *e = getenv("TLLM_BATCH_K_PARTS")) t.batch_k_parts = atoi(e);
         if (const char *e = getenv("TLLM_TALL_MAX_BATCH")) t.tall_max_batch = atoi(e);
         if (const char *e = getenv("TLLM_TALL_MIN_SHARE")) t.tall_min_share_milli = (int)(atof(e) * 1000.0 + 0.5);
@@ -35,7 +34,7 @@ std::atomic<int> *tuning_by_name(const char *name) {
         const char *name;
         std::atomic<int> *value;
     } all[] = {{"gemm_path", &t.gemm_path},           {"gemm_rowsplit", &t.gemm_rowsplit},
-               {"gemm_pingpong", &t.gemm_pingpong},   {"batch_k_parts", &t.batch_k_parts},
+               {"batch_k_parts", &t.batch_k_parts},
                {"tall_max_batch", &t.tall_max_batch}, {"tall_min_share_milli", &t.tall_min_share_milli},
                {"read_wgs_per_cu", &t.read_wgs_per_cu}, {"read_in_flight", &t.read_in_flight},
                {"stage_spin_limit", &t.stage_spin_limit}};

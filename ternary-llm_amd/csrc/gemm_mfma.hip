@@ -5,8 +5,8 @@
 // Here the product scale * w is formed exactly in fp16 (w in {-1,0,+1}), so the only difference to
 // the reference is the order of the fp32 additions.
 //
-// Three kernels, chosen per shape by a cost model (choose_config): the four-wave kernel described next, the eight-wave
-// ping-pong kernel (gemm_pp_kernel) and the row-split kernel (gemm_ns_kernel), each described where it is defined.
+// Two kernels, chosen per shape by a cost model (choose_config): the four-wave kernel described next and the row-split
+// kernel (gemm_ns_kernel), described where it is defined.
 //
 // Tiling of the four-wave kernel. A workgroup (4 waves, one per SIMD) computes 128 weight rows x BM activation rows; every wave
 // owns all 128 weight rows and BM/4 activation rows of its own. Per stage of 64 columns of K:
@@ -482,377 +482,6 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
     }
 }
 
-// ---- The eight-wave kernel for tall problems (M >= 512 or so, one workgroup per tile).
-//
-// What bounds the four-wave kernel above is not the matrix pipe (busy 45 % of the time) but what a single
-// wave per SIMD has to issue between its MFMAs, and the LDS: a workgroup-stage writes 51 KB into LDS
-// (decoded weights and, through the direct loads, activations; LDS writes run at about 84 bytes per clock
-// here, a third of the read rate) and reads 96 KB back. This kernel changes three things.
-//   * Activations do not pass through LDS. A small kernel first copies A into MFMA fragment order
-//     (tile_acts_kernel: block (m / 32, k / 16) = 1 KB, lane (li, lq) holds A[32 mb + li][16 ks + 8 lq .. + 7]),
-//     and every wave loads its B operands from that copy with fully coalesced 16-byte loads, two stages
-//     ahead, into three register sets.
-//   * Two waves per SIMD that split K, not M or N: waves w and w + 4 own the same 128 x 64 outputs and take
-//     the first / second pair of the four 16-column steps of every stage, so the fragment reads from LDS
-//     do not grow with the wave count; their sums meet once, through LDS, after the last stage.
-//   * Ping-pong. A stage is a memory half (weight fragments to registers, this thread's 16 weights of the next
-//     stage decoded into LDS) and a matrix half (16 MFMAs, with the requests to memory for later stages
-//     between them: a vector memory instruction holds its wave for 30 - 60 cycles when the address unit is
-//     busy, which costs nothing in a half that otherwise only waits for the matrix pipe). One barrier per
-//     stage, in different places for the two waves of a SIMD: first waves (kh = 0) pass it after their matrix
-//     half, second waves after their memory half. Between two barriers the first waves run memory and
-//     matrix half of stage s while the second run the matrix half of stage s - 1 and the memory half of
-//     stage s: one wave of a SIMD multiplies while the other fetches. The barrier orders the second waves'
-//     weights of stage s + 1 before the first waves' reads; three weight buffers make every other order safe.
-// Mask words and scales still come through LDS (direct loads, lane-private dwords, two buffers).
-constexpr int kPpThreads = 512;
-constexpr int kPpMaskBuf = 8 * 768;  // per wave: nz words | sign words | scale dwords, 256 bytes each
-
-// A [M, K] row-major -> fragment order, rows past M as zeros. A workgroup copies 32 rows x 256 columns in four
-// passes of 64 columns (four 16-column steps): every wave reads eight whole 128-byte lines (8 rows) per
-// pass and writes eight 128-byte runs (8 consecutive lanes of a fragment each); the four loads of a thread
-// are in flight together.
-__global__ __launch_bounds__(256) void tile_acts_kernel(const uint16_t *__restrict__ A, u4 *__restrict__ At, int M, int K) {
-    const int ksteps = K / 16, kq_count = ksteps / 4, wg_per_row = (kq_count + 3) / 4;
-    const int mb = (int)blockIdx.x / wg_per_row, kq0 = ((int)blockIdx.x % wg_per_row) * 4;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int r = 8 * wave + (lane >> 3), c = lane & 7;  // row inside the block, 16-byte chunk inside the 128 bytes
-    const int row = 32 * mb + r;
-    u4 v[4];
-#pragma unroll
-    for (int q = 0; q < 4; q++) {
-        v[q] = u4{0u, 0u, 0u, 0u};
-        if (row < M && kq0 + q < kq_count)
-            v[q] = __builtin_nontemporal_load(reinterpret_cast<const u4 *>(A + (size_t)row * K + 64 * (kq0 + q) + 8 * c));
-    }
-#pragma unroll
-    for (int q = 0; q < 4; q++)
-        if (kq0 + q < kq_count) At[((size_t)mb * ksteps + 4 * (kq0 + q) + (c >> 1)) * 64 + (c & 1) * 32 + r] = v[q];
-}
-
-template <int MF>
-__global__ __launch_bounds__(kPpThreads, 1) void gemm_pp_kernel(
-    const uint16_t *__restrict__ At, const uint32_t *__restrict__ nzB, const uint32_t *__restrict__ sgB,
-    const uint16_t *__restrict__ scB, uint16_t *__restrict__ C, int M, int N, int K) {
-    constexpr int kWM = 32 * MF;   // activation rows of a wave pair
-    constexpr int BM = 4 * kWM;
-    constexpr int kMaskBase = 3 * kWBytes;
-    constexpr int kReq = 2 * MF + 3;  // memory requests of one matrix half
-    constexpr int kTiles = 4 * MF;    // accumulator fragments per wave
-    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    typedef __attribute__((address_space(3))) unsigned char LB;
-    typedef __attribute__((address_space(1))) const unsigned char GB;
-    LB *lds_l = (LB *)lds;
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int mg = wave & 3, kh = wave >> 2;
-    const int li = lane & 31, lq = lane >> 5;
-
-    const int m_tiles = (M + BM - 1) / BM;
-    const int n0 = ((int)blockIdx.x / m_tiles) * kBN;
-    const int m0 = ((int)blockIdx.x % m_tiles) * BM + mg * kWM;
-    const int words = K / 32, groups = K / 128, ksteps = K / 16;
-    const int last = groups * 2 - 1;
-    const int mblocks = (M + 31) / 32;
-
-    // ---- activations: block (m0 / 32 + j, 4 s + 2 kh + e); the two steps of a stage lie 1 KB apart
-    const unsigned char *a_ptr[MF];
-#pragma unroll
-    for (int j = 0; j < MF; j++) {
-        const int mb = min(m0 / 32 + j, mblocks - 1);  // blocks past M repeat the last one; their results are not stored
-        a_ptr[j] = (const unsigned char *)At + ((size_t)mb * ksteps + 2 * kh) * 1024 + lane * 16;
-    }
-    const uint32_t lds0 = (uint32_t)(uintptr_t)lds_l;
-    uint32_t fw[2];  // weight fragment i of step 2 kh + e: row 32 i + li, chunk 2 (2 kh + e) + lq
-#pragma unroll
-    for (int e = 0; e < 2; e++) fw[e] = lds0 + (uint32_t)(chunk_off(li, lq) ^ ((2 * kh + e) << 5));
-
-    // ---- weights: this thread decodes 16 weights (half a mask word pair) of one row per stage
-    const int w_row = tid >> 2, w_word = (tid >> 1) & 1, w_half = tid & 1;
-    const int gn = min(n0 + w_row, N - 1);
-    const uint32_t perm_sel = w_half ? 0x07060302u : 0x05040100u;
-    uint32_t w_wr[2];
-#pragma unroll
-    for (int c = 0; c < 2; c++) w_wr[c] = lds0 + (uint32_t)chunk_off(w_row, w_word * 4 + 2 * w_half + c);
-    GB *nz_g = (GB *)nzB + ((size_t)gn * words + w_word) * 4;
-    GB *sg_g = (GB *)sgB + ((size_t)gn * words + w_word) * 4;
-    // the scale of a group travels as the aligned dword that holds it; the half flips from group to group
-    const size_t sc_elem = (size_t)gn * groups;
-    GB *sc_g = (GB *)scB + ((sc_elem * 2) & ~(size_t)3);
-    const int w_par = (int)(sc_elem & 1);
-    uint32_t m_rd = lds0 + (uint32_t)(kMaskBase + wave * 768 + lane * 4);
-    uint32_t m_rdb[3] = {m_rd, m_rd + (uint32_t)kPpMaskBuf, m_rd + 2u * (uint32_t)kPpMaskBuf};  // ds_read2 offsets are 8 bits
-    const uint32_t s_rd_a = m_rd + 512u + 2u * (uint32_t)w_par;
-#define TLLM_GPTR(p) ((__attribute__((address_space(1))) const void *)(p))
-#define TLLM_LPTR(p) ((__attribute__((address_space(3))) void *)(p))
-    // request `which` (0: nz word, 1: sign word, 2: scale dword) for the masks of stage `stage` into buffer `buf`
-    auto dma_mask = [&](int buf, int stage, int which) {
-        const int st = min(stage, last);
-        LB *dst = lds_l + kMaskBase + buf * kPpMaskBuf + wave * 768;
-        if (which == 0) __builtin_amdgcn_global_load_lds(TLLM_GPTR(nz_g + st * 8), TLLM_LPTR(dst), 4, 0, 0);
-        else if (which == 1) __builtin_amdgcn_global_load_lds(TLLM_GPTR(sg_g + st * 8), TLLM_LPTR(dst + 256), 4, 0, 0);
-        else __builtin_amdgcn_global_load_lds(TLLM_GPTR(sc_g + ((w_par + (st >> 1)) >> 1) * 4), TLLM_LPTR(dst + 512), 4, 0, 0);
-    };
-#define TLLM_LDS_READ128(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "i"(off))
-#define TLLM_LDS_WRITE128(addr, val, off) asm volatile("ds_write_b128 %0, %1 offset:%2" ::"v"(addr), "v"(val), "i"(off) : "memory")
-#define TLLM_GLOAD128(dst, ptr, off) asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(dst) : "v"(ptr), "i"(off) : "memory")
-#define TLLM_FENCE() __builtin_amdgcn_sched_barrier(0)
-    auto decode_store = [&](uint32_t m_nz, uint32_t m_sg, uint32_t m_sc, auto WB) {
-        constexpr int wb = decltype(WB)::value;
-        const uint32_t neg = m_nz & ~m_sg;
-        const uint32_t t0 = __builtin_amdgcn_bitop3_b32(neg << 1, m_nz, 0xAAAAAAAAu, 0xE4);
-        const uint32_t t1 = __builtin_amdgcn_bitop3_b32(neg, m_nz >> 1, 0xAAAAAAAAu, 0xE4);
-        const uint32_t q = __builtin_amdgcn_perm(t1, t0, perm_sel);  // low half: even weights of this thread's 16, high half: odd
-        const h2 sp = __builtin_bit_cast(h2, m_sc | (m_sc << 16));
-        uint32_t o[8];
-#pragma unroll
-        for (int d = 0; d < 8; d++) {
-            us2 v = __builtin_bit_cast(us2, q);
-            v = v << (uint16_t)(14 - 2 * d);
-            const uint32_t top = __builtin_bit_cast(uint32_t, v) & 0xC000C000u;  // 0, +2.0 or -2.0
-            o[d] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, top) * sp);
-        }
-        const u4 v0 = {o[0], o[1], o[2], o[3]}, v1 = {o[4], o[5], o[6], o[7]};
-        const uint32_t wa0 = w_wr[0], wa1 = w_wr[1];
-        TLLM_LDS_WRITE128(wa0, v0, wb * kWBytes);
-        TLLM_LDS_WRITE128(wa1, v1, wb * kWBytes);
-    };
-
-    f16v acc[4][MF];
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-#pragma unroll
-        for (int j = 0; j < MF; j++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
-    u4 Ra[2][4];
-    u4 Rb[3][2][MF];  // activation fragments of three stages
-#pragma unroll
-    for (int q = 0; q < 3; q++)
-#pragma unroll
-        for (int e = 0; e < 2; e++)
-#pragma unroll
-            for (int j = 0; j < MF; j++) Rb[q][e][j] = u4{0u, 0u, 0u, 0u};
-    // request r (0 .. kReq - 1) of the group a matrix half makes: activations of stage `a_stage` into register
-    // set Q, masks of stage `m_stage` into mask buffer UB
-    auto request = [&](auto Q, auto UB, int r, int a_stage, int m_stage) {
-        constexpr int q = decltype(Q)::value;
-        constexpr int ub = decltype(UB)::value;
-        u4(&R)[2][MF] = Rb[q];
-        if (r < 2 * MF) {
-            const unsigned char *p = a_ptr[r >> 1] + (size_t)min(a_stage, last) * 4096;
-            if (r & 1) TLLM_GLOAD128(R[1][r >> 1], p, 1024);
-            else TLLM_GLOAD128(R[0][r >> 1], p, 0);
-        } else {
-            dma_mask(ub, m_stage, r - 2 * MF);
-        }
-    };
-
-    // ---- prologue: masks of stages 0 .. 2, activations of stages 0 and 1; weights of stage 0 decoded
-    std::integral_constant<int, 0> c0;
-    std::integral_constant<int, 1> c1;
-#pragma unroll
-    for (int r = 0; r < 3; r++) dma_mask(0, 0, r);
-#pragma unroll
-    for (int r = 0; r < 2 * MF; r++) request(c0, c0, r, 0, 0);
-#pragma unroll
-    for (int r = 0; r < 3; r++) dma_mask(1, 1, r);
-#pragma unroll
-    for (int r = 0; r < 2 * MF; r++) request(c1, c0, r, 1, 0);
-#pragma unroll
-    for (int r = 0; r < 3; r++) dma_mask(2, 2, r);
-    TLLM_FENCE();
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    TLLM_FENCE();
-    {
-        uint32_t m_w[2], m_sc;
-        const uint32_t ma = m_rd, sa = s_rd_a;
-        asm volatile("ds_read2_b32 %0, %1 offset0:0 offset1:64" : "=v"(m_w) : "v"(ma));
-        asm volatile("ds_read_u16 %0, %1" : "=v"(m_sc) : "v"(sa));
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        TLLM_FENCE();
-        decode_store(m_w[0], m_w[1], m_sc, c0);
-    }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    TLLM_FENCE();
-
-    // memory half of stage s
-    auto mem = [&](auto U, const int s) {
-        constexpr int u = decltype(U)::value;
-        constexpr int wb = u % 3;
-        const uint32_t fwl[2] = {fw[0], fw[1]};
-        uint32_t m_w[2], m_sc;
-        // masks of stage s + 1: in flight behind them only the requests of the matrix half before
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kReq) : "memory");
-        TLLM_FENCE();
-        {
-            const uint32_t ma = m_rdb[(u + 1) % 3], sa = s_rd_a ^ (((min(s + 1, last) >> 1) & 1) ? 2u : 0u);
-            asm volatile("ds_read2_b32 %0, %1 offset0:0 offset1:64" : "=v"(m_w) : "v"(ma));
-            asm volatile("ds_read_u16 %0, %1 offset:%2" : "=v"(m_sc) : "v"(sa), "i"(((u + 1) % 3) * kPpMaskBuf));
-        }
-#pragma unroll
-        for (int e = 0; e < 2; e++)
-#pragma unroll
-            for (int i = 0; i < 4; i++) TLLM_LDS_READ128(Ra[e][i], fwl[e], wb * kWBytes + i * 32 * kRowBytes);
-        TLLM_FENCE();
-        asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");  // the mask words; the fragments may still be on their way
-        TLLM_FENCE();
-        decode_store(m_w[0], m_w[1], m_sc, std::integral_constant<int, (wb + 1) % 3>{});
-        TLLM_FENCE();
-        // the activations of stage s were asked for before the masks of stage s + 1: they have landed too
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        TLLM_FENCE();
-    };
-    // matrix half of stage s: asks for the activations of stage s + 2 and the masks of stage s + 3
-    auto mma = [&](auto U, const int s) {
-        constexpr int u = decltype(U)::value;
-        constexpr int rb = u % 3;
-        __builtin_amdgcn_s_setprio(3);  // the other wave of the SIMD is in its memory half: its instructions must not delay these
-#pragma unroll
-        for (int e = 0; e < 2; e++)
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-#pragma unroll
-                for (int j = 0; j < MF; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, Ra[e][i]), __builtin_bit_cast(h8, Rb[rb][e][j]),
-                                                                       acc[i][j], 0, 0, 0);
-                TLLM_FENCE();
-                if (e * 4 + i < kReq)
-                    request(std::integral_constant<int, (rb + 2) % 3>{}, std::integral_constant<int, u % 3>{}, e * 4 + i, s + 2, s + 3);
-                TLLM_FENCE();
-            }
-        __builtin_amdgcn_s_setprio(0);
-        TLLM_FENCE();
-    };
-    auto step = [&](auto U, const int s) {
-        mem(U, s);
-        if (kh) __builtin_amdgcn_s_barrier();
-        TLLM_FENCE();
-        mma(U, s);
-        if (!kh) __builtin_amdgcn_s_barrier();
-        TLLM_FENCE();
-    };
-    for (int s0 = 0; s0 <= last; s0 += 6) {  // `last` is odd: stages come in pairs
-        step(std::integral_constant<int, 0>{}, s0);
-        step(std::integral_constant<int, 1>{}, s0 + 1);
-        if (s0 + 2 > last) break;
-        step(std::integral_constant<int, 2>{}, s0 + 2);
-        step(std::integral_constant<int, 3>{}, s0 + 3);
-        if (s0 + 4 > last) break;
-        step(std::integral_constant<int, 4>{}, s0 + 4);
-        step(std::integral_constant<int, 5>{}, s0 + 5);
-    }
-    TLLM_FENCE();
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // requests past the last stage have landed (registers and LDS)
-    __builtin_amdgcn_s_barrier();
-    TLLM_FENCE();
-
-    // ---- the two waves of a pair add their sums: fragment t = i * MF + j stays with wave kh = t & 1, the other
-    // half crosses through LDS (free now); a + b = b + a, so both get the same bits whoever adds
-    {
-        // the compiler cannot see that the LDS writes below read matrix results: the slots a 16-pass
-        // product needs before its result may be read by a memory instruction
-        asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 3" ::: "memory");
-        constexpr int kKeep = kTiles / 2;
-        const uint32_t xw = lds0 + (uint32_t)(wave * kKeep * 4096 + lane * 16);
-        const uint32_t xr = lds0 + (uint32_t)((wave ^ 4) * kKeep * 4096 + lane * 16);
-#pragma unroll
-        for (int t = 0; t < kTiles; t++) {
-            const int i = t / MF, j = t % MF;
-            if ((t & 1) != kh) {
-#pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const f4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-                    asm volatile("ds_write_b128 %0, %1" ::"v"(xw + (uint32_t)(((t >> 1) * 4 + g) * 1024)), "v"(v) : "memory");
-                }
-            }
-        }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        __builtin_amdgcn_s_barrier();
-        TLLM_FENCE();
-#pragma unroll
-        for (int t = 0; t < kTiles; t++) {
-            const int i = t / MF, j = t % MF;
-            if ((t & 1) == kh) {
-                f4 v[4];
-#pragma unroll
-                for (int g = 0; g < 4; g++)
-                    asm volatile("ds_read_b128 %0, %1" : "=v"(v[g]) : "v"(xr + (uint32_t)(((t >> 1) * 4 + g) * 1024)));
-                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                TLLM_FENCE();
-#pragma unroll
-                for (int g = 0; g < 4; g++)
-#pragma unroll
-                    for (int e = 0; e < 4; e++) acc[i][j][4 * g + e] += v[g][e];
-            }
-        }
-    }
-#undef TLLM_LDS_READ128
-#undef TLLM_LDS_WRITE128
-#undef TLLM_GLOAD128
-#undef TLLM_FENCE
-#undef TLLM_GPTR
-#undef TLLM_LPTR
-
-    // ---- store the fragments this wave kept: 32 activation rows (j = kh for MF = 2) x 128 weight rows. Lane
-    // (li, lq) holds, for activation row li, four consecutive weight rows per register quad: written as they are
-    // these would be 8-byte pieces in 32 different lines per instruction. The tile goes through LDS instead
-    // (rows of 272 bytes, so that the 8-byte writes of a wave spread over the banks) and leaves as whole
-    // 256-byte runs, 16 lanes per activation row.
-    constexpr int kRowPad = 272;
-    const bool wide_store = MF == 2 && (N & 7) == 0 && (reinterpret_cast<uintptr_t>(C) & 15) == 0;
-    if (wide_store) {
-        __builtin_amdgcn_s_barrier();  // the exchange area is read: it may be overwritten
-        unsigned char *mine = lds + wave * 32 * kRowPad;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const f16v a = kh ? acc[i][MF - 1] : acc[i][0];  // the fragment this wave kept: column kh
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const uint2 hq = {(uint32_t)f2h(a[4 * g] * 0.5f) | ((uint32_t)f2h(a[4 * g + 1] * 0.5f) << 16),
-                                  (uint32_t)f2h(a[4 * g + 2] * 0.5f) | ((uint32_t)f2h(a[4 * g + 3] * 0.5f) << 16)};
-                *reinterpret_cast<uint2 *>(mine + li * kRowPad + (32 * i + 8 * g + 4 * lq) * 2) = hq;
-            }
-        }
-        // a wave reads back only what it wrote: no barrier, the compiler's wait for the LDS queue is enough
-        const int c16 = lane & 15, r4 = lane >> 4;
-#pragma unroll
-        for (int rr = 0; rr < 8; rr++) {
-            const int r = 4 * rr + r4;
-            const u4 v = *reinterpret_cast<const u4 *>(mine + r * kRowPad + c16 * 16);
-            const int m = m0 + kh * 32 + r, n = n0 + c16 * 8;
-            if (m < M && n < N) *reinterpret_cast<u4 *>(C + (size_t)m * N + n) = v;
-        }
-        return;
-    }
-    const bool vec_store = (N & 3) == 0 && (reinterpret_cast<uintptr_t>(C) & 7) == 0;
-#pragma unroll
-    for (int t = 0; t < kTiles; t++) {
-        const int i = t / MF, j = t % MF;
-        if ((t & 1) != kh) continue;
-        const int m = m0 + j * 32 + li;
-        if (m >= M) continue;
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-            const int n = n0 + i * 32 + 8 * g + 4 * lq;
-            uint16_t h[4];
-#pragma unroll
-            for (int v = 0; v < 4; v++) h[v] = f2h(acc[i][j][4 * g + v] * 0.5f);
-            uint16_t *dst = C + (size_t)m * N + n;
-            if (n + 3 < N && vec_store) {
-                *reinterpret_cast<uint2 *>(dst) = uint2{(uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
-            } else {
-#pragma unroll
-                for (int v = 0; v < 4; v++)
-                    if (n + v < N) dst[v] = h[v];
-            }
-        }
-    }
-}
-
 // ---- The row-split kernel: the waves of a workgroup split the weight rows, weights decoded straight into MFMA operand
 // registers.
 //
@@ -926,8 +555,11 @@ __global__ __launch_bounds__(512 / NF) __attribute__((amdgpu_waves_per_eu(2, 2))
     // activation tile first: whichever lets an XCD's L2 fetch fewer bytes for its share (the launcher decides)
     const int n0 = (n_fastest ? tile % n_tiles : tile / m_tiles) * kNsBN;
     const int m0 = (n_fastest ? tile / n_tiles : tile % m_tiles) * BM;
-    const int words = K / 32, groups = K / 128, blocks = K / 256;
-    const int chunks = blocks * 4;
+    // K is a multiple of 128: a last block of 128 columns runs as a whole block whose upper mask words are zero
+    // (its activation chunks past the row re-read the last chunk: they meet zero weights)
+    const int words = K / 32, groups = K / 128, blocks = (K + 255) / 256;
+    const int chunks = K / 64;
+    const bool tail_half = (K & 255) != 0;
     const int b_begin = is_split ? (int)((long)blocks * split / splits) : 0;
     const int b_end = is_split ? (int)((long)blocks * (split + 1) / splits) : blocks;
 
@@ -975,13 +607,18 @@ __global__ __launch_bounds__(512 / NF) __attribute__((amdgpu_waves_per_eu(2, 2))
         nx_sg[f] = u4{0u, 0u, 0u, 0u};
         nx_sc[f] = 0;
     }
+    auto half_block = [&](int b) { return tail_half && b >= blocks - 1; };
     auto load_masks = [&](int b) {
         const int bb = min(b, blocks - 1);
+        // a half block holds mask words 0..3 and one scale: the upper lane half, which would load words 4..7 from
+        // the next row (or from beyond the array), loads the lower words again (dropped in take_masks); the scale
+        // dword starts one scale earlier, so that it ends with the row
+        const int back = half_block(b) ? 16 * lq : 0, sc_back = half_block(b) ? 2 : 0;
 #pragma unroll
         for (int f = 0; f < NF; f++) {
-            GB *p0 = nz_g[f] + (size_t)bb * 32;
-            GB *p1 = sg_g[f] + (size_t)bb * 32;
-            GB *p2 = sc_g[f] + (size_t)bb * 4;
+            GB *p0 = nz_g[f] + (size_t)bb * 32 - back;
+            GB *p1 = sg_g[f] + (size_t)bb * 32 - back;
+            GB *p2 = sc_g[f] + (size_t)bb * 4 - sc_back;
             asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(nx_nz[f]) : "v"(p0) : "memory");
             asm volatile("global_load_dwordx4 %0, %1, off" : "+v"(nx_sg[f]) : "v"(p1) : "memory");
             asm volatile("global_load_dword %0, %1, off" : "+v"(nx_sc[f]) : "v"(p2) : "memory");
@@ -1023,7 +660,7 @@ __global__ __launch_bounds__(512 / NF) __attribute__((amdgpu_waves_per_eu(2, 2))
         if (e > 0) top &= 0xC000C000u;  // (for e = 0 the shift leaves nothing below the field)
         return __builtin_bit_cast(uint32_t, __builtin_bit_cast(h2, top) * sp[f]);
     };
-    auto take_masks = [&]() {  // the loads into nx_* are complete where this is called
+    auto take_masks = [&](bool half) {  // the loads into nx_* are complete where this is called; half: a last block of 128 columns
 #pragma unroll
         for (int f = 0; f < NF; f++) {
             asm volatile("" : "+v"(nx_nz[f]), "+v"(nx_sg[f]), "+v"(nx_sc[f]));
@@ -1033,8 +670,12 @@ __global__ __launch_bounds__(512 / NF) __attribute__((amdgpu_waves_per_eu(2, 2))
             const auto g23 = __builtin_amdgcn_permlane32_swap(nx_sg[f][2], nx_sg[f][3], false, false);
             cu_nz[f][0] = s01[0]; cu_nz[f][2] = s01[1]; cu_nz[f][1] = s23[0]; cu_nz[f][3] = s23[1];
             cu_sg[f][0] = g01[0]; cu_sg[f][2] = g01[1]; cu_sg[f][1] = g23[0]; cu_sg[f][3] = g23[1];
-            sp2[f][0] = __builtin_bit_cast(h2, __builtin_amdgcn_perm(nx_sc[f], nx_sc[f], 0x01000100u));
+            sp2[f][0] = __builtin_bit_cast(h2, __builtin_amdgcn_perm(nx_sc[f], nx_sc[f], half ? 0x03020302u : 0x01000100u));
             sp2[f][1] = __builtin_bit_cast(h2, __builtin_amdgcn_perm(nx_sc[f], nx_sc[f], 0x03020302u));
+            if (half) {  // words 4..7 do not exist: no weights there
+                cu_nz[f][2] = 0;
+                cu_nz[f][3] = 0;
+            }
 #pragma unroll
             for (int u = 0; u < 4; u++) asm volatile("" : "+v"(cu_nz[f][u]), "+v"(cu_sg[f][u]));
             asm volatile("" : "+v"(sp2[f][0]), "+v"(sp2[f][1]));
@@ -1052,7 +693,7 @@ __global__ __launch_bounds__(512 / NF) __attribute__((amdgpu_waves_per_eu(2, 2))
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kDma) : "memory");
     __builtin_amdgcn_s_barrier();
     TLLM_FENCE();
-    take_masks();
+    take_masks(half_block(b_begin));
     load_masks(b_begin + 1);
     dma_chunk(c_begin + 3, 3);
     TLLM_FENCE();
@@ -1083,7 +724,7 @@ __global__ __launch_bounds__(512 / NF) __attribute__((amdgpu_waves_per_eu(2, 2))
             __builtin_amdgcn_s_barrier();
             TLLM_FENCE();
             if (u == 3) {
-                take_masks();
+                take_masks(half_block((c + 1) / 4));
                 load_masks((c + 1) / 4 + 1);
             }
             dma_chunk(c + 4, u);
@@ -1303,9 +944,8 @@ hipError_t static_scratch(unsigned char **out) {
 }
 
 struct GemmConfig {
-    int height;   // 0: 128 activation rows per workgroup, 1: 256 (four-wave and eight-wave ping-pong kernels)
+    int height;   // four-wave kernel: 0 = 128 activation rows per workgroup, 1 = 256
     int splits;   // workgroups per tile along K (four-wave kernel: every tile; row-split kernel: the tiles after full_tiles)
-    bool pingpong;  // the eight-wave kernel (256 activation rows, one workgroup per tile, fragment-ordered activations)
     float us;     // estimated time
     bool rowsplit = false;  // the row-split kernel (256 weight rows x 128 activation rows per workgroup)
     int full_tiles = 0;     // row-split kernel: tiles computed by one workgroup each
@@ -1313,14 +953,12 @@ struct GemmConfig {
 };
 GemmConfig choose_config(const Problem &p, size_t workspace_floats);
 
-// Workspace a configuration needs, in floats: the fp32 slots of a split, or the fragment-ordered copy of the
-// activations (rows rounded up to 32) of the eight-wave kernel. The two never occur together.
+// Workspace a configuration needs, in floats: the fp32 slots of a split.
 size_t workspace_floats(const Problem &p, const GemmConfig &c) {
     if (c.rowsplit) {
         const size_t tiles = (size_t)((p.batch + 127) / 128) * ((p.rows + kNsBN - 1) / kNsBN);
         return c.splits > 1 ? (tiles - c.full_tiles) * c.splits * 128 * kNsBN : 0;
     }
-    if (c.pingpong) return (size_t)((p.batch + 31) / 32) * 32 * p.cols / 2;
     const int bm = 128 << c.height;
     const size_t tiles = (size_t)((p.batch + bm - 1) / bm) * ((p.rows + kBN - 1) / kBN);
     return c.splits > 1 ? tiles * c.splits * bm * kBN : 0;
@@ -1349,33 +987,6 @@ hipError_t launch(const Problem &p, int splits, float *partial, unsigned *arriva
     return hipGetLastError();
 }
 
-
-hipError_t launch_pingpong(const Problem &p, float *workspace, hipStream_t s) {
-    constexpr int MF = 2, BM = 128 * MF;
-    static std::mutex attr_mutex;
-    static bool attr_set[64] = {};
-    int dev = 0;
-    if (hipError_t e = hipGetDevice(&dev)) return e;
-    // loop: three weight buffers and three mask buffers; afterwards the wave pairs exchange half their sums
-    const size_t loop = 3 * (size_t)kWBytes + 3 * (size_t)kPpMaskBuf, exchange = 8 * (size_t)(2 * MF) * 4096;
-    const size_t lds = loop > exchange ? loop : exchange;
-    if (dev >= 0 && dev < 64) {
-        std::lock_guard<std::mutex> lock(attr_mutex);
-        if (!attr_set[dev]) {
-            if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_pp_kernel<MF>),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
-                return e;
-            attr_set[dev] = true;
-        }
-    }
-    u4 *At = reinterpret_cast<u4 *>(workspace);
-    tile_acts_kernel<<<(unsigned)(((p.batch + 31) / 32) * ((p.cols / 64 + 3) / 4)), 256, 0, s>>>(p.x, At, p.batch, p.cols);
-    if (hipError_t e = hipGetLastError()) return e;
-    const int m_tiles = (p.batch + BM - 1) / BM, n_tiles = (p.rows + kBN - 1) / kBN;
-    gemm_pp_kernel<MF><<<m_tiles * n_tiles, kPpThreads, lds, s>>>(reinterpret_cast<const uint16_t *>(At), p.nz, p.sg, p.scales, p.y,
-                                                                 p.batch, p.rows, p.cols);
-    return hipGetLastError();
-}
 
 template <int NF>
 hipError_t launch_rowsplit(const Problem &p, const GemmConfig &c, float *partial, unsigned *arrivals, hipStream_t s) {
@@ -1418,11 +1029,25 @@ hipError_t launch_rowsplit(const Problem &p, const GemmConfig &c, float *partial
 
 }  // namespace
 
+namespace {
+// The four-wave kernel fetches scales as aligned dwords: the array must start on one and hold an even count.
+bool scales_dword_aligned(const Problem &p) {
+    return !(reinterpret_cast<uintptr_t>(p.scales) & 3) && !(((size_t)p.rows * (p.cols / 128)) & 1);
+}
+// The row-split kernel: K a multiple of 256, or of 128 from 384 on (the last block then holds 128 columns); mask rows and
+// activations in 16-byte pieces. (Its scale loads may start on any halfword.)
+bool rowsplit_ok(const Problem &p) {
+    return (p.cols % 256 == 0 || (p.cols % 128 == 0 && p.cols >= 384)) &&
+           !((reinterpret_cast<uintptr_t>(p.x) | reinterpret_cast<uintptr_t>(p.nz) | reinterpret_cast<uintptr_t>(p.sg)) & 15);
+}
+}  // namespace
+
 bool gemm_mfma_supports(const Problem &p, int group) {
-    // scales are fetched as aligned dwords: the array must start on one and hold an even count
-    if ((reinterpret_cast<uintptr_t>(p.scales) & 3) || (((size_t)p.rows * (p.cols / 128)) & 1)) return false;
-    return group == 128 && p.batch >= 16 && p.cols % 128 == 0 && (size_t)p.rows * (p.cols / 32) < ((size_t)1 << 31) &&
-           (size_t)p.batch * p.cols < ((size_t)1 << 31);
+    if (!(group == 128 && p.batch >= 16 && p.cols % 128 == 0 && (size_t)p.rows * (p.cols / 32) < ((size_t)1 << 31) &&
+          (size_t)p.batch * p.cols < ((size_t)1 << 31)))
+        return false;
+    // (a shape-only query, pointers null: the answer for aligned arrays)
+    return scales_dword_aligned(p) || rowsplit_ok(p);
 }
 
 namespace {
@@ -1434,13 +1059,13 @@ GemmConfig choose_config(const Problem &p, size_t limit_floats) {
     const int n_cu = current_device_cus();
     const int n_tiles = (p.rows + kBN - 1) / kBN, groups = p.cols / 128;
     const float stage_us[2] = {0.70f, 1.19f};
-    GemmConfig best{0, 1, false, 0.f};
+    GemmConfig best{0, 1, 0.f};
     for (int c = 0; c < 2; c++) {
         const int bm = 128 << c;
         const long tiles = (long)n_tiles * ((p.batch + bm - 1) / bm);
         for (int splits = 1; splits <= 8; splits *= 2) {
             if (splits > 1 && (tiles * splits > n_cu || groups / splits < 4)) break;  // only to fill idle CUs
-            const GemmConfig cand{c, splits, false, 0.f};
+            const GemmConfig cand{c, splits, 0.f};
             if (workspace_floats(p, cand) > limit_floats) break;
             const long wgs = tiles * splits;
             const float stages = (float)((groups + splits - 1) / splits * 2);
@@ -1449,19 +1074,8 @@ GemmConfig choose_config(const Problem &p, size_t limit_floats) {
             // (fitted to fifteen shapes between 100 x 2048 x 2048 and 512 x 8192 x 28672)
             const float exchange = splits > 1 ? (2.0f + 0.7f * (float)splits + 0.025f * (float)(tiles * splits)) * (float)(bm / 128) : 0.0f;
             const float us = (float)((wgs + n_cu - 1) / n_cu) * stages * stage_us[c] + 5.0f + exchange;
-            if (best.us == 0.f || us < best.us) best = GemmConfig{c, splits, false, us};
+            if (best.us == 0.f || us < best.us) best = GemmConfig{c, splits, us};
         }
-    }
-    // The eight-wave kernel: 0.85 us per stage (0.69 - 0.92 measured, the clock falls with the load), 9 us of
-    // start, first loads, pair exchange and stores, and the copy of the activations into fragment order
-    // (read + write at about 4 TB/s behind 2.5 us of its own start).
-    const int forced = tuning().gemm_pingpong.load(std::memory_order_relaxed);  // 0: never, 1: whenever the shape allows
-    const GemmConfig pp{1, 1, true, 0.f};
-    if (forced != 0 && workspace_floats(p, pp) <= limit_floats) {
-        const long tiles = (long)n_tiles * ((p.batch + 255) / 256);
-        const float us = (float)((tiles + n_cu - 1) / n_cu) * (float)(groups * 2) * 0.85f + 9.0f + 2.5f +
-                         (float)p.batch * (float)p.cols * 4.0f / 4.0e6f;
-        if (forced == 1 || us < best.us) best = GemmConfig{1, 1, true, us};
     }
     // The row-split kernel: 3.3 us per block of 256 columns (1490 - 1530 cycles per chunk of 64 at the 1.8 GHz the chip
     // holds under this load), 9 us of launch, first loads and stores. The tiles that do not fill the last round over the
@@ -1469,13 +1083,13 @@ GemmConfig choose_config(const Problem &p, size_t limit_floats) {
     // workspace) when that is cheaper than a last round of whole tiles; an exchange costs about 6 us + 1.5 us per part
     // (fitted to 4096 x 14336 at M = 128 ... 512). Tiles are 128 activation rows high: not for fewer than 96.
     const int forced_rs = tuning().gemm_rowsplit.load(std::memory_order_relaxed);  // 0: never, 1 / 2: whenever the shape allows, in its eight-wave / four-wave form
-    const bool rs_ok = p.cols % 256 == 0 && !((reinterpret_cast<uintptr_t>(p.x) | reinterpret_cast<uintptr_t>(p.nz) |
-                                                reinterpret_cast<uintptr_t>(p.sg)) & 15);
-    if (forced_rs != 0 && rs_ok && forced != 1 && (forced_rs >= 1 || p.batch >= 96)) {
-        const int blocks = p.cols / 256;
+    const bool rs_ok = rowsplit_ok(p), four_ok = scales_dword_aligned(p);
+    // (a shape whose scales the four-wave kernel cannot fetch runs the row-split kernel whatever its size)
+    if ((forced_rs != 0 || !four_ok) && rs_ok && (forced_rs >= 1 || p.batch >= 96 || !four_ok)) {
+        const int blocks = (p.cols + 255) / 256;
         const int tiles = ((p.batch + 127) / 128) * ((p.rows + kNsBN - 1) / kNsBN);
         const float block_us = 3.3f, fixed_us = 9.0f;
-        GemmConfig rs{0, 1, false, 0.f};
+        GemmConfig rs{0, 1, 0.f};
         rs.rowsplit = true;
         rs.full_tiles = tiles;
         rs.us = (float)((tiles + n_cu - 1) / n_cu) * (float)blocks * block_us + fixed_us;
@@ -1510,7 +1124,7 @@ GemmConfig choose_config(const Problem &p, size_t limit_floats) {
             two.us = (float)(tiles / slots) * (float)blocks * 5.3f + (last > n_cu ? 5.3f : last > 0 ? 3.7f : 0.f) * (float)blocks + fixed_us;
             if (forced_rs == 2 || (forced_rs != 1 && two.us < rs.us)) rs = two;
         }
-        if (forced_rs >= 1 || rs.us < best.us) best = rs;
+        if (forced_rs >= 1 || !four_ok || rs.us < best.us) best = rs;
     }
     return best;
 }
@@ -1524,7 +1138,6 @@ const char *gemm_mfma_kernel_name(const Problem &p) {
     const GemmConfig c = choose_config(p, kStaticSlotFloats);
     if (c.rowsplit && c.frags == 2) return "tllm::gemm_ns_kernel<4, 2>";
     if (c.rowsplit) return c.splits > 1 ? "tllm::gemm_ns_kernel<4, 1>, last tiles K split" : "tllm::gemm_ns_kernel<4, 1>";
-    if (c.pingpong) return "tllm::gemm_pp_kernel<2> after tllm::tile_acts_kernel";
     if (c.height == 1) return c.splits > 1 ? "tllm::gemm_mfma_kernel<2>, K split" : "tllm::gemm_mfma_kernel<2>";
     return c.splits > 1 ? "tllm::gemm_mfma_kernel<1>, K split" : "tllm::gemm_mfma_kernel<1>";
 }
@@ -1532,7 +1145,6 @@ const char *gemm_mfma_kernel_name(const Problem &p) {
 namespace {
 hipError_t launch_config(const Problem &p, const GemmConfig &c, float *workspace, unsigned *arrivals, hipStream_t s) {
     if (c.rowsplit) return c.frags == 2 ? launch_rowsplit<2>(p, c, workspace, arrivals, s) : launch_rowsplit<1>(p, c, workspace, arrivals, s);
-    if (c.pingpong) return launch_pingpong(p, workspace, s);
     return c.height == 1 ? launch<2>(p, c.splits, workspace, arrivals, s) : launch<1>(p, c.splits, workspace, arrivals, s);
 }
 }  // namespace

@@ -129,7 +129,7 @@ def test_tuning_switches_round_trip():
     """The kernel-choice switches are plain values behind tllm_debug_set_tuning / tllm_debug_get_tuning (no
     environment reads on any call path): set, read back, restore; unknown names are rejected."""
     import ternary_llm_amd as tl
-    for name, default in (("gemm_rowsplit", -1), ("gemm_pingpong", -1), ("batch_k_parts", 0), ("tall_max_batch", 4),
+    for name, default in (("gemm_rowsplit", -1), ("stage_spin_limit", 0), ("batch_k_parts", 0), ("tall_max_batch", 4),
                           ("tall_min_share_milli", 1000), ("gemm_path", 0)):
         assert tl.get_tuning(name) == default, name
         with tl.tuning(**{name: 7}):

@@ -63,14 +63,13 @@ def assert_close(oracle, got, ref, tol=TOL, what=""):
 
 
 class gemm_forced:
-    """Forces the GEMM kernel choice through the library's tuning switches (tllm_debug_set_tuning):
-    gemm_forced(pingpong=1), gemm_forced(rowsplit=1), gemm_forced(pingpong=0, rowsplit=0), gemm_forced() for the
-    library's own choice. The switches are put back on exit."""
-    NAMES = {"pingpong": "gemm_pingpong", "rowsplit": "gemm_rowsplit"}
+    """Forces the GEMM kernel choice through the library's tuning switch (tllm_debug_set_tuning):
+    gemm_forced(rowsplit=1) / (rowsplit=2) the row-split kernel in its eight-wave / four-wave form wherever the shape
+    allows, gemm_forced(rowsplit=0) the four-wave kernel, gemm_forced() the library's own choice. The switch is put
+    back on exit."""
 
-    def __init__(self, **kw):
-        self.want = {name: -1 for name in self.NAMES.values()}
-        self.want.update({self.NAMES[k]: int(v) for k, v in kw.items()})
+    def __init__(self, rowsplit=-1):
+        self.want = {"gemm_rowsplit": int(rowsplit)}
 
     def __enter__(self):
         import ternary_llm_amd as tl
@@ -261,21 +260,43 @@ def test_gemm_vs_oracle(dev, oracle, M, N, K):
 
 @pytest.mark.parametrize("M,N,K", [(600, 300, 640), (33, 128, 128), (257, 1000, 1152), (100, 129, 256), (512, 136, 384),
                                    (16, 64, 128), (1023, 260, 640)])  # K not a multiple of 512: these go to the GEMM kernels
-def test_gemm_eight_wave_kernel_edges(dev, oracle, M, N, K):
-    """The eight-wave kernel (chosen by itself only for tall problems) forced onto shapes with ragged edges:
-    M not a multiple of 256 or of 32, N not a multiple of 128 or of 8 (the narrow store path), a single
-    scale group, more tiles than CUs. Against the fp64 oracle, and against the four-wave kernel (the two
-    differ only in the order of the fp32 additions)."""
+def test_gemm_four_wave_kernel_edges(dev, oracle, M, N, K):
+    """The four-wave kernel forced onto shapes with ragged edges: M not a multiple of 256 or of 32, N not a multiple
+    of 128 or of 8 (the narrow store path), a single scale group, more tiles than CUs. Against the fp64 oracle, and
+    against the library's own choice (the kernels differ only in the order of the fp32 additions)."""
     nz, sg, s, _ = synth.problem(M * 7 + N, N, K, dontcare_sign=True)
     A = synth.acts_f16(np.random.default_rng(M + K + 5), M, K)
     ref = oracle.gemm_f64(A.view(np.uint16), nz, sg, s.view(np.uint16))
-    with gemm_forced(pingpong=1, rowsplit=0):
+    with gemm_forced(rowsplit=0):
         got = run_gemm(dev, A, nz, sg, s)
-    with gemm_forced(pingpong=0, rowsplit=0):
-        other = run_gemm(dev, A, nz, sg, s)
-    assert_close(oracle, got, ref, what=f"eight-wave gemm {M}x{N}x{K}")
-    assert_close(oracle, other, ref, what=f"four-wave gemm {M}x{N}x{K}")
-    assert_close(oracle, got, other, tol=2e-3, what=f"eight-wave against four-wave {M}x{N}x{K}")
+    other = run_gemm(dev, A, nz, sg, s)
+    assert_close(oracle, got, ref, what=f"four-wave gemm {M}x{N}x{K}")
+    assert_close(oracle, other, ref, what=f"gemm as chosen {M}x{N}x{K}")
+    assert_close(oracle, got, other, tol=2e-3, what=f"four-wave against the chosen kernel {M}x{N}x{K}")
+
+
+@pytest.mark.parametrize("M,N,K", [(600, 300, 640), (257, 1000, 1152), (512, 136, 384), (1023, 261, 896), (130, 200, 2688),
+                                   (200, 301, 5248), (96, 17, 384)])
+def test_gemm_row_split_kernel_last_half_block(dev, oracle, M, N, K):
+    """K a multiple of 128 but not of 256: the row-split kernel runs the last 128 columns as a block whose upper mask
+    words are zero. Scale rows then hold an odd number of groups (rows start on any halfword; 1023 x 261 and 96 x 17
+    have an odd number of scales in all, which the four-wave kernel cannot fetch: the library then takes the row-split
+    kernel by itself). Both forms, every output against the fp64 oracle, the last weight row and the last activation
+    row included, and the same bits on every call."""
+    torch, tl = dev
+    nz, sg, s, _ = synth.problem(M * 3 + N + K, N, K, dontcare_sign=True)
+    A = synth.acts_f16(np.random.default_rng(M + K + 11), M, K)
+    ref = oracle.gemm_f64(A.view(np.uint16), nz, sg, s.view(np.uint16))
+    if (N * (K // 128)) % 2:
+        assert "gemm_ns_kernel" in tl.gemm_kernel(M, N, K)
+        assert_close(oracle, run_gemm(dev, A, nz, sg, s), ref, what=f"odd scale count, as chosen, {M}x{N}x{K}")
+    for form in (1, 2):
+        with gemm_forced(rowsplit=form):
+            assert f"gemm_ns_kernel<4, {form}>" in tl.gemm_kernel(M, N, K)
+            got = run_gemm(dev, A, nz, sg, s)
+            again = run_gemm(dev, A, nz, sg, s)
+        assert_close(oracle, got, ref, what=f"row-split gemm with a half block, form {form}, {M}x{N}x{K}")
+        assert np.array_equal(got, again)
 
 
 @pytest.mark.parametrize("M,N,K", [(600, 300, 768), (33, 130, 256), (257, 1000, 1280), (100, 129, 512), (1023, 260, 512),
@@ -289,7 +310,7 @@ def test_gemm_row_split_kernel_edges(dev, oracle, M, N, K):
     nz, sg, s, _ = synth.problem(M * 5 + N + K, N, K, dontcare_sign=True)
     A = synth.acts_f16(np.random.default_rng(M + K + 9), M, K)
     ref = oracle.gemm_f64(A.view(np.uint16), nz, sg, s.view(np.uint16))
-    with gemm_forced(pingpong=0, rowsplit=0):
+    with gemm_forced(rowsplit=0):
         other = run_gemm(dev, A, nz, sg, s)
     for form in (1, 2):  # eight waves with one weight fragment each / four waves with two
         with gemm_forced(rowsplit=form):
@@ -1325,7 +1346,7 @@ def _dense_weights(torch, nz, sg, sc):
     (512, 1024, 4096),     # few tiles: K split eight ways
     (256, 256, 8192),
     (130, 512, 2048),
-    (1024, 14336, 4096),   # the eight-wave kernel
+    (1024, 14336, 4096),
     (300, 2048, 2176),
 ])
 def test_gemm_every_output_against_dense_product(dev, oracle, M, N, K):
@@ -1333,8 +1354,7 @@ def test_gemm_every_output_against_dense_product(dev, oracle, M, N, K):
     multiplied by the activations in fp32 (torch), which is itself checked against the fp64 oracle on sampled
     rows and columns. A fault confined to a few lanes and registers of one exchange step (1 output in 256)
     passes a sampled check more often than not; this test is the one that sees it. Each shape runs as the
-    library chooses, with the eight-wave kernel forced, with the row-split kernel forced in both its forms and with
-    the four-wave kernels only."""
+    library chooses, with the row-split kernel forced in both its forms and with the four-wave kernels only."""
     torch, tl = dev
     gen = torch.Generator(device="cuda")
     gen.manual_seed(7000 + M + N + K)
@@ -1345,7 +1365,7 @@ def test_gemm_every_output_against_dense_product(dev, oracle, M, N, K):
     del W
     _check_sampled(oracle, torch, A, nz, sg, sc, ref, 4, 40, M + K, f"dense fp32 product {M}x{N}x{K}")
     tau = float(torch.sqrt(torch.mean(ref * ref)).item()) / 64.0
-    for force in ({}, {"pingpong": 1, "rowsplit": 0}, {"rowsplit": 1}, {"rowsplit": 2}, {"pingpong": 0, "rowsplit": 0}):
+    for force in ({}, {"rowsplit": 1}, {"rowsplit": 2}, {"rowsplit": 0}):
         with gemm_forced(**force):
             for rep in range(2):
                 Cm = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda")

@@ -219,6 +219,7 @@ struct PlanDevice {
     int *status = nullptr;
     int spin_limit = 0;
     size_t barrier_bytes = 0;  // all barriers and the status word: cleared when a timeout is read
+    bool stage_fence = false;  // the workgroups invalidate their cache behind each barrier (else: loads of device scope)
 };
 hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out);
 // A plan whose problems run in stages inside one launch (Problem::stage, ascending); batch 1, shapes the wide-tile

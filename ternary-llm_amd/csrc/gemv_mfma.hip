@@ -113,6 +113,10 @@ struct Sched {
     int spin_limit;
     int *barrier;
     int *status;
+    // How a stage sees what the stage before wrote. 0: its loads of activations and residuals ask for memory's copy
+    // themselves (loads of device scope, no cache is invalidated: every problem's row is staged in one pass from
+    // registers). 1: every workgroup invalidates its cache behind the barrier (any shape; costs about 2 us per stage).
+    int stage_fence;
 };
 // Layout of a stage barrier, in ints: [0] the flag, [32] the top counter, [64 + 32 g] the counter of group g: every
 // word that takes atomics from many workgroups sits on a 128-byte line of its own.
@@ -514,10 +518,35 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
             if (n_seg == 1 && p.batch == 1 && pieces <= kKeep * kThreads) {
                 // one pass over x: all loads are issued together and kept for the image
                 uint4 keep[kKeep];
+                if (kExtras && staged && !sc.stage_fence) {
+                    // The stage before wrote these activations, maybe on another XCD: loads of device scope fetch
+                    // memory's copy instead of a stale line of this XCD's cache. The compiler does not count loads it
+                    // cannot see, so the wait is written out; it names the registers, so that nothing reads them before.
+                    u4 got[kKeep];
+#pragma unroll
+                    for (int k = 0; k < kKeep; k++) {
+                        const int c8 = stid + k * kThreads;
+                        got[k] = u4{0u, 0u, 0u, 0u};
+                        const int slice = seg_lo + (c8 * 8) / G::kCols;
+                        const int chunk = ((c8 * 8) % G::kCols) / kChunkCols;
+                        const int g = min(slice * G::kChunks, groups - G::kChunks) + chunk;
+                        if (c8 < pieces && g >= slice * G::kChunks) {
+                            const uint4 *src = reinterpret_cast<const uint4 *>(p.x) + (g * kChunkCols + (c8 * 8) % kChunkCols) / 8;
+                            asm volatile("global_load_dwordx4 %0, %1, off sc1" : "+v"(got[k]) : "v"(src) : "memory");
+                        }
+                    }
+                    asm volatile("s_waitcnt vmcnt(0)"
+                                 : "+v"(got[0]), "+v"(got[1]), "+v"(got[2]), "+v"(got[3]), "+v"(got[4]), "+v"(got[5]), "+v"(got[6]), "+v"(got[7])
+                                 :
+                                 : "memory");
+#pragma unroll
+                    for (int k = 0; k < kKeep; k++) keep[k] = uint4{got[k][0], got[k][1], got[k][2], got[k][3]};
+                } else {
 #pragma unroll
                 for (int k = 0; k < kKeep; k++) {
                     const int c8 = stid + k * kThreads;
                     keep[k] = c8 < pieces ? piece_of(0, c8) : uint4{0u, 0u, 0u, 0u};
+                }
                 }
                 if (kExtras && p.norm_w) {
                     // RMSNorm prologue, reference kernels/rmsnorm.cu:20-106 without residual: the kept
@@ -927,7 +956,8 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                 if (kExtras && p.residual) {
                     // the reference's add_forward behind the projection (src/transformer.cpp:247-250, 293-296): one
                     // correctly rounded fp16 add of the residual stream and the fp16-rounded projection
-                    const _Float16 res = __builtin_bit_cast(_Float16, p.residual[r_begin + rl]);
+                    // (a load of device scope: an earlier stage may have written the residual stream)
+                    const _Float16 res = __builtin_bit_cast(_Float16, __hip_atomic_load(p.residual + r_begin + rl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
                     out = __builtin_bit_cast(uint16_t, (_Float16)(res + __builtin_bit_cast(_Float16, out)));
                 }
                 uint16_t *dst = p.y + (size_t)b * p.rows + r_begin + rl;
@@ -979,10 +1009,10 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
         __syncthreads();
         if (!stage_reached) break;  // (the same for the whole workgroup: every wave leaves through the code below)
         // what the stage before wrote is read from memory, not from a stale line of this XCD's cache
-#ifndef TLLM_STAGE_NO_FENCE
-        if (wave == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-        __syncthreads();
-#endif
+        if (sc.stage_fence) {
+            if (wave == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+            __syncthreads();
+        }
         cur = -1;
     }
     }  // stages
@@ -1543,6 +1573,10 @@ hipError_t plan_device_create_staged(const std::vector<Problem> &host, PlanDevic
     }
     d.n_stages = stage + 1;
     d.max_batch = 1;
+    // rows that the one-pass staging holds in registers (K <= 16384) and are not quantised inside the launch are
+    // read with loads of device scope; anything else makes the workgroups invalidate their cache behind each barrier
+    for (const Problem &p : host)
+        if (p.cols > 16384 || (p.flags & kProblemQuantInput)) d.stage_fence = true;
     const int mats = has_pairs ? 2 : 1;
     if (whole + kNW * kFineUnit * 4 * mats > kLdsLimit) return hipErrorInvalidValue;  // whole rows in LDS (K <= 28672)
     const int max_units = max_units_for(whole, 1, kFineUnit, mats);
@@ -1661,6 +1695,7 @@ hipError_t plan_device_launch(const PlanDevice &plan, hipStream_t s) {
     if (plan.n_stages > 0) {
         sc.n_stages = plan.n_stages;
         sc.barrier = plan.stage_counters + slot * kBarrierInts;
+        sc.stage_fence = plan.stage_fence ? 1 : 0;
         sc.status = plan.status;
         const int limit = tuning().stage_spin_limit.load(std::memory_order_relaxed);
         sc.spin_limit = limit > 0 ? limit : plan.spin_limit;

@@ -380,7 +380,8 @@ const char *tllm_linear_plan_kernel(const tllm_linear_plan *plan) {
     const tllm::PlanDevice &d = plan->dev;
     if (d.batch_kernel) return "tllm::gemv_batch_kernel";
     if (!d.use_mfma) return "tllm::gemv_rowwave_f16_table_kernel";
-    if (d.n_stages > 0) return "tllm::gemv_mfma_kernel<Wide, extras, fine>, staged";
+    if (d.n_stages > 0 && d.exchange) return "tllm::gemv_mfma_kernel<Wide, extras, fine>, staged, results handed over as tagged words";
+    if (d.n_stages > 0) return "tllm::gemv_mfma_kernel<Wide, extras, fine>, staged, barriers between the stages";
     if (!d.wide) return d.fine ? "tllm::gemv_mfma_kernel<Tall, fine>" : "tllm::gemv_mfma_kernel<Tall>";
     if (d.extras) return d.fine ? "tllm::gemv_mfma_kernel<Wide, extras, fine>" : "tllm::gemv_mfma_kernel<Wide, extras>";
     return d.fine ? "tllm::gemv_mfma_kernel<Wide, fine>" : "tllm::gemv_mfma_kernel<Wide>";

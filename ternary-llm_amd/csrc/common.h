@@ -43,10 +43,26 @@ struct Problem {
     // optional epilogue (staged plans): the output is fp16(residual[r] + fp16(projection)), the reference's add_forward
     // behind the projection; may point at the output itself (in place)
     const uint16_t *residual;
+    // Staged plans that hand results from stage to stage as tagged words (PlanDevice::exchange): where the launch
+    // finds the problem's activations / its residual / where it leaves its output, as an index into the launch
+    // slot's array of 32-bit words (fp16 bits | tag << 16), or -1: activations and residual are read from x and
+    // residual as they are (nothing in the plan writes them), no later stage reads the output.
+    int32_t x_words, res_words, y_words;
+    int32_t pad_;
 };
-static_assert(sizeof(Problem) == sizeof(tllm_linear_problem) + 24, "tllm_linear_problem, then the prologue and the epilogue");
+static_assert(sizeof(Problem) == sizeof(tllm_linear_problem) + 40, "tllm_linear_problem, then the prologue, the epilogue and the hand-over");
+// What a workgroup of a staged plan needs to start a stage, in one 128-byte record (one round trip to memory instead
+// of three dependent ones: its span, the span's place in the unit prefix, the problem): the span, the problem its
+// first unit lies in, that problem's first unit and number of units, and the problem itself.
+struct WgStart {
+    int32_t u, u_end, pi, first_unit, p_units, pad[3];
+    Problem p;
+};
+static_assert(sizeof(WgStart) == 128, "one record per 128-byte line");
 constexpr int kProblemSwigluGate = TLLM_PROBLEM_SWIGLU_GATE;
 constexpr int kProblemInt8Input = 0x100;  // set by tllm_linear_plan_create_i8, not a public flag
+// staged plans, set by the library: a later stage overwrites y, so the store to y is complete before the tagged word goes out
+constexpr int kProblemOrderedStore = 0x200;
 // fp16 activations that the kernel quantises to int8 itself (absmax, reference kernels/activations.cu:88-142) before it
 // multiplies: quantize_absmax_int8 + ternary_gemv_int8 in one launch, bit for bit (batch 1)
 constexpr int kProblemQuantInput = TLLM_PROBLEM_QUANTIZE_INPUT;
@@ -60,6 +76,7 @@ struct Tuning {
     std::atomic<int> batch_k_parts{0};          // TLLM_BATCH_K_PARTS: n parts where they fit, 1 never share out K
     std::atomic<int> tall_max_batch{4};         // TLLM_TALL_MAX_BATCH: most activation rows of a plan on the tall-tile kernel
     std::atomic<int> tall_min_share_milli{1000};  // TLLM_TALL_MIN_SHARE (x 1000): share of the plan per workgroup, in units, from which tall tiles run
+    std::atomic<int> stage_exchange{1};         // staged plans hand results over as tagged words where the plan allows (0: always the barrier)
     std::atomic<int> stage_spin_limit{0};       // polls a workgroup of a staged plan waits for a stage (0: the plan's own limit); tests force a wait to expire with 1
     std::atomic<int> read_wgs_per_cu{8};        // TLLM_READ_SHAPE="wgs_per_cu,loads_in_flight" of tllm_read_stream
     std::atomic<int> read_in_flight{8};
@@ -220,6 +237,12 @@ struct PlanDevice {
     int spin_limit = 0;
     size_t barrier_bytes = 0;  // all barriers and the status word: cleared when a timeout is read
     bool stage_fence = false;  // the workgroups invalidate their cache behind each barrier (else: loads of device scope)
+    // Hand-over by tagged words instead of barriers: per launch slot an array of words_per_slot 32-bit words (one per
+    // output row that a later stage reads) and one launch count per workgroup (epochs), from which the tag comes.
+    bool exchange = false;
+    WgStart *starts = nullptr;  // [n_stages * grid]
+    uint32_t *words = nullptr;  // per launch slot: the words, then one launch count per workgroup
+    size_t words_per_slot = 0, ints_per_slot = 0;
 };
 hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out);
 // A plan whose problems run in stages inside one launch (Problem::stage, ascending); batch 1, shapes the wide-tile

@@ -117,6 +117,18 @@ struct Sched {
     // themselves (loads of device scope, no cache is invalidated: every problem's row is staged in one pass from
     // registers). 1: every workgroup invalidates its cache behind the barrier (any shape; costs about 2 us per stage).
     int stage_fence;
+    // Hand-over without barriers (exchange != 0). A problem whose output a later stage reads also stores every
+    // output row as a 32-bit word, fp16 bits | tag << 16, written through to memory (words + Problem::y_words); the
+    // problems that read it poll those words with loads of device scope until every one carries the tag of this
+    // launch, and take the values from them: a workgroup waits for exactly the data it needs, and the wait and the
+    // transfer are one round trip. The tag is the low 16 bits of (launches of this slot so far + 1): every workgroup
+    // keeps that count in a word of its own (epochs[blockIdx.x]), reads it when it starts and adds one when it
+    // leaves, so all workgroups agree on it without talking, also when a captured launch is replayed. Every word is
+    // rewritten by every launch, so a stale word carries the tag before. Waits are bounded as at the barrier.
+    int exchange;
+    uint32_t *words;
+    int *epochs;
+    const WgStart *starts;  // staged plans: [n_stages * grid] what each workgroup starts each stage with
 };
 // Layout of a stage barrier, in ints: [0] the flag, [32] the top counter, [64 + 32 g] the counter of group g: every
 // word that takes atomics from many workgroups sits on a 128-byte line of its own.
@@ -228,6 +240,41 @@ __device__ __forceinline__ f4 tile_product(const u4 nz, const u4 sg, const u4 (&
     return d0 + d1;
 }
 
+// Loads of device scope (they fetch memory's copy, not a line of this XCD's cache that another XCD has made stale),
+// issued together and waited for inside ONE asm statement: the compiler never sees a register whose load is still in
+// flight, so it cannot copy or spill one (it takes the outputs of an asm statement for complete when it ends).
+__device__ __forceinline__ void load8_device_scope(const uint4 *const (&src)[8], u4 (&got)[8]) {
+    asm volatile(
+        "global_load_dwordx4 %0, %8, off sc1\n\t"
+        "global_load_dwordx4 %1, %9, off sc1\n\t"
+        "global_load_dwordx4 %2, %10, off sc1\n\t"
+        "global_load_dwordx4 %3, %11, off sc1\n\t"
+        "global_load_dwordx4 %4, %12, off sc1\n\t"
+        "global_load_dwordx4 %5, %13, off sc1\n\t"
+        "global_load_dwordx4 %6, %14, off sc1\n\t"
+        "global_load_dwordx4 %7, %15, off sc1\n\t"
+        "s_waitcnt vmcnt(0)"
+        : "=&v"(got[0]), "=&v"(got[1]), "=&v"(got[2]), "=&v"(got[3]), "=&v"(got[4]), "=&v"(got[5]), "=&v"(got[6]), "=&v"(got[7])
+        : "v"(src[0]), "v"(src[1]), "v"(src[2]), "v"(src[3]), "v"(src[4]), "v"(src[5]), "v"(src[6]), "v"(src[7])
+        : "memory");
+}
+// the same for four runs of eight 32-bit words (32 bytes each)
+__device__ __forceinline__ void load4x8_words_device_scope(const uint32_t *const (&src)[4], u4 (&lo)[4], u4 (&hi)[4]) {
+    asm volatile(
+        "global_load_dwordx4 %0, %8, off sc1\n\t"
+        "global_load_dwordx4 %1, %8, off offset:16 sc1\n\t"
+        "global_load_dwordx4 %2, %9, off sc1\n\t"
+        "global_load_dwordx4 %3, %9, off offset:16 sc1\n\t"
+        "global_load_dwordx4 %4, %10, off sc1\n\t"
+        "global_load_dwordx4 %5, %10, off offset:16 sc1\n\t"
+        "global_load_dwordx4 %6, %11, off sc1\n\t"
+        "global_load_dwordx4 %7, %11, off offset:16 sc1\n\t"
+        "s_waitcnt vmcnt(0)"
+        : "=&v"(lo[0]), "=&v"(hi[0]), "=&v"(lo[1]), "=&v"(hi[1]), "=&v"(lo[2]), "=&v"(hi[2]), "=&v"(lo[3]), "=&v"(hi[3])
+        : "v"(src[0]), "v"(src[1]), "v"(src[2]), "v"(src[3])
+        : "memory");
+}
+
 // kExtras: the table may hold SwiGLU pairs and RMSNorm prologues (a separate instance, so that plans
 // without them keep the register allocation of the plain kernel).
 // kFine: units of one tile per wave (16 rows for wide tiles) instead of kAhead, for launches
@@ -259,7 +306,11 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
     const int li = lane & 15;  // MFMA A row / D column
     const int lq = lane >> 4;  // MFMA k quarter / D row quad
 
+    // (Fine-grained wide tiles in units of 8 rows, where the waves share out the slices of two row blocks, were
+    // measured: a 4096 x 14336 matrix then spreads over twice the workgroups and every wave fetches half the tiles,
+    // but twice as many workgroups stage the 28 KB of activations, and a call takes the same time.)
     constexpr int kUnitRows = kNW * G::kRows * (kFine ? 1 : G::kAhead);
+    constexpr int kChunkStep = G::kRows * (kFine ? 1 : G::kAhead);  // a wave's share of a task's rows is a multiple of this
     int u = 0, u_end = 0, pi = 0;
     if (sc.table) {
         u = sc.wg_first[blockIdx.x];
@@ -283,15 +334,27 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
     // the flag of the stage barrier as this launch finds it (only thread 0 uses it): no workgroup can flip it before
     // every workgroup has read it here, because flipping takes the arrival of all of them
     int barrier_sense = 0;
-    if (kExtras && sc.n_stages > 1 && tid == 0) barrier_sense = __hip_atomic_load(sc.barrier, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (kExtras && sc.n_stages > 1 && !sc.exchange && tid == 0) barrier_sense = __hip_atomic_load(sc.barrier, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const int n_stages = kExtras && sc.n_stages > 0 ? sc.n_stages : 1;
     const bool staged = kExtras && sc.n_stages > 0;
+    const bool exchange = staged && sc.exchange != 0;
+    int epoch = 0;
+    if (exchange) epoch = sc.epochs[blockIdx.x];
+    const uint32_t tag_hi = (uint32_t)((epoch + 1) & 0xFFFF) << 16;
+    bool gave_up = false;  // a bounded wait of this workgroup expired (the same value in every thread)
     for (int stage = 0; stage < n_stages; stage++) {
+    bool from_record = false;  // the first task of the stage takes its problem and unit numbers from the record
+    int rec_first = 0, rec_units = 0;
+    Problem rec_p = single;
     if (staged) {
-        const int *spans = sc.wg_first + stage * (2 * (int)gridDim.x + 1);
-        u = spans[blockIdx.x];
-        u_end = spans[blockIdx.x + 1];
-        pi = spans[gridDim.x + 1 + blockIdx.x];
+        const WgStart &ws = sc.starts[(size_t)stage * gridDim.x + blockIdx.x];
+        u = ws.u;
+        u_end = ws.u_end;
+        pi = ws.pi;
+        rec_first = ws.first_unit;
+        rec_units = ws.p_units;
+        rec_p = ws.p;
+        from_record = true;
     }
     for (;;) {
         if (u >= u_end) {
@@ -307,17 +370,23 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
         }
         int first_unit = 0;
         int p_units = (single.rows + kUnitRows - 1) / kUnitRows;
-        if (sc.table) {
+        if (kExtras && from_record) {
+            first_unit = rec_first;
+            p_units = rec_units;
+        } else if (sc.table) {
             while (sc.unit_prefix[pi + 1] <= u) pi++;
             first_unit = sc.unit_prefix[pi];
             p_units = sc.unit_prefix[pi + 1] - first_unit;
         }
+        const bool with_record = kExtras && from_record;
+        from_record = false;
         const int n_units = min(min(u_end - u, first_unit + p_units - u), sc.max_units);
         const int task_first_row = (u - first_unit) * kUnitRows;
         u += n_units;
         const bool fresh = pi != cur;
         if (fresh) {
-            if (sc.table) p = sc.table[pi];
+            if (with_record) p = rec_p;
+            else if (sc.table) p = sc.table[pi];
             cur = pi;
             cur_seg = -1;
             words = p.cols / 32;
@@ -345,6 +414,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
             // (the list of outliers belongs to the whole row: it starts again with the row's first segment; the
             // barrier that ended the task before lies between its last reader and this write)
             if (seg == 0 && tid == 0) n_outliers = 0;
+            if (kExtras && tid == 0) stage_reached = 1;  // (a wave whose wait for tagged words expires clears it)
             __syncthreads();  // every wave is done with the image that was staged before
             cur_seg = seg;
             seg_lo = seg * seg_len;
@@ -518,29 +588,87 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
             if (n_seg == 1 && p.batch == 1 && pieces <= kKeep * kThreads) {
                 // one pass over x: all loads are issued together and kept for the image
                 uint4 keep[kKeep];
-                if (kExtras && staged && !sc.stage_fence) {
+                // RMSNorm prologue on a row of up to 8192 columns: the norm weights are asked for now, with (or before)
+                // the activations, not after the sum of squares: one round trip to memory less
+                uint4 early_w[kKeep / 2];
+                const bool early_norm = kExtras && p.norm_w != nullptr && pieces <= (kKeep / 2) * kThreads;
+                if (early_norm) {
+#pragma unroll
+                    for (int k = 0; k < kKeep / 2; k++) {
+                        const int c8 = stid + k * kThreads;
+                        early_w[k] = c8 < pieces ? norm_piece(c8) : uint4{0u, 0u, 0u, 0u};
+                    }
+                }
+                if (kExtras && exchange && p.x_words >= 0) {
+                    // The activations are the tagged words of an earlier stage: eight words per piece, asked for
+                    // again until all of this wave's carry the tag of this launch (four pieces at a time: 32
+                    // registers in flight). The fp16 bits are then packed into the piece as if loaded from x.
+                    const uint32_t *xw = sc.words + p.x_words;
+                    bool wave_ok = true;
+#pragma unroll
+                    for (int half = 0; half < 2; half++) {
+                        u4 lo[kKeep / 2], hi[kKeep / 2];
+                        for (int spins = 0;; spins++) {
+                            uint32_t bad = 0;
+                            const uint32_t *src[kKeep / 2];
+                            bool live[kKeep / 2];
+#pragma unroll
+                            for (int k = 0; k < kKeep / 2; k++) {
+                                const int c8 = stid + (half * (kKeep / 2) + k) * kThreads;
+                                const int slice = seg_lo + (c8 * 8) / G::kCols;
+                                const int chunk = ((c8 * 8) % G::kCols) / kChunkCols;
+                                const int g = min(slice * G::kChunks, groups - G::kChunks) + chunk;
+                                live[k] = c8 < pieces && g >= slice * G::kChunks;
+                                // (pieces that are not needed load the row's first words and count as zeros)
+                                src[k] = live[k] ? xw + g * kChunkCols + (c8 * 8) % kChunkCols : xw;
+                            }
+                            load4x8_words_device_scope(src, lo, hi);
+#pragma unroll
+                            for (int k = 0; k < kKeep / 2; k++) {
+                                if (!live[k]) lo[k] = hi[k] = u4{tag_hi, tag_hi, tag_hi, tag_hi};
+#pragma unroll
+                                for (int e = 0; e < 4; e++) bad |= (lo[k][e] ^ tag_hi) | (hi[k][e] ^ tag_hi);
+                            }
+                            if (__builtin_amdgcn_ballot_w64((bad >> 16) != 0) == 0) break;  // (uniform in the wave)
+                            if (spins >= sc.spin_limit ||
+                                ((spins & 15) == 15 && __hip_atomic_load(sc.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)) {
+                                wave_ok = false;
+                                break;
+                            }
+                            __builtin_amdgcn_s_sleep(2);
+                        }
+#pragma unroll
+                        for (int k = 0; k < kKeep / 2; k++)
+                            keep[half * (kKeep / 2) + k] = uint4{__builtin_amdgcn_perm(lo[k][1], lo[k][0], 0x05040100u),
+                                                                 __builtin_amdgcn_perm(lo[k][3], lo[k][2], 0x05040100u),
+                                                                 __builtin_amdgcn_perm(hi[k][1], hi[k][0], 0x05040100u),
+                                                                 __builtin_amdgcn_perm(hi[k][3], hi[k][2], 0x05040100u)};
+                        if (pieces <= (kKeep / 2) * kThreads) {  // (rows of up to 8192 columns: the second half holds nothing)
+#pragma unroll
+                            for (int k = kKeep / 2; k < kKeep; k++) keep[k] = uint4{0u, 0u, 0u, 0u};
+                            break;
+                        }
+                    }
+                    if (!wave_ok && lane == 0) stage_reached = 0;
+                } else if (kExtras && staged && !exchange && !sc.stage_fence) {
                     // The stage before wrote these activations, maybe on another XCD: loads of device scope fetch
-                    // memory's copy instead of a stale line of this XCD's cache. The compiler does not count loads it
-                    // cannot see, so the wait is written out; it names the registers, so that nothing reads them before.
+                    // memory's copy instead of a stale line of this XCD's cache.
                     u4 got[kKeep];
+                    const uint4 *src[kKeep];
+                    bool live[kKeep];
 #pragma unroll
                     for (int k = 0; k < kKeep; k++) {
                         const int c8 = stid + k * kThreads;
-                        got[k] = u4{0u, 0u, 0u, 0u};
                         const int slice = seg_lo + (c8 * 8) / G::kCols;
                         const int chunk = ((c8 * 8) % G::kCols) / kChunkCols;
                         const int g = min(slice * G::kChunks, groups - G::kChunks) + chunk;
-                        if (c8 < pieces && g >= slice * G::kChunks) {
-                            const uint4 *src = reinterpret_cast<const uint4 *>(p.x) + (g * kChunkCols + (c8 * 8) % kChunkCols) / 8;
-                            asm volatile("global_load_dwordx4 %0, %1, off sc1" : "+v"(got[k]) : "v"(src) : "memory");
-                        }
+                        live[k] = c8 < pieces && g >= slice * G::kChunks;
+                        // (pieces that are not needed load the row's first one and become zeros)
+                        src[k] = reinterpret_cast<const uint4 *>(p.x) + (live[k] ? (g * kChunkCols + (c8 * 8) % kChunkCols) / 8 : 0);
                     }
-                    asm volatile("s_waitcnt vmcnt(0)"
-                                 : "+v"(got[0]), "+v"(got[1]), "+v"(got[2]), "+v"(got[3]), "+v"(got[4]), "+v"(got[5]), "+v"(got[6]), "+v"(got[7])
-                                 :
-                                 : "memory");
+                    load8_device_scope(src, got);
 #pragma unroll
-                    for (int k = 0; k < kKeep; k++) keep[k] = uint4{got[k][0], got[k][1], got[k][2], got[k][3]};
+                    for (int k = 0; k < kKeep; k++) keep[k] = live[k] ? uint4{got[k][0], got[k][1], got[k][2], got[k][3]} : uint4{0u, 0u, 0u, 0u};
                 } else {
 #pragma unroll
                 for (int k = 0; k < kKeep; k++) {
@@ -575,11 +703,13 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                     // rarely run code below that of the tile loop
 #pragma unroll
                     for (int half = 0; half < 2; half++) {
+                        if (early_norm && half == 1) break;  // (nothing in the second half of the pieces)
                         uint4 wk[kKeep / 2];
 #pragma unroll
                         for (int k = 0; k < kKeep / 2; k++) {
                             const int c8 = stid + (half * (kKeep / 2) + k) * kThreads;
-                            wk[k] = c8 < pieces ? norm_piece(c8) : uint4{0u, 0u, 0u, 0u};
+                            if (early_norm) wk[k] = early_w[k];
+                            else wk[k] = c8 < pieces ? norm_piece(c8) : uint4{0u, 0u, 0u, 0u};
                         }
 #pragma unroll
                         for (int k = 0; k < kKeep / 2; k++) {
@@ -660,6 +790,10 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                 }
             }
             __syncthreads();
+            if (kExtras && exchange && !stage_reached) {  // (the same in every thread: read behind the barrier)
+                gave_up = true;
+                break;
+            }
         }
 
         // The task's rows are cut into kNW chunks; a "walk" is one chunk under one slice (the B
@@ -668,13 +802,20 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
         // slices of the same rows: the cache lines of a row (masks and, above all, the 2-byte
         // scales) are fetched from HBM once and shared, not once per slice.
         // chunk size: a quarter of the rows that exist, rounded up to whole groups of G::kAhead tiles
-        const int chunk_rows = ((r_end - r_begin + kNW - 1) / kNW + kUnitRows / kNW - 1) / (kUnitRows / kNW) * (kUnitRows / kNW);
+        const int chunk_rows = ((r_end - r_begin + kNW - 1) / kNW + kChunkStep - 1) / kChunkStep * kChunkStep;
         const int n_walks = kNW * seg_n;
         const int my_walks = seg_n;  // walks wave, wave + kNW, ...
+        // fine-grained instances: only the walks of chunks that have rows (the first ones of every wave)
+        const int live_walks = (r_end - r_begin + chunk_rows - 1) / chunk_rows * seg_n;
+        const int my_live = max(0, (live_walks - wave + kNW - 1) / kNW);
+        const int park_walk = kFine ? wave + (max(my_live, 1) - 1) * kNW : n_walks - kNW + wave;
         // A SwiGLU pair (flag on the gate problem; the up problem follows it in the table, same shape
         // and activations, no units of its own) runs the walks twice over the same rows, with the same
         // operand image, into two partial-sum areas; the epilogue below joins them.
-        for (int mat = 0; mat < (pair ? 2 : 1); mat++) {
+        // (The fine-grained instance that knows pairs takes both matrices in ONE pass, below: the tiles of gate and
+        // up travel through the same ring, so a unit's four tiles at K = 4096 are one round trip to memory, not two.)
+        constexpr bool kBothInOnePass = kFine && kExtras && G::kRows == 4;
+        for (int mat = 0; mat < (pair && !kBothInOnePass ? 2 : 1); mat++) {
         const uint32_t *w_nz = p.nz, *w_sg = p.sg;
         const uint16_t *w_sc = p.scales;
         if (mat == 1) {
@@ -757,7 +898,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
             int l_walk = wave, l_slot = 0;
             auto next_load = [&]() -> Tile<G> {
                 // past the last walk the cursor parks on the wave's last tile
-                const int w_ = min(l_walk, n_walks - kNW + wave);
+                const int w_ = min(l_walk, park_walk);
                 const int c = w_ / seg_n, sl = w_ - c * seg_n;
                 const int live_tiles = max(chunk_tiles(c), 1);
                 const Tile<G> t = load_tile(sl, r_begin + c * chunk_rows + min(l_slot, live_tiles - 1) * G::kRows);
@@ -765,10 +906,12 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                 return t;
             };
             Tile<G> ring[G::kAhead];
+            if constexpr (!kBothInOnePass) {
 #pragma unroll
-            for (int k = 0; k < G::kAhead; k++) {
-                ring[k] = next_load();
-                __builtin_amdgcn_sched_barrier(0);  // same issue order as in the loop below
+                for (int k = 0; k < G::kAhead; k++) {
+                    ring[k] = next_load();
+                    __builtin_amdgcn_sched_barrier(0);  // same issue order as in the loop below
+                }
             }
 
             const u4 zero4 = {0u, 0u, 0u, 0u};
@@ -849,13 +992,80 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                                             lane_select(bias[2], bias[3], odd_lanes), hi_lanes);
                 bias = bias * gf;
             };
-            if constexpr (kFine) {
+            if constexpr (kBothInOnePass) {
+                // One flat sequence of (walk, matrix, slot) triples through a ring of four tiles. Per matrix the
+                // tiles come in the order of the two-pass form, so every partial sum adds up in the same order;
+                // the B operands of a walk serve both matrices.
+                constexpr int kRing = 4;
+                const int n_mats = pair ? 2 : 1;
+                const char GB *bases[2][3] = {{nz_g, sg_g, sc_g}, {nz_g, sg_g, sc_g}};
+                if (pair) {
+                    bases[1][0] = reinterpret_cast<const char GB *>(as_global(sc.table[pi + 1].nz));
+                    bases[1][1] = reinterpret_cast<const char GB *>(as_global(sc.table[pi + 1].sg));
+                    bases[1][2] = reinterpret_cast<const char GB *>(as_global(sc.table[pi + 1].scales));
+                }
+                float *const part0 = my_part;
+                int lw = wave, lm = 0, ls = 0;  // load cursor; past the last walk it parks on the wave's last walk
+                auto next_of_both = [&]() -> Tile<G> {
+                    const int w_ = min(lw, park_walk);
+                    const int c = w_ / seg_n, sl = w_ - c * seg_n;
+                    const int live_tiles = max(chunk_tiles(c), 1);
+                    nz_g = bases[lm][0];
+                    sg_g = bases[lm][1];
+                    sc_g = bases[lm][2];
+                    const Tile<G> t = load_tile(sl, r_begin + c * chunk_rows + min(ls, live_tiles - 1) * G::kRows);
+                    if (++ls == n_slots) {
+                        ls = 0;
+                        if (++lm == n_mats) {
+                            lm = 0;
+                            lw += kNW;
+                        }
+                    }
+                    return t;
+                };
+                Tile<G> ring4[kRing];
+#pragma unroll
+                for (int k = 0; k < kRing; k++) {
+                    ring4[k] = next_of_both();
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                u4 B[kMfmaPerTile];
+                f4 bias;
+                float bias_sel = 0.0f, gf = 0.0f;
+                int wi = 0, m = 0, j = 0, c_begin = 0, n_rb = 0;
+                const int total = my_live * n_mats * n_slots;
+                for (int t0 = 0; t0 < total; t0 += kRing) {
+#pragma unroll
+                    for (int k = 0; k < kRing; k++) {
+                        if (t0 + k < total) {
+                            if (j == 0 && m == 0) {
+                                const int walk = wave + wi * kNW;
+                                const int chunk = walk / seg_n, slice = walk - chunk * seg_n;
+                                c_begin = r_begin + chunk * chunk_rows;
+                                n_rb = chunk_tiles(chunk);
+                                load_operands(slice, B, bias, bias_sel, gf);
+                            }
+                            my_part = part0 + (size_t)m * sc.pair_stride;
+                            process_tile(ring4[k], c_begin + min(j, max(n_rb, 1) - 1) * G::kRows, j < n_rb, B, bias, bias_sel, gf);
+                            if (++j == n_slots) {
+                                j = 0;
+                                if (++m == n_mats) {
+                                    m = 0;
+                                    wi++;
+                                }
+                            }
+                        }
+                        ring4[k] = next_of_both();
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            } else if constexpr (kFine) {
                 // one flat sequence of (walk, slot) pairs, three at a time through the ring
                 u4 B[kMfmaPerTile];
                 f4 bias;
                 float bias_sel = 0.0f, gf = 0.0f;
                 int wi = 0, j = 0, c_begin = 0, n_rb = 0;
-                const int total = my_walks * n_slots;
+                const int total = my_live * n_slots;
                 for (int t0 = 0; t0 < total; t0 += G::kAhead) {
 #pragma unroll
                     for (int k = 0; k < G::kAhead; k++) {
@@ -907,6 +1117,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
         }
         }  // matrices of the task
         }  // segments of the row
+        if (kExtras && gave_up) break;
         // last task of the span, or a pool task: ask for the next pool task now (not earlier: a
         // request is a claim, and a workgroup must not claim work long before it can start it); the
         // answer arrives while the partial sums are added up
@@ -957,7 +1168,27 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                     // the reference's add_forward behind the projection (src/transformer.cpp:247-250, 293-296): one
                     // correctly rounded fp16 add of the residual stream and the fp16-rounded projection
                     // (a load of device scope: an earlier stage may have written the residual stream)
-                    const _Float16 res = __builtin_bit_cast(_Float16, __hip_atomic_load(p.residual + r_begin + rl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+                    uint16_t res_bits;
+                    if (exchange && p.res_words >= 0) {
+                        // the tagged word of the stage that wrote the residual stream (it has arrived long ago when the
+                        // stages in between have run; the wait is bounded all the same)
+                        uint32_t w = 0;
+                        for (int spins = 0;; spins++) {
+                            w = __hip_atomic_load(sc.words + p.res_words + r_begin + rl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            if (((w ^ tag_hi) >> 16) == 0) break;
+                            if (spins >= sc.spin_limit) {
+                                __hip_atomic_store(sc.status, stage + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                                break;
+                            }
+                            __builtin_amdgcn_s_sleep(2);
+                        }
+                        res_bits = (uint16_t)w;
+                    } else if (exchange) {
+                        res_bits = p.residual[r_begin + rl];  // (nothing in the plan writes it, or only this row's own store below)
+                    } else {
+                        res_bits = __hip_atomic_load(p.residual + r_begin + rl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                    const _Float16 res = __builtin_bit_cast(_Float16, res_bits);
                     out = __builtin_bit_cast(uint16_t, (_Float16)(res + __builtin_bit_cast(_Float16, out)));
                 }
                 uint16_t *dst = p.y + (size_t)b * p.rows + r_begin + rl;
@@ -965,12 +1196,24 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                 // XCD they run on)
                 if (staged) __hip_atomic_store(dst, out, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 else *dst = out;
+                if (exchange && p.y_words >= 0) {
+                    // (a later stage stores to y as well: this store has reached memory before any workgroup can know
+                    // that the stage is complete, so the two stores cannot arrive in the wrong order)
+                    if (p.flags & kProblemOrderedStore) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    __hip_atomic_store(sc.words + p.y_words + r_begin + rl, (uint32_t)out | tag_hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
             }
         }
         if (request) pool_task = requested;
         __syncthreads();
     }
-    if (staged && stage + 1 < n_stages) {
+    if (kExtras && gave_up) {
+        if (tid == 0) __hip_atomic_store(sc.status, stage + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        break;
+    }
+    if (exchange) {
+        cur = -1;  // (the next stage waits for its own activations where it stages them)
+    } else if (staged && stage + 1 < n_stages) {
         // ---- between two stages: every output of this workgroup's span has reached memory, then count and wait
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
@@ -1016,6 +1259,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
         cur = -1;
     }
     }  // stages
+    if (exchange && tid == 0) sc.epochs[blockIdx.x] = epoch + 1;
     if (sc.pool_count != 0 && tid == 0) {
         const int left = __hip_atomic_fetch_add(sc.counters + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (left == (int)gridDim.x - 1) {  // every other workgroup has made its last request
@@ -1636,12 +1880,123 @@ hipError_t plan_device_create_staged(const std::vector<Problem> &host, PlanDevic
         }
     }
 
+    // Hand-over by tagged words (see Sched::exchange) where the plan allows: rows that the one-pass staging holds in
+    // registers, nothing quantised inside the launch, and buffers that relate in the plain ways: an input or residual
+    // is either exactly the output of an earlier stage (then it is read from that problem's words; the latest such
+    // stage counts) or touches no output of the plan (a residual may be its own problem's output: in place); two
+    // outputs are either the same buffer in different stages (the earlier store is then completed first) or apart.
+    std::vector<Problem> table(host);
+    size_t n_words = 0;
+    bool exchange = tuning().stage_exchange.load(std::memory_order_relaxed) != 0 && !d.stage_fence && d.n_stages > 1;
+    {
+        auto lo = [](const void *q) { return reinterpret_cast<uintptr_t>(q); };
+        auto cross = [&](const void *a, size_t na, const void *b, size_t nb) { return lo(a) < lo(b) + nb && lo(b) < lo(a) + na; };
+        for (Problem &p : table) p.x_words = p.res_words = p.y_words = -1, p.pad_ = 0;
+        // the producer of a buffer of `count` halfwords for a reader in stage `st`: -1 none, -2 the buffer relates
+        // to some output in a way the words cannot serve
+        auto producer_of = [&](const uint16_t *buf, int count, int st, int self) -> int {
+            int best = -1;
+            for (int j = 0; j < n && best != -2; j++) {
+                if (is_up(j) || j == self) continue;
+                const Problem &w = host[j];
+                if (!cross(buf, (size_t)count * 2, w.y, (size_t)w.rows * 2)) continue;
+                if (buf == w.y && count == w.rows) {
+                    if (w.stage < st && (best < 0 || host[best].stage <= w.stage)) best = j;
+                    else if (w.stage == st) best = -2;  // written and read in one stage
+                } else {
+                    best = -2;
+                }
+            }
+            return best;
+        };
+        for (int i = 0; i < n && exchange; i++) {
+            Problem &p = table[i];
+            const int src = producer_of(p.x, p.cols, p.stage, -1);
+            if (src == -2) exchange = false;
+            else if (src >= 0) p.x_words = src;  // (the producer's index for now; its words are numbered below)
+            if (p.residual) {
+                const bool in_place = p.residual == p.y;
+                const int r = producer_of(p.residual, p.rows, p.stage, in_place ? i : -1);
+                if (r == -2) exchange = false;
+                else if (r >= 0) p.res_words = r;
+            }
+            for (int j = 0; j < i && exchange; j++) {
+                if (is_up(i) || is_up(j) || !cross(p.y, (size_t)p.rows * 2, host[j].y, (size_t)host[j].rows * 2)) continue;
+                if (p.y == host[j].y && p.rows == host[j].rows && host[j].stage < p.stage) table[j].flags |= kProblemOrderedStore;
+                else exchange = false;
+            }
+        }
+        // Without barriers only data orders the stages: a problem may overwrite a buffer that an earlier stage's
+        // problem reads as it is (or has written) only if it comes after that problem by a chain of hand-overs.
+        if (exchange && n > 64) exchange = false;
+        if (exchange) {
+            std::vector<uint64_t> after(n, 0);  // bit j: problem i starts after problem j has stored all its outputs
+            for (int i = 0; i < n; i++)
+                for (int which = 0; which < 2; which++) {
+                    int j = which ? table[i].res_words : table[i].x_words;
+                    if (j < 0) continue;
+                    after[i] |= (uint64_t)1 << j | after[j];
+                    if (host[j].flags & kProblemSwigluGate) after[i] |= (uint64_t)1 << (j + 1);  // (the pair's up half)
+                }
+            for (int i = 0; i < n && exchange; i++) {
+                if (is_up(i)) continue;
+                const Problem &w = host[i];
+                for (int j = 0; j < n && exchange; j++) {
+                    if (j == i || host[j].stage >= w.stage) continue;
+                    const Problem &r = host[j];
+                    const bool reads_x = table[j].x_words < 0 && cross(w.y, (size_t)w.rows * 2, r.x, (size_t)r.cols * 2);
+                    const bool reads_res = r.residual && table[j].res_words < 0 && cross(w.y, (size_t)w.rows * 2, r.residual, (size_t)r.rows * 2);
+                    const bool wrote = !is_up(j) && cross(w.y, (size_t)w.rows * 2, r.y, (size_t)r.rows * 2);
+                    if ((reads_x || reads_res || wrote) && !(after[i] >> j & 1)) exchange = false;
+                }
+            }
+        }
+        if (exchange) {
+            std::vector<int> first_word(n, -1);
+            for (int i = 0; i < n; i++)
+                for (int which = 0; which < 2; which++) {
+                    const int j = which ? table[i].res_words : table[i].x_words;
+                    if (j >= 0 && first_word[j] < 0) {
+                        first_word[j] = (int)n_words;
+                        n_words += ((size_t)host[j].rows + 31) / 32 * 32;
+                    }
+                }
+            for (int i = 0; i < n; i++) {
+                if (table[i].x_words >= 0) table[i].x_words = first_word[table[i].x_words];
+                if (table[i].res_words >= 0) table[i].res_words = first_word[table[i].res_words];
+                table[i].y_words = first_word[i];
+            }
+        } else {
+            for (Problem &p : table) p.x_words = p.res_words = p.y_words = -1, p.pad_ = 0, p.flags &= ~kProblemOrderedStore;
+        }
+    }
+    d.exchange = exchange;
+    d.words_per_slot = n_words;
+    d.ints_per_slot = n_words + (size_t)grid;
+    // what every workgroup starts every stage with (spans: per stage [grid + 1] first units, then [grid] problems)
+    std::vector<WgStart> starts((size_t)d.n_stages * grid);
+    for (int st = 0; st < d.n_stages; st++) {
+        const int *first = spans.data() + (size_t)st * (2 * grid + 1);
+        for (int g = 0; g < grid; g++) {
+            WgStart &ws = starts[(size_t)st * grid + g];
+            ws = WgStart{};
+            ws.u = first[g];
+            ws.u_end = first[g + 1];
+            ws.pi = first[grid + 1 + g];
+            ws.first_unit = prefix[ws.pi];
+            ws.p_units = prefix[ws.pi + 1] - prefix[ws.pi];
+            ws.p = table[ws.pi];
+        }
+    }
+
     auto round16 = [](size_t v) { return (v + 15) / 16 * 16; };
     const size_t bytes_table = round16(sizeof(Problem) * n), bytes_prefix = round16(sizeof(int) * prefix.size());
     const size_t bytes_spans = round16(sizeof(int) * spans.size());
     const size_t bytes_counters = round16(sizeof(int) * (32 + kPlanSlots * kBarrierInts + 32)) + 128;
+    const size_t bytes_words = exchange ? (size_t)kPlanSlots * d.ints_per_slot * 4 + 128 : 0;
+    const size_t bytes_starts = sizeof(WgStart) * starts.size() + 128;
     char *base = nullptr;
-    if (hipError_t e = hipMalloc(&base, bytes_table + bytes_prefix + bytes_spans + bytes_counters)) return e;
+    if (hipError_t e = hipMalloc(&base, bytes_table + bytes_prefix + bytes_spans + bytes_counters + bytes_words + bytes_starts)) return e;
     d.problems = reinterpret_cast<Problem *>(base);
     d.unit_prefix = reinterpret_cast<int *>(base + bytes_table);
     d.wg_first = reinterpret_cast<int *>(base + bytes_table + bytes_prefix);
@@ -1652,10 +2007,18 @@ hipError_t plan_device_create_staged(const std::vector<Problem> &host, PlanDevic
     d.barrier_bytes = sizeof(int) * ((size_t)kPlanSlots * kBarrierInts + 1);
     // a poll is an uncached load and a short sleep, a microsecond or two: the wait gives up after about a second
     d.spin_limit = 500000;
-    hipError_t e = hipMemcpy(d.problems, host.data(), sizeof(Problem) * n, hipMemcpyHostToDevice);
+    if (exchange) {
+        // the words of all launch slots (each on a 128-byte line), then every slot's launch counts
+        char *w0 = reinterpret_cast<char *>((reinterpret_cast<uintptr_t>(base + bytes_table + bytes_prefix + bytes_spans + bytes_counters) + 127) / 128 * 128);
+        d.words = reinterpret_cast<uint32_t *>(w0);
+    }
+    d.starts = reinterpret_cast<WgStart *>((reinterpret_cast<uintptr_t>(base + bytes_table + bytes_prefix + bytes_spans + bytes_counters + bytes_words) + 127) / 128 * 128);
+    hipError_t e = hipMemcpy(d.problems, table.data(), sizeof(Problem) * n, hipMemcpyHostToDevice);
+    if (!e) e = hipMemcpy(d.starts, starts.data(), sizeof(WgStart) * starts.size(), hipMemcpyHostToDevice);
     if (!e) e = hipMemcpy(d.unit_prefix, prefix.data(), sizeof(int) * prefix.size(), hipMemcpyHostToDevice);
     if (!e) e = hipMemcpy(d.wg_first, spans.data(), sizeof(int) * spans.size(), hipMemcpyHostToDevice);
     if (!e) e = hipMemset(d.counters, 0, bytes_counters);
+    if (!e && exchange) e = hipMemset(d.words, 0, (size_t)kPlanSlots * d.ints_per_slot * 4);
     d.next_slot = new (std::nothrow) std::atomic<unsigned>(0);
     if (!e && !d.next_slot) e = hipErrorOutOfMemory;
     if (e) {
@@ -1699,6 +2062,12 @@ hipError_t plan_device_launch(const PlanDevice &plan, hipStream_t s) {
         sc.status = plan.status;
         const int limit = tuning().stage_spin_limit.load(std::memory_order_relaxed);
         sc.spin_limit = limit > 0 ? limit : plan.spin_limit;
+        sc.starts = plan.starts;
+        if (plan.exchange) {
+            sc.exchange = 1;
+            sc.words = plan.words + (size_t)slot * plan.ints_per_slot;
+            sc.epochs = reinterpret_cast<int *>(sc.words + plan.words_per_slot);
+        }
     }
     Problem none{};
     if (plan.extras && plan.fine)

@@ -1775,12 +1775,16 @@ def _chain_staged(torch, tl, w, xs, att, hbuf, q, k, v, h, qd, kvd, ffn, eps):
     return tl.LinearPlan(probs, norm_weights=norms, eps=eps, stages=[0, 1, 1, 2, 3, 3, 3], residuals=residuals)
 
 
+@pytest.mark.parametrize("handover", ["words", "barriers"])
 @pytest.mark.parametrize("h,qd,kvd,ffn", [(4096, 4096, 1024, 14336), (2048, 2048, 512, 8192), (2048, 2304, 256, 5632)])
-def test_staged_plan_equals_the_separate_launches(dev, oracle, h, qd, kvd, ffn):
+def test_staged_plan_equals_the_separate_launches(dev, oracle, tuned, h, qd, kvd, ffn, handover):
     """o_proj (+ residual) -> RMSNorm, gate/up, SiLU * up -> down_proj (+ residual) -> RMSNorm, q/k/v of the next
     layer as ONE launch with waits between the stages: the residual stream, the FFN activation and q, k, v hold the
-    bits of the twelve separate launches, launch after launch; the projection rows are within the bar of the oracle."""
+    bits of the twelve separate launches, launch after launch; the projection rows are within the bar of the oracle.
+    Both ways of handing results from stage to stage: tagged words that the next stage polls (the residual stream is
+    updated in place twice, as the reference does), and barriers."""
     torch, tl = dev
+    tuned(stage_exchange=1 if handover == "words" else 0)
     gen = torch.Generator(device="cuda")
     gen.manual_seed(h + ffn)
     eps = 1e-5
@@ -1792,7 +1796,7 @@ def test_staged_plan_equals_the_separate_launches(dev, oracle, h, qd, kvd, ffn):
     xs, hbuf = x.clone(), torch.full((1, ffn), float("nan"), **f16)
     q, k, v = torch.full((1, qd), float("nan"), **f16), torch.full((1, kvd), float("nan"), **f16), torch.full((1, kvd), float("nan"), **f16)
     plan = _chain_staged(torch, tl, w, xs, att, hbuf, q, k, v, h, qd, kvd, ffn, eps)
-    assert "staged" in plan.kernel
+    assert "staged" in plan.kernel and ("tagged words" if handover == "words" else "barriers") in plan.kernel
     for launch in range(3):
         xs.copy_(x)
         for t in (hbuf, q, k, v):
@@ -1815,10 +1819,13 @@ def test_staged_plan_equals_the_separate_launches(dev, oracle, h, qd, kvd, ffn):
     plan2.close()
 
 
-def test_staged_plan_in_a_captured_graph_and_on_a_second_stream(dev, oracle):
-    """The staged launch under graph capture (no allocation, counters that reset themselves): replays, with eager
-    launches of the same plan on another stream between them, give the eager bits every time."""
+@pytest.mark.parametrize("handover", ["words", "barriers"])
+def test_staged_plan_in_a_captured_graph_and_on_a_second_stream(dev, oracle, tuned, handover):
+    """The staged launch under graph capture (no allocation, counters that reset themselves, tags that every
+    workgroup advances by itself): replays, with eager launches of the same plan on another stream between them, give
+    the eager bits every time."""
     torch, tl = dev
+    tuned(stage_exchange=1 if handover == "words" else 0)
     h, qd, kvd, ffn, eps = 2048, 2048, 512, 8192, 1e-5
     gen = torch.Generator(device="cuda")
     gen.manual_seed(31)
@@ -1857,11 +1864,13 @@ def test_staged_plan_in_a_captured_graph_and_on_a_second_stream(dev, oracle):
     plan.close()
 
 
-def test_staged_plan_wait_that_expires_is_reported(dev, oracle, tuned):
+@pytest.mark.parametrize("handover", ["words", "barriers"])
+def test_staged_plan_wait_that_expires_is_reported(dev, oracle, tuned, handover):
     """A wait between two stages is bounded: with the bound forced down to one poll (tuning switch) the workgroups
     that arrive early give up, every workgroup ends normally, tllm_linear_plan_status reports the timeout once, and
     the next launch with the ordinary bound is complete and correct."""
     torch, tl = dev
+    tuned(stage_exchange=1 if handover == "words" else 0)
     h, qd, kvd, ffn, eps = 2048, 2048, 512, 8192, 1e-5
     gen = torch.Generator(device="cuda")
     gen.manual_seed(32)

@@ -128,7 +128,7 @@ struct Sched {
     int exchange;
     uint32_t *words;
     int *epochs;
-    const WgStart *starts;  // staged plans: [n_stages * grid] what each workgroup starts each stage with
+    const WgStart *starts;  // plans: [grid] (staged plans: [n_stages * grid]) what each workgroup starts (each stage) with
 };
 // Layout of a stage barrier, in ints: [0] the flag, [32] the top counter, [64 + 32 g] the counter of group g: every
 // word that takes atomics from many workgroups sits on a 128-byte line of its own.
@@ -313,9 +313,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
     constexpr int kChunkStep = G::kRows * (kFine ? 1 : G::kAhead);  // a wave's share of a task's rows is a multiple of this
     int u = 0, u_end = 0, pi = 0;
     if (sc.table) {
-        u = sc.wg_first[blockIdx.x];
-        u_end = sc.wg_first[blockIdx.x + 1];
-        pi = sc.wg_first[gridDim.x + 1 + blockIdx.x];  // no scan over the problems before this span
+        // (plans: the span, its place among the units and the problem come in one record, below)
     } else {
         const int total = (single.rows + kUnitRows - 1) / kUnitRows;
         u = (int)((int64_t)total * blockIdx.x / gridDim.x);
@@ -346,7 +344,8 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
     bool from_record = false;  // the first task of the stage takes its problem and unit numbers from the record
     int rec_first = 0, rec_units = 0;
     Problem rec_p = single;
-    if (staged) {
+    if (sc.table) {
+        // one round trip to memory instead of three dependent ones (the span, the unit prefix around it, the problem)
         const WgStart &ws = sc.starts[(size_t)stage * gridDim.x + blockIdx.x];
         u = ws.u;
         u_end = ws.u_end;
@@ -370,7 +369,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
         }
         int first_unit = 0;
         int p_units = (single.rows + kUnitRows - 1) / kUnitRows;
-        if (kExtras && from_record) {
+        if (from_record) {
             first_unit = rec_first;
             p_units = rec_units;
         } else if (sc.table) {
@@ -378,7 +377,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
             first_unit = sc.unit_prefix[pi];
             p_units = sc.unit_prefix[pi + 1] - first_unit;
         }
-        const bool with_record = kExtras && from_record;
+        const bool with_record = from_record;
         from_record = false;
         const int n_units = min(min(u_end - u, first_unit + p_units - u), sc.max_units);
         const int task_first_row = (u - first_unit) * kUnitRows;
@@ -508,18 +507,31 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                 }
                 return m;
             };
+            // Where the eight elements of a piece go inside their (slice, chunk) and what power of two they take
+            // depends on the piece's place in its 128-column chunk, which is the same for every piece a thread
+            // handles (a thread's pieces are a multiple of 16 pieces apart): worked out once per staging, not per
+            // element (a row of 14336 columns is seven pieces per thread).
+            int el_at[8], el_exp[8];
+            {
+                int t16 = tid & 15;
+                asm volatile("" : "+v"(t16));  // (keeps these sixteen values out of the registers of the tile loop)
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const OperandSlot s = chunk_slot(t16 * 8 + e);
+                    el_at[e] = image_index(s.t, 0, s.e, G::kChunks);
+                    el_exp[e] = 127 + 14 - s.p;
+                }
+            }
             auto write_piece = [&](uint16_t *img, int c8, const uint4 &v, int ex) {
                 const int slice = (c8 * 8) / G::kCols;
                 const int chunk = ((c8 * 8) % G::kCols) / kChunkCols;
-                const int cc0 = (c8 * 8) % kChunkCols;
                 const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
-                uint16_t *dst = img + slice * G::kCols;
+                uint16_t *dst = img + slice * G::kCols + chunk * 8;
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
-                    const OperandSlot s = chunk_slot(cc0 + e);
-                    const float mult = __builtin_bit_cast(float, (uint32_t)(127 + 14 - ex - s.p) << 23);
+                    const float mult = __builtin_bit_cast(float, (uint32_t)(el_exp[e] - ex) << 23);
                     const uint16_t hx = (uint16_t)(w4[e >> 1] >> (16 * (e & 1)));
-                    dst[image_index(s.t, chunk, s.e, G::kChunks)] = f2h(h2f(hx) * mult);
+                    dst[el_at[e]] = f2h(h2f(hx) * mult);
                 }
             };
             // One piece into the image. The 16 pieces of a 128-column group are held by 16 neighbouring threads
@@ -1764,8 +1776,24 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
     const size_t bytes_prefix = round16(sizeof(int) * prefix.size());
     const size_t bytes_wg = round16(sizeof(int) * wg_first.size());
     const size_t bytes_pool = round16(sizeof(int) * pool_first.size());
+    // what every workgroup of the MFMA kernel starts with (wg_first: [grid + 1] first units, then [grid] problems)
+    std::vector<WgStart> starts;
+    if (d.use_mfma && !d.batch_kernel) {
+        starts.resize(d.grid);
+        for (int g = 0; g < d.grid; g++) {
+            WgStart &ws = starts[g];
+            ws = WgStart{};
+            ws.u = wg_first[g];
+            ws.u_end = wg_first[g + 1];
+            ws.pi = wg_first[d.grid + 1 + g];
+            ws.first_unit = prefix[ws.pi];
+            ws.p_units = prefix[ws.pi + 1] - prefix[ws.pi];
+            ws.p = ordered[ws.pi];
+        }
+    }
+    const size_t bytes_starts = starts.empty() ? 0 : sizeof(WgStart) * starts.size() + 128;
     char *base = nullptr;
-    if (hipError_t e = hipMalloc(&base, bytes_table + bytes_prefix + bytes_wg + bytes_pool + 8 * kPlanSlots)) return e;
+    if (hipError_t e = hipMalloc(&base, bytes_table + bytes_prefix + bytes_wg + bytes_pool + round16(8 * kPlanSlots) + bytes_starts)) return e;
     d.problems = reinterpret_cast<Problem *>(base);
     d.unit_prefix = reinterpret_cast<int *>(base + bytes_table);
     d.wg_first = reinterpret_cast<int *>(base + bytes_table + bytes_prefix);
@@ -1778,6 +1806,10 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
     if (!e && !pool_first.empty())
         e = hipMemcpy(d.pool_first, pool_first.data(), sizeof(int) * pool_first.size(), hipMemcpyHostToDevice);
     if (!e) e = hipMemset(d.counters, 0, 8 * kPlanSlots);
+    if (!e && !starts.empty()) {
+        d.starts = reinterpret_cast<WgStart *>((reinterpret_cast<uintptr_t>(d.counters) + round16(8 * kPlanSlots) + 127) / 128 * 128);
+        e = hipMemcpy(d.starts, starts.data(), sizeof(WgStart) * starts.size(), hipMemcpyHostToDevice);
+    }
     d.next_slot = new (std::nothrow) std::atomic<unsigned>(0);
     if (!e && !d.next_slot) e = hipErrorOutOfMemory;
     if (e) {
@@ -2055,6 +2087,7 @@ hipError_t plan_device_launch(const PlanDevice &plan, hipStream_t s) {
     sc.max_units = plan.max_units;
     sc.max_batch = plan.max_batch;
     sc.image_bytes = plan.image_bytes;
+    sc.starts = plan.starts;
     if (plan.n_stages > 0) {
         sc.n_stages = plan.n_stages;
         sc.barrier = plan.stage_counters + slot * kBarrierInts;
@@ -2062,7 +2095,6 @@ hipError_t plan_device_launch(const PlanDevice &plan, hipStream_t s) {
         sc.status = plan.status;
         const int limit = tuning().stage_spin_limit.load(std::memory_order_relaxed);
         sc.spin_limit = limit > 0 ? limit : plan.spin_limit;
-        sc.starts = plan.starts;
         if (plan.exchange) {
             sc.exchange = 1;
             sc.words = plan.words + (size_t)slot * plan.ints_per_slot;

@@ -301,9 +301,21 @@ int tllm_linear_plan_create_i8(tllm_linear_plan **plan, const tllm_linear_proble
 /*
  * A plan whose problems DEPEND on each other, run in stages inside ONE launch: stages[i] (HOST array, ascending from 0,
  * at most 8 stages) says after which problems problem i runs; the problems of one stage are independent, and every
- * problem of stage s + 1 may read what stage s stored. Between two stages the workgroups of the launch wait for each
- * other at a counter in device memory instead of ending the kernel, which saves the start, the drain and the launch gap
- * of a kernel per stage. Replaces the dependent launches of a decode step, reference src/transformer.cpp:239-296, e.g.
+ * problem of stage s + 1 may read what stage s stored. The kernel does not end between two stages. How a stage gets
+ * the results of the stage before, chosen when the plan is created:
+ *   - as tagged words (the usual case): a problem whose output a later stage reads also stores every output row as a
+ *     32-bit word (fp16 bits and a tag of the launch) in memory the plan owns; the workgroups that need it poll those
+ *     words and take the values from them, so each waits for exactly the data it needs. This needs buffers that
+ *     relate plainly: an input or residual is either exactly one earlier stage's output (same pointer, same length)
+ *     or touches no output of the plan (a residual may be its own problem's output: in place); two outputs are
+ *     either the same buffer in different stages (the reference's residual stream, updated in place twice) or do
+ *     not overlap; a buffer that a later stage overwrites is only overwritten by a problem that depends, through
+ *     such hand-overs, on every problem that reads or writes it earlier; rows of at most 16384 columns, no
+ *     TLLM_PROBLEM_QUANTIZE_INPUT, at most 64 problems.
+ *   - otherwise at a barrier in device memory between every two stages (counters, bounded polling), after which
+ *     the outputs of the stage before are read from memory, not from a stale cache line.
+ * tllm_linear_plan_kernel names the way a plan runs. Either way the launches of a decode step that depend on each
+ * other become one, reference src/transformer.cpp:239-296, e.g.
  *   stage 0  o_proj, residuals[0] = the residual stream (output = stream + projection, in place allowed)
  *   stage 1  gate / up as a SwiGLU pair with norm_weights = the FFN norm: reads the stream through RMSNorm
  *   stage 2  down_proj on the pair's output, residuals = the stream again
@@ -356,7 +368,9 @@ int tllm_read_stream(const void *src, size_t bytes, uint32_t *sink, tllm_stream_
  * TLLM_TALL_MIN_SHARE, TLLM_READ_SHAPE) when the library first needs one; no operator call reads the environment.
  * These two calls change and read them afterwards, by name: "gemm_path" (0 cost model, 1 prefill GEMM, 2 passes of
  * the decode kernel), "gemm_rowsplit" (-1 cost model, 0 never, 1 or 2 forced), "batch_k_parts", "tall_max_batch",
- * "tall_min_share_milli", "stage_spin_limit", "read_wgs_per_cu", "read_in_flight". An unknown name returns
+ * "tall_min_share_milli", "stage_spin_limit" (polls a staged plan waits; 0: about a second), "stage_exchange" (read when
+ * a staged plan is created: 0 makes it wait at barriers even where tagged words would do), "read_wgs_per_cu",
+ * "read_in_flight". An unknown name returns
  * TLLM_ERR_BAD_SHAPE. Results never depend on them beyond the order of fp32 additions. Not for concurrent use
  * with operator calls whose choice should be stable. No counterpart in the reference.
  */

@@ -507,31 +507,18 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                 }
                 return m;
             };
-            // Where the eight elements of a piece go inside their (slice, chunk) and what power of two they take
-            // depends on the piece's place in its 128-column chunk, which is the same for every piece a thread
-            // handles (a thread's pieces are a multiple of 16 pieces apart): worked out once per staging, not per
-            // element (a row of 14336 columns is seven pieces per thread).
-            int el_at[8], el_exp[8];
-            {
-                int t16 = tid & 15;
-                asm volatile("" : "+v"(t16));  // (keeps these sixteen values out of the registers of the tile loop)
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const OperandSlot s = chunk_slot(t16 * 8 + e);
-                    el_at[e] = image_index(s.t, 0, s.e, G::kChunks);
-                    el_exp[e] = 127 + 14 - s.p;
-                }
-            }
             auto write_piece = [&](uint16_t *img, int c8, const uint4 &v, int ex) {
                 const int slice = (c8 * 8) / G::kCols;
                 const int chunk = ((c8 * 8) % G::kCols) / kChunkCols;
+                const int cc0 = (c8 * 8) % kChunkCols;
                 const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
-                uint16_t *dst = img + slice * G::kCols + chunk * 8;
+                uint16_t *dst = img + slice * G::kCols;
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
-                    const float mult = __builtin_bit_cast(float, (uint32_t)(el_exp[e] - ex) << 23);
+                    const OperandSlot s = chunk_slot(cc0 + e);
+                    const float mult = __builtin_bit_cast(float, (uint32_t)(127 + 14 - ex - s.p) << 23);
                     const uint16_t hx = (uint16_t)(w4[e >> 1] >> (16 * (e & 1)));
-                    dst[el_at[e]] = f2h(h2f(hx) * mult);
+                    dst[image_index(s.t, chunk, s.e, G::kChunks)] = f2h(h2f(hx) * mult);
                 }
             };
             // One piece into the image. The 16 pieces of a 128-column group are held by 16 neighbouring threads

@@ -1819,6 +1819,43 @@ def test_staged_plan_equals_the_separate_launches(dev, oracle, tuned, h, qd, kvd
     plan2.close()
 
 
+def test_staged_plan_whose_buffers_rule_out_tagged_words_waits_at_barriers(dev, oracle):
+    """A stage that reads only PART of an earlier output (a view into it) cannot take it from the producer's tagged
+    words; the plan then runs with barriers between its stages, and gives the bits of the separate launches. The same
+    two problems on whole buffers run with tagged words."""
+    torch, tl = dev
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(77)
+    f16 = dict(dtype=torch.float16, device="cuda")
+    wa, wb = _rand_weight(torch, gen, 4096, 2048), _rand_weight(torch, gen, 1024, 2048)
+    wc = _rand_weight(torch, gen, 1024, 4096)
+    x = torch.randn((1, 2048), device="cuda", generator=gen).to(torch.float16)
+    ya, yb, yc = torch.zeros((1, 4096), **f16), torch.zeros((1, 1024), **f16), torch.zeros((1, 1024), **f16)
+    tl.ternary_gemv(*wa, x, ya, 4096, 2048, 128)
+    tl.ternary_gemv(*wb, ya[:, 2048:].contiguous(), yb, 1024, 2048, 128)
+    tl.ternary_gemv(*wc, ya, yc, 1024, 4096, 128)
+    want_a, want_b, want_c = ya.clone(), yb.clone(), yc.clone()
+    part = ya[:, 2048:]                                  # the second half of the first stage's output, in place
+    plan = tl.LinearPlan([(*wa, x, ya, 4096, 2048, 1), (*wb, part, yb, 1024, 2048, 1)], stages=[0, 1])
+    assert "barriers" in plan.kernel
+    whole = tl.LinearPlan([(*wa, x, ya, 4096, 2048, 1), (*wc, ya, yc, 1024, 4096, 1)], stages=[0, 1])
+    assert "tagged words" in whole.kernel
+    for launch in range(3):
+        for t in (ya, yb, yc):
+            t.fill_(float("nan"))
+        plan.launch()
+        torch.cuda.synchronize()
+        plan.status()
+        assert torch.equal(ya.view(torch.int16), want_a.view(torch.int16)) and torch.equal(yb.view(torch.int16), want_b.view(torch.int16))
+        ya.fill_(float("nan"))
+        whole.launch()
+        torch.cuda.synchronize()
+        whole.status()
+        assert torch.equal(ya.view(torch.int16), want_a.view(torch.int16)) and torch.equal(yc.view(torch.int16), want_c.view(torch.int16))
+    plan.close()
+    whole.close()
+
+
 @pytest.mark.parametrize("handover", ["words", "barriers"])
 def test_staged_plan_in_a_captured_graph_and_on_a_second_stream(dev, oracle, tuned, handover):
     """The staged launch under graph capture (no allocation, counters that reset themselves, tags that every

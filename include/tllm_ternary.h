@@ -369,7 +369,8 @@ int tllm_read_stream(const void *src, size_t bytes, uint32_t *sink, tllm_stream_
  * These two calls change and read them afterwards, by name: "gemm_path" (0 cost model, 1 prefill GEMM, 2 passes of
  * the decode kernel), "gemm_rowsplit" (-1 cost model, 0 never, 1 or 2 forced), "batch_k_parts", "tall_max_batch",
  * "tall_min_share_milli", "stage_spin_limit" (polls a staged plan waits; 0: about a second), "stage_exchange" (read when
- * a staged plan is created: 0 makes it wait at barriers even where tagged words would do), "read_wgs_per_cu",
+ * a staged plan is created: 0 makes it wait at barriers even where tagged words would do), "stage_epoch_start" (the
+ * launch count a staged plan created afterwards starts its 16-bit tags from: tests put it just below the wrap), "read_wgs_per_cu",
  * "read_in_flight". An unknown name returns
  * TLLM_ERR_BAD_SHAPE. Results never depend on them beyond the order of fp32 additions. Not for concurrent use
  * with operator calls whose choice should be stable. No counterpart in the reference.

@@ -77,6 +77,7 @@ struct Tuning {
     std::atomic<int> tall_max_batch{4};         // TLLM_TALL_MAX_BATCH: most activation rows of a plan on the tall-tile kernel
     std::atomic<int> tall_min_share_milli{1000};  // TLLM_TALL_MIN_SHARE (x 1000): share of the plan per workgroup, in units, from which tall tiles run
     std::atomic<int> stage_exchange{1};         // staged plans hand results over as tagged words where the plan allows (0: always the barrier)
+    std::atomic<int> stage_epoch_start{0};      // launch count a new staged plan starts its tags from (tests put it just below the 16-bit wrap)
     std::atomic<int> stage_spin_limit{0};       // polls a workgroup of a staged plan waits for a stage (0: the plan's own limit); tests force a wait to expire with 1
     std::atomic<int> read_wgs_per_cu{8};        // TLLM_READ_SHAPE="wgs_per_cu,loads_in_flight" of tllm_read_stream
     std::atomic<int> read_in_flight{8};

@@ -37,7 +37,7 @@ std::atomic<int> *tuning_by_name(const char *name) {
                {"batch_k_parts", &t.batch_k_parts},
                {"tall_max_batch", &t.tall_max_batch}, {"tall_min_share_milli", &t.tall_min_share_milli},
                {"read_wgs_per_cu", &t.read_wgs_per_cu}, {"read_in_flight", &t.read_in_flight},
-               {"stage_spin_limit", &t.stage_spin_limit}, {"stage_exchange", &t.stage_exchange}};
+               {"stage_spin_limit", &t.stage_spin_limit}, {"stage_exchange", &t.stage_exchange}, {"stage_epoch_start", &t.stage_epoch_start}};
     for (const auto &e : all)
         if (name && !strcmp(name, e.name)) return e.value;
     return nullptr;

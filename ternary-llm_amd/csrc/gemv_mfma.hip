@@ -2038,6 +2038,12 @@ hipError_t plan_device_create_staged(const std::vector<Problem> &host, PlanDevic
     if (!e) e = hipMemcpy(d.wg_first, spans.data(), sizeof(int) * spans.size(), hipMemcpyHostToDevice);
     if (!e) e = hipMemset(d.counters, 0, bytes_counters);
     if (!e && exchange) e = hipMemset(d.words, 0, (size_t)kPlanSlots * d.ints_per_slot * 4);
+    if (const int start = tuning().stage_epoch_start.load(std::memory_order_relaxed); !e && exchange && start != 0) {
+        // (every workgroup of every slot starts counting its launches from `start`)
+        const std::vector<int> counts((size_t)grid, start);
+        for (int slot = 0; slot < kPlanSlots && !e; slot++)
+            e = hipMemcpy(d.words + (size_t)slot * d.ints_per_slot + n_words, counts.data(), sizeof(int) * counts.size(), hipMemcpyHostToDevice);
+    }
     d.next_slot = new (std::nothrow) std::atomic<unsigned>(0);
     if (!e && !d.next_slot) e = hipErrorOutOfMemory;
     if (e) {

@@ -1901,6 +1901,36 @@ def test_staged_plan_in_a_captured_graph_and_on_a_second_stream(dev, oracle, tun
     plan.close()
 
 
+def test_staged_plan_tags_wrap_around(dev, oracle, tuned):
+    """The tag of the words that hand results from stage to stage is the low 16 bits of a launch count. A plan created
+    with that count just below the wrap is launched across it (more launches than launch slots times the distance to
+    the wrap): every launch gives the bits of the separate launches."""
+    torch, tl = dev
+    tuned(stage_exchange=1, stage_epoch_start=65531)
+    h, qd, kvd, ffn, eps = 2048, 2048, 512, 8192, 1e-5
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(33)
+    w = _chain_layer(torch, tl, gen, h, qd, kvd, ffn)
+    f16 = dict(dtype=torch.float16, device="cuda")
+    x = torch.randn((1, h), device="cuda", generator=gen).to(torch.float16)
+    att = torch.randn((1, qd), device="cuda", generator=gen).to(torch.float16)
+    want = _chain_separate(torch, tl, w, x, att, h, qd, kvd, ffn, eps)
+    xs, hbuf = x.clone(), torch.zeros((1, ffn), **f16)
+    q, k, v = torch.zeros((1, qd), **f16), torch.zeros((1, kvd), **f16), torch.zeros((1, kvd), **f16)
+    plan = _chain_staged(torch, tl, w, xs, att, hbuf, q, k, v, h, qd, kvd, ffn, eps)
+    assert "tagged words" in plan.kernel
+    for launch in range(16 * 8):          # sixteen launch slots, each crosses the wrap at its fifth launch
+        xs.copy_(x)
+        for t in (hbuf, q, k, v):
+            t.fill_(float("nan"))
+        plan.launch()
+        torch.cuda.synchronize()
+        plan.status()
+        for name, got, ref in zip(("residual stream", "silu(gate) * up", "q", "k", "v"), (xs, hbuf, q, k, v), want):
+            assert torch.equal(got.view(torch.int16), ref.view(torch.int16)), f"launch {launch}: {name}"
+    plan.close()
+
+
 @pytest.mark.parametrize("handover", ["words", "barriers"])
 def test_staged_plan_wait_that_expires_is_reported(dev, oracle, tuned, handover):
     """A wait between two stages is bounded: with the bound forced down to one poll (tuning switch) the workgroups

@@ -1901,6 +1901,46 @@ def test_staged_plan_in_a_captured_graph_and_on_a_second_stream(dev, oracle, tun
     plan.close()
 
 
+def test_staged_plan_many_launches_back_to_back(dev, oracle):
+    """Five hundred launches of one staged plan queued without a synchronisation between them (they take the plan's
+    sixteen launch slots in turn; every launch reads its inputs from buffers no launch writes): the outputs of the last
+    one, and of a launch in the middle that is copied out on the stream, are the bits of the separate launches."""
+    torch, tl = dev
+    h, qd, ffn, eps = 4096, 4096, 14336, 1e-5
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(35)
+    w = _chain_layer(torch, tl, gen, h, qd, 1024, ffn)
+    f16 = dict(dtype=torch.float16, device="cuda")
+    x = torch.randn((1, h), device="cuda", generator=gen).to(torch.float16)
+    att = torch.randn((1, qd), device="cuda", generator=gen).to(torch.float16)
+    o, x1, xn = torch.zeros((1, h), **f16), torch.zeros((1, h), **f16), torch.zeros((1, h), **f16)
+    g, u, d, x2 = torch.zeros((1, ffn), **f16), torch.zeros((1, ffn), **f16), torch.zeros((1, h), **f16), torch.zeros((1, h), **f16)
+    tl.ternary_gemv(*w["o"], att, o, h, qd, 128)
+    tl.add(x, o, x1, h)
+    tl.rmsnorm(x1, w["n2"], xn, None, None, 1, h, eps)
+    tl.ternary_gemv(*w["g"], xn, g, ffn, h, 128)
+    tl.ternary_gemv(*w["u"], xn, u, ffn, h, 128)
+    tl.silu_mul(g, u, g, ffn)
+    tl.ternary_gemv(*w["d"], g, d, h, ffn, 128)
+    tl.add(x1, d, x2, h)
+    s1, act, s2 = torch.zeros((1, h), **f16), torch.zeros((1, ffn), **f16), torch.zeros((1, h), **f16)
+    plan = tl.LinearPlan([(*w["o"], att, s1, h, qd, 1), (*w["g"], s1, act, ffn, h, 1, tl.SWIGLU_GATE), (*w["u"], s1, None, ffn, h, 1),
+                          (*w["d"], act, s2, h, ffn, 1)],
+                         norm_weights=[None, w["n2"], w["n2"], None], eps=eps, stages=[0, 1, 1, 2], residuals=[x, None, None, s1])
+    assert "tagged words" in plan.kernel
+    middle = None
+    for launch in range(500):
+        plan.launch()
+        if launch == 250:
+            middle = (s1.clone(), act.clone(), s2.clone())
+    torch.cuda.synchronize()
+    plan.status()
+    for tag, got in (("launch 250", middle), ("last launch", (s1, act, s2))):
+        for name, a_, b_ in zip(("stream after o_proj", "silu(gate) * up", "stream after down_proj"), got, (x1, g, x2)):
+            assert torch.equal(a_.view(torch.int16), b_.view(torch.int16)), f"{tag}: {name}"
+    plan.close()
+
+
 def test_staged_plan_tags_wrap_around(dev, oracle, tuned):
     """The tag of the words that hand results from stage to stage is the low 16 bits of a launch count. A plan created
     with that count just below the wrap is launched across it (more launches than launch slots times the distance to

@@ -1059,7 +1059,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
                     }
                 }
             } else if constexpr (kFine) {
-                // one flat sequence of (walk, slot) pairs, three at a time through the ring
+                // one flat sequence of (walk, slot) pairs, G::kAhead at a time through the ring
                 u4 B[kMfmaPerTile];
                 f4 bias;
                 float bias_sel = 0.0f, gf = 0.0f;

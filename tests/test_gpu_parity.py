@@ -1901,6 +1901,64 @@ def test_staged_plan_in_a_captured_graph_and_on_a_second_stream(dev, oracle, tun
     plan.close()
 
 
+def test_staged_plan_of_int8_linears_and_of_long_rows(dev, oracle):
+    """Two kinds of problem make a staged plan wait at barriers and read the stage before with an invalidated cache:
+    inputs that the launch quantises itself (the reference's INT8 decode path, src/transformer.cpp:244-250 and 288-296:
+    o_proj and down_proj as ternary_linear_int8 with the residual add behind them) and rows too long to be staged from
+    registers (the 70B down_proj, K = 28672, behind its gate/up pair). Both give the bits of the separate launches."""
+    torch, tl = dev
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(36)
+    f16 = dict(dtype=torch.float16, device="cuda")
+    # (1) o_proj(int8) + residual -> down-like projection (int8) + residual, 8B sizes
+    h, mid = 4096, 14336
+    wa, wb = _rand_weight(torch, gen, mid, h), _rand_weight(torch, gen, h, mid)
+    x = torch.randn((1, h), device="cuda", generator=gen).to(torch.float16)
+    r1 = torch.randn((1, mid), device="cuda", generator=gen).to(torch.float16)
+    r2 = torch.randn((1, h), device="cuda", generator=gen).to(torch.float16)
+    ya, yb = torch.zeros((1, mid), **f16), torch.zeros((1, h), **f16)
+    tl.ternary_linear_int8(*wa, x, ya, mid, h, 128)
+    tl.add(r1, ya, ya, mid)
+    tl.ternary_linear_int8(*wb, ya, yb, h, mid, 128)
+    tl.add(r2, yb, yb, h)
+    want_a, want_b = ya.clone(), yb.clone()
+    plan = tl.LinearPlan([(*wa, x, ya, mid, h, 1, tl.QUANTIZE_INPUT), (*wb, ya, yb, h, mid, 1, tl.QUANTIZE_INPUT)],
+                         stages=[0, 1], residuals=[r1, r2])
+    assert "barriers" in plan.kernel
+    for launch in range(3):
+        ya.fill_(float("nan")); yb.fill_(float("nan"))
+        plan.launch()
+        torch.cuda.synchronize()
+        plan.status()
+        assert torch.equal(ya.view(torch.int16), want_a.view(torch.int16)), f"launch {launch}: first stage"
+        assert torch.equal(yb.view(torch.int16), want_b.view(torch.int16)), f"launch {launch}: second stage"
+    plan.close()
+    # (2) 70B FFN: RMSNorm + gate/up pair 28672 x 8192 -> down_proj 8192 x 28672 + residual
+    h, ffn, eps = 8192, 28672, 1e-5
+    wg, wu, wd = _rand_weight(torch, gen, ffn, h), _rand_weight(torch, gen, ffn, h), _rand_weight(torch, gen, h, ffn)
+    nw = (torch.randn(h, device="cuda", generator=gen) * 0.1 + 1.0).to(torch.float16)
+    x = torch.randn((1, h), device="cuda", generator=gen).to(torch.float16)
+    xn, g, u, d = torch.zeros((1, h), **f16), torch.zeros((1, ffn), **f16), torch.zeros((1, ffn), **f16), torch.zeros((1, h), **f16)
+    tl.rmsnorm(x, nw, xn, None, None, 1, h, eps)
+    tl.ternary_gemv(*wg, xn, g, ffn, h, 128)
+    tl.ternary_gemv(*wu, xn, u, ffn, h, 128)
+    tl.silu_mul(g, u, g, ffn)
+    tl.ternary_gemv(*wd, g, d, h, ffn, 128)
+    tl.add(x, d, d, h)
+    act, out = torch.zeros((1, ffn), **f16), torch.zeros((1, h), **f16)
+    plan = tl.LinearPlan([(*wg, x, act, ffn, h, 1, tl.SWIGLU_GATE), (*wu, x, None, ffn, h, 1), (*wd, act, out, h, ffn, 1)],
+                         norm_weights=[nw, nw, None], eps=eps, stages=[0, 0, 1], residuals=[None, None, x])
+    assert "barriers" in plan.kernel
+    for launch in range(2):
+        act.fill_(float("nan")); out.fill_(float("nan"))
+        plan.launch()
+        torch.cuda.synchronize()
+        plan.status()
+        assert torch.equal(act.view(torch.int16), g.view(torch.int16)), f"launch {launch}: silu(gate) * up"
+        assert torch.equal(out.view(torch.int16), d.view(torch.int16)), f"launch {launch}: stream after down_proj"
+    plan.close()
+
+
 def test_staged_plan_many_launches_back_to_back(dev, oracle):
     """Five hundred launches of one staged plan queued without a synchronisation between them (they take the plan's
     sixteen launch slots in turn; every launch reads its inputs from buffers no launch writes): the outputs of the last

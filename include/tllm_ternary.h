@@ -310,8 +310,8 @@ int tllm_linear_plan_create_i8(tllm_linear_plan **plan, const tllm_linear_proble
  *     or touches no output of the plan (a residual may be its own problem's output: in place); two outputs are
  *     either the same buffer in different stages (the reference's residual stream, updated in place twice) or do
  *     not overlap; a buffer that a later stage overwrites is only overwritten by a problem that depends, through
- *     such hand-overs, on every problem that reads or writes it earlier; rows of at most 16384 columns, no
- *     TLLM_PROBLEM_QUANTIZE_INPUT, at most 64 problems.
+ *     such hand-overs, on every problem that reads or writes it earlier; rows of at most 16384 columns, at most
+ *     64 problems.
  *   - otherwise at a barrier in device memory between every two stages (counters, bounded polling), after which
  *     the outputs of the stage before are read from memory, not from a stale cache line.
  * tllm_linear_plan_kernel names the way a plan runs. Either way the launches of a decode step that depend on each

@@ -1836,10 +1836,11 @@ hipError_t plan_device_create_staged(const std::vector<Problem> &host, PlanDevic
     }
     d.n_stages = stage + 1;
     d.max_batch = 1;
-    // rows that the one-pass staging holds in registers (K <= 16384) and are not quantised inside the launch are
-    // read with loads of device scope; anything else makes the workgroups invalidate their cache behind each barrier
+    // rows that the one-pass staging holds in registers (K <= 16384; also when the launch quantises them: it does so
+    // from those registers) are read with loads of device scope, or as tagged words; longer rows make the workgroups
+    // wait at barriers and invalidate their cache behind each
     for (const Problem &p : host)
-        if (p.cols > 16384 || (p.flags & kProblemQuantInput)) d.stage_fence = true;
+        if (p.cols > 16384) d.stage_fence = true;
     const int mats = has_pairs ? 2 : 1;
     if (whole + kNW * kFineUnit * 4 * mats > kLdsLimit) return hipErrorInvalidValue;  // whole rows in LDS (K <= 28672)
     const int max_units = max_units_for(whole, 1, kFineUnit, mats);

@@ -1902,10 +1902,11 @@ def test_staged_plan_in_a_captured_graph_and_on_a_second_stream(dev, oracle, tun
 
 
 def test_staged_plan_of_int8_linears_and_of_long_rows(dev, oracle):
-    """Two kinds of problem make a staged plan wait at barriers and read the stage before with an invalidated cache:
-    inputs that the launch quantises itself (the reference's INT8 decode path, src/transformer.cpp:244-250 and 288-296:
-    o_proj and down_proj as ternary_linear_int8 with the residual add behind them) and rows too long to be staged from
-    registers (the 70B down_proj, K = 28672, behind its gate/up pair). Both give the bits of the separate launches."""
+    """Inputs that the launch quantises itself (the reference's INT8 decode path, src/transformer.cpp:244-250 and
+    288-296: o_proj and down_proj as ternary_linear_int8 with the residual add behind them) in a staged plan, with
+    either way of handing results over; and rows too long to be staged from registers (the 70B down_proj, K = 28672,
+    behind its gate/up pair), which make a staged plan wait at barriers and read the stage before with an invalidated
+    cache. All give the bits of the separate launches."""
     torch, tl = dev
     gen = torch.Generator(device="cuda")
     gen.manual_seed(36)
@@ -1922,17 +1923,19 @@ def test_staged_plan_of_int8_linears_and_of_long_rows(dev, oracle):
     tl.ternary_linear_int8(*wb, ya, yb, h, mid, 128)
     tl.add(r2, yb, yb, h)
     want_a, want_b = ya.clone(), yb.clone()
-    plan = tl.LinearPlan([(*wa, x, ya, mid, h, 1, tl.QUANTIZE_INPUT), (*wb, ya, yb, h, mid, 1, tl.QUANTIZE_INPUT)],
-                         stages=[0, 1], residuals=[r1, r2])
-    assert "barriers" in plan.kernel
-    for launch in range(3):
-        ya.fill_(float("nan")); yb.fill_(float("nan"))
-        plan.launch()
-        torch.cuda.synchronize()
-        plan.status()
-        assert torch.equal(ya.view(torch.int16), want_a.view(torch.int16)), f"launch {launch}: first stage"
-        assert torch.equal(yb.view(torch.int16), want_b.view(torch.int16)), f"launch {launch}: second stage"
-    plan.close()
+    for handover in ("tagged words", "barriers"):
+        with tl.tuning(stage_exchange=1 if handover == "tagged words" else 0):
+            plan = tl.LinearPlan([(*wa, x, ya, mid, h, 1, tl.QUANTIZE_INPUT), (*wb, ya, yb, h, mid, 1, tl.QUANTIZE_INPUT)],
+                                 stages=[0, 1], residuals=[r1, r2])
+        assert handover in plan.kernel
+        for launch in range(3):
+            ya.fill_(float("nan")); yb.fill_(float("nan"))
+            plan.launch()
+            torch.cuda.synchronize()
+            plan.status()
+            assert torch.equal(ya.view(torch.int16), want_a.view(torch.int16)), f"{handover}, launch {launch}: first stage"
+            assert torch.equal(yb.view(torch.int16), want_b.view(torch.int16)), f"{handover}, launch {launch}: second stage"
+        plan.close()
     # (2) 70B FFN: RMSNorm + gate/up pair 28672 x 8192 -> down_proj 8192 x 28672 + residual
     h, ffn, eps = 8192, 28672, 1e-5
     wg, wu, wd = _rand_weight(torch, gen, ffn, h), _rand_weight(torch, gen, ffn, h), _rand_weight(torch, gen, h, ffn)

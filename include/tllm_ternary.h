@@ -242,7 +242,7 @@ typedef struct tllm_linear_problem {
     int32_t rows;
     int32_t cols;
     int32_t batch; /* 1..TLLM_MAX_PLAN_BATCH */
-    int32_t flags; /* 0, TLLM_PROBLEM_SWIGLU_GATE or TLLM_PROBLEM_QUANTIZE_INPUT */
+    int32_t flags; /* 0 or any of TLLM_PROBLEM_SWIGLU_GATE, TLLM_PROBLEM_QUANTIZE_INPUT */
 } tllm_linear_problem;
 
 enum { TLLM_MAX_PLAN_BATCH = 16 };
@@ -259,11 +259,15 @@ enum { TLLM_MAX_PLAN_BATCH = 16 };
 enum { TLLM_PROBLEM_SWIGLU_GATE = 1 };
 
 /*
- * Flag of a problem whose fp16 input the launch quantises to int8 itself before it multiplies (batch 1, not with
- * a SwiGLU pair or an RMSNorm prologue): the output is what tllm_quantize_absmax_i8 followed by
- * tllm_ternary_gemv_i8_dscale stores for that matrix, bit for bit, without the int8 vector and its scale ever being
- * written. Replaces the reference's ternary_linear_int8 (src/transformer.cpp:126-143: quantise, copy the scale to
- * the host, int8 GEMV) for every linear of a group in one launch.
+ * Flag of a problem whose fp16 input the launch quantises to int8 itself before it multiplies (batch 1): the output
+ * is what tllm_quantize_absmax_i8 followed by tllm_ternary_gemv_i8_dscale stores for that matrix, bit for bit, without
+ * the int8 vector and its scale ever being written. Replaces the reference's ternary_linear_int8
+ * (src/transformer.cpp:126-143: quantise, copy the scale to the host, int8 GEMV) for every linear of a group in one
+ * launch. It combines with the other two fusions in the order of the reference's INT8 decode step
+ * (src/transformer.cpp:193-217, 258-286): behind an RMSNorm prologue the normalised, fp16-rounded row is what gets
+ * quantised (rmsnorm_forward, then quantize_absmax_int8, then the projections that share the int8 vector); on the gate
+ * problem of a SwiGLU pair both halves multiply the same quantised row and the epilogue stores silu(gate) * up of the
+ * two fp16-rounded INT8 results (the up problem carries no flag of its own).
  */
 enum { TLLM_PROBLEM_QUANTIZE_INPUT = 2 };
 

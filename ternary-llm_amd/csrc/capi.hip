@@ -259,9 +259,10 @@ static int create_plan(tllm_linear_plan **plan, const tllm_linear_problem *probl
         if (q.batch < 1 || q.batch > TLLM_MAX_PLAN_BATCH) return TLLM_ERR_BAD_PLAN;
         if (q.flags & ~(TLLM_PROBLEM_SWIGLU_GATE | TLLM_PROBLEM_QUANTIZE_INPUT)) return TLLM_ERR_BAD_PLAN;
         if (q.flags & TLLM_PROBLEM_QUANTIZE_INPUT) {
-            // quantised inside the launch: one activation row, fp16 input, neither pair nor prologue
-            if (q.batch != 1 || (q.flags & TLLM_PROBLEM_SWIGLU_GATE) || input_scales || (norm_weights && norm_weights[i]))
-                return TLLM_ERR_BAD_PLAN;
+            // quantised inside the launch: one activation row, fp16 input. A norm prologue comes first (the normalised,
+            // fp16-rounded row is what gets quantised, as when rmsnorm_forward runs in front of the quantiser); the two
+            // halves of a SwiGLU pair share the quantised row (the flag sits on the gate problem).
+            if (q.batch != 1 || input_scales) return TLLM_ERR_BAD_PLAN;
         }
         const bool is_up = i > 0 && (problems[i - 1].flags & TLLM_PROBLEM_SWIGLU_GATE);
         if (is_up) {

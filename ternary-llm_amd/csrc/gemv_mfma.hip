@@ -1668,7 +1668,7 @@ hipError_t plan_device_create(const std::vector<Problem> &host, PlanDevice *out)
     for (const Problem &p : host) {
         has_pairs = has_pairs || (p.flags & kProblemSwigluGate);
         has_norm = has_norm || (p.norm_w != nullptr && !(p.flags & kProblemInt8Input));
-        has_quant = has_quant || (p.flags & kProblemQuantInput);  // (batch 1, no pair, no prologue: the caller has checked)
+        has_quant = has_quant || (p.flags & kProblemQuantInput);  // (batch 1: the caller has checked)
     }
     // int8 activations: all problems or none, batch 1 (the caller has checked), MFMA kernel only
     bool any_i8 = false, all_i8 = true;

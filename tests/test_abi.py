@@ -86,9 +86,7 @@ def test_validation_codes():
                 [P(0x1000, 0x2000, 0x3000, 0x4000, 0x9000, 64, 2048, 2, GATE),
                  P(0x1000, 0x2000, 0x3000, 0x4000, 0, 64, 2048, 2, 0)],               # batch 2
                 [P(0x1000, 0x2000, 0x3000, 0x4000, 0x9000, 64, 2048, 1, 4)],          # unknown flag
-                [P(0x1000, 0x2000, 0x3000, 0x4000, 0x9000, 64, 2048, 2, ops.QUANTIZE_INPUT)],   # quantised input: one row only
-                [P(0x1000, 0x2000, 0x3000, 0x4000, 0x9000, 64, 2048, 1, GATE | ops.QUANTIZE_INPUT),
-                 P(0x1000, 0x2000, 0x3000, 0x4000, 0, 64, 2048, 1, 0)]):              # ... and not in a pair
+                [P(0x1000, 0x2000, 0x3000, 0x4000, 0x9000, 64, 2048, 2, ops.QUANTIZE_INPUT)]):  # quantised input: one row only
         arr = (P * len(bad))(*bad)
         assert L.tllm_linear_plan_create(C.byref(h), arr, len(bad), 128) == -6
     # RMSNorm prologue: batch 1, cols <= 16384, aligned weights, same weights on both halves of a pair

@@ -1729,9 +1729,62 @@ def test_fused_int8_linear_special_inputs(dev, oracle):
     for pr, ref in zip(probs, pairs):
         assert torch.equal(pr[4][0].view(torch.int16), ref.view(torch.int16))
     plan.close()
-    with pytest.raises(tl.TllmError):      # not together with a SwiGLU pair
-        tl.LinearPlan([(*probs[1][:3], dx.view(1, -1), probs[1][4], 1024, cols, 1, tl.QUANTIZE_INPUT | tl.SWIGLU_GATE),
-                       (*probs[2][:3], dx.view(1, -1), None, 1024, cols, 1)])
+
+
+@pytest.mark.parametrize("h,ffn,qd,kvd", [(4096, 14336, 4096, 1024), (2048, 8192, 2048, 512), (8192, 28672, 8192, 1024)])
+def test_int8_decode_step_fusions_equal_the_reference_launches(dev, oracle, h, ffn, qd, kvd):
+    """The reference's INT8 decode step (src/transformer.cpp:193-217 and 258-286): rmsnorm_forward, quantize_absmax_int8
+    once, then the projections of the group on the shared int8 vector, then silu_mul_forward behind gate and up. As
+    plans: the RMSNorm prologue, the quantisation inside the launch and the SwiGLU pair in ONE launch per group, with
+    the bits of the separate launches; also the pair on an input that is quantised without a prologue."""
+    torch, tl = dev
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(h + 7)
+    f16 = dict(dtype=torch.float16, device="cuda")
+    eps = 1e-5
+    w = _chain_layer(torch, tl, gen, h, qd, kvd, ffn)
+    x = (torch.randn((1, h), device="cuda", generator=gen) * 1.7).to(torch.float16)
+    xn = torch.zeros((1, h), **f16)
+    i8, i8s = torch.zeros(h, dtype=torch.int8, device="cuda"), torch.zeros(1, dtype=torch.float32, device="cuda")
+    tl.rmsnorm(x, w["n2"], xn, None, None, 1, h, eps)
+    tl.quantize_absmax_int8(xn, i8, i8s, h)
+    g, u = torch.zeros((1, ffn), **f16), torch.zeros((1, ffn), **f16)
+    tl.ternary_gemv_int8(*w["g"], i8, i8s, g, ffn, h, 128)
+    tl.ternary_gemv_int8(*w["u"], i8, i8s, u, ffn, h, 128)
+    tl.silu_mul(g, u, g, ffn)
+    tl.rmsnorm(x, w["n1"], xn, None, None, 1, h, eps)
+    tl.quantize_absmax_int8(xn, i8, i8s, h)
+    want_qkv = []
+    for name, r in (("q", qd), ("k", kvd), ("v", kvd)):
+        o = torch.zeros((1, r), **f16)
+        tl.ternary_gemv_int8(*w[name], i8, i8s, o, r, h, 128)
+        want_qkv.append(o)
+    act = torch.full((1, ffn), float("nan"), **f16)
+    ffn_plan = tl.LinearPlan([(*w["g"], x, act, ffn, h, 1, tl.SWIGLU_GATE | tl.QUANTIZE_INPUT), (*w["u"], x, None, ffn, h, 1)],
+                             norm_weights=[w["n2"], w["n2"]], eps=eps)
+    outs = [torch.full((1, r), float("nan"), **f16) for r in (qd, kvd, kvd)]
+    qkv_plan = tl.LinearPlan([(*w[name], x, o, r, h, 1, tl.QUANTIZE_INPUT) for name, o, r in zip("qkv", outs, (qd, kvd, kvd))],
+                             norm_weights=[w["n1"]] * 3, eps=eps)
+    for launch in range(2):
+        ffn_plan.launch()
+        qkv_plan.launch()
+        torch.cuda.synchronize()
+        assert torch.equal(act.view(torch.int16), g.view(torch.int16)), "RMSNorm + quantise + gate/up + SiLU * up"
+        for name, got, ref in zip("qkv", outs, want_qkv):
+            assert torch.equal(got.view(torch.int16), ref.view(torch.int16)), f"RMSNorm + quantise + {name}_proj"
+    ffn_plan.close()
+    qkv_plan.close()
+    # the pair on a row that is quantised as it is (no prologue)
+    tl.quantize_absmax_int8(x, i8, i8s, h)
+    tl.ternary_gemv_int8(*w["g"], i8, i8s, g, ffn, h, 128)
+    tl.ternary_gemv_int8(*w["u"], i8, i8s, u, ffn, h, 128)
+    tl.silu_mul(g, u, g, ffn)
+    act.fill_(float("nan"))
+    plain = tl.LinearPlan([(*w["g"], x, act, ffn, h, 1, tl.SWIGLU_GATE | tl.QUANTIZE_INPUT), (*w["u"], x, None, ffn, h, 1)])
+    plain.launch()
+    torch.cuda.synchronize()
+    assert torch.equal(act.view(torch.int16), g.view(torch.int16)), "quantise + gate/up + SiLU * up"
+    plain.close()
 
 
 def _chain_layer(torch, tl, gen, h, qd, kvd, ffn):
@@ -1773,6 +1826,75 @@ def _chain_staged(torch, tl, w, xs, att, hbuf, q, k, v, h, qd, kvd, ffn, eps):
     norms = [None, w["n2"], w["n2"], None, w["n1"], w["n1"], w["n1"]]
     residuals = [xs, None, None, xs, None, None, None]
     return tl.LinearPlan(probs, norm_weights=norms, eps=eps, stages=[0, 1, 1, 2, 3, 3, 3], residuals=residuals)
+
+
+def _chain_separate_int8(torch, tl, w, x, att, h, qd, kvd, ffn, eps):
+    """The reference's INT8 decode launches (src/transformer.cpp:193-217, 244-296 with use_int8): every linear on the
+    int8 quantisation of its input, the vectors shared inside a group."""
+    f16 = dict(dtype=torch.float16, device="cuda")
+    o, xn = torch.zeros((1, h), **f16), torch.zeros((1, h), **f16)
+    g, u, d = torch.zeros((1, ffn), **f16), torch.zeros((1, ffn), **f16), torch.zeros((1, h), **f16)
+    q, k, v = torch.zeros((1, qd), **f16), torch.zeros((1, kvd), **f16), torch.zeros((1, kvd), **f16)
+    i8, i8s = torch.zeros(max(h, qd), dtype=torch.int8, device="cuda"), torch.zeros(1, dtype=torch.float32, device="cuda")
+    xs = x.clone()
+    tl.ternary_linear_int8(*w["o"], att, o, h, qd, 128)
+    tl.add(xs, o, xs, h)
+    tl.rmsnorm(xs, w["n2"], xn, None, None, 1, h, eps)
+    tl.quantize_absmax_int8(xn, i8, i8s, h)
+    tl.ternary_gemv_int8(*w["g"], i8, i8s, g, ffn, h, 128)
+    tl.ternary_gemv_int8(*w["u"], i8, i8s, u, ffn, h, 128)
+    tl.silu_mul(g, u, g, ffn)
+    tl.ternary_linear_int8(*w["d"], g, d, h, ffn, 128)
+    tl.add(xs, d, xs, h)
+    tl.rmsnorm(xs, w["n1"], xn, None, None, 1, h, eps)
+    tl.quantize_absmax_int8(xn, i8, i8s, h)
+    tl.ternary_gemv_int8(*w["q"], i8, i8s, q, qd, h, 128)
+    tl.ternary_gemv_int8(*w["k"], i8, i8s, k, kvd, h, 128)
+    tl.ternary_gemv_int8(*w["v"], i8, i8s, v, kvd, h, 128)
+    return xs, g, q, k, v
+
+
+def _chain_staged_int8(torch, tl, w, xs, att, hbuf, q, k, v, h, qd, kvd, ffn, eps):
+    Q = tl.QUANTIZE_INPUT
+    probs = [(*w["o"], att, xs, h, qd, 1, Q),
+             (*w["g"], xs, hbuf, ffn, h, 1, tl.SWIGLU_GATE | Q), (*w["u"], xs, None, ffn, h, 1),
+             (*w["d"], hbuf, xs, h, ffn, 1, Q),
+             (*w["q"], xs, q, qd, h, 1, Q), (*w["k"], xs, k, kvd, h, 1, Q), (*w["v"], xs, v, kvd, h, 1, Q)]
+    norms = [None, w["n2"], w["n2"], None, w["n1"], w["n1"], w["n1"]]
+    residuals = [xs, None, None, xs, None, None, None]
+    return tl.LinearPlan(probs, norm_weights=norms, eps=eps, stages=[0, 1, 1, 2, 3, 3, 3], residuals=residuals)
+
+
+@pytest.mark.parametrize("handover", ["words", "barriers"])
+@pytest.mark.parametrize("h,qd,kvd,ffn", [(4096, 4096, 1024, 14336), (2048, 2048, 512, 8192)])
+def test_staged_int8_decode_layer_equals_the_reference_launches(dev, oracle, tuned, h, qd, kvd, ffn, handover):
+    """The linear side of the reference's INT8 decode layer (fourteen launches and four copies of a scale to the host)
+    as ONE launch: every input quantised inside the launch, behind the RMSNorm prologue where the reference normalises
+    first. The residual stream, the FFN activation and q, k, v hold the bits of the separate launches."""
+    torch, tl = dev
+    tuned(stage_exchange=1 if handover == "words" else 0)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(h + ffn + 1)
+    eps = 1e-5
+    w = _chain_layer(torch, tl, gen, h, qd, kvd, ffn)
+    f16 = dict(dtype=torch.float16, device="cuda")
+    x = torch.randn((1, h), device="cuda", generator=gen).to(torch.float16)
+    att = torch.randn((1, qd), device="cuda", generator=gen).to(torch.float16)
+    want = _chain_separate_int8(torch, tl, w, x, att, h, qd, kvd, ffn, eps)
+    xs, hbuf = x.clone(), torch.full((1, ffn), float("nan"), **f16)
+    q, k, v = torch.full((1, qd), float("nan"), **f16), torch.full((1, kvd), float("nan"), **f16), torch.full((1, kvd), float("nan"), **f16)
+    plan = _chain_staged_int8(torch, tl, w, xs, att, hbuf, q, k, v, h, qd, kvd, ffn, eps)
+    assert ("tagged words" if handover == "words" else "barriers") in plan.kernel
+    for launch in range(3):
+        xs.copy_(x)
+        for t in (hbuf, q, k, v):
+            t.fill_(float("nan"))
+        plan.launch()
+        torch.cuda.synchronize()
+        plan.status()
+        for name, got, ref in zip(("residual stream", "silu(gate) * up", "q", "k", "v"), (xs, hbuf, q, k, v), want):
+            assert torch.equal(got.view(torch.int16), ref.view(torch.int16)), f"launch {launch}: {name} differs from the separate launches"
+    plan.close()
 
 
 @pytest.mark.parametrize("handover", ["words", "barriers"])

@@ -525,6 +525,55 @@ def decode_chain(torch, tl, problems, model, layers):
         w["qkv_s"] = tl.LinearPlan([(*w["q"], x3, q, qd, h, 1), (*w["k"], x3, k, kvd, h, 1), (*w["v"], x3, v, kvd, h, 1)],
                                    norm_weights=[w["n1"]] * 3, eps=eps)
 
+    # The reference's decode step proper is INT8 (src/transformer.cpp:176: use_int8 = n_tokens == 1): every linear runs
+    # on the absmax-quantised input, the int8 vector shared inside a group. Its launches (the four copies of the scale
+    # to the host per layer left out: the scale stays on the device here), the same as four launches per layer (norm
+    # prologue + quantisation inside the launch + SwiGLU pair), and as one staged launch per layer.
+    Q = tl.QUANTIZE_INPUT
+    i8, i8s = torch.zeros(max(h, qd, ffn), dtype=torch.int8, device="cuda"), torch.zeros(1, dtype=torch.float32, device="cuda")
+    for l, w in enumerate(L):
+        nxt = L[l + 1] if l + 1 < len(L) else None
+        w["qkv_q"] = tl.LinearPlan([(*w["q"], x, q, qd, h, 1, Q), (*w["k"], x, k, kvd, h, 1, Q), (*w["v"], x, v, kvd, h, 1, Q)],
+                                   norm_weights=[w["n1"]] * 3, eps=eps)
+        w["gu_q"] = tl.LinearPlan([(*w["g"], x, g, ffn, h, 1, tl.SWIGLU_GATE | Q), (*w["u"], x, None, ffn, h, 1)],
+                                  norm_weights=[w["n2"]] * 2, eps=eps)
+        ogd = [(*w["o"], att, xs, h, qd, 1, Q), (*w["g"], xs, g, ffn, h, 1, tl.SWIGLU_GATE | Q), (*w["u"], xs, None, ffn, h, 1),
+               (*w["d"], g, x3, h, ffn, 1, Q)]
+        norms, res, stages = [None, w["n2"], w["n2"], None], [x, None, None, xs], [0, 1, 1, 2]
+        if nxt is not None:
+            ogd = ogd + [(*nxt["q"], x3, q, qd, h, 1, Q), (*nxt["k"], x3, k, kvd, h, 1, Q), (*nxt["v"], x3, v, kvd, h, 1, Q)]
+            norms, res, stages = norms + [nxt["n1"]] * 3, res + [None] * 3, stages + [3, 3, 3]
+        w["ogdq_q"] = tl.LinearPlan(ogd, norm_weights=norms, eps=eps, stages=stages, residuals=res)
+
+    def int8_reference():
+        for w in L:
+            tl.rmsnorm(x, w["n1"], xn, None, None, 1, h, eps)
+            tl.quantize_absmax_int8(xn, i8, i8s, h)
+            tl.ternary_gemv_int8(*w["q"], i8, i8s, q, qd, h, 128)
+            tl.ternary_gemv_int8(*w["k"], i8, i8s, k, kvd, h, 128)
+            tl.ternary_gemv_int8(*w["v"], i8, i8s, v, kvd, h, 128)
+            tl.quantize_absmax_int8(att, i8, i8s, qd)
+            tl.ternary_gemv_int8(*w["o"], i8, i8s, o, h, qd, 128)
+            tl.rmsnorm(x, w["n2"], xn, None, None, 1, h, eps)
+            tl.quantize_absmax_int8(xn, i8, i8s, h)
+            tl.ternary_gemv_int8(*w["g"], i8, i8s, g, ffn, h, 128)
+            tl.ternary_gemv_int8(*w["u"], i8, i8s, u, ffn, h, 128)
+            tl.silu_mul(g, u, g, ffn)
+            tl.quantize_absmax_int8(g, i8, i8s, ffn)
+            tl.ternary_gemv_int8(*w["d"], i8, i8s, d, h, ffn, 128)
+
+    def int8_four():
+        for w in L:
+            w["qkv_q"].launch()
+            tl.ternary_linear_int8(*w["o"], att, o, h, qd, 128)
+            w["gu_q"].launch()
+            tl.ternary_linear_int8(*w["d"], g, d, h, ffn, 128)
+
+    def int8_one():
+        L[0]["qkv_q"].launch()
+        for w in L:
+            w["ogdq_q"].launch()
+
     def two():
         for w in L:
             w["qkv_s"].launch()
@@ -537,7 +586,7 @@ def decode_chain(torch, tl, problems, model, layers):
 
     def close():
         for w in L:
-            for key in ("qkv", "gu", "qkv_n", "gu_n", "qkv_s", "ogd"):
+            for key in ("qkv", "gu", "qkv_n", "gu_n", "qkv_s", "ogd", "qkv_q", "gu_q", "ogdq_q"):
                 w[key].close()
             if w["ogdq"] is not w["ogd"]:
                 w["ogdq"].close()
@@ -545,7 +594,10 @@ def decode_chain(torch, tl, problems, model, layers):
     return {"variants": (("the reference's 10 launches per layer", ten, 10), ("q/k/v and gate/up as plans: 7 per layer", seven, 7),
                          ("RMSNorm prologue + SwiGLU pair: 4 per layer", four, 4),
                          ("staged plan o_proj -> gate/up -> down_proj with the residual adds, q/k/v apart: 2 launches per layer", two, 2),
-                         ("staged plan o_proj -> gate/up -> down_proj -> q/k/v of the next layer: 1 launch per layer", one, 1)),
+                         ("staged plan o_proj -> gate/up -> down_proj -> q/k/v of the next layer: 1 launch per layer", one, 1),
+                         ("INT8 decode as the reference issues it: 14 launches per layer, scales kept on the device", int8_reference, 14),
+                         ("INT8 decode, RMSNorm prologue + quantisation in the launch + SwiGLU pair: 4 per layer", int8_four, 4),
+                         ("INT8 decode as one staged launch per layer", int8_one, 1)),
             "close": close}
 
 

@@ -402,6 +402,44 @@ def gemm_rows(torch, tl, orc, timer, seed, m_list, p_zero, calls, warm):
     return rows
 
 
+def ffn_front_rows(torch, tl, timer, seed, m_list, p_zero, calls, warm):
+    """The FFN front half of a prefill step on the 8B shapes (reference src/transformer.cpp:264-286 at n_tokens > 1):
+    ternary_gemm on gate, ternary_gemm on up and silu_mul as the reference issues them, and as ONE launch
+    (tllm_ternary_gemm_swiglu_f16). Flops counted for both products (4*M*N*K); the outputs are compared bit for bit."""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(seed + 44)
+    n, k = 14336, 4096
+    rows = []
+    g_nz, g_sg = gen_masks(torch, n, k, p_zero, gen)
+    u_nz, u_sg = gen_masks(torch, n, k, p_zero, gen)
+    g_sc = (torch.rand((n, k // 128), device="cuda", generator=gen) * 0.02 + 0.01).to(torch.float16)
+    u_sc = (torch.rand((n, k // 128), device="cuda", generator=gen) * 0.02 + 0.01).to(torch.float16)
+    for m in m_list:
+        if m <= 16:
+            continue
+        a = torch.randn((m, k), device="cuda", generator=gen).to(torch.float16)
+        g, u, one = (torch.zeros((m, n), dtype=torch.float16, device="cuda") for _ in range(3))
+
+        def three():
+            tl.ternary_gemm(a, g_nz, g_sg, g_sc, g, m, n, k, 128)
+            tl.ternary_gemm(a, u_nz, u_sg, u_sc, u, m, n, k, 128)
+            tl.silu_mul(g, u, g, m * n)
+
+        t3 = timer.run(three, calls, warm)
+        t1 = timer.run(lambda: tl.ternary_gemm_swiglu(a, g_nz, g_sg, g_sc, u_nz, u_sg, u_sc, one, m, n, k, 128), calls, warm)
+        floor = float(torch.sqrt(torch.mean(g.float() ** 2)).item()) / 64.0
+        rel = float(((one.float() - g.float()).abs() / torch.clamp(g.float().abs(), min=floor)).max().item())
+        flops = 4.0 * m * n * k
+        for name, t, kern in (("gate GEMM + up GEMM + SiLU*mul, three launches", t3, tl.gemm_kernel(m, n, k) + " x 2, silu_mul_kernel"),
+                              ("gate/up/SiLU*mul in one launch", t1, "tllm::gemm_ns_kernel<4, 2, pair>")):
+            tf = flops / (t["mean_ms"] * 1e-3) / 1e12
+            rows.append({"config": f"cfg4: prefill FFN front half M={m}, 2 x W {n}x{k}: {name}", "M": m, "N": n, "K": k, **stats_us(t),
+                         "tflops": round(tf, 1), "bound": "mfma", "frac_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
+                         "kernel": kern, "max_rel_one_launch_vs_three": rel})
+        del a, g, u, one
+    return rows
+
+
 def single_call_rows(torch, tl, timer, problems, model, layers):
     """The reference's call pattern on the headline weights: one operator call per matrix
     (src/transformer.cpp:102-118), all calls of a sweep captured once into a HIP graph and replayed, so the
@@ -820,6 +858,7 @@ def main():
             gemm_m = [int(v) for v in args.gemm_m.split(",") if v.strip()]
             g = gemm_rows(torch, tl, orc, timer, args.seed, gemm_m, 0.42, args.gemm_calls, args.gemm_warm)
             cfgs += g
+            cfgs += ffn_front_rows(torch, tl, timer, args.seed, [m for m in gemm_m if m in (512, 2048)], 0.42, args.gemm_calls, args.gemm_warm)
             m512 = [c for c in g if c["M"] == 512]
             if m512:
                 agg = sum(2.0 * c["M"] * c["N"] * c["K"] for c in m512) / sum(c["us"] for c in m512) / 1e6

@@ -97,6 +97,18 @@ inline void ternary_linear_int8(const uint32_t *nonzero_masks, const uint32_t *s
                                         reinterpret_cast<uint16_t *>(output), rows, cols, group_size, stream));
 }
 
+// The FFN front half of a prefill step as one call (no counterpart in include/kernels.cuh: there it is ternary_gemm on
+// the gate matrix, ternary_gemm on the up matrix and silu_mul_forward, src/transformer.cpp:264-286). C = silu(A gate^T) * (A up^T).
+inline void ternary_gemm_swiglu(const half *A, const uint32_t *nz_gate, const uint32_t *sign_gate, const half *scales_gate,
+                                const uint32_t *nz_up, const uint32_t *sign_up, const half *scales_up, half *C, int M,
+                                int N, int K, int group_size, hipStream_t stream = 0) {
+    report("ternary_gemm_swiglu",
+           tllm_ternary_gemm_swiglu_f16(reinterpret_cast<const uint16_t *>(A), nz_gate, sign_gate,
+                                        reinterpret_cast<const uint16_t *>(scales_gate), nz_up, sign_up,
+                                        reinterpret_cast<const uint16_t *>(scales_up), reinterpret_cast<uint16_t *>(C), M, N,
+                                        K, group_size, stream));
+}
+
 // Reference include/kernels.cuh:37-40.
 inline void ternary_gemm(const half *A, const uint32_t *nz_B, const uint32_t *sign_B,
                          const half *scales_B, half *C, int M, int N, int K, int group_size,

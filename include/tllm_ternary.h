@@ -132,6 +132,22 @@ int tllm_ternary_gemm_f16(const uint16_t *A, const uint32_t *nz_B, const uint32_
                           int group_size, tllm_stream_t stream);
 
 /*
+ * The FFN front half of a prefill step in ONE launch: C[m, n] = fp16( silu(g) * u ) with g = fp16(A[m, :] . gate row n),
+ * u = fp16(A[m, :] . up row n), i.e. what tllm_ternary_gemm_f16 on the gate matrix, tllm_ternary_gemm_f16 on the up
+ * matrix and tllm_silu_mul_f16 store (reference src/transformer.cpp:264-286 at n_tokens > 1: ternary_linear(gate),
+ * ternary_linear(up), silu_mul_forward). A workgroup multiplies one tile of the activations with the same 128 rows of
+ * both matrices, so the activations are fetched once and the two M x N intermediates are never written. Same arithmetic
+ * as tllm_ternary_gemm_f16 (fp32 accumulation; the order of the additions is that of its row-split kernel in the
+ * four-wave form). Both matrices are [N, K] in the packed layout; group_size 128; K a multiple of 256, or of 128 from
+ * 384 on (else TLLM_ERR_BAD_SHAPE / TLLM_ERR_BAD_GROUP: issue the three launches); A and the mask planes 16-byte aligned.
+ * Any M >= 1 (for M = 1 the decode plans with TLLM_PROBLEM_SWIGLU_GATE are the faster form). Allocation-free.
+ */
+int tllm_ternary_gemm_swiglu_f16(const uint16_t *A, const uint32_t *nz_gate, const uint32_t *sign_gate,
+                                 const uint16_t *scales_gate, const uint32_t *nz_up, const uint32_t *sign_up,
+                                 const uint16_t *scales_up, uint16_t *C, int M, int N, int K, int group_size,
+                                 tllm_stream_t stream);
+
+/*
  * tllm_ternary_gemm_f16 for callers that cannot allocate device memory (code under HIP graph capture,
  * serving loops and harnesses that forbid hipMalloc): same arguments, same kernels, same results bit for
  * bit, but the workspace (the split-K exchange) is a fixed array of

@@ -102,6 +102,21 @@ int tllm_ternary_gemm_f16_static(const uint16_t *A, const uint32_t *nz_B, const 
     return (int)tllm::dispatch_linear(p, group_size, (hipStream_t)stream, true);
 }
 
+int tllm_ternary_gemm_swiglu_f16(const uint16_t *A, const uint32_t *nz_gate, const uint32_t *sign_gate,
+                                 const uint16_t *scales_gate, const uint32_t *nz_up, const uint32_t *sign_up,
+                                 const uint16_t *scales_up, uint16_t *C, int M, int N, int K, int group_size,
+                                 tllm_stream_t stream) {
+    if (M < 1) return TLLM_ERR_BAD_SHAPE;
+    Problem gate{nz_gate, sign_gate, scales_gate, A, C, N, K, M, 0};
+    Problem up{nz_up, sign_up, scales_up, A, C, N, K, M, 0};
+    if (int e = tllm::check_linear(gate, group_size)) return e;
+    if (int e = tllm::check_weight(nz_up, sign_up, scales_up, N, K, group_size)) return e;
+    // (one kernel serves the pair: group 128, K a multiple of 256 or of 128 from 384 on; other shapes: the three launches)
+    if (group_size != 128) return TLLM_ERR_BAD_GROUP;
+    if (!tllm::gemm_swiglu_supports(gate, up)) return TLLM_ERR_BAD_SHAPE;
+    return (int)tllm::launch_gemm_swiglu(gate, up, (hipStream_t)stream);
+}
+
 int tllm_gemm_workspace_reserve(int M, int N, int K, int group_size, tllm_stream_t stream) {
     if (M < 1 || N < 1 || K < 1 || K % 32 != 0) return TLLM_ERR_BAD_SHAPE;
     if (group_size < 32 || group_size % 32 != 0 || K % group_size != 0) return TLLM_ERR_BAD_GROUP;

@@ -186,6 +186,10 @@ hipError_t split_exchange_memory(hipStream_t s, size_t floats, bool fixed, float
 hipError_t gemm_mfma_reserve(const Problem &p, hipStream_t s);
 void gemm_mfma_release_all();  // frees every split-K workspace (nothing may still be running on them)
 // The same launch with the split-K exchange in the library's fixed device array (no allocation, ever).
+// The prefill form of a SwiGLU pair in one launch (gate.y = silu(gate product) * up product); shapes: K a multiple of 128
+// from 384 on, 16-byte aligned masks and activations.
+bool gemm_swiglu_supports(const Problem &gate, const Problem &up);
+hipError_t launch_gemm_swiglu(const Problem &gate, const Problem &up, hipStream_t s);
 bool gemm_mfma_static_fits(const Problem &p);
 hipError_t launch_gemm_mfma_static(const Problem &p, hipStream_t s);
 

@@ -514,12 +514,20 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_mfma_kernel(
 constexpr int kNsBN = 256;
 constexpr int kNsPitch = 2 * kNsBN + 16;  // bytes per activation row of the output tile in LDS
 
-template <int MF, int NF>
+// kPair (NF = 2 only): the prefill form of a SwiGLU pair (reference src/transformer.cpp:264-286 at n_tokens > 1: gate GEMM,
+// up GEMM, silu_mul_forward). A wave's two weight fragments are the SAME 32 rows of the gate matrix (B arrays) and of the
+// up matrix (U arrays), so every activation fragment read from LDS feeds one MFMA of each, the activation tile is
+// fetched once for both matrices, and the two accumulators that meet in the epilogue sit in the same lane: the tile
+// (128 rows of each matrix x 128 activation rows) is stored once, as fp16(silu(fp16 gate) * fp16 up). No K split.
+template <int MF, int NF, bool kPair = false>
 __global__ __launch_bounds__(512 / NF) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_ns_kernel(
     const uint16_t *__restrict__ A, const uint32_t *__restrict__ nzB, const uint32_t *__restrict__ sgB,
     const uint16_t *__restrict__ scB, uint16_t *__restrict__ C, int M, int N, int K, int full_tiles, int splits,
-    int n_fastest, float *__restrict__ partial, unsigned *__restrict__ arrivals) {
+    int n_fastest, float *__restrict__ partial, unsigned *__restrict__ arrivals, const uint32_t *__restrict__ nzU = nullptr,
+    const uint32_t *__restrict__ sgU = nullptr, const uint16_t *__restrict__ scU = nullptr) {
+    static_assert(!kPair || NF == 2, "a pair is the two fragments of a wave");
     constexpr int BM = 32 * MF;
+    constexpr int kTileN = kPair ? kNsBN / 2 : kNsBN;  // weight rows (of each matrix) per workgroup
     constexpr int kWaves = 8 / NF, kNsThreads = 64 * kWaves;
     constexpr int kChunk = 4 * MF * 1024;    // bytes of one chunk: four steps of MF fragments
     constexpr int kDma = MF * 4 / kWaves;    // 1 KB pieces per wave and chunk
@@ -536,7 +544,7 @@ __global__ __launch_bounds__(512 / NF) __attribute__((amdgpu_waves_per_eu(2, 2))
 
     // ---- which tile, which part of K. Workgroup ids go round the XCDs: XCD x takes the x-th eighth of the whole tiles
     // first and the x-th eighth of the parts of split tiles afterwards.
-    const int m_tiles = (M + BM - 1) / BM, n_tiles = (N + kNsBN - 1) / kNsBN;
+    const int m_tiles = (M + BM - 1) / BM, n_tiles = (N + kTileN - 1) / kTileN;
     const int tiles = m_tiles * n_tiles, parts = (tiles - full_tiles) * splits;
     const int full_per = (full_tiles + 7) / 8, part_per = (parts + 7) / 8;
     const int xcd = (int)blockIdx.x & 7, slot_in_xcd = (int)blockIdx.x >> 3;
@@ -553,7 +561,7 @@ __global__ __launch_bounds__(512 / NF) __attribute__((amdgpu_waves_per_eu(2, 2))
     const bool is_split = tile >= full_tiles && splits > 1;
     // consecutive tiles (one XCD's share) walk the activation tiles of one weight tile first, or the weight tiles of one
     // activation tile first: whichever lets an XCD's L2 fetch fewer bytes for its share (the launcher decides)
-    const int n0 = (n_fastest ? tile % n_tiles : tile / m_tiles) * kNsBN;
+    const int n0 = (n_fastest ? tile % n_tiles : tile / m_tiles) * kTileN;
     const int m0 = (n_fastest ? tile / n_tiles : tile % m_tiles) * BM;
     // K is a multiple of 128: a last block of 128 columns runs as a whole block whose upper mask words are zero
     // (its activation chunks past the row re-read the last chunk: they meet zero weights)
@@ -567,10 +575,11 @@ __global__ __launch_bounds__(512 / NF) __attribute__((amdgpu_waves_per_eu(2, 2))
     GB *nz_g[NF], *sg_g[NF], *sc_g[NF];
 #pragma unroll
     for (int f = 0; f < NF; f++) {
-        const int row = min(n0 + 32 * (NF * wave + f) + li, N - 1);
-        nz_g[f] = (GB *)nzB + ((size_t)row * words + 4 * lq) * 4;
-        sg_g[f] = (GB *)sgB + ((size_t)row * words + 4 * lq) * 4;
-        sc_g[f] = (GB *)scB + (size_t)row * groups * 2;  // two scales per block: one aligned dword (groups is even)
+        const int row = min(n0 + (kPair ? 32 * wave : 32 * (NF * wave + f)) + li, N - 1);
+        const bool up = kPair && f == 1;
+        nz_g[f] = (GB *)(up ? nzU : nzB) + ((size_t)row * words + 4 * lq) * 4;
+        sg_g[f] = (GB *)(up ? sgU : sgB) + ((size_t)row * words + 4 * lq) * 4;
+        sc_g[f] = (GB *)(up ? scU : scB) + (size_t)row * groups * 2;  // two scales per block: one aligned dword (groups is even)
     }
 
     // activation pieces this wave copies per chunk: piece p = wave * kDma + i covers fragment j = p / 4, rows
@@ -831,7 +840,49 @@ __global__ __launch_bounds__(512 / NF) __attribute__((amdgpu_waves_per_eu(2, 2))
     // m0 + 32 j + li: stored as they are these are 8-byte pieces in 32 different lines per instruction. The tile goes
     // through LDS instead (the ring is free now) and leaves as whole 512-byte rows, two rows per instruction.
     const bool wide_store = (N & 7) == 0 && (reinterpret_cast<uintptr_t>(C) & 15) == 0;
-    if (wide_store) {
+    if constexpr (kPair) {
+        // silu(gate) * up on the fp16-rounded products, in fp32: what the two GEMMs and the element-wise kernel store
+        auto joined = [&](int j, int r) -> uint16_t {
+            const float g = h2f(f2h(acc[0][j][r] * 0.5f)), u = h2f(f2h(acc[1][j][r] * 0.5f));
+            return f2h(g / (1.0f + expf(-g)) * u);
+        };
+        if (wide_store) {
+            __syncthreads();  // every wave is done with the ring
+#pragma unroll
+            for (int j = 0; j < MF; j++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    uint16_t hv[4];
+#pragma unroll
+                    for (int v = 0; v < 4; v++) hv[v] = joined(j, 4 * g + v);
+                    *reinterpret_cast<uint2 *>(lds + (32 * j + li) * kNsPitch + (32 * wave + 8 * g + 4 * lq) * 2) =
+                        uint2{(uint32_t)hv[0] | ((uint32_t)hv[1] << 16), (uint32_t)hv[2] | ((uint32_t)hv[3] << 16)};
+                }
+            __syncthreads();
+            // rows of 128 outputs = 256 bytes: sixteen lanes per activation row, four rows per instruction
+            const int piece = lane & 15;
+            const int n = n0 + piece * 8;
+#pragma unroll
+            for (int r = 0; r < BM / (4 * kWaves); r++) {
+                const int ml = wave * (BM / kWaves) + 4 * r + (lane >> 4);
+                const int m = m0 + ml;
+                if (m < M && n < N) *reinterpret_cast<u4 *>(C + (size_t)m * N + n) = *reinterpret_cast<const u4 *>(lds + ml * kNsPitch + piece * 16);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < MF; j++) {
+                const int m = m0 + j * 32 + li;
+                if (m >= M) continue;
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int n = n0 + 32 * wave + 8 * g + 4 * lq;
+#pragma unroll
+                    for (int v = 0; v < 4; v++)
+                        if (n + v < N) C[(size_t)m * N + n + v] = joined(j, 4 * g + v);
+                }
+            }
+        }
+    } else if (wide_store) {
         __syncthreads();  // every wave is done with the ring
 #pragma unroll
         for (int fj = 0; fj < NF * MF; fj++)
@@ -1196,6 +1247,44 @@ void gemm_mfma_release_all() {
     }
     g_ws.clear();
     (void)hipSetDevice(dev);
+}
+
+// The prefill form of a SwiGLU pair: one launch of the row-split kernel in its pair form. `gate.y` receives
+// fp16(silu(fp16 gate product) * fp16 up product) [batch, rows]; `up` has the gate's shape and activations.
+bool gemm_swiglu_supports(const Problem &gate, const Problem &up) {
+    return gemm_mfma_supports(Problem{nullptr, nullptr, nullptr, nullptr, nullptr, gate.rows, gate.cols, std::max(gate.batch, 16), 0}, 128) &&
+           rowsplit_ok(gate) && rowsplit_ok(up);
+}
+hipError_t launch_gemm_swiglu(const Problem &gate, const Problem &up, hipStream_t s) {
+    constexpr int MF = 4, BM = 32 * MF, kTileN = kNsBN / 2;
+    static std::mutex attr_mutex;
+    static bool attr_set[64] = {};
+    int dev = 0;
+    if (hipError_t e = hipGetDevice(&dev)) return e;
+    const size_t ring = 4 * (size_t)(4 * MF * 1024), out_tile = (size_t)BM * kNsPitch;
+    const size_t lds = ring > out_tile ? ring : out_tile;
+    if (dev >= 0 && dev < 64) {
+        std::lock_guard<std::mutex> lock(attr_mutex);
+        if (!attr_set[dev]) {
+            if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_ns_kernel<MF, 2, true>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
+                return e;
+            attr_set[dev] = true;
+        }
+    }
+    const int m_tiles = (gate.batch + BM - 1) / BM, n_tiles = (gate.rows + kTileN - 1) / kTileN;
+    const int tiles = m_tiles * n_tiles;
+    const int wgs = 8 * ((tiles + 7) / 8);
+    // (the order of the tiles inside an XCD's share: as for the single matrix, with 128 rows of two matrices per tile)
+    const long per = (tiles + 7) / 8;
+    const double a_bytes = 128.0 * gate.cols * 2, w_bytes = 256.0 * gate.cols * 0.265625;
+    auto touched = [](long per_, long inner, long outer) { return std::pair<long, long>(std::min(inner, per_), std::min(outer, (per_ + inner - 1) / inner + 1)); };
+    const auto mf = touched(per, m_tiles, n_tiles);
+    const auto nf = touched(per, n_tiles, m_tiles);
+    const int n_fastest = nf.first <= 16 && 1.5 * (nf.second * a_bytes + nf.first * w_bytes) < mf.first * a_bytes + mf.second * w_bytes;
+    gemm_ns_kernel<MF, 2, true><<<wgs, 256, lds, s>>>(gate.x, gate.nz, gate.sg, gate.scales, gate.y, gate.batch, gate.rows, gate.cols,
+                                                      tiles, 1, n_fastest, nullptr, nullptr, up.nz, up.sg, up.scales);
+    return hipGetLastError();
 }
 
 bool gemm_mfma_static_fits(const Problem &p) { return workspace_floats(p, choose_config(p, kStaticSlotFloats)) <= kStaticSlotFloats; }

@@ -1378,6 +1378,82 @@ def test_gemm_every_output_against_dense_product(dev, oracle, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [
+    (512, 14336, 4096),   # the 8B FFN at a prefill of 512 tokens
+    (200, 1000, 2048),    # ragged in M and N (N not a multiple of 8: the narrow store path)
+    (130, 520, 2176),     # K = 128 (mod 256): a last half block; N a multiple of 8 only
+    (1, 256, 384),        # a single activation row, the smallest K
+    (2048, 2048, 2048),
+])
+def test_prefill_swiglu_pair_against_the_three_launches(dev, oracle, M, N, K):
+    """tllm_ternary_gemm_swiglu_f16: gate GEMM, up GEMM and SiLU * up in one launch (reference
+    src/transformer.cpp:264-286 at n_tokens > 1). Every output equals, bit for bit, what ternary_gemm on each matrix
+    (forced to the four-wave row-split kernel, whose order of additions the pair kernel shares) followed by silu_mul
+    stores; with the library's own choice of GEMM kernel for the separate launches the outputs agree to one rounding
+    of either projection (2.5e-3 of the larger of |result| and a floor); and the gate projection inside the pair is
+    within the bar of the fp32 product of the expanded weights (an up matrix of all-ones rows of weight makes the pair
+    return silu(gate) * sum(x), which is checked directly)."""
+    torch, tl = dev
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(7700 + M + N + K)
+    g_nz, g_sg, g_sc = _device_problem(torch, N, K, 0.42, 0.01, 0.03, gen)
+    u_nz, u_sg, u_sc = _device_problem(torch, N, K, 0.42, 0.01, 0.03, gen)
+    A = torch.randn((M, K), device="cuda", generator=gen).to(torch.float16)
+    f16 = dict(dtype=torch.float16, device="cuda")
+    out = torch.full((M, N), float("nan"), **f16)
+    tl.ternary_gemm_swiglu(A, g_nz, g_sg, g_sc, u_nz, u_sg, u_sc, out, M, N, K, 128)
+    torch.cuda.synchronize()
+    G, U = torch.zeros((M, N), **f16), torch.zeros((M, N), **f16)
+    with gemm_forced(rowsplit=2):
+        tl.ternary_gemm(A, g_nz, g_sg, g_sc, G, M, N, K, 128)
+        tl.ternary_gemm(A, u_nz, u_sg, u_sc, U, M, N, K, 128)
+    want = G.clone()
+    tl.silu_mul(want, U, want, M * N)
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16)), \
+        f"{int((out.view(torch.int16) != want.view(torch.int16)).sum())} of {M * N} outputs differ from the three launches"
+    # the library's own kernel choice for the separate launches: other order of additions, same results to a rounding
+    tl.ternary_gemm(A, g_nz, g_sg, g_sc, G, M, N, K, 128)
+    tl.ternary_gemm(A, u_nz, u_sg, u_sc, U, M, N, K, 128)
+    tl.silu_mul(G, U, G, M * N)
+    torch.cuda.synchronize()
+    floor = float(torch.sqrt(torch.mean(G.float() ** 2)).item()) / 64.0
+    rel = (out.float() - G.float()).abs() / torch.clamp(G.float().abs(), min=floor)
+    assert float(rel.max()) <= 2.5e-3, f"max_rel {float(rel.max()):.3e} against the three launches as the library runs them"
+    # against the fp32 product of the expanded weights
+    Wg, Wu = _dense_weights(torch, g_nz, g_sg, g_sc), _dense_weights(torch, u_nz, u_sg, u_sc)
+    g32 = (A.float() @ Wg.t()).half().float()
+    u32 = (A.float() @ Wu.t()).half().float()
+    ref = g32 / (1.0 + torch.exp(-g32)) * u32
+    del Wg, Wu
+    floor = float(torch.sqrt(torch.mean(ref * ref)).item()) / 64.0
+    rel = (out.float() - ref).abs() / torch.clamp(ref.abs(), min=floor)
+    assert float(rel.max()) <= 4e-3, f"max_rel {float(rel.max()):.3e} against silu(fp16(A gate^T)) * fp16(A up^T) in fp32"
+    # twice the same bits
+    again = torch.full((M, N), float("nan"), **f16)
+    tl.ternary_gemm_swiglu(A, g_nz, g_sg, g_sc, u_nz, u_sg, u_sc, again, M, N, K, 128)
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), again.view(torch.int16))
+
+
+def test_prefill_swiglu_pair_rejects_what_it_cannot_run(dev, oracle):
+    torch, tl = dev
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(7799)
+    nz, sg, sc = _device_problem(torch, 256, 128, 0.42, 0.01, 0.03, gen)
+    A = torch.randn((32, 128), device="cuda", generator=gen).to(torch.float16)
+    out = torch.zeros((32, 256), dtype=torch.float16, device="cuda")
+    with pytest.raises(tl.TllmError) as err:       # K = 128: neither a multiple of 256 nor at least 384
+        tl.ternary_gemm_swiglu(A, nz, sg, sc, nz, sg, sc, out, 32, 256, 128, 128)
+    assert err.value.code == -2
+    with pytest.raises(tl.TllmError) as err:       # group size other than 128
+        tl.ternary_gemm_swiglu(A, nz, sg, sc, nz, sg, sc, out, 32, 256, 128, 64)
+    assert err.value.code == -3
+    with pytest.raises(tl.TllmError) as err:       # the output over the activations
+        tl.ternary_gemm_swiglu(A, nz, sg, sc, nz, sg, sc, A, 32, 128, 128, 128)
+    assert err.value.code < 0
+
+
+@pytest.mark.parametrize("M,N,K", [
     (16, 4096, 14336),   # 64 blocks of 64 rows, four workgroups each
     (9, 1000, 4096),     # ragged last block, two parts of two steps
     (16, 192, 6144),     # three parts

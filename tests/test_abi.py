@@ -120,7 +120,7 @@ def test_cpp_dropin_call_shapes(tmp_path):
     subprocess.run(cmd, check=True, capture_output=True, text=True)
     out = subprocess.run([str(exe)], capture_output=True, text=True)
     assert out.returncode == 0, out.stdout + out.stderr
-    assert "rejected=10" in out.stdout
+    assert "rejected=12" in out.stdout
 
 
 def test_tuning_switches_round_trip():

@@ -607,7 +607,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
 #pragma unroll
                     for (int half = 0; half < 2; half++) {
                         u4 lo[kKeep / 2], hi[kKeep / 2];
-                        for (int spins = 0;; spins++) {
+                        for (int spins = wave_ok ? 0 : sc.spin_limit;; spins++) {  // (a wave that has given up asks once more, no longer)
                             uint32_t bad = 0;
                             const uint32_t *src[kKeep / 2];
                             bool live[kKeep / 2];

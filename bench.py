@@ -43,9 +43,9 @@ MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense FP16 matrix peak
 # profiled on: `sha256_16` is the first 16 hex digits of the sha256 of that csrc file then. The bench recomputes the
 # hash and marks the figure `traffic_stale` when the file has changed since.
 TRAFFIC = {
-    "headline": {"bytes": 1922930278, "file": "gemv_mfma.hip", "sha256_16": "4cdd2404f5a86d22",
+    "headline": {"bytes": 1922930278, "file": "gemv_mfma.hip", "sha256_16": "a91bf3a0bdad1f50",
                  "source": "rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this workload (profiles/gemv_mfma_wide__llama8b_sweep_b1.md), not read in this run"},
-    4: {"bytes": 2251384729, "file": "gemv_mfma.hip", "sha256_16": "4cdd2404f5a86d22",
+    4: {"bytes": 2251384729, "file": "gemv_mfma.hip", "sha256_16": "a91bf3a0bdad1f50",
         "source": "rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this workload (profiles/gemv_batch__llama8b_sweep_b4_b16.md), not read in this run"},
     16: {"bytes": 2085173453, "file": "gemv_batch.hip", "sha256_16": "8f870ce9ea664d7b",
          "source": "rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this workload (profiles/gemv_batch__llama8b_sweep_b4_b16.md), not read in this run"},

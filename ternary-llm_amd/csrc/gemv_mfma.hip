@@ -336,9 +336,9 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
     const int n_stages = kExtras && sc.n_stages > 0 ? sc.n_stages : 1;
     const bool staged = kExtras && sc.n_stages > 0;
     const bool exchange = staged && sc.exchange != 0;
-    int epoch = 0;
-    if (exchange) epoch = sc.epochs[blockIdx.x];
-    const uint32_t tag_hi = (uint32_t)((epoch + 1) & 0xFFFF) << 16;
+    uint32_t epoch = 0;  // (launches of this slot so far; counted modulo 2^32, used modulo 2^16)
+    if (exchange) epoch = (uint32_t)sc.epochs[blockIdx.x];
+    const uint32_t tag_hi = ((epoch + 1u) & 0xFFFFu) << 16;
     bool gave_up = false;  // a bounded wait of this workgroup expired (the same value in every thread)
     for (int stage = 0; stage < n_stages; stage++) {
     bool from_record = false;  // the first task of the stage takes its problem and unit numbers from the record
@@ -1258,7 +1258,7 @@ __global__ __launch_bounds__(kThreads, kExtras ? 2 : G::kWgPerCu) void gemv_mfma
         cur = -1;
     }
     }  // stages
-    if (exchange && tid == 0) sc.epochs[blockIdx.x] = epoch + 1;
+    if (exchange && tid == 0) sc.epochs[blockIdx.x] = (int)(epoch + 1u);
     if (sc.pool_count != 0 && tid == 0) {
         const int left = __hip_atomic_fetch_add(sc.counters + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (left == (int)gridDim.x - 1) {  // every other workgroup has made its last request

@@ -440,6 +440,47 @@ def ffn_front_rows(torch, tl, timer, seed, m_list, p_zero, calls, warm):
     return rows
 
 
+def qkv_prefill_rows(torch, tl, timer, seed, m_list, p_zero, calls, warm):
+    """The q, k and v projections of a prefill step on the 8B shapes (reference src/transformer.cpp:199-217 at
+    n_tokens > 1): three ternary_gemm calls as the reference issues them, and ONE launch whose tiles are dealt to the
+    workgroups together (tllm_ternary_gemm_group_f16). Flops of the three products; the outputs of the two ways are
+    compared (same arithmetic; where a tile is split along K the order of the fp32 additions may differ)."""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(seed + 45)
+    k, ns = 4096, (4096, 1024, 1024)
+    ws = []
+    for n in ns:
+        nz, sg = gen_masks(torch, n, k, p_zero, gen)
+        ws.append((nz, sg, (torch.rand((n, k // 128), device="cuda", generator=gen) * 0.02 + 0.01).to(torch.float16)))
+    rows = []
+    for m in m_list:
+        if m <= 16:
+            continue
+        a = torch.randn((m, k), device="cuda", generator=gen).to(torch.float16)
+        sep = [torch.zeros((m, n), dtype=torch.float16, device="cuda") for n in ns]
+        grp = [torch.zeros((m, n), dtype=torch.float16, device="cuda") for n in ns]
+
+        def three():
+            for n, w, o in zip(ns, ws, sep):
+                tl.ternary_gemm(a, *w, o, m, n, k, 128)
+
+        t3 = timer.run(three, calls, warm)
+        t1 = timer.run(lambda: tl.ternary_gemm_group(a, ws, grp, m, k), calls, warm)
+        rel = 0.0
+        for x, y in zip(sep, grp):
+            floor = float(torch.sqrt(torch.mean(x.float() ** 2)).item()) / 64.0
+            rel = max(rel, float(((y.float() - x.float()).abs() / torch.clamp(x.float().abs(), min=floor)).max().item()))
+        flops = 2.0 * m * sum(ns) * k
+        for name, t, kern in (("three launches", t3, " + ".join(tl.gemm_kernel(m, n, k) for n in ns)),
+                              ("one launch", t1, "tllm::gemm_ns_kernel<4, 1, group>")):
+            tf = flops / (t["mean_ms"] * 1e-3) / 1e12
+            rows.append({"config": f"cfg4: prefill q/k/v M={m}, W 4096+1024+1024 x {k}: {name}", "M": m, "N": sum(ns), "K": k, **stats_us(t),
+                         "tflops": round(tf, 1), "bound": "mfma", "frac_mfma_peak": round(tf / MFMA_F16_PEAK_TFLOPS, 4),
+                         "kernel": kern, "max_rel_one_launch_vs_three": rel})
+        del a, sep, grp
+    return rows
+
+
 def single_call_rows(torch, tl, timer, problems, model, layers):
     """The reference's call pattern on the headline weights: one operator call per matrix
     (src/transformer.cpp:102-118), all calls of a sweep captured once into a HIP graph and replayed, so the
@@ -859,6 +900,7 @@ def main():
             g = gemm_rows(torch, tl, orc, timer, args.seed, gemm_m, 0.42, args.gemm_calls, args.gemm_warm)
             cfgs += g
             cfgs += ffn_front_rows(torch, tl, timer, args.seed, [m for m in gemm_m if m in (512, 2048)], 0.42, args.gemm_calls, args.gemm_warm)
+            cfgs += qkv_prefill_rows(torch, tl, timer, args.seed, [m for m in gemm_m if m in (128, 512, 2048)], 0.42, args.gemm_calls, args.gemm_warm)
             m512 = [c for c in g if c["M"] == 512]
             if m512:
                 agg = sum(2.0 * c["M"] * c["N"] * c["K"] for c in m512) / sum(c["us"] for c in m512) / 1e6

@@ -109,6 +109,18 @@ inline void ternary_gemm_swiglu(const half *A, const uint32_t *nz_gate, const ui
                                         K, group_size, stream));
 }
 
+// The q, k and v projections of a prefill step (or any `count` <= TLLM_MAX_GEMM_GROUP matrices on the same activations)
+// as one launch; no counterpart in include/kernels.cuh: there it is one ternary_gemm per matrix
+// (src/transformer.cpp:199-217). C[i] = A B[i]^T, the pointer arrays live in host memory.
+inline void ternary_gemm_group(const half *A, const uint32_t *const *nz_B, const uint32_t *const *sign_B,
+                               const half *const *scales_B, half *const *C, const int *N, int count, int M, int K,
+                               int group_size, hipStream_t stream = 0) {
+    report("ternary_gemm_group",
+           tllm_ternary_gemm_group_f16(reinterpret_cast<const uint16_t *>(A), nz_B, sign_B,
+                                       reinterpret_cast<const uint16_t *const *>(scales_B),
+                                       reinterpret_cast<uint16_t *const *>(C), N, count, M, K, group_size, stream));
+}
+
 // Reference include/kernels.cuh:37-40.
 inline void ternary_gemm(const half *A, const uint32_t *nz_B, const uint32_t *sign_B,
                          const half *scales_B, half *C, int M, int N, int K, int group_size,

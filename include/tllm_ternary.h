@@ -132,6 +132,23 @@ int tllm_ternary_gemm_f16(const uint16_t *A, const uint32_t *nz_B, const uint32_
                           int group_size, tllm_stream_t stream);
 
 /*
+ * Up to TLLM_MAX_GEMM_GROUP weight matrices on the SAME activations in one launch: C[i][m, n] = fp16(A[m, :] . row n of
+ * matrix i), what `count` calls of tllm_ternary_gemm_f16 store (reference src/transformer.cpp:199-217 at n_tokens > 1:
+ * ternary_linear on q_proj, k_proj and v_proj with the same hidden_buf_). The tiles of all matrices are dealt to the
+ * workgroups together, so three small matrices fill the chip where each alone leaves most of it idle. nz, sign,
+ * scales, C and N are HOST arrays of `count` entries (device pointers / row counts); every matrix is [N[i], K] in the
+ * packed layout, every output [M, N[i]], no two outputs overlapping. Same arithmetic as tllm_ternary_gemm_f16 in its
+ * row-split kernel (fp32 accumulation; tiles that do not fill the last round over the CUs are split along K through
+ * the stream's workspace, like there: tllm_gemm_workspace_reserve(M, 256 * sum over i of ceil(N[i] / 256), K, ...)
+ * reserves it; under graph capture without it the tiles run whole). group_size 128; K a multiple of 256, or of 128 from
+ * 384 on; A and the mask planes 16-byte aligned (else TLLM_ERR_BAD_SHAPE / TLLM_ERR_BAD_GROUP: issue the calls one by one).
+ */
+enum { TLLM_MAX_GEMM_GROUP = 4 };
+int tllm_ternary_gemm_group_f16(const uint16_t *A, const uint32_t *const *nz, const uint32_t *const *sign,
+                                const uint16_t *const *scales, uint16_t *const *C, const int *N, int count, int M, int K,
+                                int group_size, tllm_stream_t stream);
+
+/*
  * The FFN front half of a prefill step in ONE launch: C[m, n] = fp16( silu(g) * u ) with g = fp16(A[m, :] . gate row n),
  * u = fp16(A[m, :] . up row n), i.e. what tllm_ternary_gemm_f16 on the gate matrix, tllm_ternary_gemm_f16 on the up
  * matrix and tllm_silu_mul_f16 store (reference src/transformer.cpp:264-286 at n_tokens > 1: ternary_linear(gate),

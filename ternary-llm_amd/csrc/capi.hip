@@ -117,6 +117,23 @@ int tllm_ternary_gemm_swiglu_f16(const uint16_t *A, const uint32_t *nz_gate, con
     return (int)tllm::launch_gemm_swiglu(gate, up, (hipStream_t)stream);
 }
 
+int tllm_ternary_gemm_group_f16(const uint16_t *A, const uint32_t *const *nz, const uint32_t *const *sign,
+                                const uint16_t *const *scales, uint16_t *const *C, const int *N, int count, int M, int K,
+                                int group_size, tllm_stream_t stream) {
+    if (!nz || !sign || !scales || !C || !N) return TLLM_ERR_NULL_POINTER;
+    if (count < 1 || count > TLLM_MAX_GEMM_GROUP || M < 1) return TLLM_ERR_BAD_SHAPE;
+    Problem ps[TLLM_MAX_GEMM_GROUP];
+    for (int i = 0; i < count; i++) {
+        ps[i] = Problem{nz[i], sign[i], scales[i], A, C[i], N[i], K, M, 0};
+        if (int e = tllm::check_linear(ps[i], group_size)) return e;
+        for (int j = 0; j < i; j++)
+            if (tllm::overlaps(C[i], (size_t)M * N[i] * 2, C[j], (size_t)M * N[j] * 2)) return TLLM_ERR_ALIAS;
+    }
+    if (group_size != 128) return TLLM_ERR_BAD_GROUP;
+    if (!tllm::gemm_group_supports(ps, count)) return TLLM_ERR_BAD_SHAPE;
+    return (int)tllm::launch_gemm_group(ps, count, (hipStream_t)stream);
+}
+
 int tllm_gemm_workspace_reserve(int M, int N, int K, int group_size, tllm_stream_t stream) {
     if (M < 1 || N < 1 || K < 1 || K % 32 != 0) return TLLM_ERR_BAD_SHAPE;
     if (group_size < 32 || group_size % 32 != 0 || K % group_size != 0) return TLLM_ERR_BAD_GROUP;

@@ -186,6 +186,10 @@ hipError_t split_exchange_memory(hipStream_t s, size_t floats, bool fixed, float
 hipError_t gemm_mfma_reserve(const Problem &p, hipStream_t s);
 void gemm_mfma_release_all();  // frees every split-K workspace (nothing may still be running on them)
 // The same launch with the split-K exchange in the library's fixed device array (no allocation, ever).
+// Up to four weight matrices on the same activations in one launch of the prefill GEMM (same x, batch and cols; K a
+// multiple of 256 or of 128 from 384 on; 16-byte aligned masks and activations).
+bool gemm_group_supports(const Problem *ps, int count);
+hipError_t launch_gemm_group(const Problem *ps, int count, hipStream_t s);
 // The prefill form of a SwiGLU pair in one launch (gate.y = silu(gate product) * up product); shapes: K a multiple of 128
 // from 384 on, 16-byte aligned masks and activations.
 bool gemm_swiglu_supports(const Problem &gate, const Problem &up);

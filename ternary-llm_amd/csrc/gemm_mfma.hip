@@ -519,13 +519,34 @@ constexpr int kNsPitch = 2 * kNsBN + 16;  // bytes per activation row of the out
 // up matrix (U arrays), so every activation fragment read from LDS feeds one MFMA of each, the activation tile is
 // fetched once for both matrices, and the two accumulators that meet in the epilogue sit in the same lane: the tile
 // (128 rows of each matrix x 128 activation rows) is stored once, as fp16(silu(fp16 gate) * fp16 up). No K split.
-template <int MF, int NF, bool kPair = false>
+// kGroup: up to four weight matrices that share the activations in one launch (the q, k and v projections of a prefill
+// step, reference src/transformer.cpp:199-217 at n_tokens > 1: three ternary_gemm calls on the same input). The tiles of
+// the matrices are numbered one after the other (matrix g owns tiles prefix[g] .. prefix[g + 1] - 1) and dealt to the
+// workgroups, whole or split along K, exactly as the tiles of one matrix are: three small matrices fill the chip
+// together where each alone leaves most of it idle. Every output is what the single call computes when its tiles are
+// split the same way.
+struct GemmGroup {
+    int count;
+    int prefix[5];
+    int N[4];
+    const uint32_t *nz[4];
+    const uint32_t *sg[4];
+    const uint16_t *sc[4];
+    uint16_t *C[4];
+};
+template <int MF, int NF, bool kPair = false, bool kGroup = false>
 __global__ __launch_bounds__(512 / NF) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_ns_kernel(
-    const uint16_t *__restrict__ A, const uint32_t *__restrict__ nzB, const uint32_t *__restrict__ sgB,
-    const uint16_t *__restrict__ scB, uint16_t *__restrict__ C, int M, int N, int K, int full_tiles, int splits,
+    const uint16_t *__restrict__ A, const uint32_t *__restrict__ nzB_, const uint32_t *__restrict__ sgB_,
+    const uint16_t *__restrict__ scB_, uint16_t *__restrict__ C_, int M, int N_, int K, int full_tiles, int splits,
     int n_fastest, float *__restrict__ partial, unsigned *__restrict__ arrivals, const uint32_t *__restrict__ nzU = nullptr,
-    const uint32_t *__restrict__ sgU = nullptr, const uint16_t *__restrict__ scU = nullptr) {
+    const uint32_t *__restrict__ sgU = nullptr, const uint16_t *__restrict__ scU = nullptr, GemmGroup grp = GemmGroup{}) {
     static_assert(!kPair || NF == 2, "a pair is the two fragments of a wave");
+    static_assert(!(kPair && kGroup), "one or the other");
+    const uint32_t *__restrict__ nzB = nzB_;
+    const uint32_t *__restrict__ sgB = sgB_;
+    const uint16_t *__restrict__ scB = scB_;
+    uint16_t *__restrict__ C = C_;
+    int N = N_;
     constexpr int BM = 32 * MF;
     constexpr int kTileN = kPair ? kNsBN / 2 : kNsBN;  // weight rows (of each matrix) per workgroup
     constexpr int kWaves = 8 / NF, kNsThreads = 64 * kWaves;
@@ -544,8 +565,9 @@ __global__ __launch_bounds__(512 / NF) __attribute__((amdgpu_waves_per_eu(2, 2))
 
     // ---- which tile, which part of K. Workgroup ids go round the XCDs: XCD x takes the x-th eighth of the whole tiles
     // first and the x-th eighth of the parts of split tiles afterwards.
-    const int m_tiles = (M + BM - 1) / BM, n_tiles = (N + kTileN - 1) / kTileN;
-    const int tiles = m_tiles * n_tiles, parts = (tiles - full_tiles) * splits;
+    const int m_tiles = (M + BM - 1) / BM;
+    int n_tiles = (N + kTileN - 1) / kTileN;
+    const int tiles = kGroup ? grp.prefix[grp.count] : m_tiles * n_tiles, parts = (tiles - full_tiles) * splits;
     const int full_per = (full_tiles + 7) / 8, part_per = (parts + 7) / 8;
     const int xcd = (int)blockIdx.x & 7, slot_in_xcd = (int)blockIdx.x >> 3;
     int tile, split = 0;
@@ -561,8 +583,21 @@ __global__ __launch_bounds__(512 / NF) __attribute__((amdgpu_waves_per_eu(2, 2))
     const bool is_split = tile >= full_tiles && splits > 1;
     // consecutive tiles (one XCD's share) walk the activation tiles of one weight tile first, or the weight tiles of one
     // activation tile first: whichever lets an XCD's L2 fetch fewer bytes for its share (the launcher decides)
-    const int n0 = (n_fastest ? tile % n_tiles : tile / m_tiles) * kTileN;
-    const int m0 = (n_fastest ? tile / n_tiles : tile % m_tiles) * BM;
+    int local = tile;  // the tile's number inside its matrix
+    if constexpr (kGroup) {
+        int g = 0;
+#pragma unroll
+        for (int k = 1; k < 4; k++) g += k < grp.count && tile >= grp.prefix[k];
+        local = tile - grp.prefix[g];
+        nzB = grp.nz[g];
+        sgB = grp.sg[g];
+        scB = grp.sc[g];
+        C = grp.C[g];
+        N = grp.N[g];
+        n_tiles = (N + kTileN - 1) / kTileN;
+    }
+    const int n0 = (n_fastest ? local % n_tiles : local / m_tiles) * kTileN;
+    const int m0 = (n_fastest ? local / n_tiles : local % m_tiles) * BM;
     // K is a multiple of 128: a last block of 128 columns runs as a whole block whose upper mask words are zero
     // (its activation chunks past the row re-read the last chunk: they meet zero weights)
     const int words = K / 32, groups = K / 128, blocks = (K + 255) / 256;
@@ -1102,6 +1137,48 @@ bool gemm_mfma_supports(const Problem &p, int group) {
 }
 
 namespace {
+// The row-split kernel's configuration for `tiles` tiles of 256 weight rows x 128 activation rows (of one matrix, or of
+// several that share the activations) over `blocks` blocks of 256 columns.
+GemmConfig rowsplit_config(int tiles, int blocks, int n_cu, size_t limit_floats, int forced_rs) {
+    const float block_us = 3.3f, fixed_us = 9.0f;
+    GemmConfig rs{0, 1, 0.f};
+    rs.rowsplit = true;
+    rs.full_tiles = tiles;
+    rs.us = (float)((tiles + n_cu - 1) / n_cu) * (float)blocks * block_us + fixed_us;
+    const int rem = tiles % n_cu;
+    if (rem) {
+        int splits = n_cu / rem;
+        if (splits > 8) splits = 8;
+        if (splits > blocks / 2) splits = blocks / 2;
+        while (splits > 1 && (size_t)rem * splits * 128 * kNsBN > limit_floats) splits--;
+        if (splits > 1) {
+            const float exchange = 6.0f + 1.5f * (float)splits;
+            // (a launch that leaves CUs idle runs its blocks and its exchange faster: down to 3/4 of the time)
+            const float parts = (float)rem * (float)splits;
+            const float thin = tiles < n_cu ? 0.75f + 0.25f * std::min(1.0f, parts / (float)n_cu) : 1.0f;
+            const float us = (float)(tiles / n_cu) * (float)blocks * block_us +
+                             thin * ((float)((blocks + splits - 1) / splits) * block_us + exchange + fixed_us);
+            if (us < rs.us) {
+                rs.splits = splits;
+                rs.full_tiles = tiles - rem;
+                rs.us = us;
+            }
+        }
+    }
+    // Two workgroups of four waves per CU: a workgroup alone on its CU takes 3.7 us per block, two together 5.3 us
+    // each; pays when there are more tiles than CUs. (No K split in this form.) TLLM_GEMM_ROWSPLIT=2 forces it.
+    if (tiles > n_cu || forced_rs == 2) {
+        const int slots = 2 * n_cu, last = tiles % slots;
+        GemmConfig two = rs;
+        two.frags = 2;
+        two.splits = 1;
+        two.full_tiles = tiles;
+        two.us = (float)(tiles / slots) * (float)blocks * 5.3f + (last > n_cu ? 5.3f : last > 0 ? 3.7f : 0.f) * (float)blocks + fixed_us;
+        if (forced_rs == 2 || (forced_rs != 1 && two.us < rs.us)) rs = two;
+    }
+    return rs;
+}
+
 // One workgroup occupies a CU (LDS). Taller tiles do more per stage, shorter tiles fill the chip
 // when there are few of them, and when even those leave CUs idle K is split across workgroups.
 // Estimate: (rounds of workgroups over the CUs) x (stages per workgroup) x (time of one stage,
@@ -1137,44 +1214,7 @@ GemmConfig choose_config(const Problem &p, size_t limit_floats) {
     const bool rs_ok = rowsplit_ok(p), four_ok = scales_dword_aligned(p);
     // (a shape whose scales the four-wave kernel cannot fetch runs the row-split kernel whatever its size)
     if ((forced_rs != 0 || !four_ok) && rs_ok && (forced_rs >= 1 || p.batch >= 96 || !four_ok)) {
-        const int blocks = (p.cols + 255) / 256;
-        const int tiles = ((p.batch + 127) / 128) * ((p.rows + kNsBN - 1) / kNsBN);
-        const float block_us = 3.3f, fixed_us = 9.0f;
-        GemmConfig rs{0, 1, 0.f};
-        rs.rowsplit = true;
-        rs.full_tiles = tiles;
-        rs.us = (float)((tiles + n_cu - 1) / n_cu) * (float)blocks * block_us + fixed_us;
-        const int rem = tiles % n_cu;
-        if (rem) {
-            int splits = n_cu / rem;
-            if (splits > 8) splits = 8;
-            if (splits > blocks / 2) splits = blocks / 2;
-            while (splits > 1 && (size_t)rem * splits * 128 * kNsBN > limit_floats) splits--;
-            if (splits > 1) {
-                const float exchange = 6.0f + 1.5f * (float)splits;
-                // (a launch that leaves CUs idle runs its blocks and its exchange faster: down to 3/4 of the time)
-                const float parts = (float)rem * (float)splits;
-                const float thin = tiles < n_cu ? 0.75f + 0.25f * std::min(1.0f, parts / (float)n_cu) : 1.0f;
-                const float us = (float)(tiles / n_cu) * (float)blocks * block_us +
-                                 thin * ((float)((blocks + splits - 1) / splits) * block_us + exchange + fixed_us);
-                if (us < rs.us) {
-                    rs.splits = splits;
-                    rs.full_tiles = tiles - rem;
-                    rs.us = us;
-                }
-            }
-        }
-        // Two workgroups of four waves per CU: a workgroup alone on its CU takes 3.7 us per block, two together 5.3 us
-        // each; pays when there are more tiles than CUs. (No K split in this form.) TLLM_GEMM_ROWSPLIT=2 forces it.
-        if (tiles > n_cu || forced_rs == 2) {
-            const int slots = 2 * n_cu, last = tiles % slots;
-            GemmConfig two = rs;
-            two.frags = 2;
-            two.splits = 1;
-            two.full_tiles = tiles;
-            two.us = (float)(tiles / slots) * (float)blocks * 5.3f + (last > n_cu ? 5.3f : last > 0 ? 3.7f : 0.f) * (float)blocks + fixed_us;
-            if (forced_rs == 2 || (forced_rs != 1 && two.us < rs.us)) rs = two;
-        }
+        const GemmConfig rs = rowsplit_config(((p.batch + 127) / 128) * ((p.rows + kNsBN - 1) / kNsBN), (p.cols + 255) / 256, n_cu, limit_floats, forced_rs);
         if (forced_rs >= 1 || !four_ok || rs.us < best.us) best = rs;
     }
     return best;
@@ -1247,6 +1287,81 @@ void gemm_mfma_release_all() {
     }
     g_ws.clear();
     (void)hipSetDevice(dev);
+}
+
+// Several weight matrices on the same activations in one launch of the row-split kernel (its group form): the
+// problems share x, batch and cols; each stores its own [batch, rows] output. `fixed`: the exchange of split tiles uses
+// the library's fixed device array (the entry point that never allocates is not offered for groups: false everywhere).
+bool gemm_group_supports(const Problem *ps, int count) {
+    if (count < 1 || count > 4) return false;
+    for (int i = 0; i < count; i++) {
+        const Problem shape{nullptr, nullptr, nullptr, nullptr, nullptr, ps[i].rows, ps[i].cols, std::max(ps[i].batch, 16), 0};
+        if (!gemm_mfma_supports(shape, 128) || !rowsplit_ok(ps[i])) return false;
+        if (ps[i].x != ps[0].x || ps[i].batch != ps[0].batch || ps[i].cols != ps[0].cols) return false;
+    }
+    return true;
+}
+namespace {
+template <int NF>
+hipError_t launch_group_form(const GemmGroup &grp, const Problem &first, const GemmConfig &c, float *partial, unsigned *arrivals,
+                             hipStream_t s) {
+    constexpr int MF = 4, BM = 32 * MF, kNsThreads = 512 / NF;
+    static std::mutex attr_mutex;
+    static bool attr_set[64] = {};
+    int dev = 0;
+    if (hipError_t e = hipGetDevice(&dev)) return e;
+    const size_t ring = 4 * (size_t)(4 * MF * 1024), out_tile = (size_t)BM * kNsPitch;
+    const size_t lds = ring > out_tile ? ring : out_tile;
+    if (dev >= 0 && dev < 64) {
+        std::lock_guard<std::mutex> lock(attr_mutex);
+        if (!attr_set[dev]) {
+            if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_ns_kernel<MF, NF, false, true>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
+                return e;
+            attr_set[dev] = true;
+        }
+    }
+    const int tiles = grp.prefix[grp.count];
+    const int parts = (tiles - c.full_tiles) * c.splits;
+    const int wgs = 8 * ((c.full_tiles + 7) / 8 + (parts + 7) / 8);
+    // (consecutive tiles of a matrix walk its activation tiles first: the weight tile stays, the few activation tiles
+    // of a prefill step are shared by everybody anyway)
+    gemm_ns_kernel<MF, NF, false, true><<<wgs, kNsThreads, lds, s>>>(first.x, nullptr, nullptr, nullptr, nullptr, first.batch, 0,
+                                                                      first.cols, c.full_tiles, c.splits, 0, partial, arrivals,
+                                                                      nullptr, nullptr, nullptr, grp);
+    return hipGetLastError();
+}
+}  // namespace
+hipError_t launch_gemm_group(const Problem *ps, int count, hipStream_t s) {
+    constexpr int BM = 128;
+    GemmGroup grp{};
+    grp.count = count;
+    const int m_tiles = (ps[0].batch + BM - 1) / BM;
+    for (int i = 0; i < count; i++) {
+        grp.prefix[i + 1] = grp.prefix[i] + m_tiles * ((ps[i].rows + kNsBN - 1) / kNsBN);
+        grp.N[i] = ps[i].rows;
+        grp.nz[i] = ps[i].nz;
+        grp.sg[i] = ps[i].sg;
+        grp.sc[i] = ps[i].scales;
+        grp.C[i] = ps[i].y;
+    }
+    for (int i = count; i < 4; i++) grp.prefix[i + 1] = grp.prefix[count];
+    const int tiles = grp.prefix[count], blocks = (ps[0].cols + 255) / 256;
+    const int forced = tuning().gemm_rowsplit.load(std::memory_order_relaxed);
+    GemmConfig c = rowsplit_config(tiles, blocks, current_device_cus(), kStaticSlotFloats, forced > 0 ? forced : -1);
+    float *workspace = nullptr;
+    unsigned *arrivals = nullptr;
+    if (c.splits > 1) {
+        const size_t need = (size_t)(tiles - c.full_tiles) * c.splits * 128 * kNsBN;
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipError_t e = hipStreamIsCapturing(s, &cap)) return e;
+        if (hipError_t e = split_workspace(s, need, cap == hipStreamCaptureStatusNone, &workspace, &arrivals)) return e;
+        if (!workspace) {  // under capture without a reserved workspace: whole tiles only
+            c.splits = 1;
+            c.full_tiles = tiles;
+        }
+    }
+    return c.frags == 2 ? launch_group_form<2>(grp, ps[0], c, workspace, arrivals, s) : launch_group_form<1>(grp, ps[0], c, workspace, arrivals, s);
 }
 
 // The prefill form of a SwiGLU pair: one launch of the row-split kernel in its pair form. `gate.y` receives

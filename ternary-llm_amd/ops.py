@@ -19,7 +19,7 @@ ABI_SYMBOLS = (
     "tllm_linear_plan_destroy", "tllm_rmsnorm_f16", "tllm_silu_mul_f16", "tllm_linear_plan_create_normed", "tllm_linear_plan_create_i8",
     "tllm_add_f16", "tllm_rope_f16", "tllm_embedding_lookup_f16", "tllm_copy_to_kv_cache_f16",
     "tllm_linear_plan_kernel", "tllm_gemm_workspace_reserve", "tllm_gemm_workspace_release",
-    "tllm_ternary_gemm_f16_static", "tllm_ternary_gemm_swiglu_f16", "tllm_read_stream", "tllm_ternary_gemm_kernel",
+    "tllm_ternary_gemm_f16_static", "tllm_ternary_gemm_swiglu_f16", "tllm_ternary_gemm_group_f16", "tllm_read_stream", "tllm_ternary_gemm_kernel",
     "tllm_debug_set_tuning", "tllm_debug_get_tuning", "tllm_ternary_linear_int8_f16",
     "tllm_linear_plan_create_staged", "tllm_linear_plan_status",
 )
@@ -82,6 +82,7 @@ def lib():
     L.tllm_ternary_gemm_f16.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, vp]
     L.tllm_ternary_gemm_f16_static.argtypes = [vp, vp, vp, vp, vp, i, i, i, i, vp]
     L.tllm_ternary_gemm_swiglu_f16.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i, i, i, i, vp]
+    L.tllm_ternary_gemm_group_f16.argtypes = [vp, vp, vp, vp, vp, vp, i, i, i, i, vp]
     L.tllm_gemm_workspace_reserve.argtypes = [i, i, i, i, vp]
     L.tllm_read_stream.argtypes = [vp, C.c_size_t, vp, vp]
     L.tllm_gemm_workspace_release.argtypes = []
@@ -189,6 +190,16 @@ def ternary_gemm_swiglu(A, nz_gate, sign_gate, scales_gate, nz_up, sign_up, scal
     (reference src/transformer.cpp:264-286 at n_tokens > 1)."""
     check(lib().tllm_ternary_gemm_swiglu_f16(_ptr(A), _ptr(nz_gate), _ptr(sign_gate), _ptr(scales_gate), _ptr(nz_up),
                                              _ptr(sign_up), _ptr(scales_up), _ptr(Cout), M, N, K, group_size, _stream(stream)))
+
+
+def ternary_gemm_group(A, weights, outputs, M, K, group_size=128, stream=None):
+    """Several ternary_gemm calls on the same activations in one launch (the q/k/v projections of a prefill step,
+    reference src/transformer.cpp:199-217 at n_tokens > 1). weights: [(nz, sign, scales), ...]; outputs: [C_i [M, N_i], ...]."""
+    n = len(weights)
+    arr = lambda vals: (C.c_void_p * n)(*[v.data_ptr() for v in vals])
+    rows = (C.c_int * n)(*[int(o.shape[-1]) for o in outputs])
+    check(lib().tllm_ternary_gemm_group_f16(_ptr(A), arr([w[0] for w in weights]), arr([w[1] for w in weights]),
+                                            arr([w[2] for w in weights]), arr(outputs), rows, n, M, K, group_size, _stream(stream)))
 
 
 def ternary_gemm_static(A, nz_B, sign_B, scales_B, Cout, M, N, K, group_size=128, stream=None):

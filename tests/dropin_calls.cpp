@@ -54,11 +54,17 @@ int main() {
     ternary::rope_forward(q_buf_, k_buf_, 1, n_tokens, n_heads, n_kv_heads, head_dim, start_pos, rope_theta);
     ternary::copy_to_kv_cache(k_buf_, v_buf_, k_cache, v_cache, 1, n_kv_heads, head_dim, n_tokens, start_pos, max_seq_len);
     ternary::add_forward(residual_buf_, hidden_buf_, residual_buf_, n_tokens * hidden);
-    // the two calls that replace member functions or groups of launches of the reference: ternary_linear_int8
+    // the calls that replace member functions or groups of launches of the reference: ternary_linear_int8
     // (src/transformer.cpp:126-143) and the FFN front half of a prefill step (:264-286)
     ternary::ternary_linear_int8(w.nonzero_masks, w.sign_masks, w.scales, input, output, w.out_features, w.in_features, gs);
     ternary::ternary_gemm_swiglu(hidden_buf_, w.nonzero_masks, w.sign_masks, w.scales, w.nonzero_masks, w.sign_masks, w.scales,
                                  gate_buf_, n_tokens, inter, hidden, gs);
+    // the q, k and v projections of a prefill step as one launch (:199-217)
+    const uint32_t *nzs[3] = {w.nonzero_masks, w.nonzero_masks, w.nonzero_masks}, *sgs[3] = {w.sign_masks, w.sign_masks, w.sign_masks};
+    const half *scs[3] = {w.scales, w.scales, w.scales};
+    half *outs[3] = {q_buf_, k_buf_, v_buf_};
+    const int ns[3] = {n_heads * head_dim, n_kv_heads * head_dim, n_kv_heads * head_dim};
+    ternary::ternary_gemm_group(hidden_buf_, nzs, sgs, scs, outs, ns, 3, n_tokens, hidden, gs);
     std::printf("rejected=%d\n", rejected);
-    return rejected == 12 ? 0 : 1;
+    return rejected == 13 ? 0 : 1;
 }

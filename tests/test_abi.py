@@ -103,6 +103,18 @@ def test_validation_codes():
     up_ = P(0x1000, 0x2000, 0x3000, 0x4000, 0, 64, 2048, 1, 0)
     assert normed([gate, up_], [0x7000, 0x8000]) == -6
     assert normed([gate, up_], [0x7000, None]) == -6
+    # grouped GEMMs: host arrays of device pointers, 1 to TLLM_MAX_GEMM_GROUP matrices, outputs apart, groups of 128
+    def grouped(nz=(0x10000,), sg=(0x20000,), sc=(0x30000,), out=(0x90000,), n=(256,), count=None, M=32, K=256, g=128, A=0x4000):
+        k = len(n)
+        ptrs = lambda v: (C.c_void_p * max(1, len(v)))(*v)
+        return L.tllm_ternary_gemm_group_f16(A, ptrs(nz), ptrs(sg), ptrs(sc), ptrs(out), (C.c_int * max(1, k))(*n),
+                                             k if count is None else count, M, K, g, None)
+    assert L.tllm_ternary_gemm_group_f16(0x4000, None, None, None, None, None, 1, 32, 256, 128, None) == -1
+    assert grouped(count=0) == -2 and grouped(count=5) == -2 and grouped(M=0) == -2
+    assert grouped(nz=(None,)) == -1 and grouped(A=None) == -1
+    assert grouped(g=64) == -3 and grouped(K=128) == -2                               # K = 128: not a shape of the row-split kernel
+    assert grouped(nz=(0x10000, 0x10000), sg=(0x20000, 0x20000), sc=(0x30000, 0x30000), out=(0x90000, 0x90100), n=(256, 256)) == -5
+    assert grouped(nz=(0x10004,)) == -7                                                 # mask planes in 16-byte pieces
     assert L.tllm_linear_plan_launch(None, None) == -6
     for code in range(-7, 1):
         assert L.tllm_error_string(code)
@@ -120,7 +132,7 @@ def test_cpp_dropin_call_shapes(tmp_path):
     subprocess.run(cmd, check=True, capture_output=True, text=True)
     out = subprocess.run([str(exe)], capture_output=True, text=True)
     assert out.returncode == 0, out.stdout + out.stderr
-    assert "rejected=12" in out.stdout
+    assert "rejected=13" in out.stdout
 
 
 def test_tuning_switches_round_trip():

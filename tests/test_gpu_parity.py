@@ -1435,6 +1435,57 @@ def test_prefill_swiglu_pair_against_the_three_launches(dev, oracle, M, N, K):
     assert torch.equal(out.view(torch.int16), again.view(torch.int16))
 
 
+@pytest.mark.parametrize("M,K,Ns", [
+    (512, 4096, (4096, 1024, 1024)),     # q, k, v of the 8B model at a prefill of 512 tokens
+    (200, 2176, (520, 1000)),            # ragged everywhere; K = 128 (mod 256); an N that is not a multiple of 8
+    (2048, 2048, (2048, 512, 512, 256)), # four matrices
+    (96, 8192, (1024,)),                 # a group of one
+])
+def test_gemm_group_every_output(dev, oracle, M, K, Ns):
+    """tllm_ternary_gemm_group_f16: several weight matrices on the same activations in one launch (the q/k/v
+    projections of a prefill step, reference src/transformer.cpp:199-217 at n_tokens > 1). Every output of every
+    matrix against the fp32 product of the expanded weights (sampled against the fp64 oracle); with the four-wave
+    form forced (no tile is split along K) the bits equal those of the single calls forced the same way; repeated
+    launches give the same bits."""
+    torch, tl = dev
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(7800 + M + K + sum(Ns))
+    A = torch.randn((M, K), device="cuda", generator=gen).to(torch.float16)
+    ws = [_device_problem(torch, n, K, 0.42, 0.01, 0.03, gen) for n in Ns]
+    f16 = dict(dtype=torch.float16, device="cuda")
+    outs = [torch.full((M, n), float("nan"), **f16) for n in Ns]
+    tl.ternary_gemm_group(A, ws, outs, M, K)
+    torch.cuda.synchronize()
+    first = [o.clone() for o in outs]
+    for i, (n, w) in enumerate(zip(Ns, ws)):
+        W = _dense_weights(torch, *w)
+        ref = A.float() @ W.t()
+        del W
+        _check_sampled(oracle, torch, A, *w, ref, 3, 24, M + n, f"dense fp32 product of matrix {i}")
+        tau = float(torch.sqrt(torch.mean(ref * ref)).item()) / 64.0
+        rel = (outs[i].float() - ref).abs() / torch.clamp(ref.abs(), min=tau)
+        bad = int((~(rel <= TOL)).sum().item())
+        assert bad == 0, f"matrix {i} ({M}x{n}x{K}): {bad} of {M * n} outputs beyond {TOL}, max_rel {float(rel.max()):.3e}"
+    for o in outs:
+        o.fill_(float("nan"))
+    tl.ternary_gemm_group(A, ws, outs, M, K)
+    torch.cuda.synchronize()
+    for a_, b_ in zip(outs, first):
+        assert torch.equal(a_.view(torch.int16), b_.view(torch.int16))
+    with gemm_forced(rowsplit=2):
+        tl.ternary_gemm_group(A, ws, outs, M, K)
+        compared = 0
+        for n, w, o in zip(Ns, ws, outs):
+            if "gemm_ns_kernel<4, 2>" not in tl.gemm_kernel(M, n, K):
+                continue  # (a shape that the library streams through the batched kernel whatever is forced)
+            compared += 1
+            single = torch.zeros((M, n), **f16)
+            tl.ternary_gemm(A, *w, single, M, n, K, 128)
+            torch.cuda.synchronize()
+            assert torch.equal(o.view(torch.int16), single.view(torch.int16)), f"matrix with {n} rows differs from its single call"
+        assert compared or M < 128
+
+
 def test_prefill_swiglu_pair_rejects_what_it_cannot_run(dev, oracle):
     torch, tl = dev
     gen = torch.Generator(device="cuda")

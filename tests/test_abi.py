@@ -147,3 +147,29 @@ def test_tuning_switches_round_trip():
         assert tl.get_tuning(name) == default
     with pytest.raises(tl.TllmError):
         tl.set_tuning("no_such_switch", 1)
+
+
+def test_kernel_choice_by_shape():
+    """Host logic of the dispatcher (reference src/transformer.cpp:112-116: one token -> ternary_gemv, more ->
+    ternary_gemm; here one entry point chooses among four kernels by shape, csrc/dispatch.hip). Asked through
+    tllm_ternary_gemm_kernel, which touches no GPU (without one the cost model assumes the MI355X's 256 CUs)."""
+    k = ops.gemm_kernel
+    assert "gemv_mfma_kernel" in k(1, 4096, 4096) and "gemv_mfma_kernel" in k(1, 4096, 14336)
+    for m in (2, 4, 16):
+        assert "gemv_batch_kernel" in k(m, 4096, 4096)
+    assert k(16, 4096, 14336) == "tllm::gemv_batch_kernel, K shared out"       # 64 blocks for 256 CUs: K is shared out
+    assert k(16, 14336, 4096) == "tllm::gemv_batch_kernel"
+    assert "gemm_ns_kernel<4, 1>" in k(512, 14336, 4096) and "gemm_ns_kernel<4, 1>" in k(512, 4096, 14336)
+    assert k(2048, 14336, 4096) == "tllm::gemm_ns_kernel<4, 2>"                 # more tiles than CUs: two workgroups per CU
+    assert "gemm_mfma_kernel" in k(100, 1000, 1536)                            # few rows: the four-wave kernel, K split
+    assert k(1, 64, 96, 32)                                                    # any group size runs somewhere
+    assert k(512, 4096, 4096, 64)
+    for bad in ((0, 4096, 4096, 128), (4, 4096, 100, 128), (4, 4096, 4096, 48), (4, 4096, 160, 128)):
+        assert k(*bad) == ""
+    # the forced forms of the tests answer to their switch and leave it as it was
+    before = ops.get_tuning("gemm_rowsplit")
+    with ops.tuning(gemm_rowsplit=0):
+        assert "gemm_mfma_kernel" in k(512, 14336, 4096)
+    with ops.tuning(gemm_rowsplit=2):
+        assert k(512, 14336, 4096) == "tllm::gemm_ns_kernel<4, 2>"
+    assert ops.get_tuning("gemm_rowsplit") == before

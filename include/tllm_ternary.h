@@ -141,7 +141,8 @@ int tllm_ternary_gemm_f16(const uint16_t *A, const uint32_t *nz_B, const uint32_
  * row-split kernel (fp32 accumulation; tiles that do not fill the last round over the CUs are split along K through
  * the stream's workspace, like there: tllm_gemm_workspace_reserve(M, 256 * sum over i of ceil(N[i] / 256), K, ...)
  * reserves it; under graph capture without it the tiles run whole). group_size 128; K a multiple of 256, or of 128 from
- * 384 on; A and the mask planes 16-byte aligned (else TLLM_ERR_BAD_SHAPE / TLLM_ERR_BAD_GROUP: issue the calls one by one).
+ * 384 on (another K: TLLM_ERR_BAD_SHAPE, another group size: TLLM_ERR_BAD_GROUP; issue the calls one by one then); count
+ * outside 1 .. TLLM_MAX_GEMM_GROUP: TLLM_ERR_BAD_SHAPE; outputs that overlap each other or A: TLLM_ERR_ALIAS.
  */
 enum { TLLM_MAX_GEMM_GROUP = 4 };
 int tllm_ternary_gemm_group_f16(const uint16_t *A, const uint32_t *const *nz, const uint32_t *const *sign,
